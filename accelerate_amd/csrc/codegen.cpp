@@ -1,0 +1,926 @@
+#include "codegen.hpp"
+
+#include <cmath>
+#include <cstdio>
+#include <cstdlib>
+#include <cstring>
+#include <set>
+
+namespace acchip {
+
+// ------------------------------------------------------------------------------------
+// values
+
+ValP vUnit() {
+  static ValP u = std::make_shared<Val>();
+  return u;
+}
+ValP vLeaf(ST st, const std::string& ex) {
+  auto v = std::make_shared<Val>();
+  v->k = Val::Leaf;
+  v->st = st;
+  v->ex = ex;
+  return v;
+}
+ValP vPair(ValP a, ValP b) {
+  auto v = std::make_shared<Val>();
+  v->k = Val::Pair;
+  v->a = std::move(a);
+  v->b = std::move(b);
+  return v;
+}
+TypeP valType(const ValP& v) {
+  if (v->k == Val::Unit) return tUnit();
+  if (v->k == Val::Leaf) return tScalar(v->st);
+  return tPair(valType(v->a), valType(v->b));
+}
+void valLeaves(const ValP& v, std::vector<ValP>& out) {
+  if (v->k == Val::Leaf) out.push_back(v);
+  else if (v->k == Val::Pair) {
+    valLeaves(v->a, out);
+    valLeaves(v->b, out);
+  }
+}
+static std::vector<ValP> leavesOf(const ValP& v) {
+  std::vector<ValP> o;
+  valLeaves(v, o);
+  return o;
+}
+
+static const ValP& leaf1(const ValP& v, const char* what) {
+  if (v->k != Val::Leaf) throw Error(std::string("expected a scalar operand for ") + what);
+  return v;
+}
+
+// ------------------------------------------------------------------------------------
+// literals
+
+std::string literalText(ST st, const std::string& tok) {
+  char buf[96];
+  if (stIsFloat(st)) {
+    double d;
+    if (tok == "nan") d = NAN;
+    else if (tok == "inf") d = INFINITY;
+    else if (tok == "-inf") d = -INFINITY;
+    else {
+      char* end = nullptr;
+      d = std::strtod(tok.c_str(), &end);
+      if (!end || *end) throw Error("malformed floating literal '" + tok + "'");
+    }
+    const char* T = stName(st);
+    if (std::isnan(d)) { snprintf(buf, sizeof buf, "((%s)__builtin_nanf(\"\"))", T); return buf; }
+    if (std::isinf(d)) { snprintf(buf, sizeof buf, "((%s)%s__builtin_inff())", T, d < 0 ? "-" : ""); return buf; }
+    if (st == ST::F64) snprintf(buf, sizeof buf, "(%a)", d);
+    else if (st == ST::F32) snprintf(buf, sizeof buf, "(%af)", (double)(float)d);
+    else snprintf(buf, sizeof buf, "((f16)%af)", (double)(float)d);
+    return buf;
+  }
+  // integers: accept anything that fits the signed or unsigned range, wrap to the type
+  errno = 0;
+  char* end = nullptr;
+  unsigned long long u;
+  if (!tok.empty() && tok[0] == '-') u = (unsigned long long)std::strtoll(tok.c_str(), &end, 0);
+  else u = std::strtoull(tok.c_str(), &end, 0);
+  if (!end || *end || tok.empty()) throw Error("malformed integer literal '" + tok + "'");
+  int bits = stBits(st);
+  if (bits < 64) u &= ((1ULL << bits) - 1);
+  snprintf(buf, sizeof buf, "((%s)0x%llxULL)", stName(st), u);
+  return buf;
+}
+
+// ------------------------------------------------------------------------------------
+// array slots
+
+const ArraySlot& Codegen::slotForVar(int idx) {
+  if (idx < 0 || idx >= (int)aenv_.size()) throw Error("array variable index out of range");
+  std::string name = "a" + std::to_string(idx);
+  auto it = used_.find(name);
+  if (it == used_.end()) {
+    ArraySlot s;
+    s.name = name;
+    s.r = aenv_[idx];
+    s.index = idx;
+    it = used_.emplace(name, s).first;
+  }
+  return it->second;
+}
+
+std::string Codegen::addTemp(const ArrayR& r) {
+  ArraySlot s;
+  s.name = "t" + std::to_string(temps_.size());
+  s.r = r;
+  s.temp = true;
+  s.index = (int)temps_.size();
+  temps_.push_back(s);
+  return s.name;
+}
+
+const ArraySlot& Codegen::slotByName(const std::string& name) {
+  auto it = used_.find(name);
+  if (it != used_.end()) return it->second;
+  if (name[0] == 't') {
+    int k = std::atoi(name.c_str() + 1);
+    if (k < 0 || k >= (int)temps_.size()) throw Error("unknown temporary slot " + name);
+    return used_.emplace(name, temps_[k]).first->second;
+  }
+  if (name == "out") throw Error("output extent slot not declared");
+  return slotForVar(std::atoi(name.c_str() + 1));
+}
+
+// ------------------------------------------------------------------------------------
+// small emit helpers
+
+ValP Codegen::bindLeaf(ST st, const std::string& ex, Emit& em) {
+  std::string n = fresh();
+  em.line(std::string("const ") + stName(st) + " " + n + " = " + ex + ";");
+  return vLeaf(st, n);
+}
+
+ValP Codegen::declareVars(const TypeP& t, Emit& em) {
+  if (t->k == Type::Unit) return vUnit();
+  if (t->k == Type::Scalar) {
+    std::string n = fresh();
+    em.line(std::string(stName(t->st)) + " " + n + ";");
+    return vLeaf(t->st, n);
+  }
+  ValP a = declareVars(t->a, em);
+  return vPair(a, declareVars(t->b, em));
+}
+
+void Codegen::assign(const ValP& dst, const ValP& src, Emit& em) {
+  auto d = leavesOf(dst), s = leavesOf(src);
+  if (d.size() != s.size()) throw Error("internal: assignment between values of different shape");
+  for (size_t i = 0; i < d.size(); ++i) {
+    if (d[i]->st != s[i]->st) throw Error("type mismatch between branches of a conditional or loop");
+    em.line(d[i]->ex + " = " + s[i]->ex + ";");
+  }
+}
+
+ValP Codegen::copyToVars(const ValP& v, Emit& em) {
+  if (v->k == Val::Unit) return v;
+  if (v->k == Val::Leaf) {
+    std::string n = fresh();
+    em.line(std::string(stName(v->st)) + " " + n + " = " + v->ex + ";");
+    return vLeaf(v->st, n);
+  }
+  ValP a = copyToVars(v->a, em);
+  return vPair(a, copyToVars(v->b, em));
+}
+
+static void pushLhs(const Sx& lhs, const ValP& v, Codegen::Env& env) {
+  if (lhs.is("single")) {
+    if (v->k != Val::Leaf) throw Error("left-hand side binds a scalar but the value is a tuple: " + lhs.str());
+    env.push_back(v);
+  } else if (lhs.is("wild")) {
+  } else if (lhs.is("pair")) {
+    if (v->k != Val::Pair) throw Error("left-hand side is a pair but the value is not: " + lhs.str());
+    pushLhs(lhs.at(1), v->a, env);
+    pushLhs(lhs.at(2), v->b, env);
+  } else {
+    throw Error("malformed left-hand side " + lhs.str());
+  }
+}
+
+ValP Codegen::shapeOf(const ArraySlot& s) {
+  ValP v = vUnit();
+  for (int d = 0; d < s.r.rank; ++d) v = vPair(v, vLeaf(ST::I64, "env." + s.name + "_d" + std::to_string(d)));
+  return v;
+}
+
+static void shapeDims(const ValP& sh, std::vector<std::string>& out) {
+  if (sh->k == Val::Unit) return;
+  if (sh->k != Val::Pair || sh->b->k != Val::Leaf) throw Error("expected a shape value");
+  shapeDims(sh->a, out);
+  out.push_back(sh->b->ex);
+}
+
+std::string Codegen::toIndex(const ValP& sh, const ValP& ix, Emit& em) {
+  std::vector<std::string> d, i;
+  shapeDims(sh, d);
+  shapeDims(ix, i);
+  if (d.size() != i.size()) throw Error("toIndex: rank mismatch between shape and index");
+  if (d.empty()) return "((i64)0)";
+  std::string e = i[0];
+  for (size_t k = 1; k < d.size(); ++k) e = "(" + e + " * " + d[k] + " + " + i[k] + ")";
+  return bindLeaf(ST::I64, e, em)->ex;
+}
+
+ValP Codegen::fromIndex(int rank, const ValP& sh, const std::string& lin, Emit& em) {
+  std::vector<std::string> d;
+  shapeDims(sh, d);
+  if ((int)d.size() != rank) throw Error("fromIndex: rank mismatch");
+  if (rank == 0) return vUnit();
+  std::vector<std::string> ix(rank);
+  std::string cur = lin;
+  for (int k = rank - 1; k >= 1; --k) {
+    ix[k] = bindLeaf(ST::I64, "acc_rem(" + cur + ", " + d[k] + ")", em)->ex;
+    cur = bindLeaf(ST::I64, "acc_quot(" + cur + ", " + d[k] + ")", em)->ex;
+  }
+  ix[0] = cur;  // the outermost component needs no remainder (Shape.hs:110-120)
+  ValP v = vUnit();
+  for (int k = 0; k < rank; ++k) v = vPair(v, vLeaf(ST::I64, ix[k]));
+  return v;
+}
+
+ValP Codegen::readArray(const ArraySlot& s, const std::string& lin, Emit& em) {
+  int leaf = 0;
+  struct R {
+    static ValP go(Codegen& cg, const TypeP& t, const ArraySlot& s, const std::string& lin, int& leaf, Emit& em) {
+      if (t->k == Type::Unit) return vUnit();
+      if (t->k == Type::Scalar)
+        return cg.bindLeaf(t->st, "env." + s.name + "_" + std::to_string(leaf++) + "[" + lin + "]", em);
+      ValP a = go(cg, t->a, s, lin, leaf, em);
+      return vPair(a, go(cg, t->b, s, lin, leaf, em));
+    }
+  };
+  return R::go(*this, s.r.elt, s, lin, leaf, em);
+}
+
+ValP Codegen::operandLinear(const Operand& o, const std::string& lin, Emit& em) {
+  if (o.delayed) return applyFun(o.linearD, {vLeaf(ST::I64, lin)}, {}, em);
+  return readArray(slotByName(o.slot), lin, em);
+}
+
+ValP Codegen::operandIndex(const Operand& o, const ValP& ix, Emit& em) {
+  if (o.delayed) return applyFun(o.indexD, {ix}, {}, em);
+  const ArraySlot& s = slotByName(o.slot);
+  return readArray(s, toIndex(shapeOf(s), ix, em), em);
+}
+
+ValP Codegen::operandShape(const Operand& o, Emit& em) {
+  if (o.delayed) return exp(o.extent, {}, em);
+  return shapeOf(slotByName(o.slot));
+}
+
+// ------------------------------------------------------------------------------------
+// primitives (semantics: Interpreter.hs:1154-1416)
+
+static int primTypeParams(const std::string& n) {
+  if (n == "land" || n == "lor" || n == "lnot") return 0;
+  if (n == "truncate" || n == "round" || n == "floor" || n == "ceiling" || n == "fromintegral" || n == "tofloating")
+    return 2;
+  return 1;
+}
+
+ValP Codegen::prim(const std::string& name, const std::vector<ST>& tys, const ValP& arg, Emit& em) {
+  auto T = [](ST t) { return std::string(stName(t)); };
+  auto bin = [&](std::string& a, std::string& b) {
+    if (arg->k != Val::Pair) throw Error("primitive '" + name + "' expects a pair argument");
+    a = leaf1(arg->a, name.c_str())->ex;
+    b = leaf1(arg->b, name.c_str())->ex;
+  };
+  auto un = [&]() { return leaf1(arg, name.c_str())->ex; };
+  auto fcall1 = [&](ST t, const char* fn, const std::string& a) {
+    if (t == ST::F64) return std::string(fn) + "(" + a + ")";
+    if (t == ST::F32) return std::string(fn) + "f(" + a + ")";
+    return "(f16)" + std::string(fn) + "f((f32)" + a + ")";
+  };
+  auto fcall2 = [&](ST t, const char* fn, const std::string& a, const std::string& b) {
+    if (t == ST::F64) return std::string(fn) + "(" + a + ", " + b + ")";
+    if (t == ST::F32) return std::string(fn) + "f(" + a + ", " + b + ")";
+    return "(f16)" + std::string(fn) + "f((f32)" + a + ", (f32)" + b + ")";
+  };
+  auto arith = [&](ST t, const char* op, const std::string& a, const std::string& b) {
+    if (stIsInt(t)) return "(" + T(t) + ")((" + stWide(t) + ")" + a + " " + op + " (" + stWide(t) + ")" + b + ")";
+    if (t == ST::F16) return "(f16)((f32)" + a + " " + op + " (f32)" + b + ")";
+    return a + " " + op + " " + b;
+  };
+  auto needInt = [&](ST t) {
+    if (!stIsInt(t)) throw Error("primitive '" + name + "' needs an integral type");
+  };
+  auto needFloat = [&](ST t) {
+    if (!stIsFloat(t)) throw Error("primitive '" + name + "' needs a floating type");
+  };
+  const ST t = tys.empty() ? ST::U8 : tys[0];
+  const std::string bits = std::to_string(stBits(t));
+  const std::string U = T(stUnsigned(t));
+  std::string a, b;
+
+  if (name == "add" || name == "sub" || name == "mul") {
+    bin(a, b);
+    return bindLeaf(t, arith(t, name == "add" ? "+" : name == "sub" ? "-" : "*", a, b), em);
+  }
+  if (name == "neg") {
+    a = un();
+    if (stIsInt(t)) return bindLeaf(t, "(" + T(t) + ")((" + stWide(t) + ")0 - (" + stWide(t) + ")" + a + ")", em);
+    return bindLeaf(t, "-" + a, em);
+  }
+  if (name == "abs") {
+    a = un();
+    if (stIsInt(t)) {
+      if (!stIsSigned(t)) return arg;
+      return bindLeaf(t, "(" + a + " < 0) ? (" + T(t) + ")((" + stWide(t) + ")0 - (" + stWide(t) + ")" + a + ") : " + a, em);
+    }
+    return bindLeaf(t, fcall1(t, "fabs", a), em);
+  }
+  if (name == "sig") {
+    a = un();
+    if (stIsInt(t)) return bindLeaf(t, "(" + T(t) + ")((" + a + " > 0) - (" + a + " < 0))", em);
+    // GHC.Float: signum x | x > 0 = 1 | x < 0 = -1 | otherwise = x
+    return bindLeaf(t, "(" + a + " > 0) ? (" + T(t) + ")1 : ((" + a + " < 0) ? (" + T(t) + ")-1 : " + a + ")", em);
+  }
+  if (name == "quot" || name == "rem" || name == "idiv" || name == "mod" || name == "quotrem" || name == "divmod") {
+    needInt(t);
+    bin(a, b);
+    ValP q = bindLeaf(t, "(" + T(t) + ")(" + a + " / " + b + ")", em);
+    ValP r = bindLeaf(t, "(" + T(t) + ")(" + a + " % " + b + ")", em);
+    if (name == "quot") return q;
+    if (name == "rem") return r;
+    if (name == "quotrem") return vPair(q, r);
+    if (!stIsSigned(t)) return name == "idiv" ? q : name == "mod" ? r : vPair(q, r);
+    // floor division (Haskell div / mod): adjust when the remainder's sign differs from the divisor's
+    ValP adj = bindLeaf(ST::U8, "(u8)((" + r->ex + " != 0) & ((" + r->ex + " < 0) != (" + b + " < 0)))", em);
+    ValP d = bindLeaf(t, adj->ex + " ? (" + T(t) + ")(" + q->ex + " - 1) : " + q->ex, em);
+    ValP m = bindLeaf(t, adj->ex + " ? (" + T(t) + ")(" + r->ex + " + " + b + ") : " + r->ex, em);
+    if (name == "idiv") return d;
+    if (name == "mod") return m;
+    return vPair(d, m);
+  }
+  if (name == "band" || name == "bor" || name == "bxor") {
+    needInt(t);
+    bin(a, b);
+    const char* op = name == "band" ? "&" : name == "bor" ? "|" : "^";
+    return bindLeaf(t, "(" + T(t) + ")(" + a + " " + op + " " + b + ")", em);
+  }
+  if (name == "bnot") {
+    needInt(t);
+    return bindLeaf(t, "(" + T(t) + ")(~" + un() + ")", em);
+  }
+  if (name == "shl") {
+    needInt(t);
+    bin(a, b);
+    return bindLeaf(t, "((u64)" + b + " >= " + bits + ") ? (" + T(t) + ")0 : (" + T(t) + ")((" + stWide(t) + ")" + a + " << " + b + ")", em);
+  }
+  if (name == "shr") {
+    needInt(t);
+    bin(a, b);
+    std::string over = stIsSigned(t) ? "(" + T(t) + ")(" + a + " < 0 ? -1 : 0)" : "(" + T(t) + ")0";
+    return bindLeaf(t, "((u64)" + b + " >= " + bits + ") ? " + over + " : (" + T(t) + ")(" + a + " >> " + b + ")", em);
+  }
+  if (name == "rotl" || name == "rotr") {
+    needInt(t);
+    bin(a, b);
+    // rotate by (n mod bits), Data.Bits semantics; rotr n = rotl (-n)
+    std::string n = name == "rotl" ? b : "(-" + b + ")";
+    ValP k = bindLeaf(ST::I32, "(i32)(((" + n + " % " + bits + ") + " + bits + ") % " + bits + ")", em);
+    ValP u = bindLeaf(stUnsigned(t), "(" + U + ")" + a, em);
+    std::string W = stWide(t);
+    return bindLeaf(t, "(" + k->ex + " == 0) ? " + a + " : (" + T(t) + ")(((" + W + ")" + u->ex + " << " + k->ex + ") | ((" + W + ")" + u->ex + " >> (" + bits + " - " + k->ex + ")))", em);
+  }
+  if (name == "popcount") {
+    needInt(t);
+    return bindLeaf(ST::I64, "(i64)__builtin_popcountll((u64)(" + U + ")" + un() + ")", em);
+  }
+  if (name == "clz") {
+    needInt(t);
+    a = un();
+    return bindLeaf(ST::I64, "((" + U + ")" + a + " == 0) ? (i64)" + bits + " : (i64)(__builtin_clzll((u64)(" + U + ")" + a + ") - (64 - " + bits + "))", em);
+  }
+  if (name == "ctz") {
+    needInt(t);
+    a = un();
+    return bindLeaf(ST::I64, "((" + U + ")" + a + " == 0) ? (i64)" + bits + " : (i64)__builtin_ctzll((u64)(" + U + ")" + a + ")", em);
+  }
+  if (name == "fdiv") {
+    needFloat(t);
+    bin(a, b);
+    return bindLeaf(t, arith(t, "/", a, b), em);
+  }
+  if (name == "recip") {
+    needFloat(t);
+    return bindLeaf(t, arith(t, "/", "(" + T(t) + ")1", un()), em);
+  }
+  static const char* unaryMath[] = {"sin", "cos", "tan", "asin", "acos", "atan", "sinh", "cosh", "tanh",
+                                    "asinh", "acosh", "atanh", "exp", "sqrt", "log"};
+  for (const char* m : unaryMath)
+    if (name == m) {
+      needFloat(t);
+      return bindLeaf(t, fcall1(t, m, un()), em);
+    }
+  if (name == "fpow") {
+    needFloat(t);
+    bin(a, b);
+    return bindLeaf(t, fcall2(t, "pow", a, b), em);
+  }
+  if (name == "atan2") {
+    needFloat(t);
+    bin(a, b);
+    return bindLeaf(t, fcall2(t, "atan2", a, b), em);
+  }
+  if (name == "logbase") {  // logBase x y = log y / log x
+    needFloat(t);
+    bin(a, b);
+    ValP ly = bindLeaf(t, fcall1(t, "log", b), em), lx = bindLeaf(t, fcall1(t, "log", a), em);
+    return bindLeaf(t, arith(t, "/", ly->ex, lx->ex), em);
+  }
+  if (name == "truncate" || name == "round" || name == "floor" || name == "ceiling") {
+    if (tys.size() != 2) throw Error("primitive '" + name + "' needs two type parameters");
+    needFloat(tys[0]);
+    if (!stIsInt(tys[1])) throw Error("primitive '" + name + "' converts to an integral type");
+    const char* fn = name == "truncate" ? "trunc" : name == "round" ? "rint" : name == "floor" ? "floor" : "ceil";
+    std::string x = tys[0] == ST::F64 ? std::string(fn) + "(" + un() + ")" : std::string(fn) + "f((f32)" + un() + ")";
+    // go through i64 so that narrow targets wrap like fromIntegral would
+    return bindLeaf(tys[1], "(" + T(tys[1]) + ")(i64)" + x, em);
+  }
+  if (name == "isnan" || name == "isinf") {
+    needFloat(t);
+    std::string x = t == ST::F16 ? "(f32)" + un() : un();
+    return bindLeaf(ST::U8, std::string("(u8)(") + (name == "isnan" ? "__builtin_isnan(" : "__builtin_isinf(") + x + ") != 0)", em);
+  }
+  static const struct { const char* n; const char* op; } cmps[] = {{"lt", "<"}, {"gt", ">"}, {"lte", "<="},
+                                                                   {"gte", ">="}, {"eq", "=="}, {"neq", "!="}};
+  for (auto& c : cmps)
+    if (name == c.n) {
+      bin(a, b);
+      return bindLeaf(ST::U8, "(u8)(" + a + " " + c.op + " " + b + ")", em);
+    }
+  if (name == "max") {  // Ord default: max x y = if x <= y then y else x
+    bin(a, b);
+    return bindLeaf(t, "(" + a + " <= " + b + ") ? " + b + " : " + a, em);
+  }
+  if (name == "min") {  // min x y = if x <= y then x else y
+    bin(a, b);
+    return bindLeaf(t, "(" + a + " <= " + b + ") ? " + a + " : " + b, em);
+  }
+  if (name == "land" || name == "lor") {
+    bin(a, b);
+    return bindLeaf(ST::U8, "(u8)((" + a + " != 0) " + (name == "land" ? "&" : "|") + " (" + b + " != 0))", em);
+  }
+  if (name == "lnot") return bindLeaf(ST::U8, "(u8)(" + un() + " == 0)", em);
+  if (name == "fromintegral" || name == "tofloating") {
+    if (tys.size() != 2) throw Error("primitive '" + name + "' needs two type parameters");
+    a = un();
+    ST to = tys[1];
+    if (to == ST::F16 && stIsInt(tys[0])) return bindLeaf(to, "(f16)(f32)" + a, em);  // Half goes through Float
+    return bindLeaf(to, "(" + T(to) + ")" + a, em);
+  }
+  throw Error("unknown primitive '" + name + "'");
+}
+
+// ------------------------------------------------------------------------------------
+// expressions
+
+static void sliceRestrict(const Sx& spec, size_t k, const ValP& slix, const ValP& sh, ValP& out) {
+  // IndexSlice (Interpreter.hs:944-953); spec lists all/fixed from the innermost dimension outwards
+  if (k == spec.size()) { out = vUnit(); return; }
+  if (slix->k != Val::Pair || sh->k != Val::Pair) throw Error("indexslice: slice index does not match the specification");
+  ValP rest;
+  sliceRestrict(spec, k + 1, slix->a, sh->a, rest);
+  out = spec.at(k).isAtom("all") ? vPair(rest, sh->b) : rest;
+}
+
+static void sliceExtend(const Sx& spec, size_t k, const ValP& slix, const ValP& sl, ValP& out) {
+  // IndexFull (Interpreter.hs:955-965)
+  if (k == spec.size()) { out = vUnit(); return; }
+  if (slix->k != Val::Pair) throw Error("indexfull: slice index does not match the specification");
+  ValP rest;
+  if (spec.at(k).isAtom("all")) {
+    if (sl->k != Val::Pair) throw Error("indexfull: slice shape does not match the specification");
+    sliceExtend(spec, k + 1, slix->a, sl->a, rest);
+    out = vPair(rest, sl->b);
+  } else {
+    sliceExtend(spec, k + 1, slix->a, sl, rest);
+    out = vPair(rest, slix->b);
+  }
+}
+
+ValP Codegen::applyFun(const Sx& f, const std::vector<ValP>& args, const Env& env, Emit& em) {
+  Env e2 = env;
+  const Sx* cur = &f;
+  for (const ValP& a : args) {
+    if (!cur->is("lam")) throw Error("function applied to too many arguments: " + f.str().substr(0, 120));
+    pushLhs(cur->at(1), a, e2);
+    cur = &cur->at(2);
+  }
+  if (cur->is("lam")) throw Error("function applied to too few arguments");
+  return exp(*cur, e2, em);
+}
+
+ValP Codegen::exp(const Sx& e, const Env& env, Emit& em) {
+  if (e.isAtom("nil")) return vUnit();
+  if (e.atom) throw Error("unexpected atom '" + e.s + "' in scalar expression");
+  const std::string& h = e.head();
+  if (h == "var") {
+    long long ix = e.at(1).asInt();
+    if (ix < 0 || ix >= (long long)env.size()) throw Error("scalar variable index out of range");
+    return env[env.size() - 1 - ix];
+  }
+  if (h == "let") {
+    ValP v = exp(e.at(2), env, em);
+    Env e2 = env;
+    pushLhs(e.at(1), v, e2);
+    return exp(e.at(3), e2, em);
+  }
+  if (h == "pair") {
+    ValP a = exp(e.at(1), env, em);
+    return vPair(a, exp(e.at(2), env, em));
+  }
+  if (h == "const") {
+    ST t = parseST(e.at(1));
+    return vLeaf(t, literalText(t, e.at(2).s));
+  }
+  if (h == "undef") {
+    ST t = parseST(e.at(1));
+    return vLeaf(t, literalText(t, "0"));
+  }
+  if (h == "minbound" || h == "maxbound") {
+    ST t = parseST(e.at(1));
+    if (!stIsInt(t)) throw Error(h + " needs an integral type");
+    int bits = stBits(t);
+    unsigned long long v;
+    if (h == "minbound") v = stIsSigned(t) ? (1ULL << (bits - 1)) : 0ULL;
+    else v = stIsSigned(t) ? ((1ULL << (bits - 1)) - 1) : (bits == 64 ? ~0ULL : ((1ULL << bits) - 1));
+    char buf[64];
+    snprintf(buf, sizeof buf, "((%s)0x%llxULL)", stName(t), v);
+    return vLeaf(t, buf);
+  }
+  if (h == "pi") {
+    ST t = parseST(e.at(1));
+    return vLeaf(t, literalText(t, "0x1.921fb54442d18p+1"));
+  }
+  if (h == "prim") {
+    std::string name = e.at(1).s;
+    int nt = primTypeParams(name);
+    std::vector<ST> tys;
+    for (int k = 0; k < nt; ++k) tys.push_back(parseST(e.at(2 + k)));
+    ValP arg = exp(e.at(2 + nt), env, em);
+    return prim(name, tys, arg, em);
+  }
+  if (h == "toindex") {
+    ValP sh = exp(e.at(2), env, em), ix = exp(e.at(3), env, em);
+    return vLeaf(ST::I64, toIndex(sh, ix, em));
+  }
+  if (h == "fromindex") {
+    ValP sh = exp(e.at(2), env, em), i = exp(e.at(3), env, em);
+    return fromIndex((int)e.at(1).asInt(), sh, leaf1(i, "fromindex")->ex, em);
+  }
+  if (h == "indexslice" || h == "indexfull") {
+    ValP slix = exp(e.at(2), env, em), sh = exp(e.at(3), env, em), out;
+    if (h == "indexslice") sliceRestrict(e.at(1), 0, slix, sh, out);
+    else sliceExtend(e.at(1), 0, slix, sh, out);
+    return out;
+  }
+  if (h == "cond") {
+    ValP c = exp(e.at(1), env, em);
+    Emit et, ee;
+    et.ind = ee.ind = em.ind + 2;
+    ValP tv = exp(e.at(2), env, et), ev = exp(e.at(3), env, ee);
+    if (!typeEq(valType(tv), valType(ev))) throw Error("branches of a conditional have different types");
+    const std::string cx = "(" + leaf1(c, "cond")->ex + " != 0)";
+    if (et.code.empty() && ee.code.empty()) {
+      auto tl = leavesOf(tv), el = leavesOf(ev);
+      std::vector<ValP> rl;
+      for (size_t i = 0; i < tl.size(); ++i)
+        rl.push_back(tl[i]->ex == el[i]->ex ? tl[i] : bindLeaf(tl[i]->st, cx + " ? " + tl[i]->ex + " : " + el[i]->ex, em));
+      size_t pos = 0;
+      struct B {
+        static ValP go(const ValP& shape, const std::vector<ValP>& rl, size_t& pos) {
+          if (shape->k == Val::Unit) return shape;
+          if (shape->k == Val::Leaf) return rl[pos++];
+          ValP a = go(shape->a, rl, pos);
+          return vPair(a, go(shape->b, rl, pos));
+        }
+      };
+      return B::go(tv, rl, pos);
+    }
+    // only the chosen branch may run (a branch can guard an out-of-bounds index)
+    ValP res = declareVars(valType(tv), em);
+    em.line("if " + cx + " {");
+    em.code += et.code;
+    em.ind += 2;
+    assign(res, tv, em);
+    em.ind -= 2;
+    em.line("} else {");
+    em.code += ee.code;
+    em.ind += 2;
+    assign(res, ev, em);
+    em.ind -= 2;
+    em.line("}");
+    return res;
+  }
+  if (h == "case") {
+    ValP tag = exp(e.at(1), env, em);
+    const Sx& alts = e.at(2);
+    std::vector<Emit> ems(alts.size() + 1);
+    std::vector<ValP> vals;
+    for (size_t k = 0; k < alts.size(); ++k) {
+      ems[k].ind = em.ind + 4;
+      vals.push_back(exp(alts.at(k).at(1), env, ems[k]));
+    }
+    bool hasDef = !e.at(3).isAtom("none");
+    if (hasDef) {
+      ems.back().ind = em.ind + 4;
+      vals.push_back(exp(e.at(3), env, ems.back()));
+    }
+    if (vals.empty()) throw Error("case without alternatives");
+    ValP res = declareVars(valType(vals[0]), em);
+    em.line("switch ((int)" + leaf1(tag, "case")->ex + ") {");
+    for (size_t k = 0; k < vals.size(); ++k) {
+      bool def = k == alts.size();
+      em.line(def ? "  default: {" : "  case " + std::to_string(alts.at(k).at(0).asInt()) + ": {");
+      em.code += ems[k].code;
+      em.ind += 4;
+      assign(res, vals[k], em);
+      em.ind -= 4;
+      em.line("  } break;");
+    }
+    em.line("}");
+    return res;
+  }
+  if (h == "while") {
+    ValP seed = exp(e.at(3), env, em);
+    ValP st = copyToVars(seed, em);
+    em.line("for (;;) {");
+    em.ind += 2;
+    ValP c = applyFun(e.at(1), {st}, env, em);
+    em.line("if (" + leaf1(c, "while")->ex + " == 0) break;");
+    ValP nv = applyFun(e.at(2), {st}, env, em);
+    ValP tmp = copyToVars(nv, em);  // the new state may mention the old one
+    assign(st, tmp, em);
+    em.ind -= 2;
+    em.line("}");
+    return st;
+  }
+  if (h == "index") {
+    const ArraySlot& s = slotForVar((int)e.at(1).asInt());
+    ValP ix = exp(e.at(2), env, em);
+    return readArray(s, toIndex(shapeOf(s), ix, em), em);
+  }
+  if (h == "linearindex") {
+    const ArraySlot& s = slotForVar((int)e.at(1).asInt());
+    ValP i = exp(e.at(2), env, em);
+    return readArray(s, leaf1(i, "linearindex")->ex, em);
+  }
+  if (h == "shape") return shapeOf(slotForVar((int)e.at(1).asInt()));
+  if (h == "shapesize") {
+    ValP sh = exp(e.at(2), env, em);
+    std::vector<std::string> d;
+    shapeDims(sh, d);
+    if (d.empty()) return vLeaf(ST::I64, "((i64)1)");
+    std::string neg, prod;
+    for (size_t k = 0; k < d.size(); ++k) {
+      neg += (k ? " || " : "") + ("(" + d[k] + " <= 0)");
+      prod += (k ? " * " : "") + d[k];
+    }
+    return bindLeaf(ST::I64, "(" + neg + ") ? (i64)0 : (i64)(" + prod + ")", em);
+  }
+  if (h == "coerce") {
+    ST t1 = parseST(e.at(1)), t2 = parseST(e.at(2));
+    if (stSize(t1) != stSize(t2)) throw Error("coerce between types of different width");
+    ValP v = exp(e.at(3), env, em);
+    return bindLeaf(t2, std::string("__builtin_bit_cast(") + stName(t2) + ", (" + stName(t1) + ")" + leaf1(v, "coerce")->ex + ")", em);
+  }
+  if (h == "foreign") {
+    ValP v = exp(e.at(2), env, em);
+    return applyFun(e.at(1), {v}, {}, em);  // the pure fallback, in an empty environment
+  }
+  throw Error("unknown scalar expression '" + h + "'");
+}
+
+TypeP Codegen::typeOfExp(const Sx& e) {
+  Emit scratch;
+  int save = next_;
+  auto usedSave = used_;
+  TypeP t = valType(exp(e, {}, scratch));
+  next_ = save;
+  used_ = usedSave;
+  return t;
+}
+
+// ------------------------------------------------------------------------------------
+// translation-unit assembly
+
+static std::string leafDecls(const std::vector<ST>& leaves, const char* prefix, bool pointer, bool constPtr) {
+  std::string s;
+  for (size_t k = 0; k < leaves.size(); ++k) {
+    s += "  ";
+    if (pointer && constPtr) s += "const ";
+    s += stName(leaves[k]);
+    if (pointer) s += "*";
+    s += " " + std::string(prefix) + std::to_string(k) + ";\n";
+  }
+  return s;
+}
+
+std::string Codegen::eltStruct(const TypeP& t, const std::string& name) {
+  return "struct " + name + " {\n" + leafDecls(typeLeaves(t), "c", false, false) + "};\n";
+}
+
+std::string Codegen::outStruct(const std::vector<ST>& leaves) {
+  return "struct Out {\n  i64 _pad;\n" + leafDecls(leaves, "o", true, false) + "};\n";
+}
+
+std::string Codegen::envStruct(std::vector<ArraySlot>& order) {
+  std::string s = "struct Env {\n  i64 _pad;\n";
+  order.clear();
+  for (auto& kv : used_) order.push_back(kv.second);
+  for (auto& a : order) {
+    auto lv = typeLeaves(a.r.elt);
+    for (size_t k = 0; k < lv.size(); ++k)
+      s += std::string("  const ") + stName(lv[k]) + "* __restrict__ " + a.name + "_" + std::to_string(k) + ";\n";
+    for (int d = 0; d < a.r.rank; ++d) s += "  i64 " + a.name + "_d" + std::to_string(d) + ";\n";
+  }
+  return s + "};\n";
+}
+
+ValP Codegen::eltVal(const TypeP& t, const std::string& var) {
+  int leaf = 0;
+  struct R {
+    static ValP go(const TypeP& t, const std::string& var, int& leaf) {
+      if (t->k == Type::Unit) return vUnit();
+      if (t->k == Type::Scalar) return vLeaf(t->st, var + ".c" + std::to_string(leaf++));
+      ValP a = go(t->a, var, leaf);
+      return vPair(a, go(t->b, var, leaf));
+    }
+  };
+  return R::go(t, var, leaf);
+}
+
+std::string Codegen::returnElt(const ValP& v, Emit& em) {
+  auto lv = leavesOf(v);
+  em.line("Elt r_;");
+  for (size_t k = 0; k < lv.size(); ++k) em.line("r_.c" + std::to_string(k) + " = " + lv[k]->ex + ";");
+  em.line("return r_;");
+  return em.code;
+}
+
+bool Codegen::isCommutative(const Sx& f, std::string* op, ST* st) {
+  // \x y -> prim OP T (x, y)   or   (y, x), for OP in a fixed set of commutative primitives
+  if (!f.is("lam") || !f.at(1).is("single")) return false;
+  const Sx& g = f.at(2);
+  if (!g.is("lam") || !g.at(1).is("single")) return false;
+  const Sx& b = g.at(2);
+  if (!b.is("prim") || b.size() != 4) return false;
+  static const char* ops[] = {"add", "mul", "min", "max", "band", "bor", "bxor"};
+  bool ok = false;
+  for (const char* o : ops) ok = ok || b.at(1).s == o;
+  if (!ok || !isST(b.at(2))) return false;
+  const Sx& arg = b.at(3);
+  if (!arg.is("pair") || !arg.at(1).is("var") || !arg.at(2).is("var")) return false;
+  long long i = arg.at(1).at(1).asInt(), j = arg.at(2).at(1).asInt();
+  if (!((i == 0 && j == 1) || (i == 1 && j == 0))) return false;
+  if (op) *op = b.at(1).s;
+  if (st) *st = parseST(b.at(2));
+  return true;
+}
+
+static int vecFor(const std::vector<ST>& leaves, const std::vector<ArraySlot>& arrays) {
+  int maxLeaf = 1, eltBytes = 0;
+  for (ST s : leaves) {
+    maxLeaf = std::max(maxLeaf, stSize(s));
+    eltBytes += stSize(s);
+  }
+  for (auto& a : arrays)
+    for (ST s : typeLeaves(a.r.elt)) maxLeaf = std::max(maxLeaf, stSize(s));
+  int v = 16 / maxLeaf;
+  while (v > 1 && v * eltBytes > 64) v >>= 1;
+  return std::max(1, std::min(v, 8));
+}
+
+KernelSource Codegen::finish(const std::string& specBody, const TypeP& elt, const std::vector<ST>& outLeaves,
+                             const std::string& skeleton, int vec) {
+  KernelSource ks;
+  std::string envS = envStruct(ks.arrays);
+  ks.outLeaves = outLeaves;
+  ks.vec = vec > 0 ? vec : vecFor(outLeaves, ks.arrays);
+  std::string s = deviceHeader("prelude.hpp");
+  s += "\n" + envS + eltStruct(elt, "Elt") + outStruct(outLeaves);
+  s += "struct Spec {\n  typedef ::Env Env;\n  typedef ::Elt Elt;\n  typedef ::Out Out;\n";
+  s += "  static constexpr int V = " + std::to_string(ks.vec) + ";\n";
+  s += specBody;
+  // Out <-> Elt when both have the same leaves
+  auto el = typeLeaves(elt);
+  if (el == outLeaves) {
+    s += "  ACC_DEV Elt load(const Out& o, i64 i) {\n    Elt r_;\n";
+    for (size_t k = 0; k < el.size(); ++k) s += "    r_.c" + std::to_string(k) + " = o.o" + std::to_string(k) + "[i];\n";
+    s += "    return r_;\n  }\n";
+    s += "  ACC_DEV void store(const Out& o, i64 i, const Elt& v) {\n";
+    for (size_t k = 0; k < el.size(); ++k) s += "    o.o" + std::to_string(k) + "[i] = v.c" + std::to_string(k) + ";\n";
+    s += "  }\n";
+  }
+  s += "};\n\n" + deviceHeader(skeleton);
+  ks.source = std::move(s);
+  return ks;
+}
+
+// ------------------------------------------------------------------------------------
+// skeleton instantiations
+
+static std::string fnHead(const char* ret, const char* name, const char* params) {
+  return std::string("  ACC_DEV ") + ret + " " + name + "(" + params + ") {\n";
+}
+
+KernelSource Codegen::fold(const Sx& f, const Sx* seed, const Operand& src) {
+  const TypeP elt = src.r.elt;
+  std::string body;
+  bool comm = isCommutative(f);
+  body += std::string("  static constexpr bool kCommutative = ") + (comm ? "true" : "false") + ";\n";
+  body += std::string("  static constexpr bool kSeeded = ") + (seed ? "true" : "false") + ";\n";
+  {
+    Emit em;
+    em.ind = 4;
+    ValP r = applyFun(f, {eltVal(elt, "x"), eltVal(elt, "y")}, {}, em);
+    if (!typeEq(valType(r), elt)) throw Error("fold: combination function does not return the element type");
+    body += fnHead("Elt", "combine", "const Env& env, const Elt& x, const Elt& y") + returnElt(r, em) + "  }\n";
+  }
+  {
+    Emit em;
+    em.ind = 4;
+    if (seed) {
+      ValP z = exp(*seed, {}, em);
+      if (!typeEq(valType(z), elt)) throw Error("fold: seed does not have the element type");
+      returnElt(z, em);
+    } else {
+      em.line("Elt r_{};");
+      em.line("return r_;");
+    }
+    body += fnHead("Elt", "seed", "const Env& env") + em.code + "  }\n";
+  }
+  {
+    Emit em;
+    em.ind = 4;
+    ValP v = operandLinear(src, "i", em);
+    if (!typeEq(valType(v), elt)) throw Error("fold: fused producer does not return the element type");
+    body += fnHead("Elt", "in_linear", "const Env& env, i64 i") + returnElt(v, em) + "  }\n";
+  }
+  KernelSource ks = finish(body, elt, typeLeaves(elt), "fold.hpp", 0);
+  ks.commutative = comm;
+  return ks;
+}
+
+KernelSource Codegen::map(const TypeP& outElt, const Sx* f, const Operand& src) {
+  Emit em;
+  em.ind = 4;
+  ValP v = operandLinear(src, "i", em);
+  ValP r = f ? applyFun(*f, {v}, {}, em) : v;
+  if (!typeEq(valType(r), outElt)) throw Error("map: function result does not match the declared element type");
+  std::string body = fnHead("Elt", "produce", "const Env& env, i64 i") + returnElt(r, em) + "  }\n";
+  return finish(body, outElt, typeLeaves(outElt), "map.hpp", 0);
+}
+
+static void declareOut(std::map<std::string, ArraySlot>& used, int rank) {
+  ArraySlot s;
+  s.name = "out";
+  s.r.rank = rank;
+  s.r.elt = tUnit();
+  s.index = -1;
+  used.emplace("out", s);
+}
+
+KernelSource Codegen::zipWith(const TypeP& outElt, const Sx& f, const Operand& a, const Operand& b, int rank) {
+  Emit em;
+  em.ind = 4;
+  ValP x, y;
+  if (rank <= 1) {
+    // rank <= 1: the linear index of the intersection is the linear index of both operands
+    x = operandLinear(a, "i", em);
+    y = operandLinear(b, "i", em);
+  } else {
+    declareOut(used_, rank);
+    ArraySlot o = used_.at("out");
+    ValP ix = fromIndex(rank, shapeOf(o), "i", em);
+    x = operandIndex(a, ix, em);
+    y = operandIndex(b, ix, em);
+  }
+  ValP r = applyFun(f, {x, y}, {}, em);
+  if (!typeEq(valType(r), outElt)) throw Error("zipWith: function result does not match the declared element type");
+  std::string body = fnHead("Elt", "produce", "const Env& env, i64 i") + returnElt(r, em) + "  }\n";
+  return finish(body, outElt, typeLeaves(outElt), "map.hpp", 0);
+}
+
+KernelSource Codegen::generate(const ArrayR& out, const Sx& f) {
+  Emit em;
+  em.ind = 4;
+  declareOut(used_, out.rank);
+  ArraySlot o = used_.at("out");
+  ValP ix = fromIndex(out.rank, shapeOf(o), "i", em);
+  ValP r = applyFun(f, {ix}, {}, em);
+  if (!typeEq(valType(r), out.elt)) throw Error("generate: function result does not match the declared element type");
+  std::string body = fnHead("Elt", "produce", "const Env& env, i64 i") + returnElt(r, em) + "  }\n";
+  return finish(body, out.elt, typeLeaves(out.elt), "map.hpp", 0);
+}
+
+KernelSource Codegen::backpermute(int outRank, const Sx& p, const Sx* f, const TypeP& outElt, const Operand& src) {
+  Emit em;
+  em.ind = 4;
+  declareOut(used_, outRank);
+  ArraySlot o = used_.at("out");
+  ValP ix = fromIndex(outRank, shapeOf(o), "i", em);
+  ValP sx = applyFun(p, {ix}, {}, em);
+  ValP v = operandIndex(src, sx, em);
+  ValP r = f ? applyFun(*f, {v}, {}, em) : v;
+  if (!typeEq(valType(r), outElt)) throw Error("backpermute: result does not match the declared element type");
+  std::string body = fnHead("Elt", "produce", "const Env& env, i64 i") + returnElt(r, em) + "  }\n";
+  return finish(body, outElt, typeLeaves(outElt), "map.hpp", 0);
+}
+
+KernelSource Codegen::scalarKernel(const Sx& e) {
+  Emit em;
+  em.ind = 4;
+  ValP r = exp(e, {}, em);
+  TypeP t = valType(r);
+  std::string body = fnHead("Elt", "produce", "const Env& env, i64 i") + returnElt(r, em) + "  }\n";
+  return finish(body, t, typeLeaves(t), "map.hpp", 1);
+}
+
+}  // namespace acchip

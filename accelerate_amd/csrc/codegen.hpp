@@ -1,0 +1,125 @@
+// Lowering of the scalar language (OpenExp / OpenFun / PrimFun, AST.hs:494-753) to HIP C++
+// text, and assembly of one translation unit per array node: prelude + generated `Spec`
+// (element type, scalar functions, fused producers) + one hand-written skeleton.
+#pragma once
+#include <map>
+#include <memory>
+#include <string>
+#include <vector>
+
+#include "types.hpp"
+
+namespace acchip {
+
+// A value during code generation: a tree whose leaves are C++ expressions that are cheap
+// and pure to repeat (a variable name or a literal).
+struct Val;
+using ValP = std::shared_ptr<Val>;
+struct Val {
+  enum K { Unit, Leaf, Pair } k = Unit;
+  ST st = ST::I64;
+  std::string ex;
+  ValP a, b;
+};
+ValP vUnit();
+ValP vLeaf(ST st, const std::string& ex);
+ValP vPair(ValP a, ValP b);
+TypeP valType(const ValP& v);
+void valLeaves(const ValP& v, std::vector<ValP>& out);
+
+// An array a kernel reads: a variable of the node's array environment, or a temporary the
+// executor materialised for a nested manifest operand.
+struct ArraySlot {
+  std::string name;   // "a<deBruijn>" or "t<k>"
+  ArrayR r;
+  bool temp = false;
+  int index = 0;      // de Bruijn index or temporary number
+};
+
+// Operand of a consumer: fused (Delayed) or a real array.
+struct Operand {
+  bool delayed = false;
+  ArrayR r;
+  Sx extent, indexD, linearD;  // when delayed
+  std::string slot;            // when manifest: name of the array slot
+};
+
+// Everything the executor needs to launch a generated kernel.
+struct KernelSource {
+  std::string source;                 // full translation unit
+  std::vector<ArraySlot> arrays;      // Env fields, in order (per array: leaf pointers, then extents)
+  std::vector<ST> outLeaves;          // element leaves of Spec::Out
+  int vec = 1;                        // Spec::V
+  bool commutative = false;
+  std::string permuteMode;            // permute only: "atomic", "cas", "lock", "store"
+};
+
+class Codegen {
+ public:
+  // aenv[i] is the type of array variable with de Bruijn index i at this node
+  explicit Codegen(std::vector<ArrayR> aenv) : aenv_(std::move(aenv)) {}
+
+  std::string addTemp(const ArrayR& r);  // returns slot name for a materialised operand
+
+  KernelSource fold(const Sx& f, const Sx* seed, const Operand& src);
+  KernelSource map(const TypeP& outElt, const Sx* f, const Operand& src);
+  KernelSource zipWith(const TypeP& outElt, const Sx& f, const Operand& a, const Operand& b, int rank);
+  KernelSource generate(const ArrayR& out, const Sx& f);
+  KernelSource backpermute(int outRank, const Sx& p, const Sx* f, const TypeP& outElt, const Operand& src);
+  KernelSource scan(const Sx& f, const Sx* seed, const Operand& src, bool right);
+  KernelSource foldSeg(const Sx& f, const Sx* seed, const Operand& src, const Operand& seg, ST segType);
+  KernelSource permute(const Sx& f, const ArrayR& dst, const Sx& p, const Operand& src);
+  KernelSource stencil(const std::vector<Sx>& patterns, const TypeP& outElt, const Sx& f,
+                       const std::vector<Sx>& boundaries, const std::vector<Operand>& srcs);
+  KernelSource scalarKernel(const Sx& exp);  // evaluates a closed Exp with one thread
+
+  // type of a closed scalar expression / result of a function, without emitting code
+  TypeP typeOfExp(const Sx& e);
+
+  struct Emit {
+    std::string code;
+    int ind = 2;
+    void line(const std::string& s) { code.append(ind, ' ').append(s).append("\n"); }
+  };
+  using Env = std::vector<ValP>;  // scalar environment; back() has de Bruijn index 0
+
+ private:
+  friend struct CodegenImpl;
+  std::vector<ArrayR> aenv_;
+  std::map<std::string, ArraySlot> used_;
+  std::vector<ArraySlot> temps_;
+  int next_ = 0;
+
+  std::string fresh() { return "v" + std::to_string(next_++); }
+  const ArraySlot& slotForVar(int idx);
+  const ArraySlot& slotByName(const std::string& name);
+
+  ValP exp(const Sx& e, const Env& env, Emit& em);
+  ValP applyFun(const Sx& f, const std::vector<ValP>& args, const Env& env, Emit& em);
+  ValP prim(const std::string& name, const std::vector<ST>& tys, const ValP& arg, Emit& em);
+  ValP bindLeaf(ST st, const std::string& ex, Emit& em);  // const T vN = ex;
+  ValP readArray(const ArraySlot& s, const std::string& lin, Emit& em);
+  ValP shapeOf(const ArraySlot& s);
+  std::string toIndex(const ValP& sh, const ValP& ix, Emit& em);
+  ValP fromIndex(int rank, const ValP& sh, const std::string& lin, Emit& em);
+  ValP operandLinear(const Operand& o, const std::string& lin, Emit& em);
+  ValP operandIndex(const Operand& o, const ValP& ix, Emit& em);
+  ValP operandShape(const Operand& o, Emit& em);
+  ValP declareVars(const TypeP& t, Emit& em);                // uninitialised mutable variables
+  void assign(const ValP& dst, const ValP& src, Emit& em);
+  ValP copyToVars(const ValP& v, Emit& em);
+
+  std::string eltStruct(const TypeP& t, const std::string& name);
+  std::string outStruct(const std::vector<ST>& leaves);
+  std::string envStruct(std::vector<ArraySlot>& order);
+  ValP eltVal(const TypeP& t, const std::string& var);
+  std::string returnElt(const ValP& v, Emit& em);
+  bool isCommutative(const Sx& f, std::string* op = nullptr, ST* st = nullptr);
+  KernelSource finish(const std::string& specBody, const TypeP& elt, const std::vector<ST>& outLeaves,
+                      const std::string& skeleton, int vec);
+};
+
+std::string literalText(ST st, const std::string& tok);
+const std::string& deviceHeader(const std::string& name);  // embedded device/*.hpp text
+
+}  // namespace acchip

@@ -1,0 +1,171 @@
+// Fold / Fold1 skeleton: reduction of the innermost dimension, one result per outer row.
+// Reference semantics: foldOp / fold1Op (Interpreter.hs:371-387) with Shape.iter's left
+// fold seeded once by z (Representation/Shape.hs:127-132).
+//
+// A row is cut into `bpr` contiguous chunks, one per workgroup; a chunk is cut into one
+// contiguous span per wave.  Each lane reads S::V consecutive elements per step (one
+// 128-bit request when the source is a plain array) so that a wave's step is one fully
+// coalesced tile of 64*V elements.
+//   commutative operator: lanes keep private accumulators over all their tiles and one
+//     wave reduction runs at the end;
+//   otherwise: every tile is reduced in lane order and chained onto a carry in lane 0,
+//     which keeps operands strictly left to right (associativity only).
+// Wave results meet in LDS and are combined in wave order.  With bpr > 1 the chunk
+// results go to `tmp` (rows x bpr) and acc_fold_final reduces them, again in order, and
+// applies the seed exactly once on the left.
+
+struct FoldParams {
+  i64 rows;   // number of outer rows
+  i64 n;      // extent of the innermost dimension
+  i64 bpr;    // workgroups per row
+  i64 chunk;  // elements per workgroup (multiple of ACC_WAVES * 64 * V)
+};
+
+template <class S, class Src>
+ACC_DEV bool acc_fold_span(const typename S::Env& env, const Src& src, i64 off, i64 lo, i64 hi,
+                           typename S::Elt& result) {
+  typedef typename S::Elt Elt;
+  const int V = S::V;
+  const i64 T = (i64)ACC_WAVE * V;
+  const int lane = acc_lane();
+  Elt acc;
+  bool have = false;
+  if (S::kCommutative) {
+    i64 base = lo;
+    bool full = false;
+    if (base + T <= hi) {
+      i64 p = off + base + (i64)lane * V;
+      acc = src(p);
+#pragma unroll
+      for (int k = 1; k < V; ++k) acc = S::combine(env, acc, src(p + k));
+      base += T;
+      full = true;
+#pragma unroll 4
+      for (; base + T <= hi; base += T) {
+        i64 q = off + base + (i64)lane * V;
+        Elt x[S::V];
+#pragma unroll
+        for (int k = 0; k < V; ++k) x[k] = src(q + k);
+#pragma unroll
+        for (int k = 0; k < V; ++k) acc = S::combine(env, acc, x[k]);
+      }
+    }
+    have = full;
+    i64 p0 = base + (i64)lane * V;
+#pragma unroll
+    for (int k = 0; k < V; ++k) {
+      if (p0 + k < hi) {
+        Elt x = src(off + p0 + k);
+        acc = have ? S::combine(env, acc, x) : x;
+        have = true;
+      }
+    }
+    i64 cnt = hi - base;
+    int nvalid = full ? ACC_WAVE : (cnt <= 0 ? 0 : (int)((cnt + V - 1) / V));
+    acc = acc_wave_reduce<S>(env, acc, lane, nvalid);
+    result = acc;
+    return nvalid > 0;
+  } else {
+    Elt carry;
+    for (i64 base = lo; base < hi; base += T) {
+      i64 cnt = hi - base < T ? hi - base : T;
+      int nl = (int)((cnt + V - 1) / V);
+      i64 p0 = base + (i64)lane * V;
+      Elt t;
+      if (p0 < hi) {
+        t = src(off + p0);
+#pragma unroll
+        for (int k = 1; k < V; ++k)
+          if (p0 + k < hi) t = S::combine(env, t, src(off + p0 + k));
+      }
+      t = acc_wave_reduce<S>(env, t, lane, nl);
+      carry = have ? S::combine(env, carry, t) : t;
+      have = true;
+    }
+    result = carry;
+    return have;
+  }
+}
+
+// Reduce [lo, hi) of one row with the whole workgroup; the result is valid in thread 0.
+template <class S, class Src>
+ACC_DEV bool acc_fold_block(const typename S::Env& env, const Src& src, i64 off, i64 lo, i64 hi,
+                            typename S::Elt& result) {
+  typedef typename S::Elt Elt;
+  __shared__ Elt sh_v[ACC_WAVES];
+  __shared__ int sh_ok[ACC_WAVES];
+  const i64 T = (i64)ACC_WAVE * S::V;
+  i64 span = hi - lo;
+  i64 wlen = (span + ACC_WAVES - 1) / ACC_WAVES;
+  wlen = (wlen + T - 1) / T * T;
+  const int w = acc_wave();
+  i64 wlo = lo + (i64)w * wlen;
+  i64 whi = wlo + wlen < hi ? wlo + wlen : hi;
+  Elt r;
+  bool ok = acc_fold_span<S>(env, src, off, wlo, whi, r);
+  if (acc_lane() == 0) {
+    sh_v[w] = r;
+    sh_ok[w] = ok ? 1 : 0;
+  }
+  __syncthreads();
+  bool have = false;
+  if (threadIdx.x == 0) {
+#pragma unroll
+    for (int k = 0; k < ACC_WAVES; ++k) {
+      if (sh_ok[k]) {
+        result = have ? S::combine(env, result, sh_v[k]) : sh_v[k];
+        have = true;
+      }
+    }
+  }
+  return have;
+}
+
+template <class S> struct AccFoldSrcIn {
+  const typename S::Env& env;
+  __device__ __forceinline__ typename S::Elt operator()(i64 i) const { return S::in_linear(env, i); }
+};
+template <class S> struct AccFoldSrcTmp {
+  const typename S::Out& tmp;
+  __device__ __forceinline__ typename S::Elt operator()(i64 i) const { return S::load(tmp, i); }
+};
+
+template <class S>
+ACC_DEV void acc_fold_finish(const typename S::Env& env, const typename S::Out& out, i64 row, bool have,
+                             const typename S::Elt& r) {
+  if (threadIdx.x != 0) return;
+  if (S::kSeeded) {
+    typename S::Elt z = S::seed(env);
+    S::store(out, row, have ? S::combine(env, z, r) : z);
+  } else if (have) {
+    S::store(out, row, r);
+  }
+}
+
+extern "C" __global__ void __launch_bounds__(ACC_BLOCK)
+acc_fold_main(Spec::Env env, Spec::Out out, Spec::Out tmp, FoldParams p) {
+  typedef Spec S;
+  i64 bid = (i64)blockIdx.x;
+  i64 row = bid / p.bpr;
+  i64 b = bid - row * p.bpr;
+  i64 lo = b * p.chunk;
+  i64 hi = lo + p.chunk < p.n ? lo + p.chunk : p.n;
+  AccFoldSrcIn<S> src{env};
+  S::Elt r;
+  bool have = acc_fold_block<S>(env, src, row * p.n, lo, hi, r);
+  if (p.bpr == 1) {
+    acc_fold_finish<S>(env, out, row, have, r);
+  } else if (threadIdx.x == 0 && have) {
+    S::store(tmp, bid, r);
+  }
+}
+
+extern "C" __global__ void __launch_bounds__(ACC_BLOCK)
+acc_fold_final(Spec::Env env, Spec::Out out, Spec::Out tmp, FoldParams p) {
+  typedef Spec S;
+  i64 row = (i64)blockIdx.x;
+  AccFoldSrcTmp<S> src{tmp};
+  S::Elt r;
+  bool have = acc_fold_block<S>(env, src, row * p.bpr, 0, p.bpr, r);
+  acc_fold_finish<S>(env, out, row, have, r);
+}

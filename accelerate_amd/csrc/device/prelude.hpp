@@ -1,0 +1,91 @@
+// Device-side prelude shared by every generated kernel (gfx950, wave64).
+// Compiled at run time by hipRTC together with the generated scalar code and one
+// skeleton; nothing here is host code.
+
+typedef signed char i8;
+typedef short i16;
+typedef int i32;
+typedef long long i64;
+typedef unsigned char u8;
+typedef unsigned short u16;
+typedef unsigned int u32;
+typedef unsigned long long u64;
+typedef _Float16 f16;
+typedef float f32;
+typedef double f64;
+
+#define ACC_DEV static __device__ __forceinline__
+#define ACC_WAVE 64
+#define ACC_BLOCK 256
+#define ACC_WAVES (ACC_BLOCK / ACC_WAVE)
+
+// Index arithmetic is 64-bit in the source language (Int); array extents almost always
+// fit 32 bits, where the hardware divide is several times cheaper.
+ACC_DEV i64 acc_quot(i64 a, i64 b) {
+  if ((((u64)a | (u64)b) >> 32) == 0) return (i64)((u32)a / (u32)b);
+  return a / b;
+}
+ACC_DEV i64 acc_rem(i64 a, i64 b) {
+  if ((((u64)a | (u64)b) >> 32) == 0) return (i64)((u32)a % (u32)b);
+  return a % b;
+}
+
+ACC_DEV int acc_lane() { return (int)(threadIdx.x & (ACC_WAVE - 1)); }
+ACC_DEV int acc_wave() { return (int)(threadIdx.x / ACC_WAVE); }
+
+// Word-wise cross-lane movement of any trivially copyable value.
+template <class T> struct AccWords { enum { N = (sizeof(T) + 3) / 4 }; };
+
+template <class T> ACC_DEV void acc_to_words(const T& v, u32* w) {
+  for (int k = 0; k < AccWords<T>::N; ++k) w[k] = 0;
+  __builtin_memcpy(w, &v, sizeof(T));
+}
+template <class T> ACC_DEV T acc_from_words(const u32* w) {
+  T r;
+  __builtin_memcpy(&r, w, sizeof(T));
+  return r;
+}
+
+template <class T> ACC_DEV T acc_shfl_up(const T& v, int delta) {
+  u32 w[AccWords<T>::N];
+  acc_to_words(v, w);
+#pragma unroll
+  for (int k = 0; k < AccWords<T>::N; ++k) w[k] = (u32)__shfl_up((int)w[k], delta, ACC_WAVE);
+  return acc_from_words<T>(w);
+}
+template <class T> ACC_DEV T acc_shfl_down(const T& v, int delta) {
+  u32 w[AccWords<T>::N];
+  acc_to_words(v, w);
+#pragma unroll
+  for (int k = 0; k < AccWords<T>::N; ++k) w[k] = (u32)__shfl_down((int)w[k], delta, ACC_WAVE);
+  return acc_from_words<T>(w);
+}
+template <class T> ACC_DEV T acc_shfl(const T& v, int src) {
+  u32 w[AccWords<T>::N];
+  acc_to_words(v, w);
+#pragma unroll
+  for (int k = 0; k < AccWords<T>::N; ++k) w[k] = (u32)__shfl((int)w[k], src, ACC_WAVE);
+  return acc_from_words<T>(w);
+}
+
+// Ordered reduction of the values held by lanes [0, nvalid) of a wave: the result, in
+// lane 0, is v0 (+) v1 (+) .. with operands kept left to right, so the operator need
+// only be associative.
+template <class S> ACC_DEV typename S::Elt acc_wave_reduce(const typename S::Env& env, typename S::Elt v, int lane, int nvalid) {
+#pragma unroll
+  for (int d = 1; d < ACC_WAVE; d <<= 1) {
+    typename S::Elt o = acc_shfl_down(v, d);
+    if (lane + d < nvalid) v = S::combine(env, v, o);
+  }
+  return v;
+}
+
+// Ordered inclusive scan across the lanes of a wave (valid lanes must form a prefix).
+template <class S> ACC_DEV typename S::Elt acc_wave_scan(const typename S::Env& env, typename S::Elt v, int lane) {
+#pragma unroll
+  for (int d = 1; d < ACC_WAVE; d <<= 1) {
+    typename S::Elt o = acc_shfl_up(v, d);
+    if (lane >= d) v = S::combine(env, o, v);
+  }
+  return v;
+}

@@ -1,0 +1,793 @@
+#include "exec.hpp"
+
+#include <algorithm>
+#include <cstring>
+
+namespace acchip {
+
+// ------------------------------------------------------------------------------------
+// array types
+
+static ATyP atUnit() {
+  static ATyP u = std::make_shared<ATy>();
+  return u;
+}
+static ATyP atArr(const ArrayR& r) {
+  auto t = std::make_shared<ATy>();
+  t->k = ATy::Arr;
+  t->r = r;
+  return t;
+}
+static ATyP atPair(ATyP a, ATyP b) {
+  auto t = std::make_shared<ATy>();
+  t->k = ATy::Pair;
+  t->a = std::move(a);
+  t->b = std::move(b);
+  return t;
+}
+static const ArrayR& oneArray(const ATyP& t, const char* what) {
+  if (t->k != ATy::Arr) throw Error(std::string(what) + ": expected a single array");
+  return t->r;
+}
+
+static AValP avUnit() {
+  static AValP u = std::make_shared<AVal>();
+  return u;
+}
+static AValP avArr(DArrayP a) {
+  auto v = std::make_shared<AVal>();
+  v->k = AVal::Arr;
+  v->arr = std::move(a);
+  return v;
+}
+static AValP avPair(AValP a, AValP b) {
+  auto v = std::make_shared<AVal>();
+  v->k = AVal::Pair;
+  v->a = std::move(a);
+  v->b = std::move(b);
+  return v;
+}
+
+static ATyP lhsType(const Sx& lhs) {
+  if (lhs.is("single")) return atArr(parseArrayR(lhs.at(1)));
+  if (lhs.is("wild")) {
+    const Sx& t = lhs.at(1);
+    if (t.isAtom("unit")) return atUnit();
+    if (t.is("array")) return atArr(parseArrayR(t));
+    if (t.is("pair")) {
+      Sx l, r;
+      l.kids = {Sx{true, "wild", {}}, t.at(1)};
+      r.kids = {Sx{true, "wild", {}}, t.at(2)};
+      return atPair(lhsType(l), lhsType(r));
+    }
+    throw Error("malformed array left-hand side " + lhs.str());
+  }
+  if (lhs.is("pair")) return atPair(lhsType(lhs.at(1)), lhsType(lhs.at(2)));
+  throw Error("malformed array left-hand side " + lhs.str());
+}
+
+static void pushTypes(const Sx& lhs, std::vector<ArrayR>& tenv) {
+  if (lhs.is("single")) tenv.push_back(parseArrayR(lhs.at(1)));
+  else if (lhs.is("pair")) {
+    pushTypes(lhs.at(1), tenv);
+    pushTypes(lhs.at(2), tenv);
+  }
+}
+static int lhsCount(const Sx& lhs) {
+  if (lhs.is("single")) return 1;
+  if (lhs.is("pair")) return lhsCount(lhs.at(1)) + lhsCount(lhs.at(2));
+  return 0;
+}
+static void pushVals(const Sx& lhs, const AValP& v, std::vector<DArrayP>& aenv) {
+  if (lhs.is("single")) {
+    if (v->k != AVal::Arr) throw Error("array left-hand side binds one array but the value is a tuple");
+    aenv.push_back(v->arr);
+  } else if (lhs.is("pair")) {
+    if (v->k != AVal::Pair) throw Error("array left-hand side is a pair but the value is not");
+    pushVals(lhs.at(1), v->a, aenv);
+    pushVals(lhs.at(2), v->b, aenv);
+  }
+}
+
+// ------------------------------------------------------------------------------------
+// host evaluation of simple scalar expressions (extents, predicates)
+
+static HValP hvUnit() {
+  static HValP u = std::make_shared<HVal>();
+  return u;
+}
+static HValP hvInt(ST st, int64_t i) {
+  auto v = std::make_shared<HVal>();
+  v->k = HVal::Leaf;
+  v->st = st;
+  v->i = i;
+  return v;
+}
+static HValP hvPair(HValP a, HValP b) {
+  auto v = std::make_shared<HVal>();
+  v->k = HVal::Pair;
+  v->a = std::move(a);
+  v->b = std::move(b);
+  return v;
+}
+
+static bool hostPrimOk(const std::string& n) {
+  static const char* ok[] = {"add", "sub", "mul", "min", "max", "quot", "rem", "idiv", "mod", "lt", "gt", "lte",
+                             "gte", "eq", "neq", "land", "lor", "lnot", "fromintegral", "neg", "abs"};
+  for (const char* o : ok)
+    if (n == o) return true;
+  return false;
+}
+
+// structural test: can hostEval handle this term without touching array contents?
+static bool hostSupported(const Sx& e) {
+  if (e.isAtom("nil")) return true;
+  if (e.atom) return false;
+  const std::string& h = e.head();
+  if (h == "var" || h == "shape") return true;
+  if (h == "const") return isST(e.at(1)) && !stIsFloat(parseST(e.at(1)));
+  if (h == "let") return hostSupported(e.at(2)) && hostSupported(e.at(3));
+  if (h == "pair") return hostSupported(e.at(1)) && hostSupported(e.at(2));
+  if (h == "cond") return hostSupported(e.at(1)) && hostSupported(e.at(2)) && hostSupported(e.at(3));
+  if (h == "toindex" || h == "fromindex") return hostSupported(e.at(2)) && hostSupported(e.at(3));
+  if (h == "indexslice" || h == "indexfull") return hostSupported(e.at(2)) && hostSupported(e.at(3));
+  if (h == "shapesize") return hostSupported(e.at(2));
+  if (h == "prim") {
+    if (!hostPrimOk(e.at(1).s)) return false;
+    for (size_t k = 2; k + 1 < e.size(); ++k)
+      if (!isST(e.at(k)) || stIsFloat(parseST(e.at(k)))) return false;
+    return hostSupported(e.at(e.size() - 1));
+  }
+  return false;
+}
+
+static int64_t wrapTo(ST st, int64_t v) {
+  switch (st) {
+    case ST::I8: return (int8_t)v;
+    case ST::I16: return (int16_t)v;
+    case ST::I32: return (int32_t)v;
+    case ST::U8: return (uint8_t)v;
+    case ST::U16: return (uint16_t)v;
+    case ST::U32: return (uint32_t)v;
+    default: return v;
+  }
+}
+
+static void hPush(const Sx& lhs, const HValP& v, std::vector<HValP>& env) {
+  if (lhs.is("single")) env.push_back(v);
+  else if (lhs.is("pair")) {
+    if (v->k != HVal::Pair) throw Error("host evaluation: left-hand side does not match the value");
+    hPush(lhs.at(1), v->a, env);
+    hPush(lhs.at(2), v->b, env);
+  }
+}
+
+static void hDims(const HValP& sh, std::vector<int64_t>& out) {
+  if (sh->k == HVal::Unit) return;
+  if (sh->k != HVal::Pair || sh->b->k != HVal::Leaf) throw Error("host evaluation: expected a shape");
+  hDims(sh->a, out);
+  out.push_back(sh->b->i);
+}
+static void hLeaves(const HValP& v, std::vector<int64_t>& out) {
+  if (v->k == HVal::Leaf) out.push_back(v->i);
+  else if (v->k == HVal::Pair) {
+    hLeaves(v->a, out);
+    hLeaves(v->b, out);
+  }
+}
+static HValP hShape(const std::vector<int64_t>& d) {
+  HValP v = hvUnit();
+  for (int64_t x : d) v = hvPair(v, hvInt(ST::I64, x));
+  return v;
+}
+
+static HValP hostEval(const Sx& e, std::vector<HValP> env, const std::vector<DArrayP>& aenv) {
+  if (e.isAtom("nil")) return hvUnit();
+  const std::string& h = e.head();
+  if (h == "var") {
+    size_t ix = (size_t)e.at(1).asInt();
+    if (ix >= env.size()) throw Error("host evaluation: scalar variable out of range");
+    return env[env.size() - 1 - ix];
+  }
+  if (h == "shape") {
+    size_t ix = (size_t)e.at(1).asInt();
+    if (ix >= aenv.size()) throw Error("host evaluation: array variable out of range");
+    return hShape(aenv[aenv.size() - 1 - ix]->shape);
+  }
+  if (h == "const") {
+    ST st = parseST(e.at(1));
+    const std::string& tok = e.at(2).s;
+    int64_t v = (!tok.empty() && tok[0] == '-') ? std::strtoll(tok.c_str(), nullptr, 0)
+                                                 : (int64_t)std::strtoull(tok.c_str(), nullptr, 0);
+    return hvInt(st, wrapTo(st, v));
+  }
+  if (h == "let") {
+    HValP v = hostEval(e.at(2), env, aenv);
+    hPush(e.at(1), v, env);
+    return hostEval(e.at(3), env, aenv);
+  }
+  if (h == "pair") {
+    HValP a = hostEval(e.at(1), env, aenv);
+    return hvPair(a, hostEval(e.at(2), env, aenv));
+  }
+  if (h == "cond") {
+    HValP c = hostEval(e.at(1), env, aenv);
+    return hostEval(c->i != 0 ? e.at(2) : e.at(3), env, aenv);
+  }
+  if (h == "toindex") {
+    std::vector<int64_t> d, i;
+    hDims(hostEval(e.at(2), env, aenv), d);
+    hDims(hostEval(e.at(3), env, aenv), i);
+    if (d.size() != i.size()) throw Error("host evaluation: toIndex rank mismatch");
+    int64_t lin = 0;
+    for (size_t k = 0; k < d.size(); ++k) lin = lin * d[k] + i[k];
+    return hvInt(ST::I64, lin);
+  }
+  if (h == "fromindex") {
+    std::vector<int64_t> d;
+    hDims(hostEval(e.at(2), env, aenv), d);
+    int64_t cur = hostEval(e.at(3), env, aenv)->i;
+    std::vector<int64_t> ix(d.size());
+    for (size_t k = d.size(); k-- > 1;) {
+      if (d[k] == 0) throw Error("host evaluation: fromIndex into an empty shape");
+      ix[k] = cur % d[k];
+      cur /= d[k];
+    }
+    if (!d.empty()) ix[0] = cur;
+    return hShape(ix);
+  }
+  if (h == "shapesize") {
+    std::vector<int64_t> d;
+    hDims(hostEval(e.at(2), env, aenv), d);
+    int64_t n = 1;
+    for (int64_t x : d) {
+      if (x <= 0) return hvInt(ST::I64, 0);
+      n *= x;
+    }
+    return hvInt(ST::I64, n);
+  }
+  if (h == "indexslice" || h == "indexfull") {
+    const Sx& spec = e.at(1);
+    HValP slix = hostEval(e.at(2), env, aenv), sh = hostEval(e.at(3), env, aenv);
+    struct R {
+      static HValP restrict_(const Sx& spec, size_t k, const HValP& slix, const HValP& sh) {
+        if (k == spec.size()) return hvUnit();
+        if (slix->k != HVal::Pair || sh->k != HVal::Pair) throw Error("host evaluation: malformed slice");
+        HValP rest = restrict_(spec, k + 1, slix->a, sh->a);
+        return spec.at(k).isAtom("all") ? hvPair(rest, sh->b) : rest;
+      }
+      static HValP extend(const Sx& spec, size_t k, const HValP& slix, const HValP& sl) {
+        if (k == spec.size()) return hvUnit();
+        if (slix->k != HVal::Pair) throw Error("host evaluation: malformed slice");
+        if (spec.at(k).isAtom("all")) {
+          if (sl->k != HVal::Pair) throw Error("host evaluation: malformed slice");
+          return hvPair(extend(spec, k + 1, slix->a, sl->a), sl->b);
+        }
+        return hvPair(extend(spec, k + 1, slix->a, sl), slix->b);
+      }
+    };
+    return h == "indexslice" ? R::restrict_(spec, 0, slix, sh) : R::extend(spec, 0, slix, sh);
+  }
+  if (h == "prim") {
+    const std::string& n = e.at(1).s;
+    HValP arg = hostEval(e.at(e.size() - 1), env, aenv);
+    ST st = e.size() > 3 ? parseST(e.at(2)) : ST::U8;
+    auto B = [](bool b) { return hvInt(ST::U8, b ? 1 : 0); };
+    if (n == "lnot") return B(arg->i == 0);
+    if (n == "neg") return hvInt(st, wrapTo(st, (int64_t)(0 - (uint64_t)arg->i)));
+    if (n == "abs") return hvInt(st, wrapTo(st, arg->i < 0 ? (int64_t)(0 - (uint64_t)arg->i) : arg->i));
+    if (n == "fromintegral") {
+      ST to = parseST(e.at(3));
+      return hvInt(to, wrapTo(to, arg->i));
+    }
+    if (arg->k != HVal::Pair) throw Error("host evaluation: primitive expects a pair");
+    int64_t a = arg->a->i, b = arg->b->i;
+    bool uns = !stIsSigned(st) && stSize(st) == 8;
+    uint64_t ua = (uint64_t)a, ub = (uint64_t)b;
+    if (n == "add") return hvInt(st, wrapTo(st, (int64_t)(ua + ub)));
+    if (n == "sub") return hvInt(st, wrapTo(st, (int64_t)(ua - ub)));
+    if (n == "mul") return hvInt(st, wrapTo(st, (int64_t)(ua * ub)));
+    auto le = [&](int64_t x, int64_t y) { return uns ? (uint64_t)x <= (uint64_t)y : x <= y; };
+    auto ltf = [&](int64_t x, int64_t y) { return uns ? (uint64_t)x < (uint64_t)y : x < y; };
+    if (n == "min") return hvInt(st, le(a, b) ? a : b);
+    if (n == "max") return hvInt(st, le(a, b) ? b : a);
+    if (n == "lt") return B(ltf(a, b));
+    if (n == "gt") return B(ltf(b, a));
+    if (n == "lte") return B(le(a, b));
+    if (n == "gte") return B(le(b, a));
+    if (n == "eq") return B(a == b);
+    if (n == "neq") return B(a != b);
+    if (n == "land") return B(a != 0 && b != 0);
+    if (n == "lor") return B(a != 0 || b != 0);
+    if (b == 0) throw Error("divide by zero");
+    if (uns) {
+      if (n == "quot" || n == "idiv") return hvInt(st, (int64_t)(ua / ub));
+      return hvInt(st, (int64_t)(ua % ub));
+    }
+    int64_t q = a / b, r = a % b;
+    if (n == "quot") return hvInt(st, wrapTo(st, q));
+    if (n == "rem") return hvInt(st, wrapTo(st, r));
+    bool adj = r != 0 && ((r < 0) != (b < 0));
+    if (n == "idiv") return hvInt(st, wrapTo(st, adj ? q - 1 : q));
+    if (n == "mod") return hvInt(st, wrapTo(st, adj ? r + b : r));
+  }
+  throw Error("host evaluation: unsupported expression '" + h + "'");
+}
+
+// ------------------------------------------------------------------------------------
+// preparation (type inference + code generation for every node)
+
+Program::Program(Context& ctx, const char* text, size_t len) : ctx_(ctx) {
+  root_ = parseSx(text, len);
+  const Sx* f = &root_;
+  TEnv tenv;
+  while (f->is("alam")) {
+    argTypes.push_back(lhsType(f->at(1)));
+    pushTypes(f->at(1), tenv);
+    lams_.push_back(f);
+    f = &f->at(2);
+  }
+  body_ = f;
+  resultType = prepare(*body_, tenv);
+}
+
+std::vector<ArrayR> Program::aenvOf(const TEnv& tenv) {
+  std::vector<ArrayR> a(tenv.rbegin(), tenv.rend());  // index 0 = most recently bound
+  return a;
+}
+
+Operand Program::operandOf(const Sx& o, Codegen& cg, TEnv& tenv, Plan& plan) {
+  Operand op;
+  if (o.is("delayed")) {
+    op.delayed = true;
+    op.r = parseArrayR(o.at(1));
+    op.extent = o.at(2);
+    op.indexD = o.at(3);
+    op.linearD = o.at(4);
+    prepareHostExp(o.at(2), tenv, plan);
+    return op;
+  }
+  if (o.is("avar")) {
+    size_t ix = (size_t)o.at(1).asInt();
+    if (ix >= tenv.size()) throw Error("array variable index out of range");
+    op.r = tenv[tenv.size() - 1 - ix];
+    op.slot = "a" + std::to_string(ix);
+    return op;
+  }
+  // a nested manifest term: evaluated to a temporary before this node's kernel runs
+  ATyP t = prepare(o, tenv);
+  op.r = oneArray(t, "array operand");
+  op.slot = cg.addTemp(op.r);
+  plan.temps.push_back(&o);
+  return op;
+}
+
+void Program::prepareHostExp(const Sx& e, TEnv& tenv, Plan& plan) {
+  if (hostSupported(e)) return;
+  Codegen cg(aenvOf(tenv));
+  plan.scalarKernels[&e] = ctx_.kernel(cg.scalarKernel(e));
+}
+
+ATyP Program::prepareFun(const Sx& f, TEnv& tenv, std::vector<ATyP>* params) {
+  if (f.is("alam")) {
+    if (params) params->push_back(lhsType(f.at(1)));
+    size_t mark = tenv.size();
+    pushTypes(f.at(1), tenv);
+    ATyP r = prepareFun(f.at(2), tenv, params);
+    tenv.resize(mark);
+    return r;
+  }
+  return prepare(f, tenv);
+}
+
+ATyP Program::prepare(const Sx& n, TEnv& tenv) {
+  if (n.isAtom("anil")) return atUnit();
+  if (n.atom) throw Error("unexpected atom '" + n.s + "' in array term");
+  const std::string& h = n.head();
+  auto seedOf = [&](const Sx& s) -> const Sx* {
+    if (s.isAtom("nothing")) return nullptr;
+    if (s.is("just")) return &s.at(1);
+    throw Error("expected (just e) or nothing, got " + s.str());
+  };
+
+  if (h == "avar") {
+    size_t ix = (size_t)n.at(1).asInt();
+    if (ix >= tenv.size()) throw Error("array variable index out of range");
+    return atArr(tenv[tenv.size() - 1 - ix]);
+  }
+  if (h == "alet") {
+    prepare(n.at(2), tenv);
+    size_t mark = tenv.size();
+    pushTypes(n.at(1), tenv);
+    ATyP r = prepare(n.at(3), tenv);
+    tenv.resize(mark);
+    return r;
+  }
+  if (h == "apair") {
+    ATyP a = prepare(n.at(1), tenv);
+    return atPair(a, prepare(n.at(2), tenv));
+  }
+  if (h == "apply") {
+    prepare(n.at(2), tenv);
+    return prepareFun(n.at(1), tenv, nullptr);
+  }
+  if (h == "acond") {
+    Plan& plan = plans_[&n];
+    prepareHostExp(n.at(1), tenv, plan);
+    ATyP a = prepare(n.at(2), tenv);
+    prepare(n.at(3), tenv);
+    return a;
+  }
+  if (h == "awhile") {
+    ATyP t = prepare(n.at(3), tenv);
+    prepareFun(n.at(1), tenv, nullptr);
+    prepareFun(n.at(2), tenv, nullptr);
+    return t;
+  }
+  if (h == "use") return atArr(parseArrayR(n.at(1)));
+  if (h == "delayed") throw Error("expected manifest array");  // Interpreter.hs:180
+
+  Plan& plan = plans_[&n];
+  Codegen cg(aenvOf(tenv));
+  auto done = [&](const ArrayR& r) {
+    plan.ty = atArr(r);
+    return plan.ty;
+  };
+
+  if (h == "unit") {
+    ArrayR r;
+    r.rank = 0;
+    r.elt = parseType(n.at(1));
+    plan.k = ctx_.kernel(cg.scalarKernel(n.at(2)));
+    return done(r);
+  }
+  if (h == "reshape") {
+    prepareHostExp(n.at(2), tenv, plan);
+    ATyP t = prepare(n.at(3), tenv);
+    ArrayR r = oneArray(t, "reshape");
+    r.rank = (int)n.at(1).asInt();
+    return done(r);
+  }
+  if (h == "generate") {
+    ArrayR r = parseArrayR(n.at(1));
+    prepareHostExp(n.at(2), tenv, plan);
+    plan.k = ctx_.kernel(cg.generate(r, n.at(3)));
+    return done(r);
+  }
+  if (h == "transform") {
+    ArrayR r = parseArrayR(n.at(1));
+    prepareHostExp(n.at(2), tenv, plan);
+    Operand src = operandOf(n.at(5), cg, tenv, plan);
+    plan.k = ctx_.kernel(cg.backpermute(r.rank, n.at(3), &n.at(4), r.elt, src));
+    return done(r);
+  }
+  if (h == "backpermute") {
+    int rank = (int)n.at(1).asInt();
+    prepareHostExp(n.at(2), tenv, plan);
+    Operand src = operandOf(n.at(4), cg, tenv, plan);
+    ArrayR r;
+    r.rank = rank;
+    r.elt = src.r.elt;
+    plan.k = ctx_.kernel(cg.backpermute(rank, n.at(3), nullptr, r.elt, src));
+    return done(r);
+  }
+  if (h == "map") {
+    Operand src = operandOf(n.at(3), cg, tenv, plan);
+    ArrayR r;
+    r.rank = src.r.rank;
+    r.elt = parseType(n.at(1));
+    plan.k = ctx_.kernel(cg.map(r.elt, &n.at(2), src));
+    return done(r);
+  }
+  if (h == "zipwith") {
+    Operand a = operandOf(n.at(3), cg, tenv, plan);
+    Operand b = operandOf(n.at(4), cg, tenv, plan);
+    if (a.r.rank != b.r.rank) throw Error("zipWith: operands of different rank");
+    ArrayR r;
+    r.rank = a.r.rank;
+    r.elt = parseType(n.at(1));
+    plan.k = ctx_.kernel(cg.zipWith(r.elt, n.at(2), a, b, r.rank));
+    return done(r);
+  }
+  if (h == "fold") {
+    Operand src = operandOf(n.at(3), cg, tenv, plan);
+    if (src.r.rank < 1) throw Error("fold: operand must have rank >= 1");
+    plan.k = ctx_.kernel(cg.fold(n.at(1), seedOf(n.at(2)), src));
+    ArrayR r;
+    r.rank = src.r.rank - 1;
+    r.elt = src.r.elt;
+    return done(r);
+  }
+  throw Error("unsupported array term '" + h + "'");
+}
+
+// ------------------------------------------------------------------------------------
+// execution
+
+DArrayP Program::alloc(const ArrayR& r, const std::vector<int64_t>& shape) {
+  auto a = std::make_shared<DArray>();
+  a->r = r;
+  a->shape = shape;
+  int64_t n = a->size();
+  for (ST st : typeLeaves(r.elt)) {
+    auto b = std::make_shared<Buffer>();
+    b->ctx = &ctx_;
+    b->bytes = (size_t)n * stSize(st);
+    b->p = ctx_.malloc(b->bytes);
+    if (!b->p) throw Error("Remote memory exhausted");  // Array/Remote/LRU.hs:258-303
+    b->owned = true;
+    a->bufs.push_back(b);
+  }
+  return a;
+}
+
+void Program::packOut(std::vector<uint64_t>& args, const DArray& a) {
+  args.push_back(0);
+  for (auto& b : a.bufs) args.push_back((uint64_t)(uintptr_t)b->p);
+}
+
+std::vector<uint64_t> Program::packArgs(const KernelSource& ks, const AEnv& aenv, const std::vector<DArrayP>& temps,
+                                        const std::vector<int64_t>& outShape) {
+  std::vector<uint64_t> args;
+  args.push_back(0);
+  for (const ArraySlot& s : ks.arrays) {
+    if (s.name == "out") {
+      if ((int)outShape.size() != s.r.rank) throw Error("internal: result rank does not match the generated kernel");
+      for (int64_t d : outShape) args.push_back((uint64_t)d);
+      continue;
+    }
+    DArrayP a;
+    if (s.temp) {
+      if (s.index >= (int)temps.size()) throw Error("internal: missing temporary operand");
+      a = temps[s.index];
+    } else {
+      if (s.index >= (int)aenv.size()) throw Error("internal: array variable out of range at launch");
+      a = aenv[aenv.size() - 1 - s.index];
+    }
+    if (a->r.rank != s.r.rank || !typeEq(a->r.elt, s.r.elt))
+      throw Error("array bound to " + s.name + " does not have the type the program declares (rank " +
+                  std::to_string(s.r.rank) + ", " + typeStr(s.r.elt) + ")");
+    for (auto& b : a->bufs) args.push_back((uint64_t)(uintptr_t)b->p);
+    for (int64_t d : a->shape) args.push_back((uint64_t)d);
+  }
+  return args;
+}
+
+HValP Program::hostExp(const Sx& e, const AEnv& aenv, const Plan& plan) {
+  auto it = plan.scalarKernels.find(&e);
+  if (it == plan.scalarKernels.end()) return hostEval(e, {}, aenv);
+  // one-thread kernel, then read the leaves back
+  const KernelP& k = it->second;
+  ArrayR r;
+  r.rank = 0;
+  TypeP t = tUnit();
+  // rebuild the element type from the leaves (flat tuple is enough to hold them)
+  for (ST st : k->meta.outLeaves) t = tPair(t, tScalar(st));
+  r.elt = t;
+  DArrayP out = alloc(r, {});
+  std::vector<uint64_t> args = packArgs(k->meta, aenv, {}, {});
+  packOut(args, *out);
+  args.push_back(1);
+  ctx_.launch(k, "acc_map", 1, 256, args);
+  std::vector<HValP> leaves;
+  for (size_t i = 0; i < out->bufs.size(); ++i) {
+    ST st = k->meta.outLeaves[i];
+    unsigned char raw[8] = {0};
+    ctx_.peek(raw, out->bufs[i]->p, stSize(st));
+    auto v = std::make_shared<HVal>();
+    v->k = HVal::Leaf;
+    v->st = st;
+    switch (st) {
+      case ST::I8: v->i = *(int8_t*)raw; break;
+      case ST::I16: v->i = *(int16_t*)raw; break;
+      case ST::I32: v->i = *(int32_t*)raw; break;
+      case ST::I64: v->i = *(int64_t*)raw; break;
+      case ST::U8: v->i = *(uint8_t*)raw; break;
+      case ST::U16: v->i = *(uint16_t*)raw; break;
+      case ST::U32: v->i = *(uint32_t*)raw; break;
+      case ST::U64: v->i = (int64_t) * (uint64_t*)raw; break;
+      case ST::F32: v->f = *(float*)raw; break;
+      case ST::F64: v->f = *(double*)raw; break;
+      case ST::F16: v->f = 0; break;
+    }
+    leaves.push_back(v);
+  }
+  // the caller only needs shapes / predicates: hand back a left-nested tuple of the leaves
+  HValP v = hvUnit();
+  if (leaves.size() == 1) return leaves[0];
+  for (auto& l : leaves) v = hvPair(v, l);
+  return v;
+}
+
+std::vector<int64_t> Program::hostShape(const Sx& e, const AEnv& aenv, const Plan& plan, int rank) {
+  HValP v = hostExp(e, aenv, plan);
+  std::vector<int64_t> d;
+  hLeaves(v, d);
+  if ((int)d.size() != rank) throw Error("shape expression has rank " + std::to_string(d.size()) + ", expected " + std::to_string(rank));
+  return d;
+}
+
+std::vector<DArrayP> Program::evalTemps(const std::vector<const Sx*>& temps, AEnv& aenv) {
+  std::vector<DArrayP> out;
+  for (const Sx* t : temps) {
+    AValP v = eval(*t, aenv);
+    if (v->k != AVal::Arr) throw Error("array operand evaluated to a tuple");
+    out.push_back(v->arr);
+  }
+  return out;
+}
+
+std::vector<int64_t> Program::operandExtent(const Sx& o, const AEnv& aenv, const Plan& plan,
+                                            const std::vector<DArrayP>& temps, size_t& cursor) {
+  if (o.is("delayed")) return hostShape(o.at(2), aenv, plan, parseArrayR(o.at(1)).rank);
+  if (o.is("avar")) {
+    size_t ix = (size_t)o.at(1).asInt();
+    return aenv[aenv.size() - 1 - ix]->shape;
+  }
+  return temps.at(cursor++)->shape;
+}
+
+void Program::launchMap(const KernelP& k, const AEnv& aenv, const std::vector<DArrayP>& temps, DArray& out) {
+  int64_t n = out.size();
+  if (n == 0) return;
+  std::vector<uint64_t> args = packArgs(k->meta, aenv, temps, out.shape);
+  packOut(args, out);
+  args.push_back((uint64_t)n);
+  int64_t per = (int64_t)256 * k->meta.vec;
+  ctx_.launch(k, "acc_map", (unsigned)((n + per - 1) / per), 256, args);
+}
+
+AValP Program::evalFun(const Sx& f, AEnv& aenv, const std::vector<AValP>& args) {
+  size_t mark = aenv.size();
+  const Sx* cur = &f;
+  for (const AValP& a : args) {
+    if (!cur->is("alam")) throw Error("array function applied to too many arguments");
+    pushVals(cur->at(1), a, aenv);
+    cur = &cur->at(2);
+  }
+  if (cur->is("alam")) throw Error("array function applied to too few arguments");
+  AValP r = eval(*cur, aenv);
+  aenv.resize(mark);
+  return r;
+}
+
+AValP Program::run(const std::vector<AValP>& args, const std::vector<DArrayP>& uses) {
+  if (args.size() != lams_.size())
+    throw Error("program expects " + std::to_string(lams_.size()) + " arguments, got " + std::to_string(args.size()));
+  uses_ = &uses;
+  AEnv aenv;
+  for (size_t i = 0; i < args.size(); ++i) pushVals(lams_[i]->at(1), args[i], aenv);
+  return eval(*body_, aenv);
+}
+
+AValP Program::eval(const Sx& n, AEnv& aenv) {
+  if (n.isAtom("anil")) return avUnit();
+  const std::string& h = n.head();
+  if (h == "avar") {
+    size_t ix = (size_t)n.at(1).asInt();
+    return avArr(aenv[aenv.size() - 1 - ix]);
+  }
+  if (h == "alet") {
+    AValP v = eval(n.at(2), aenv);
+    size_t mark = aenv.size();
+    pushVals(n.at(1), v, aenv);
+    AValP r = eval(n.at(3), aenv);
+    aenv.resize(mark);
+    return r;
+  }
+  if (h == "apair") {
+    AValP a = eval(n.at(1), aenv);
+    return avPair(a, eval(n.at(2), aenv));
+  }
+  if (h == "apply") {
+    AValP a = eval(n.at(2), aenv);
+    return evalFun(n.at(1), aenv, {a});
+  }
+  if (h == "acond") {
+    const Plan& plan = plans_.at(&n);
+    HValP c = hostExp(n.at(1), aenv, plan);
+    return eval(c->i != 0 ? n.at(2) : n.at(3), aenv);
+  }
+  if (h == "awhile") {
+    // host loop reading one byte back per iteration (Interpreter.hs:222-229)
+    AValP x = eval(n.at(3), aenv);
+    for (;;) {
+      AValP p = evalFun(n.at(1), aenv, {x});
+      if (p->k != AVal::Arr || p->arr->bufs.size() != 1) throw Error("awhile: predicate must be a scalar boolean array");
+      unsigned char flag = 0;
+      ctx_.peek(&flag, p->arr->bufs[0]->p, 1);
+      if (!flag) break;
+      x = evalFun(n.at(2), aenv, {x});
+    }
+    return x;
+  }
+  if (h == "use") {
+    size_t slot = (size_t)n.at(2).asInt();
+    if (!uses_ || slot >= uses_->size()) throw Error("use: no array supplied for slot " + std::to_string(slot));
+    return avArr((*uses_)[slot]);
+  }
+
+  const Plan& plan = plans_.at(&n);
+  auto seeded = [&](const Sx& s) { return !s.isAtom("nothing"); };
+
+  if (h == "unit") {
+    DArrayP out = alloc(plan.ty->r, {});
+    launchMap(plan.k, aenv, {}, *out);
+    return avArr(out);
+  }
+  if (h == "reshape") {
+    AValP v = eval(n.at(3), aenv);
+    int rank = (int)n.at(1).asInt();
+    std::vector<int64_t> sh = hostShape(n.at(2), aenv, plan, rank);
+    auto a = std::make_shared<DArray>(*v->arr);
+    a->shape = sh;
+    a->r.rank = rank;
+    if (a->size() != v->arr->size()) throw Error("shape mismatch");  // Interpreter.hs:295
+    return avArr(a);
+  }
+  if (h == "generate" || h == "transform" || h == "backpermute") {
+    std::vector<DArrayP> temps = evalTemps(plan.temps, aenv);
+    const ArrayR& r = plan.ty->r;
+    DArrayP out = alloc(r, hostShape(n.at(2), aenv, plan, r.rank));
+    launchMap(plan.k, aenv, temps, *out);
+    return avArr(out);
+  }
+  if (h == "map") {
+    std::vector<DArrayP> temps = evalTemps(plan.temps, aenv);
+    size_t cur = 0;
+    std::vector<int64_t> ext = operandExtent(n.at(3), aenv, plan, temps, cur);
+    DArrayP out = alloc(plan.ty->r, ext);
+    launchMap(plan.k, aenv, temps, *out);
+    return avArr(out);
+  }
+  if (h == "zipwith") {
+    std::vector<DArrayP> temps = evalTemps(plan.temps, aenv);
+    size_t cur = 0;
+    std::vector<int64_t> e1 = operandExtent(n.at(3), aenv, plan, temps, cur);
+    std::vector<int64_t> e2 = operandExtent(n.at(4), aenv, plan, temps, cur);
+    for (size_t k = 0; k < e1.size(); ++k) e1[k] = std::min(e1[k], e2[k]);  // intersect, Shape.hs:81-82
+    DArrayP out = alloc(plan.ty->r, e1);
+    launchMap(plan.k, aenv, temps, *out);
+    return avArr(out);
+  }
+  if (h == "fold") {
+    std::vector<DArrayP> temps = evalTemps(plan.temps, aenv);
+    size_t cur = 0;
+    std::vector<int64_t> ext = operandExtent(n.at(3), aenv, plan, temps, cur);
+    int64_t len = std::max<int64_t>(ext.back(), 0);
+    ext.pop_back();
+    if (!seeded(n.at(2)) && len <= 0) throw Error("empty array");  // fold1, Interpreter.hs:386
+    DArrayP out = alloc(plan.ty->r, ext);
+    int64_t rows = out->size();
+    if (rows == 0) return avArr(out);
+    // geometry: enough workgroups to fill the chip, each with at least a few tiles of work
+    const int64_t tile = (int64_t)4 * 64 * plan.k->meta.vec;
+    const int64_t target = 2048;
+    int64_t bpr = 1;
+    if (rows < target && len > 8 * tile)
+      bpr = std::min((target + rows - 1) / rows, (len + 8 * tile - 1) / (8 * tile));
+    int64_t chunk = ((len + bpr - 1) / bpr + tile - 1) / tile * tile;
+    if (chunk == 0) chunk = tile;
+    bpr = std::max<int64_t>(1, (len + chunk - 1) / chunk);
+    if (rows * bpr > 0x7fffffffLL) throw Error("fold: too many rows for one launch");
+    DArrayP tmp = out;
+    if (bpr > 1) {
+      ArrayR tr = plan.ty->r;
+      tr.rank = 1;
+      tmp = alloc(tr, {rows * bpr});
+    }
+    std::vector<uint64_t> args = packArgs(plan.k->meta, aenv, temps, {});
+    packOut(args, *out);
+    packOut(args, *tmp);
+    args.push_back((uint64_t)rows);
+    args.push_back((uint64_t)len);
+    args.push_back((uint64_t)bpr);
+    args.push_back((uint64_t)chunk);
+    ctx_.launch(plan.k, "acc_fold_main", (unsigned)(rows * bpr), 256, args);
+    if (bpr > 1) ctx_.launch(plan.k, "acc_fold_final", (unsigned)rows, 256, args);
+    return avArr(out);
+  }
+  throw Error("unsupported array term '" + h + "'");
+}
+
+}  // namespace acchip

@@ -1,0 +1,120 @@
+// Executor: walks the array-level term (the counterpart of evalOpenAcc,
+// Interpreter.hs:175-259), one kernel launch per array node, host-driven control flow.
+// A Program is prepared once (parse, type inference, code generation and hipRTC for every
+// node: what `runN f` does at partial application) and executed many times.
+#pragma once
+#include <map>
+#include <memory>
+#include <vector>
+
+#include "runtime.hpp"
+
+namespace acchip {
+
+struct Buffer {
+  Context* ctx = nullptr;
+  void* p = nullptr;
+  size_t bytes = 0;
+  bool owned = false;
+  ~Buffer() {
+    if (owned && ctx) ctx->free(p);
+  }
+};
+using BufferP = std::shared_ptr<Buffer>;
+
+// A device-resident array: shape + one dense buffer per scalar leaf of the element type
+// (struct-of-arrays, Array/Data.hs:95-119; row-major, Representation/Shape.hs:98-106).
+struct DArray {
+  ArrayR r;
+  std::vector<int64_t> shape;
+  std::vector<BufferP> bufs;
+  int64_t size() const {
+    int64_t n = 1;
+    for (int64_t d : shape) n = d <= 0 ? 0 : n * d;
+    for (int64_t d : shape)
+      if (d <= 0) return 0;
+    return n;
+  }
+};
+using DArrayP = std::shared_ptr<DArray>;
+
+struct AVal;
+using AValP = std::shared_ptr<AVal>;
+struct AVal {
+  enum K { Unit, Arr, Pair } k = Unit;
+  DArrayP arr;
+  AValP a, b;
+};
+
+struct ATy;
+using ATyP = std::shared_ptr<ATy>;
+struct ATy {
+  enum K { Unit, Arr, Pair } k = Unit;
+  ArrayR r;
+  ATyP a, b;
+};
+
+// host-side scalar value (extents, predicates)
+struct HVal;
+using HValP = std::shared_ptr<HVal>;
+struct HVal {
+  enum K { Unit, Leaf, Pair } k = Unit;
+  ST st = ST::I64;
+  int64_t i = 0;   // integral leaves (any width, stored sign/zero-extended)
+  double f = 0;    // floating leaves
+  HValP a, b;
+};
+
+struct Plan {
+  KernelP k, k2;
+  std::vector<const Sx*> temps;                  // nested manifest operands, in slot order
+  std::map<const Sx*, KernelP> scalarKernels;    // expressions evaluated by a one-thread kernel
+  std::map<const Sx*, std::vector<const Sx*>> scalarTemps;
+  std::string mode;
+  ATyP ty;                                       // result type of the node
+};
+
+class Program {
+ public:
+  Program(Context& ctx, const char* text, size_t len);
+  // args: one AVal per lambda of the program, in order; uses: arrays for (use ..) slots
+  AValP run(const std::vector<AValP>& args, const std::vector<DArrayP>& uses);
+
+  std::vector<ATyP> argTypes;
+  ATyP resultType;
+  size_t kernelCount() const { return plans_.size(); }
+
+ private:
+  Context& ctx_;
+  Sx root_;
+  const Sx* body_ = nullptr;
+  std::vector<const Sx*> lams_;
+  std::map<const Sx*, Plan> plans_;
+  const std::vector<DArrayP>* uses_ = nullptr;
+
+  using TEnv = std::vector<ArrayR>;     // back() has de Bruijn index 0
+  using AEnv = std::vector<DArrayP>;
+
+  // preparation
+  ATyP prepare(const Sx& n, TEnv& tenv);
+  ATyP prepareFun(const Sx& f, TEnv& tenv, std::vector<ATyP>* params);
+  Operand operandOf(const Sx& o, Codegen& cg, TEnv& tenv, Plan& plan);
+  void prepareHostExp(const Sx& e, TEnv& tenv, Plan& plan);
+  static std::vector<ArrayR> aenvOf(const TEnv& tenv);
+
+  // execution
+  AValP eval(const Sx& n, AEnv& aenv);
+  AValP evalFun(const Sx& f, AEnv& aenv, const std::vector<AValP>& args);
+  HValP hostExp(const Sx& e, const AEnv& aenv, const Plan& plan);
+  std::vector<int64_t> hostShape(const Sx& e, const AEnv& aenv, const Plan& plan, int rank);
+  std::vector<DArrayP> evalTemps(const std::vector<const Sx*>& temps, AEnv& aenv);
+  std::vector<int64_t> operandExtent(const Sx& o, const AEnv& aenv, const Plan& plan, const std::vector<DArrayP>& temps,
+                                     size_t& tempCursor);
+  DArrayP alloc(const ArrayR& r, const std::vector<int64_t>& shape);
+  std::vector<uint64_t> packArgs(const KernelSource& ks, const AEnv& aenv, const std::vector<DArrayP>& temps,
+                                 const std::vector<int64_t>& outShape);
+  static void packOut(std::vector<uint64_t>& args, const DArray& a);
+  void launchMap(const KernelP& k, const AEnv& aenv, const std::vector<DArrayP>& temps, DArray& out);
+};
+
+}  // namespace acchip

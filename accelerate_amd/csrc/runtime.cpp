@@ -1,0 +1,337 @@
+#include "runtime.hpp"
+
+#include <dlfcn.h>
+#include <hip/hiprtc.h>
+#include <sys/stat.h>
+#include <unistd.h>
+
+#include <cstdio>
+#include <cstdlib>
+#include <cstring>
+#include <fstream>
+
+#include "sha3.hpp"
+
+namespace acchip {
+
+void hipCheck(hipError_t e, const char* what) {
+  if (e != hipSuccess) throw Error(std::string(what) + ": " + hipGetErrorString(e));
+}
+
+std::string libraryDir() {
+  Dl_info info;
+  if (dladdr((void*)&libraryDir, &info) && info.dli_fname) {
+    std::string p = info.dli_fname;
+    size_t k = p.rfind('/');
+    return k == std::string::npos ? "." : p.substr(0, k);
+  }
+  return ".";
+}
+
+static const char* kCompileOptions[] = {
+    "--offload-arch=gfx950", "-O3", "-std=c++17", "-ffp-contract=off",
+    // packed fp32 instructions are kept out of generated code on this target
+    "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"};
+static const int kNumCompileOptions = sizeof(kCompileOptions) / sizeof(kCompileOptions[0]);
+
+Context::Context(int device) : device_(device) {
+  const char* cd = std::getenv("ACCHIP_CACHE_DIR");
+  cacheDir = cd ? cd : libraryDir() + "/kcache";
+  const char* fl = std::getenv("ACCHIP_FLAGS");
+  if (fl) {
+    std::string f = fl;
+    dumpCC = f.find("dump-cc") != std::string::npos;
+    dumpExec = f.find("dump-exec") != std::string::npos;
+    forceRecomp = f.find("force-recomp") != std::string::npos;
+  }
+  if (device_ >= 0) {
+    hipCheck(hipSetDevice(device_), "hipSetDevice");
+    hipCheck(hipStreamCreateWithFlags(&stream_, hipStreamNonBlocking), "hipStreamCreate");
+  }
+}
+
+Context::~Context() {
+  if (device_ < 0) return;
+  (void)hipSetDevice(device_);
+  (void)hipStreamSynchronize(stream_);
+  for (auto& kv : kernels_)
+    if (kv.second->module) (void)hipModuleUnload(kv.second->module);
+  purge();
+  for (auto& kv : live_) (void)hipFree(kv.first);
+  if (staging_) (void)hipHostFree(staging_);
+  if (scan_.desc) (void)hipFree(scan_.desc);
+  if (scan_.ticket) (void)hipFree(scan_.ticket);
+  (void)hipStreamDestroy(stream_);
+}
+
+// ------------------------------------------------------------------------------------
+// memory
+
+static size_t roundUp(size_t bytes) {
+  const size_t chunk = 1024;  // remoteAllocationSize default (Array/Remote/Table.hs:180-190)
+  if (bytes == 0) bytes = 1;
+  return (bytes + chunk - 1) / chunk * chunk;
+}
+
+void* Context::malloc(size_t bytes) {
+  if (device_ < 0) return nullptr;
+  size_t n = roundUp(bytes);
+  {
+    std::lock_guard<std::mutex> g(mu_);
+    auto it = nursery_.find(n);
+    if (it != nursery_.end() && !it->second.empty()) {
+      void* p = it->second.back();
+      it->second.pop_back();
+      live_[p] = n;
+      stats.poolHits++;
+      return p;
+    }
+  }
+  stats.poolMisses++;
+  void* p = nullptr;
+  (void)hipSetDevice(device_);
+  hipError_t e = hipMalloc(&p, n);
+  if (e != hipSuccess) {
+    (void)hipGetLastError();
+    // work queued on the stream may still use blocks waiting in the free lists
+    (void)hipStreamSynchronize(stream_);
+    purge();
+    e = hipMalloc(&p, n);
+    if (e != hipSuccess) {
+      (void)hipGetLastError();
+      return nullptr;
+    }
+  }
+  stats.bytesAllocated += (long long)n;
+  std::lock_guard<std::mutex> g(mu_);
+  live_[p] = n;
+  return p;
+}
+
+void Context::free(void* p) {
+  if (!p) return;
+  std::lock_guard<std::mutex> g(mu_);
+  auto it = live_.find(p);
+  if (it == live_.end()) return;  // not ours (or freed twice): ignore, as the reference's table does
+  nursery_[it->second].push_back(p);
+  live_.erase(it);
+}
+
+void Context::purge() {
+  std::map<size_t, std::vector<void*>> take;
+  {
+    std::lock_guard<std::mutex> g(mu_);
+    take.swap(nursery_);
+  }
+  for (auto& kv : take)
+    for (void* p : kv.second) {
+      (void)hipFree(p);
+      stats.bytesEvicted += (long long)kv.first;
+    }
+}
+
+size_t Context::blockSize(void* p) {
+  std::lock_guard<std::mutex> g(mu_);
+  auto it = live_.find(p);
+  return it == live_.end() ? 0 : it->second;
+}
+
+void Context::memInfo(size_t* total, size_t* avail) {
+  *total = *avail = 0;
+  if (device_ < 0) return;
+  hipCheck(hipMemGetInfo(avail, total), "hipMemGetInfo");
+  std::lock_guard<std::mutex> g(mu_);
+  for (auto& kv : nursery_) *avail += kv.first * kv.second.size();  // reusable without asking the driver
+}
+
+void* Context::staging(size_t bytes) {
+  if (bytes > stagingBytes_) {
+    if (staging_) {
+      hipCheck(hipStreamSynchronize(stream_), "hipStreamSynchronize");
+      (void)hipHostFree(staging_);
+      staging_ = nullptr;
+    }
+    hipCheck(hipHostMalloc(&staging_, bytes, hipHostMallocDefault), "hipHostMalloc");
+    stagingBytes_ = bytes;
+  }
+  return staging_;
+}
+
+void Context::poke(void* dev, const void* host, size_t bytes) {
+  if (bytes == 0) return;
+  if (device_ < 0) throw Error("no device");
+  // Pageable host memory is staged through a pinned buffer in 64 MiB pieces.
+  const size_t piece = 64u << 20;
+  const char* src = static_cast<const char*>(host);
+  char* dst = static_cast<char*>(dev);
+  for (size_t off = 0; off < bytes; off += piece) {
+    size_t n = bytes - off < piece ? bytes - off : piece;
+    void* st = staging(n < piece ? n : piece);
+    std::memcpy(st, src + off, n);
+    hipCheck(hipMemcpyAsync(dst + off, st, n, hipMemcpyHostToDevice, stream_), "hipMemcpyAsync(H2D)");
+    hipCheck(hipStreamSynchronize(stream_), "hipStreamSynchronize");  // staging buffer is reused
+  }
+  stats.bytesCopiedToRemote += (long long)bytes;
+}
+
+void Context::peek(void* host, const void* dev, size_t bytes) {
+  if (bytes == 0) return;
+  if (device_ < 0) throw Error("no device");
+  const size_t piece = 64u << 20;
+  char* dst = static_cast<char*>(host);
+  const char* src = static_cast<const char*>(dev);
+  for (size_t off = 0; off < bytes; off += piece) {
+    size_t n = bytes - off < piece ? bytes - off : piece;
+    void* st = staging(n < piece ? n : piece);
+    hipCheck(hipMemcpyAsync(st, src + off, n, hipMemcpyDeviceToHost, stream_), "hipMemcpyAsync(D2H)");
+    hipCheck(hipStreamSynchronize(stream_), "hipStreamSynchronize");
+    std::memcpy(dst + off, st, n);
+  }
+  stats.bytesCopiedFromRemote += (long long)bytes;
+}
+
+void Context::copy(void* dst, const void* src, size_t bytes) {
+  if (bytes == 0) return;
+  hipCheck(hipMemcpyAsync(dst, src, bytes, hipMemcpyDeviceToDevice, stream_), "hipMemcpyAsync(D2D)");
+}
+
+void Context::fill0(void* dev, size_t bytes) {
+  if (bytes == 0) return;
+  hipCheck(hipMemsetAsync(dev, 0, bytes, stream_), "hipMemsetAsync");
+}
+
+void Context::sync() {
+  if (device_ >= 0) hipCheck(hipStreamSynchronize(stream_), "hipStreamSynchronize");
+}
+
+Context::ScanState& Context::scanState(size_t descBytes) {
+  if (!scan_.ticket) {
+    hipCheck(hipMalloc((void**)&scan_.ticket, 256), "hipMalloc(scan ticket)");
+    hipCheck(hipMemsetAsync(scan_.ticket, 0, 256, stream_), "hipMemsetAsync");
+    scan_.ticketBase = 0;
+  }
+  if (descBytes > scan_.descBytes) {
+    if (scan_.desc) {
+      hipCheck(hipStreamSynchronize(stream_), "hipStreamSynchronize");
+      (void)hipFree(scan_.desc);
+    }
+    size_t n = std::max(descBytes, (size_t)4 << 20);
+    hipCheck(hipMalloc(&scan_.desc, n), "hipMalloc(scan descriptors)");
+    hipCheck(hipMemsetAsync(scan_.desc, 0, n, stream_), "hipMemsetAsync");
+    scan_.descBytes = n;
+    scan_.epoch = 0;
+  }
+  if (++scan_.epoch == 0) {  // wrapped: stale flags could alias, start over from a clean slate
+    hipCheck(hipMemsetAsync(scan_.desc, 0, scan_.descBytes, stream_), "hipMemsetAsync");
+    scan_.epoch = 1;
+  }
+  return scan_;
+}
+
+// ------------------------------------------------------------------------------------
+// kernels
+
+static bool readFile(const std::string& path, std::string& out) {
+  std::ifstream f(path, std::ios::binary);
+  if (!f) return false;
+  out.assign(std::istreambuf_iterator<char>(f), std::istreambuf_iterator<char>());
+  return true;
+}
+
+static void writeFile(const std::string& path, const std::string& data) {
+  std::string tmp = path + ".tmp" + std::to_string((long long)getpid());
+  {
+    std::ofstream f(tmp, std::ios::binary);
+    if (!f) return;
+    f.write(data.data(), (std::streamsize)data.size());
+    if (!f) return;
+  }
+  std::rename(tmp.c_str(), path.c_str());
+}
+
+static std::string compileHipRTC(const std::string& source, std::string& log) {
+  hiprtcProgram prog;
+  if (hiprtcCreateProgram(&prog, source.c_str(), "acchip_kernel.hip", 0, nullptr, nullptr) != HIPRTC_SUCCESS)
+    throw Error("hiprtcCreateProgram failed");
+  hiprtcResult r = hiprtcCompileProgram(prog, kNumCompileOptions, kCompileOptions);
+  size_t ls = 0;
+  hiprtcGetProgramLogSize(prog, &ls);
+  log.assign(ls, '\0');
+  if (ls) hiprtcGetProgramLog(prog, &log[0]);
+  if (r != HIPRTC_SUCCESS) {
+    hiprtcDestroyProgram(&prog);
+    throw Error(std::string("hipRTC compilation failed: ") + hiprtcGetErrorString(r) + "\n" + log);
+  }
+  size_t cs = 0;
+  hiprtcGetCodeSize(prog, &cs);
+  std::string code(cs, '\0');
+  hiprtcGetCode(prog, &code[0]);
+  hiprtcDestroyProgram(&prog);
+  return code;
+}
+
+KernelP Context::kernel(const KernelSource& ks) {
+  std::string keyText = ks.source;
+  for (int i = 0; i < kNumCompileOptions; ++i) keyText += std::string("\n//opt ") + kCompileOptions[i];
+  int major = 0, minor = 0;
+  hiprtcVersion(&major, &minor);
+  keyText += "\n//hiprtc " + std::to_string(major) + "." + std::to_string(minor);
+  std::string hash = sha3_256_hex(keyText);
+  {
+    std::lock_guard<std::mutex> g(mu_);
+    auto it = kernels_.find(hash);
+    if (it != kernels_.end()) {
+      stats.kernelsFromMemory++;
+      return it->second;
+    }
+  }
+  auto k = std::make_shared<Kernel>();
+  k->hash = hash;
+  k->meta = ks;
+  k->meta.source.clear();
+  std::string path = cacheDir + "/" + hash + ".hsaco";
+  if (dumpCC) fprintf(stderr, "[acchip] kernel %s\n%s\n", hash.c_str(), ks.source.c_str());
+  if (!forceRecomp && readFile(path, k->code) && !k->code.empty()) {
+    stats.kernelsFromDisk++;
+  } else {
+    std::string log;
+    k->code = compileHipRTC(ks.source, log);
+    if (dumpCC && !log.empty()) fprintf(stderr, "[acchip] hipRTC log:\n%s\n", log.c_str());
+    stats.kernelsCompiled++;
+    ::mkdir(cacheDir.c_str(), 0777);
+    writeFile(path, k->code);
+  }
+  std::lock_guard<std::mutex> g(mu_);
+  auto ins = kernels_.emplace(hash, k);
+  return ins.first->second;
+}
+
+void Context::ensureLoaded(const KernelP& k) {
+  if (k->module) return;
+  if (device_ < 0) throw Error("this context has no device: programs can be compiled but not executed");
+  hipCheck(hipModuleLoadData(&k->module, k->code.data()), "hipModuleLoadData");
+}
+
+void Context::launch(const KernelP& k, const char* fn, unsigned grid, unsigned block, const std::vector<uint64_t>& args) {
+  if (grid == 0) return;
+  hipFunction_t f;
+  {
+    std::lock_guard<std::mutex> g(mu_);
+    ensureLoaded(k);
+    auto it = k->fns.find(fn);
+    if (it == k->fns.end()) {
+      hipCheck(hipModuleGetFunction(&f, k->module, fn), fn);
+      k->fns[fn] = f;
+    } else {
+      f = it->second;
+    }
+  }
+  size_t size = args.size() * sizeof(uint64_t);
+  void* config[] = {HIP_LAUNCH_PARAM_BUFFER_POINTER, (void*)args.data(), HIP_LAUNCH_PARAM_BUFFER_SIZE, &size,
+                    HIP_LAUNCH_PARAM_END};
+  if (dumpExec) fprintf(stderr, "[acchip] launch %s<<<%u,%u>>> %s (%zu arg bytes)\n", fn, grid, block, k->hash.substr(0, 12).c_str(), size);
+  hipCheck(hipModuleLaunchKernel(f, grid, 1, 1, block, 1, 1, 0, stream_, nullptr, config), "hipModuleLaunchKernel");
+  stats.launches++;
+}
+
+}  // namespace acchip

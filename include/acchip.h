@@ -1,0 +1,137 @@
+/* acchip -- C ABI of the MI355X (gfx950) execution backend for Accelerate programs.
+ *
+ * This is the boundary a `Data.Array.Accelerate.HIP` module binds with `foreign import
+ * ccall`: it stands where the reference's own backend stands, below the optimiser
+ * (`Trafo.convertAfun`) and behind `run / run1 / runN`
+ * (src/Data/Array/Accelerate/Interpreter.hs:93-126).  Citations name the reference
+ * interface each entry point replaces; paths are relative to
+ * src/Data/Array/Accelerate/ of the reference.
+ *
+ * Conventions: every function that can fail returns 0 on success and a non-zero code on
+ * failure, in which case acchip_last_error() describes the failure (thread-local
+ * string).  No C++ exception crosses the boundary.  All handles are opaque.  Nothing in
+ * this library falls back to a CPU implementation: without a GPU, programs can be
+ * compiled (code generation + hipRTC for gfx950) but execution entry points fail.
+ */
+#ifndef ACCHIP_H
+#define ACCHIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define ACCHIP_MAX_RANK 8
+
+typedef struct acchip_ctx acchip_ctx;         /* device + stream + memory pool + kernel cache */
+typedef struct acchip_program acchip_program; /* a prepared array function (result of runN f) */
+typedef struct acchip_array acchip_array;     /* a device-resident array (or tuple of arrays) */
+typedef struct acchip_event acchip_event;     /* a point in the context's stream */
+
+/* error codes */
+enum {
+  ACCHIP_OK = 0,
+  ACCHIP_ERROR = 1,          /* malformed program, type error, internal error: see last_error */
+  ACCHIP_NO_DEVICE = 2,      /* the context owns no GPU */
+  ACCHIP_OUT_OF_MEMORY = 3,  /* "Remote memory exhausted", Array/Remote/LRU.hs:258-303 */
+  ACCHIP_BOUNDS = 4          /* a condition the reference reports via boundsCheck (Error.hs:33-62):
+                                empty fold1, shape mismatch in reshape, empty segment descriptor */
+};
+
+const char* acchip_last_error(void);
+
+/* --- context ---------------------------------------------------------------------- */
+
+/* Create a context on HIP device `device` (one stream, default priority).  device < 0
+ * creates a compile-only context.  Replaces the implicit global state of the reference
+ * interpreter; a compiling backend creates this once per process. */
+int acchip_init(int device, acchip_ctx** out);
+void acchip_shutdown(acchip_ctx* ctx);
+
+/* totalRemoteMem / availableRemoteMem of class RemoteMemory (Array/Remote/Class.hs:47-73). */
+int acchip_mem_info(acchip_ctx* ctx, size_t* total, size_t* available);
+
+/* mallocRemote (Array/Remote/Class.hs:52-54): returns NULL when the device is exhausted
+ * even after releasing the pool's free lists (Array/Remote/Table.hs:194-206); never
+ * aborts.  Thread-safe; may be called from finaliser threads. */
+void* acchip_malloc(acchip_ctx* ctx, size_t bytes);
+/* freeRemote; the block returns to the pool's free list of its size class
+ * (Array/Remote/Nursery.hs:43-113). */
+void acchip_free(acchip_ctx* ctx, void* devptr);
+/* Release every block waiting in the free lists (Table.purge, Table.hs:247-284). */
+void acchip_purge(acchip_ctx* ctx);
+
+/* pokeRemote / peekRemote (Array/Remote/Class.hs:56-62): host <-> device copies through
+ * a pinned staging buffer on the context's stream.  poke is stream-ordered and returns
+ * once the host buffer may be reused; peek returns once the data is in `host`. */
+int acchip_poke(acchip_ctx* ctx, void* devptr, const void* host, size_t bytes);
+int acchip_peek(acchip_ctx* ctx, void* host, const void* devptr, size_t bytes);
+
+/* Counters with the meaning of cbits/monitoring.c:26-32 plus kernel-cache statistics.
+ * names: "bytes_allocated_remote", "bytes_copied_to_remote", "bytes_copied_from_remote",
+ * "bytes_evicted_from_remote", "kernels_compiled", "kernels_from_disk",
+ * "kernels_from_memory", "launches", "pool_hits", "pool_misses".  Unknown name: -1. */
+long long acchip_stat(acchip_ctx* ctx, const char* name);
+
+/* --- events: `Task` of Array/Remote/LRU.hs:105-110 --------------------------------- */
+
+int acchip_event_record(acchip_ctx* ctx, acchip_event** out); /* record on the stream */
+int acchip_event_query(acchip_event* ev, int* completed);     /* Task.completed */
+int acchip_event_sync(acchip_event* ev);
+int acchip_event_elapsed_ms(acchip_event* start, acchip_event* stop, float* ms);
+void acchip_event_destroy(acchip_event* ev);
+int acchip_sync(acchip_ctx* ctx); /* wait for everything queued on the context's stream */
+
+/* --- arrays ------------------------------------------------------------------------ */
+
+/* Describe an array whose buffers the caller owns (e.g. blocks its memory table got from
+ * acchip_malloc): rank, extents (outermost first, row-major: Representation/Shape.hs:98-106)
+ * element type as text ("f32", "(pair (pair unit i32) f32)", ...), and one device pointer
+ * per scalar leaf of the element type in left-to-right order -- the struct-of-arrays
+ * payload of Array/Data.hs:95-119.  The handle does not take ownership of the buffers. */
+int acchip_array_wrap(acchip_ctx* ctx, int rank, const int64_t* shape, const char* elt_type,
+                      void* const* buffers, int n_buffers, acchip_array** out);
+/* Allocate an array from the pool (allocateArray + mallocRemote); owned by the handle. */
+int acchip_array_new(acchip_ctx* ctx, int rank, const int64_t* shape, const char* elt_type, acchip_array** out);
+/* Build / take apart tuples of arrays (Apair / Anil of the array-level language). */
+int acchip_array_pair(acchip_array* a, acchip_array* b, acchip_array** out);
+int acchip_array_unit(acchip_array** out);
+int acchip_array_kind(const acchip_array* a);                 /* 0 unit, 1 array, 2 pair */
+int acchip_array_fst(const acchip_array* a, acchip_array** out);
+int acchip_array_snd(const acchip_array* a, acchip_array** out);
+int acchip_array_rank(const acchip_array* a);
+int acchip_array_shape(const acchip_array* a, int64_t* shape_out /* rank entries */);
+int acchip_array_num_buffers(const acchip_array* a);
+void* acchip_array_buffer(const acchip_array* a, int leaf);   /* device pointer of one leaf */
+size_t acchip_array_buffer_bytes(const acchip_array* a, int leaf);
+const char* acchip_array_elt_type(const acchip_array* a);     /* valid while the handle lives */
+/* Drop a handle; buffers the library allocated return to the pool when the last handle
+ * that shares them is released. */
+void acchip_array_release(acchip_array* a);
+
+/* --- programs ---------------------------------------------------------------------- */
+
+/* Prepare an array function: parse the textual DelayedOpenAfun (Trafo/Delayed.hs:42-59;
+ * one S-expression per constructor, de Bruijn indices as in AST/Idx.hs), infer types,
+ * generate one kernel per array node and compile it for gfx950 (memory cache, then disk
+ * cache keyed by SHA3-256 of the source as in Analysis/Hash.hs:107-111, then hipRTC).
+ * This is everything `runN f` does at partial application (Interpreter.hs:110-118). */
+int acchip_compile(acchip_ctx* ctx, const char* program_text, size_t length, acchip_program** out);
+void acchip_program_release(acchip_program* p);
+int acchip_program_arity(const acchip_program* p);
+int acchip_program_num_kernels(const acchip_program* p);
+
+/* Apply a prepared function to device-resident arguments (the `go` closure returned by
+ * runN, Interpreter.hs:118-126): args[i] is the i-th lambda's argument; uses[k] fills
+ * `(use .. k)` nodes.  All work is queued on the context's stream; the result handle may
+ * be passed to further calls without synchronising.  Results are owned by the library's
+ * pool until released. */
+int acchip_execute(acchip_ctx* ctx, acchip_program* p, acchip_array* const* args, int n_args,
+                   acchip_array* const* uses, int n_uses, acchip_array** result);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* ACCHIP_H */
