@@ -848,6 +848,71 @@ KernelSource Codegen::fold(const Sx& f, const Sx* seed, const Operand& src) {
   return ks;
 }
 
+static int structWords(const std::vector<ST>& leaves) {
+  // size of `struct { leaf0; leaf1; .. }` under the C++ layout rules, in 32-bit words
+  int off = 0, align = 1;
+  for (ST s : leaves) {
+    int a = stSize(s);
+    off = (off + a - 1) / a * a + a;
+    align = std::max(align, a);
+  }
+  if (off == 0) off = 1;
+  off = (off + align - 1) / align * align;
+  return (off + 3) / 4;
+}
+
+KernelSource Codegen::scan(const Sx& f, const Sx* seed, const Operand& src, bool right, int kind) {
+  const TypeP elt = src.r.elt;
+  if (kind != 0 && !seed) throw Error("scan: this variant needs a seed");
+  std::string body;
+  body += std::string("  static constexpr bool kSeeded = ") + (seed ? "true" : "false") + ";\n";
+  body += std::string("  static constexpr bool kRight = ") + (right ? "true" : "false") + ";\n";
+  body += "  static constexpr int kKind = " + std::to_string(kind) + ";\n";
+  auto leaves = typeLeaves(elt);
+  int eltBytes = 0;
+  for (ST s : leaves) eltBytes += stSize(s);
+  {
+    // combine(earlier, later) in traversal order; right scans apply f with the input on the
+    // left (Interpreter.hs:524-526, 547-549)
+    Emit em;
+    em.ind = 4;
+    ValP a = eltVal(elt, "x"), b = eltVal(elt, "y");
+    ValP r = right ? applyFun(f, {b, a}, {}, em) : applyFun(f, {a, b}, {}, em);
+    if (!typeEq(valType(r), elt)) throw Error("scan: combination function does not return the element type");
+    body += fnHead("Elt", "combine", "const Env& env, const Elt& x, const Elt& y") + returnElt(r, em) + "  }\n";
+  }
+  {
+    Emit em;
+    em.ind = 4;
+    if (seed) {
+      ValP z = exp(*seed, {}, em);
+      if (!typeEq(valType(z), elt)) throw Error("scan: seed does not have the element type");
+      returnElt(z, em);
+    } else {
+      em.line("Elt r_{};");
+      em.line("return r_;");
+    }
+    body += fnHead("Elt", "seed", "const Env& env") + em.code + "  }\n";
+  }
+  {
+    Emit em;
+    em.ind = 4;
+    ValP v = operandLinear(src, "i", em);
+    if (!typeEq(valType(v), elt)) throw Error("scan: fused producer does not return the element type");
+    body += fnHead("Elt", "in_linear", "const Env& env, i64 i") + returnElt(v, em) + "  }\n";
+  }
+  // V from the widest leaf; G so that a lane holds about 128 bytes of elements
+  std::vector<ArraySlot> tmpOrder;
+  for (auto& kv : used_) tmpOrder.push_back(kv.second);
+  int vec = vecFor(leaves, tmpOrder);
+  int g = std::max(1, std::min(8, 128 / std::max(1, vec * std::max(1, eltBytes))));
+  body += "  static constexpr int G = " + std::to_string(g) + ";\n";
+  KernelSource ks = finish(body, elt, leaves, "scan.hpp", vec);
+  ks.group = g;
+  ks.words = structWords(leaves);
+  return ks;
+}
+
 KernelSource Codegen::map(const TypeP& outElt, const Sx* f, const Operand& src) {
   Emit em;
   em.ind = 4;

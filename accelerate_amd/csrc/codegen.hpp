@@ -50,6 +50,8 @@ struct KernelSource {
   std::vector<ArraySlot> arrays;      // Env fields, in order (per array: leaf pointers, then extents)
   std::vector<ST> outLeaves;          // element leaves of Spec::Out
   int vec = 1;                        // Spec::V
+  int group = 1;                      // Spec::G (scan: groups per wave)
+  int words = 1;                      // 32-bit words of Spec::Elt (scan descriptors)
   bool commutative = false;
   std::string permuteMode;            // permute only: "atomic", "cas", "lock", "store"
 };
@@ -66,7 +68,8 @@ class Codegen {
   KernelSource zipWith(const TypeP& outElt, const Sx& f, const Operand& a, const Operand& b, int rank);
   KernelSource generate(const ArrayR& out, const Sx& f);
   KernelSource backpermute(int outRank, const Sx& p, const Sx* f, const TypeP& outElt, const Operand& src);
-  KernelSource scan(const Sx& f, const Sx* seed, const Operand& src, bool right);
+  // kind 0: scanl1/scanr1, 1: scanl/scanr, 2: scanl'/scanr' (seed required for 1 and 2)
+  KernelSource scan(const Sx& f, const Sx* seed, const Operand& src, bool right, int kind);
   KernelSource foldSeg(const Sx& f, const Sx* seed, const Operand& src, const Operand& seg, ST segType);
   KernelSource permute(const Sx& f, const ArrayR& dst, const Sx& p, const Operand& src);
   KernelSource stencil(const std::vector<Sx>& patterns, const TypeP& outElt, const Sx& f,

@@ -498,6 +498,23 @@ ATyP Program::prepare(const Sx& n, TEnv& tenv) {
     r.elt = src.r.elt;
     return done(r);
   }
+  if (h == "scan" || h == "scan'") {
+    bool prime = h == "scan'";
+    const std::string& dir = n.at(1).s;
+    if (dir != "l" && dir != "r") throw Error("scan direction must be l or r");
+    Operand src = operandOf(n.at(4), cg, tenv, plan);
+    if (src.r.rank < 1) throw Error("scan: operand must have rank >= 1");
+    const Sx* z = prime ? &n.at(3) : seedOf(n.at(3));
+    int kind = prime ? 2 : (z ? 1 : 0);
+    plan.k = ctx_.kernel(cg.scan(n.at(2), z, src, dir == "r", kind));
+    if (prime) {
+      ArrayR tr = src.r;
+      tr.rank -= 1;
+      plan.ty = atPair(atArr(src.r), atArr(tr));
+      return plan.ty;
+    }
+    return done(src.r);
+  }
   throw Error("unsupported array term '" + h + "'");
 }
 
@@ -786,6 +803,44 @@ AValP Program::eval(const Sx& n, AEnv& aenv) {
     ctx_.launch(plan.k, "acc_fold_main", (unsigned)(rows * bpr), 256, args);
     if (bpr > 1) ctx_.launch(plan.k, "acc_fold_final", (unsigned)rows, 256, args);
     return avArr(out);
+  }
+  if (h == "scan" || h == "scan'") {
+    const bool prime = h == "scan'";
+    const int kind = prime ? 2 : (seeded(n.at(3)) ? 1 : 0);
+    std::vector<DArrayP> temps = evalTemps(plan.temps, aenv);
+    size_t cur = 0;
+    std::vector<int64_t> ext = operandExtent(n.at(4), aenv, plan, temps, cur);
+    const int64_t len = std::max<int64_t>(ext.back(), 0);
+    std::vector<int64_t> outer(ext.begin(), ext.end() - 1);
+    std::vector<int64_t> oshape = outer;
+    oshape.push_back(kind == 1 ? len + 1 : len);
+    const ArrayR& ar = prime ? plan.ty->a->r : plan.ty->r;
+    DArrayP out = alloc(ar, oshape);
+    DArrayP tot = out;
+    if (prime) tot = alloc(plan.ty->b->r, outer);
+    int64_t rows = 1;
+    for (int64_t d : outer) rows *= std::max<int64_t>(d, 0);
+    AValP result = prime ? avPair(avArr(out), avArr(tot)) : avArr(out);
+    if (rows == 0 || (kind == 0 && len == 0)) return result;
+    const KernelSource& m = plan.k->meta;
+    const int64_t tile = (int64_t)4 * m.group * 64 * m.vec;
+    const int64_t tpr = std::max<int64_t>(1, (len + tile - 1) / tile);
+    const int64_t tiles = rows * tpr;
+    if (tiles > 0x7fffffffLL) throw Error("scan: too many tiles for one launch");
+    Context::ScanState& st = ctx_.scanState((size_t)tiles * 2 * m.words * sizeof(uint64_t));
+    std::vector<uint64_t> args = packArgs(m, aenv, temps, {});
+    packOut(args, *out);
+    packOut(args, *tot);
+    args.push_back((uint64_t)rows);
+    args.push_back((uint64_t)len);
+    args.push_back((uint64_t)tpr);
+    args.push_back((uint64_t)(uintptr_t)st.desc);
+    args.push_back((uint64_t)(uintptr_t)st.ticket);
+    args.push_back((uint64_t)st.ticketBase);
+    args.push_back((uint64_t)st.epoch);
+    ctx_.launch(plan.k, "acc_scan", (unsigned)tiles, 256, args);
+    st.ticketBase += (uint64_t)tiles;
+    return result;
   }
   throw Error("unsupported array term '" + h + "'");
 }
