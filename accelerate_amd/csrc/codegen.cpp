@@ -4,6 +4,7 @@
 #include <cstdio>
 #include <cstdlib>
 #include <cstring>
+#include <functional>
 #include <set>
 
 namespace acchip {
@@ -798,7 +799,13 @@ KernelSource Codegen::finish(const std::string& specBody, const TypeP& elt, cons
     for (size_t k = 0; k < el.size(); ++k) s += "    o.o" + std::to_string(k) + "[i] = v.c" + std::to_string(k) + ";\n";
     s += "  }\n";
   }
-  s += "};\n\n" + deviceHeader(skeleton);
+  s += "};\n\n";
+  for (size_t b = 0; b <= skeleton.size();) {  // one or more headers joined by '+'
+    size_t e = skeleton.find('+', b);
+    if (e == std::string::npos) e = skeleton.size();
+    s += deviceHeader(skeleton.substr(b, e - b)) + "\n";
+    b = e + 1;
+  }
   ks.source = std::move(s);
   return ks;
 }
@@ -848,17 +855,84 @@ KernelSource Codegen::fold(const Sx& f, const Sx* seed, const Operand& src) {
   return ks;
 }
 
-static int structWords(const std::vector<ST>& leaves) {
-  // size of `struct { leaf0; leaf1; .. }` under the C++ layout rules, in 32-bit words
-  int off = 0, align = 1;
+// size and alignment of `struct { leaf0; leaf1; .. }` under the C++ layout rules
+static void structLayout(const std::vector<ST>& leaves, int& size, int& align) {
+  int off = 0;
+  align = 1;
   for (ST s : leaves) {
     int a = stSize(s);
     off = (off + a - 1) / a * a + a;
     align = std::max(align, a);
   }
   if (off == 0) off = 1;
-  off = (off + align - 1) / align * align;
-  return (off + 3) / 4;
+  size = (off + align - 1) / align * align;
+}
+static int structWords(const std::vector<ST>& leaves) {
+  int size, align;
+  structLayout(leaves, size, align);
+  return (size + 3) / 4;
+}
+// words of `struct { Elt v; u32 f; }`
+static int flaggedWords(const std::vector<ST>& leaves) {
+  int size, align;
+  structLayout(leaves, size, align);
+  int off = (size + 3) / 4 * 4 + 4;
+  align = std::max(align, 4);
+  return ((off + align - 1) / align * align + 3) / 4;
+}
+
+KernelSource Codegen::foldSeg(const Sx& f, const Sx* seed, const Operand& src, const Operand& seg, ST segType) {
+  const TypeP elt = src.r.elt;
+  std::string body;
+  body += std::string("  static constexpr bool kSeeded = ") + (seed ? "true" : "false") + ";\n";
+  auto leaves = typeLeaves(elt);
+  int eltBytes = 4;
+  for (ST s : leaves) eltBytes += stSize(s);
+  {
+    Emit em;
+    em.ind = 4;
+    ValP r = applyFun(f, {eltVal(elt, "x"), eltVal(elt, "y")}, {}, em);
+    if (!typeEq(valType(r), elt)) throw Error("foldSeg: combination function does not return the element type");
+    body += fnHead("Elt", "combine", "const Env& env, const Elt& x, const Elt& y") + returnElt(r, em) + "  }\n";
+  }
+  {
+    Emit em;
+    em.ind = 4;
+    if (seed) {
+      ValP z = exp(*seed, {}, em);
+      if (!typeEq(valType(z), elt)) throw Error("foldSeg: seed does not have the element type");
+      returnElt(z, em);
+    } else {
+      em.line("Elt r_{};");
+      em.line("return r_;");
+    }
+    body += fnHead("Elt", "seed", "const Env& env") + em.code + "  }\n";
+  }
+  {
+    Emit em;
+    em.ind = 4;
+    ValP v = operandLinear(src, "i", em);
+    if (!typeEq(valType(v), elt)) throw Error("foldSeg: fused producer does not return the element type");
+    body += fnHead("Elt", "in_linear", "const Env& env, i64 i") + returnElt(v, em) + "  }\n";
+  }
+  {
+    Emit em;
+    em.ind = 4;
+    ValP v = operandLinear(seg, "s", em);
+    if (v->k != Val::Leaf || v->st != segType) throw Error("foldSeg: segment descriptor does not have the declared integral type");
+    em.line("return (i64)" + v->ex + ";");
+    body += fnHead("i64", "seg_at", "const Env& env, i64 s") + em.code + "  }\n";
+  }
+  std::vector<ArraySlot> tmpOrder;
+  for (auto& kv : used_)
+    if (kv.second.name != seg.slot) tmpOrder.push_back(kv.second);
+  int vec = vecFor(leaves, tmpOrder);
+  int g = std::max(1, std::min(8, 128 / std::max(1, vec * eltBytes)));
+  body += "  static constexpr int G = " + std::to_string(g) + ";\n";
+  KernelSource ks = finish(body, elt, leaves, "scan.hpp+foldseg.hpp", vec);
+  ks.group = g;
+  ks.words = flaggedWords(leaves);
+  return ks;
 }
 
 KernelSource Codegen::scan(const Sx& f, const Sx* seed, const Operand& src, bool right, int kind) {
@@ -907,7 +981,7 @@ KernelSource Codegen::scan(const Sx& f, const Sx* seed, const Operand& src, bool
   int vec = vecFor(leaves, tmpOrder);
   int g = std::max(1, std::min(8, 128 / std::max(1, vec * std::max(1, eltBytes))));
   body += "  static constexpr int G = " + std::to_string(g) + ";\n";
-  KernelSource ks = finish(body, elt, leaves, "scan.hpp", vec);
+  KernelSource ks = finish(body, elt, leaves, "scan.hpp+scan_kernel.hpp", vec);
   ks.group = g;
   ks.words = structWords(leaves);
   return ks;
@@ -975,6 +1049,215 @@ KernelSource Codegen::backpermute(int outRank, const Sx& p, const Sx* f, const T
   ValP v = operandIndex(src, sx, em);
   ValP r = f ? applyFun(*f, {v}, {}, em) : v;
   if (!typeEq(valType(r), outElt)) throw Error("backpermute: result does not match the declared element type");
+  std::string body = fnHead("Elt", "produce", "const Env& env, i64 i") + returnElt(r, em) + "  }\n";
+  return finish(body, outElt, typeLeaves(outElt), "map.hpp", 0);
+}
+
+// does the function's second argument (the old value) go unused?  `\x _ -> ..`
+static bool ignoresSecond(const Sx& f) {
+  if (!f.is("lam")) return false;
+  const Sx& g = f.at(2);
+  if (!g.is("lam")) return false;
+  struct W {
+    static bool allWild(const Sx& lhs) {
+      if (lhs.is("wild")) return true;
+      if (lhs.is("pair")) return allWild(lhs.at(1)) && allWild(lhs.at(2));
+      return false;
+    }
+  };
+  return W::allWild(g.at(1));
+}
+
+KernelSource Codegen::permute(const Sx& f, const ArrayR& dst, const Sx& p, const Operand& src) {
+  const TypeP elt = dst.elt;
+  if (!typeEq(elt, src.r.elt)) throw Error("permute: source and defaults have different element types");
+  auto leaves = typeLeaves(elt);
+  std::string body;
+  {
+    Emit em;
+    em.ind = 4;
+    ValP r = applyFun(f, {eltVal(elt, "x"), eltVal(elt, "y")}, {}, em);
+    if (!typeEq(valType(r), elt)) throw Error("permute: combination function does not return the element type");
+    body += fnHead("Elt", "combine", "const Env& env, const Elt& x, const Elt& y") + returnElt(r, em) + "  }\n";
+  }
+  {
+    Emit em;
+    em.ind = 4;
+    ValP v = operandLinear(src, "i", em);
+    if (!typeEq(valType(v), elt)) throw Error("permute: fused producer does not return the element type");
+    body += fnHead("Elt", "in_linear", "const Env& env, i64 i") + returnElt(v, em) + "  }\n";
+  }
+  {
+    // source index -> PrimMaybe destination index = (tag, ((), dst))  (AST.hs:202)
+    Emit em;
+    em.ind = 4;
+    declareOut(used_, dst.rank);
+    ArraySlot o = used_.at("out");
+    ValP ssh = operandShape(src, em);
+    ValP ix = fromIndex(src.r.rank, ssh, "i", em);
+    ValP m = applyFun(p, {ix}, {}, em);
+    if (m->k != Val::Pair || m->a->k != Val::Leaf || m->b->k != Val::Pair)
+      throw Error("permute: index function must return a Maybe index (tag, ((), ix))");
+    std::string tag = m->a->ex;
+    em.line("if (" + tag + " == 0) return false;");
+    em.line("j = " + toIndex(shapeOf(o), m->b->b, em) + ";");
+    em.line("return true;");
+    body += fnHead("bool", "target", "const Env& env, i64 i, i64& j") + em.code + "  }\n";
+  }
+  // how to combine into the destination
+  std::string mode = "lock", op;
+  ST st = ST::I32;
+  const bool single = leaves.size() == 1;
+  const bool wide = single && (stSize(leaves[0]) == 4 || stSize(leaves[0]) == 8);
+  if (ignoresSecond(f)) mode = "store";
+  else if (wide && isCommutative(f, &op, &st) && st == leaves[0] &&
+           (op == "add" ? (st != ST::F16) : (op != "mul" && stIsInt(st))))
+    mode = "atomic";
+  else if (wide) mode = "cas";
+  std::string u = "  ACC_DEV void update(const Env& env, const Out& out, i64 j, const Elt& x, u32* locks) {\n";
+  if (mode == "store") {
+    u += "    Elt y_{};\n    store(out, j, combine(env, x, y_));\n";
+  } else if (mode == "atomic") {
+    std::string fn = op == "add" ? "__hip_atomic_fetch_add" : op == "min" ? "__hip_atomic_fetch_min"
+                   : op == "max" ? "__hip_atomic_fetch_max" : op == "band" ? "__hip_atomic_fetch_and"
+                   : op == "bor" ? "__hip_atomic_fetch_or" : "__hip_atomic_fetch_xor";
+    u += "    (void)" + fn + "(&out.o0[j], x.c0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);\n";
+  } else if (mode == "cas") {
+    std::string B = stSize(leaves[0]) == 4 ? "u32" : "u64", T = stName(leaves[0]);
+    u += "    " + B + "* a_ = (" + B + "*)&out.o0[j];\n";
+    u += "    " + B + " old_ = __hip_atomic_load(a_, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);\n";
+    u += "    for (;;) {\n      Elt y_;\n      y_.c0 = __builtin_bit_cast(" + T + ", old_);\n";
+    u += "      Elt r_ = combine(env, x, y_);\n      " + B + " new_ = __builtin_bit_cast(" + B + ", r_.c0);\n";
+    u += "      if (__hip_atomic_compare_exchange_strong(a_, &old_, new_, __ATOMIC_RELAXED, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)) break;\n    }\n";
+  } else {
+    u += "    u32* lk_ = locks + j;\n    bool done_ = false;\n    while (!done_) {\n";
+    u += "      if (__hip_atomic_exchange(lk_, 1u, __ATOMIC_ACQUIRE, __HIP_MEMORY_SCOPE_AGENT) == 0u) {\n        Elt y_;\n";
+    for (size_t k = 0; k < leaves.size(); ++k)
+      u += "        y_.c" + std::to_string(k) + " = __hip_atomic_load(&out.o" + std::to_string(k) + "[j], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);\n";
+    u += "        Elt r_ = combine(env, x, y_);\n";
+    for (size_t k = 0; k < leaves.size(); ++k)
+      u += "        __hip_atomic_store(&out.o" + std::to_string(k) + "[j], r_.c" + std::to_string(k) + ", __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);\n";
+    u += "        __hip_atomic_store(lk_, 0u, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_AGENT);\n        done_ = true;\n      }\n    }\n";
+  }
+  u += "  }\n";
+  // update() uses store()/combine(): it must come after them, and finish() appends load/store
+  // last, so emit our own forward-safe copies by placing update in a trailing block
+  KernelSource ks = finish(body + "//@UPDATE@\n", elt, leaves, "permute.hpp", 1);
+  size_t at = ks.source.find("//@UPDATE@\n");
+  size_t endSpec = ks.source.find("};\n\n", at);
+  ks.source.erase(at, std::strlen("//@UPDATE@\n"));
+  endSpec -= std::strlen("//@UPDATE@\n");
+  ks.source.insert(endSpec, u);
+  ks.permuteMode = mode;
+  return ks;
+}
+
+static int stencilWidth(const Sx& sr) {
+  const std::string& h = sr.head();
+  if (h.compare(0, 4, "unit") == 0) return std::atoi(h.c_str() + 4);
+  if (h.compare(0, 3, "tup") == 0) return std::atoi(h.c_str() + 3);
+  throw Error("malformed stencil pattern " + sr.str());
+}
+
+KernelSource Codegen::stencil(const std::vector<Sx>& patterns, const TypeP& outElt, const Sx& f,
+                              const std::vector<Sx>& boundaries, const std::vector<Operand>& srcs) {
+  Emit em;
+  em.ind = 4;
+  const int rank = srcs.at(0).r.rank;
+  declareOut(used_, rank);
+  ArraySlot o = used_.at("out");
+  ValP focus = fromIndex(rank, shapeOf(o), "i", em);
+  std::vector<std::string> fx;
+  shapeDims(focus, fx);
+
+  std::vector<ValP> stencilArgs;
+  for (size_t a = 0; a < srcs.size(); ++a) {
+    const Operand& src = srcs[a];
+    const Sx& bnd = boundaries[a];
+    const std::string kind = bnd.atom ? bnd.s : bnd.head();
+    if (kind != "clamp" && kind != "mirror" && kind != "wrap" && kind != "constant" && kind != "function")
+      throw Error("unknown stencil boundary '" + kind + "'");
+    std::vector<std::string> dims;
+    {
+      ValP sh = operandShape(src, em);
+      shapeDims(sh, dims);
+    }
+    // bounded (Interpreter.hs:797-839): value of the source at focus + off
+    auto access = [&](const std::vector<int>& off) -> ValP {
+      std::vector<std::string> raw(rank), idx(rank);
+      std::string inside;
+      for (int d = 0; d < rank; ++d) {
+        if (off[d] == 0) {
+          raw[d] = idx[d] = fx[d];
+          continue;
+        }
+        raw[d] = bindLeaf(ST::I64, fx[d] + " + (i64)" + std::to_string(off[d]), em)->ex;
+        const std::string& j = raw[d];
+        const std::string& sz = dims[d];
+        if (kind == "clamp")
+          idx[d] = bindLeaf(ST::I64, off[d] < 0 ? "(" + j + " < 0) ? (i64)0 : " + j
+                                                : "(" + j + " >= " + sz + ") ? " + sz + " - 1 : " + j, em)->ex;
+        else if (kind == "mirror")
+          idx[d] = bindLeaf(ST::I64, off[d] < 0 ? "(" + j + " < 0) ? -" + j + " : " + j
+                                                : "(" + j + " >= " + sz + ") ? " + sz + " - (" + j + " - " + sz + " + 2) : " + j, em)->ex;
+        else if (kind == "wrap")
+          idx[d] = bindLeaf(ST::I64, off[d] < 0 ? "(" + j + " < 0) ? " + sz + " + " + j + " : " + j
+                                                : "(" + j + " >= " + sz + ") ? " + j + " - " + sz + " : " + j, em)->ex;
+        else {
+          idx[d] = j;
+          inside += (inside.empty() ? "" : " && ") + (off[d] < 0 ? "(" + j + " >= 0)" : "(" + j + " < " + sz + ")");
+        }
+      }
+      auto mk = [&](const std::vector<std::string>& c) {
+        ValP v = vUnit();
+        for (int d = 0; d < rank; ++d) v = vPair(v, vLeaf(ST::I64, c[d]));
+        return v;
+      };
+      if ((kind != "constant" && kind != "function") || inside.empty()) return operandIndex(src, mk(idx), em);
+      // Constant / Function: the whole index decides (no per-dimension remapping)
+      Emit ei, eo;
+      ei.ind = eo.ind = em.ind + 2;
+      ValP vin = operandIndex(src, mk(idx), ei);
+      ValP vout = kind == "constant" ? exp(bnd.at(1), {}, eo) : applyFun(bnd.at(1), {mk(raw)}, {}, eo);
+      if (!typeEq(valType(vin), valType(vout))) throw Error("stencil: boundary value does not have the element type");
+      ValP res = declareVars(valType(vin), em);
+      em.line("if (" + inside + ") {");
+      em.code += ei.code;
+      em.ind += 2;
+      assign(res, vin, em);
+      em.ind -= 2;
+      em.line("} else {");
+      em.code += eo.code;
+      em.ind += 2;
+      assign(res, vout, em);
+      em.ind -= 2;
+      em.line("}");
+      return res;
+    };
+    // stencilAccess (Interpreter.hs:670-794): the outermost tuple walks the left-most
+    // dimension, offsets -k..+k left to right
+    struct Rec {
+      static ValP go(const Sx& sr, int dim, int rank, std::vector<int>& off,
+                     const std::function<ValP(const std::vector<int>&)>& access) {
+        int w = stencilWidth(sr), k = w / 2;
+        bool unit = sr.head().compare(0, 4, "unit") == 0;
+        if (unit != (dim == rank - 1)) throw Error("stencil pattern does not match the array rank");
+        if (!unit && (int)sr.size() != w + 1) throw Error("malformed stencil pattern " + sr.str());
+        ValP v = vUnit();
+        for (int d = -k; d <= k; ++d) {
+          off[dim] = d;
+          v = vPair(v, unit ? access(off) : go(sr.at(1 + d + k), dim + 1, rank, off, access));
+        }
+        off[dim] = 0;
+        return v;
+      }
+    };
+    if (rank < 1) throw Error("stencil: rank must be at least 1");
+    std::vector<int> off(rank, 0);
+    stencilArgs.push_back(Rec::go(patterns[a], 0, rank, off, access));
+  }
+  ValP r = applyFun(f, stencilArgs, {}, em);
+  if (!typeEq(valType(r), outElt)) throw Error("stencil: function result does not match the declared element type");
   std::string body = fnHead("Elt", "produce", "const Env& env, i64 i") + returnElt(r, em) + "  }\n";
   return finish(body, outElt, typeLeaves(outElt), "map.hpp", 0);
 }

@@ -138,28 +138,22 @@ ACC_DEV bool acc_lookback(const typename S::Env& env, const u64* rowDesc, i64 ti
   return have;
 }
 
-extern "C" __global__ void __launch_bounds__(ACC_BLOCK)
-acc_scan(Spec::Env env, Spec::Out out, Spec::Out tot, ScanParams p) {
-  typedef Spec S;
-  typedef S::Elt Elt;
+// One tile of a scan over a sequence of n elements: load(t) yields element t, store(t, y)
+// receives val[t] (the inclusive combination up to t, seed included when S::kSeeded).
+// `desc` holds the descriptors of this sequence's tiles.  Called by all threads of the
+// workgroup.
+template <class S, class Load, class Store>
+ACC_DEV void acc_scan_tile(const typename S::Env& env, u64* desc, i64 tiles, i64 tile, i64 n, u64 epoch,
+                           const Load& load, const Store& store) {
+  typedef typename S::Elt Elt;
   typedef AccScanCfg<S> C;
   const int V = C::V, G = C::G, W = C::W;
-  __shared__ i64 sh_tile;
   __shared__ Elt sh_wave[ACC_WAVES];
   __shared__ Elt sh_excl;
   __shared__ int sh_has_excl;
-
-  if (threadIdx.x == 0)
-    sh_tile = (i64)(__hip_atomic_fetch_add(p.ticket, 1ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) - p.ticket_base);
-  __syncthreads();
-  const i64 gtile = sh_tile;
-  const i64 row = gtile / p.tpr;
-  const i64 tile = gtile - row * p.tpr;
-  const i64 n = p.n;
   const int lane = acc_lane(), w = acc_wave();
   const i64 tlo = tile * (i64)C::TILE;
   const i64 wlo = tlo + (i64)w * G * C::GROUP;
-  const i64 inBase = row * n;
 
   // load + lane-local scan; trailing invalid slots repeat the last valid value so that
   // x[g][V-1] is always the lane's total
@@ -171,7 +165,7 @@ acc_scan(Spec::Env env, Spec::Out out, Spec::Out tot, ScanParams p) {
     for (int k = 0; k < V; ++k) {
       const i64 t = t0 + k;
       if (t < n) {
-        Elt e = S::in_linear(env, inBase + (S::kRight ? n - 1 - t : t));
+        Elt e = load(t);
         x[g][k] = k == 0 ? e : S::combine(env, x[g][k - 1], e);
       } else if (k > 0) {
         x[g][k] = x[g][k - 1];
@@ -204,7 +198,7 @@ acc_scan(Spec::Env env, Spec::Out out, Spec::Out tot, ScanParams p) {
   __syncthreads();
 
   // a wave has data only if all earlier waves are full, so validity follows from counts
-  const i64 tcnt = n - tlo;  // elements from the tile's start to the row's end (may exceed TILE)
+  const i64 tcnt = n - tlo;  // elements from the tile's start to the end (may exceed TILE)
   const i64 perWave = (i64)G * C::GROUP;
   i64 wd = tcnt <= 0 ? 0 : (tcnt + perWave - 1) / perWave;
   const int wavesWithData = wd > ACC_WAVES ? ACC_WAVES : (int)wd;
@@ -218,7 +212,6 @@ acc_scan(Spec::Env env, Spec::Out out, Spec::Out tot, ScanParams p) {
     }
   }
 
-  u64* rowDesc = p.desc + (u64)row * (u64)p.tpr * 2 * W;
   if (w == 0) {
     Elt agg;
     bool hasAgg = false;
@@ -229,7 +222,7 @@ acc_scan(Spec::Env env, Spec::Out out, Spec::Out tot, ScanParams p) {
         hasAgg = true;
       }
     }
-    const bool successors = tile + 1 < p.tpr;
+    const bool successors = tile + 1 < tiles;
     Elt excl;
     bool hasExcl = false;
     if (tile == 0) {
@@ -238,14 +231,14 @@ acc_scan(Spec::Env env, Spec::Out out, Spec::Out tot, ScanParams p) {
         hasExcl = true;
       }
     } else {
-      if (lane == 0 && successors && hasAgg) acc_publish<Elt>(rowDesc + (tile * 2 + 0) * W, agg, p.epoch);
-      hasExcl = acc_lookback<S>(env, rowDesc, tile, p.epoch, excl);
+      if (lane == 0 && successors && hasAgg) acc_publish<Elt>(desc + (tile * 2 + 0) * W, agg, epoch);
+      hasExcl = acc_lookback<S>(env, desc, tile, epoch, excl);
     }
     if (lane == 0) {
       if (successors && hasAgg) {
         Elt inc;
         acc_join<S>(env, hasExcl, excl, hasAgg, agg, inc);
-        acc_publish<Elt>(rowDesc + (tile * 2 + 1) * W, inc, p.epoch);
+        acc_publish<Elt>(desc + (tile * 2 + 1) * W, inc, epoch);
       }
       sh_excl = excl;
       sh_has_excl = hasExcl ? 1 : 0;
@@ -256,9 +249,6 @@ acc_scan(Spec::Env env, Spec::Out out, Spec::Out tot, ScanParams p) {
   // prefix of everything before this wave
   Elt base;
   bool hasBase = acc_join<S>(env, sh_has_excl != 0, sh_excl, hasWavePre, wavePre, base);
-
-  const i64 m = S::kKind == 1 ? n + 1 : n;  // entries per output row
-  const i64 outBase = row * m;
 #pragma unroll
   for (int g = 0; g < G; ++g) {
     Elt gb;
@@ -269,21 +259,15 @@ acc_scan(Spec::Env env, Spec::Out out, Spec::Out tot, ScanParams p) {
 #pragma unroll
     for (int k = 0; k < V; ++k) {
       const i64 t = t0 + k;
-      if (t < n) {
-        Elt y = hasLp ? S::combine(env, lp, x[g][k]) : x[g][k];
-        if (S::kKind == 0) {
-          S::store(out, outBase + (S::kRight ? n - 1 - t : t), y);
-        } else {
-          const i64 u = t + 1;
-          if (S::kKind == 2 && u == n) S::store(tot, row, y);
-          else S::store(out, outBase + (S::kRight ? m - 1 - u : u), y);
-        }
-      }
+      if (t < n) store(t, hasLp ? S::combine(env, lp, x[g][k]) : x[g][k]);
     }
   }
-  if (S::kKind != 0 && tile == 0 && threadIdx.x == 0) {
-    Elt z = S::seed(env);
-    if (S::kKind == 2 && n == 0) S::store(tot, row, z);
-    else S::store(out, outBase + (S::kRight ? m - 1 : 0), z);
-  }
+}
+
+ACC_DEV i64 acc_take_ticket(u64* ticket, u64 base) {
+  __shared__ i64 sh_tile;
+  if (threadIdx.x == 0)
+    sh_tile = (i64)(__hip_atomic_fetch_add(ticket, 1ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) - base);
+  __syncthreads();
+  return sh_tile;
 }

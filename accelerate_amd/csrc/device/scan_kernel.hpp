@@ -1,0 +1,35 @@
+// Entry point of the scan skeleton: one workgroup per tile, tiles numbered by ticket in
+// row-major (row, tile-in-row) order; the tile machinery lives in scan.hpp.
+
+extern "C" __global__ void __launch_bounds__(ACC_BLOCK)
+acc_scan(Spec::Env env, Spec::Out out, Spec::Out tot, ScanParams p) {
+  typedef Spec S;
+  typedef S::Elt Elt;
+  const int W = AccScanCfg<S>::W;
+  const i64 gtile = acc_take_ticket(p.ticket, p.ticket_base);
+  const i64 row = gtile / p.tpr;
+  const i64 tile = gtile - row * p.tpr;
+  const i64 n = p.n;
+  const i64 inBase = row * n;
+  const i64 m = S::kKind == 1 ? n + 1 : n;  // entries per output row
+  const i64 outBase = row * m;
+  u64* rowDesc = p.desc + (u64)row * (u64)p.tpr * 2 * W;
+
+  auto load = [&](i64 t) -> Elt { return S::in_linear(env, inBase + (S::kRight ? n - 1 - t : t)); };
+  auto store = [&](i64 t, const Elt& y) {
+    if (S::kKind == 0) {
+      S::store(out, outBase + (S::kRight ? n - 1 - t : t), y);
+    } else {
+      const i64 u = t + 1;
+      if (S::kKind == 2 && u == n) S::store(tot, row, y);
+      else S::store(out, outBase + (S::kRight ? m - 1 - u : u), y);
+    }
+  };
+  acc_scan_tile<S>(env, rowDesc, p.tpr, tile, n, p.epoch, load, store);
+
+  if (S::kKind != 0 && tile == 0 && threadIdx.x == 0) {
+    Elt z = S::seed(env);
+    if (S::kKind == 2 && n == 0) S::store(tot, row, z);
+    else S::store(out, outBase + (S::kRight ? m - 1 : 0), z);
+  }
+}

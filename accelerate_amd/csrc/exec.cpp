@@ -498,6 +498,52 @@ ATyP Program::prepare(const Sx& n, TEnv& tenv) {
     r.elt = src.r.elt;
     return done(r);
   }
+  if (h == "permute") {
+    // (permute f defaults p source); the defaults operand is always manifest (Fusion.hs:213)
+    ATyP dt = prepare(n.at(2), tenv);
+    ArrayR dr = oneArray(dt, "permute defaults");
+    Operand src = operandOf(n.at(4), cg, tenv, plan);
+    KernelSource ks = cg.permute(n.at(1), dr, n.at(3), src);
+    plan.mode = ks.permuteMode;
+    plan.k = ctx_.kernel(ks);
+    return done(dr);
+  }
+  if (h == "stencil" || h == "stencil2") {
+    const bool two = h == "stencil2";
+    std::vector<Sx> pats, bnds;
+    std::vector<Operand> srcs;
+    TypeP outElt;
+    const Sx* f;
+    if (!two) {
+      pats = {n.at(1)};
+      outElt = parseType(n.at(2));
+      f = &n.at(3);
+      bnds = {n.at(4)};
+      srcs.push_back(operandOf(n.at(5), cg, tenv, plan));
+    } else {
+      pats = {n.at(1), n.at(2)};
+      outElt = parseType(n.at(3));
+      f = &n.at(4);
+      bnds = {n.at(5), n.at(7)};
+      srcs.push_back(operandOf(n.at(6), cg, tenv, plan));
+      srcs.push_back(operandOf(n.at(8), cg, tenv, plan));
+      if (srcs[0].r.rank != srcs[1].r.rank) throw Error("stencil2: operands of different rank");
+    }
+    plan.k = ctx_.kernel(cg.stencil(pats, outElt, *f, bnds, srcs));
+    ArrayR r;
+    r.rank = srcs[0].r.rank;
+    r.elt = outElt;
+    return done(r);
+  }
+  if (h == "foldseg") {
+    ST ity = parseST(n.at(1));
+    if (!stIsInt(ity)) throw Error("foldSeg: segment descriptor must be integral");
+    Operand src = operandOf(n.at(4), cg, tenv, plan);
+    Operand seg = operandOf(n.at(5), cg, tenv, plan);
+    if (src.r.rank < 1 || seg.r.rank != 1) throw Error("foldSeg: operands have the wrong rank");
+    plan.k = ctx_.kernel(cg.foldSeg(n.at(2), seedOf(n.at(3)), src, seg, ity));
+    return done(src.r);
+  }
   if (h == "scan" || h == "scan'") {
     bool prime = h == "scan'";
     const std::string& dir = n.at(1).s;
@@ -802,6 +848,95 @@ AValP Program::eval(const Sx& n, AEnv& aenv) {
     args.push_back((uint64_t)chunk);
     ctx_.launch(plan.k, "acc_fold_main", (unsigned)(rows * bpr), 256, args);
     if (bpr > 1) ctx_.launch(plan.k, "acc_fold_final", (unsigned)rows, 256, args);
+    return avArr(out);
+  }
+  if (h == "permute") {
+    // the destination starts as the defaults; a defaults operand that is not a variable is
+    // a fresh array nobody else can see and is updated in place (Trafo/Fusion.hs:559-566)
+    AValP dv = eval(n.at(2), aenv);
+    if (dv->k != AVal::Arr) throw Error("permute: defaults must be a single array");
+    DArrayP out = dv->arr;
+    static const char* fresh[] = {"generate", "map", "zipwith", "transform", "backpermute", "fold", "foldseg",
+                                  "scan", "permute", "stencil", "stencil2", "unit"};
+    bool inPlace = false;
+    for (const char* k : fresh) inPlace = inPlace || n.at(2).is(k);
+    if (!inPlace) {
+      out = alloc(dv->arr->r, dv->arr->shape);
+      for (size_t k = 0; k < out->bufs.size(); ++k) ctx_.copy(out->bufs[k]->p, dv->arr->bufs[k]->p, out->bufs[k]->bytes);
+    }
+    std::vector<DArrayP> temps = evalTemps(plan.temps, aenv);
+    size_t cur = 0;
+    std::vector<int64_t> ext = operandExtent(n.at(4), aenv, plan, temps, cur);
+    int64_t cnt = 1;
+    for (int64_t d : ext) cnt *= std::max<int64_t>(d, 0);
+    if (cnt == 0 || out->size() == 0) return avArr(out);
+    DArrayP locks;
+    if (plan.mode == "lock") {
+      ArrayR lr;
+      lr.rank = 1;
+      lr.elt = tScalar(ST::U32);
+      locks = alloc(lr, {out->size()});
+      ctx_.fill0(locks->bufs[0]->p, locks->bufs[0]->bytes);
+    }
+    std::vector<uint64_t> args = packArgs(plan.k->meta, aenv, temps, out->shape);
+    packOut(args, *out);
+    args.push_back((uint64_t)cnt);
+    args.push_back(locks ? (uint64_t)(uintptr_t)locks->bufs[0]->p : 0);
+    int64_t grid = std::min<int64_t>((cnt + 255) / 256, 256 * 32);
+    ctx_.launch(plan.k, "acc_permute", (unsigned)grid, 256, args);
+    return avArr(out);
+  }
+  if (h == "stencil" || h == "stencil2") {
+    const bool two = h == "stencil2";
+    std::vector<DArrayP> temps = evalTemps(plan.temps, aenv);
+    size_t cur = 0;
+    std::vector<int64_t> ext = operandExtent(n.at(two ? 6 : 5), aenv, plan, temps, cur);
+    if (two) {
+      std::vector<int64_t> e2 = operandExtent(n.at(8), aenv, plan, temps, cur);
+      for (size_t k = 0; k < ext.size(); ++k) ext[k] = std::min(ext[k], e2[k]);
+    }
+    DArrayP out = alloc(plan.ty->r, ext);
+    launchMap(plan.k, aenv, temps, *out);
+    return avArr(out);
+  }
+  if (h == "foldseg") {
+    std::vector<DArrayP> temps = evalTemps(plan.temps, aenv);
+    size_t cur = 0;
+    std::vector<int64_t> ext = operandExtent(n.at(4), aenv, plan, temps, cur);
+    std::vector<int64_t> sext = operandExtent(n.at(5), aenv, plan, temps, cur);
+    if (sext[0] <= 0) throw Error("empty segment descriptor");  // Interpreter.hs:400
+    const int64_t len = std::max<int64_t>(ext.back(), 0), nseg = sext[0] - 1;
+    std::vector<int64_t> oshape(ext.begin(), ext.end() - 1);
+    int64_t rows = 1;
+    for (int64_t d : oshape) rows *= std::max<int64_t>(d, 0);
+    oshape.push_back(nseg);
+    DArrayP out = alloc(plan.ty->r, oshape);
+    if (rows == 0 || nseg == 0) return avArr(out);
+    const KernelSource& m = plan.k->meta;
+    const int64_t tile = (int64_t)4 * m.group * 64 * m.vec;
+    const int64_t total = rows * len;
+    const int64_t tiles = std::max<int64_t>(1, (total + tile - 1) / tile);
+    if (tiles > 0x7ffffff0LL) throw Error("foldSeg: too many tiles for one launch");
+    ArrayR pr;
+    pr.rank = 1;
+    pr.elt = tScalar(ST::I64);
+    DArrayP part = alloc(pr, {tiles + 1});
+    Context::ScanState& st = ctx_.scanState((size_t)tiles * 2 * m.words * sizeof(uint64_t));
+    std::vector<uint64_t> args = packArgs(m, aenv, temps, {});
+    packOut(args, *out);
+    args.push_back((uint64_t)rows);
+    args.push_back((uint64_t)len);
+    args.push_back((uint64_t)nseg);
+    args.push_back((uint64_t)total);
+    args.push_back((uint64_t)tiles);
+    args.push_back((uint64_t)(uintptr_t)part->bufs[0]->p);
+    args.push_back((uint64_t)(uintptr_t)st.desc);
+    args.push_back((uint64_t)(uintptr_t)st.ticket);
+    args.push_back((uint64_t)st.ticketBase);
+    args.push_back((uint64_t)st.epoch);
+    ctx_.launch(plan.k, "acc_foldseg_partition", (unsigned)((tiles + 1 + 255) / 256), 256, args);
+    ctx_.launch(plan.k, "acc_foldseg", (unsigned)tiles, 256, args);
+    st.ticketBase += (uint64_t)tiles;
     return avArr(out);
   }
   if (h == "scan" || h == "scan'") {
