@@ -4,6 +4,7 @@
 
 #include "../../include/acchip.h"
 #include "exec.hpp"
+#include "sha3.hpp"
 
 using namespace acchip;
 
@@ -304,6 +305,13 @@ int acchip_compile(acchip_ctx* ctx, const char* program_text, size_t length, acc
 void acchip_program_release(acchip_program* p) { delete p; }
 int acchip_program_arity(const acchip_program* p) { return (int)p->prog.argTypes.size(); }
 int acchip_program_num_kernels(const acchip_program* p) { return (int)p->prog.kernelCount(); }
+
+int acchip_sha3_256(const void* data, size_t length, uint8_t digest[32]) {
+  ACCHIP_TRY
+  sha3_256(data, length, digest);
+  return ACCHIP_OK;
+  ACCHIP_END
+}
 
 int acchip_execute(acchip_ctx* ctx, acchip_program* p, acchip_array* const* args, int n_args,
                    acchip_array* const* uses, int n_uses, acchip_array** result) {

@@ -77,6 +77,7 @@ def lib():
         "acchip_program_release": (None, [vp]),
         "acchip_program_arity": (C.c_int, [vp]),
         "acchip_program_num_kernels": (C.c_int, [vp]),
+        "acchip_sha3_256": (C.c_int, [vp, C.c_size_t, C.c_char_p]),
         "acchip_execute": (C.c_int, [vp, vp, C.POINTER(vp), C.c_int, C.POINTER(vp), C.c_int, C.POINTER(vp)]),
     }
     for name, (res, args) in sigs.items():
@@ -272,14 +273,15 @@ class Program:
     def __init__(self, ctx, program):
         self.ctx = ctx
         self.text = program.text() if isinstance(program, ir.Node) else str(program)
+        self._h = C.c_void_p()
+        raw = self.text.encode()
+        _check(lib().acchip_compile(ctx._h, raw, len(raw), C.byref(self._h)))
+        # the library accepted the text, so it is well formed: read the argument types off it
         sx = _parse_type(self.text)
         self.arg_types = []
         while isinstance(sx, tuple) and sx and sx[0] == "alam":
             self.arg_types.append(_lhs_type(sx[1]))
             sx = sx[2]
-        self._h = C.c_void_p()
-        raw = self.text.encode()
-        _check(lib().acchip_compile(ctx._h, raw, len(raw), C.byref(self._h)))
 
     @property
     def num_kernels(self):

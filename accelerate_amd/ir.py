@@ -433,6 +433,13 @@ def shape(av):
     return Raw("shape", _AIdx(av))
 
 
+def untup_shape(av):
+    """Extents of an array variable as a list of expressions, outermost first."""
+    rank = int(av.ty[1])
+    sht = tshape(rank)
+    return [let(sht, shape(av), (lambda k: lambda s: _untup(s)[k])(k)) for k in range(rank)]
+
+
 def shapesize(rank, sh_):
     return Raw("shapesize", rank, sh_)
 

@@ -123,6 +123,10 @@ void acchip_program_release(acchip_program* p);
 int acchip_program_arity(const acchip_program* p);
 int acchip_program_num_kernels(const acchip_program* p);
 
+/* SHA3-256 digest used for kernel cache keys; same function as the reference's
+ * Crypto.Hash.XKCP (src/Crypto/Hash/XKCP.hs:93-170, cbits/xkcp SHA3_256). */
+int acchip_sha3_256(const void* data, size_t length, uint8_t digest[32]);
+
 /* Apply a prepared function to device-resident arguments (the `go` closure returned by
  * runN, Interpreter.hs:118-126): args[i] is the i-th lambda's argument; uses[k] fills
  * `(use .. k)` nodes.  All work is queued on the context's stream; the result handle may

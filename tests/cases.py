@@ -1,0 +1,187 @@
+"""Test cases shared by the CPU suite (oracle vs. the reference's known answers) and the GPU
+suite (HIP backend vs. oracle and known answers)."""
+from __future__ import annotations
+
+import json
+import os
+
+import numpy as np
+
+from accelerate_amd import ir as A
+from accelerate_amd import programs as P
+
+from . import progs as Q
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+VEC = json.load(open(os.path.join(HERE, "golden", "vectors.json")))
+I64 = np.int64
+
+
+def golden_cases():
+    """(id, program, args, expected): expected is what the reference's own doctests /
+    regression tests state (tests/golden/vectors.json)."""
+    v = VEC
+    out = []
+    add = lambda *c: out.append(c)
+    add("fold_sum_seed42", P.fold_sum(A.Int, 2, 42), [np.array(v["fold_sum_seed42"]["mat"], I64)],
+        np.array(v["fold_sum_seed42"]["expected"], I64))
+    add("mss", Q.mss(), [np.array(v["mss"]["vec"], I64)], np.array(v["mss"]["expected"], I64))
+    add("scanl_vec", P.scan_sum("l", A.Int, 1, v["scanl_vec"]["seed"]), [np.array(v["scanl_vec"]["vec"], I64)],
+        np.array(v["scanl_vec"]["expected"], I64))
+    add("scanl_mat", P.scan_sum("l", A.Int, 2, 0), [np.array(v["scanl_mat"]["mat"], I64)],
+        np.array(v["scanl_mat"]["expected"], I64))
+    add("scanl_prime_vec", P.scan_prime_sum("l", A.Int, 1, 0), [np.array(v["scanl_prime_vec"]["vec"], I64)],
+        (np.array(v["scanl_prime_vec"]["expected"], I64), np.array(v["scanl_prime_vec"]["expected_sum"], I64)))
+    add("scanl_prime_mat", P.scan_prime_sum("l", A.Int, 2, 0), [np.array(v["scanl_prime_mat"]["mat"], I64)],
+        (np.array(v["scanl_prime_mat"]["expected"], I64), np.array(v["scanl_prime_mat"]["expected_sum"], I64)))
+    add("scanl1_mat", P.scanl1_sum(A.Int, 2), [np.array(v["scanl1_mat"]["mat"], I64)],
+        np.array(v["scanl1_mat"]["expected"], I64))
+    r, c = v["misc_scanl1"]["rows"], v["misc_scanl1"]["cols"]
+    arr = np.arange(1, r * c + 1, dtype=I64).reshape(r, c)
+    intsum = lambda n, m: m * (m + 1) // 2 - (n - 1) * n // 2
+    ref = np.array([[intsum(1 + i * c, 1 + i * c + j) for j in range(c)] for i in range(r)], I64)
+    add("misc_scanl1", P.scanl1_sum(A.Int, 2), [arr], ref)
+    add("foldseg_doctest", P.foldseg_sum(A.Int, A.Int, 2, 0),
+        [np.array(v["foldseg_doctest"]["mat"], I64), np.array(v["foldseg_doctest"]["seg"], I64)],
+        np.array(v["foldseg_doctest"]["expected"], I64))
+    add("histogram_doctest", P.histogram(v["histogram_doctest"]["bins"], A.Int, A.Int),
+        [np.array(v["histogram_doctest"]["keys"], I64)], np.array(v["histogram_doctest"]["expected"], I64))
+    add("identity_permute", Q.identity_permute(), [np.array(v["identity_permute"]["n"], I64)],
+        np.array(v["identity_permute"]["expected"], I64))
+    add("transpose_backpermute", Q.transpose(), [np.array(v["transpose_backpermute"]["mat"], I64)],
+        np.array(v["transpose_backpermute"]["expected"], I64))
+    t = v["issue228"]
+    pair_in = [np.array(t["fst"], I64), np.array(t["snd"], I64)]
+    pair_out = [np.array(t["expected"][0], I64), np.array(t["expected"][1], I64)]
+    add("issue228_fold", Q.issue228(True), [pair_in], pair_out)
+    add("issue228_fold1", Q.issue228(False), [pair_in], pair_out)
+    for k in (4, 5):
+        add("issue362_%dtuple" % k, Q.tuple_scanl1(k), [[np.array(v["issue362"]["vec"], I64)] * k],
+            [np.array(v["issue362"]["expected"], I64)] * k)
+    for name in ("issue185_A", "issue185_B"):
+        t = v[name]
+        add(name, Q.scatter(), [np.array(t["to"], I64), np.array(t["over"], I64), np.array(t["xs"], I64)],
+            np.array(t["expected"], I64))
+    t = v["issue185_E"]
+    add("issue185_E", Q.gather(), [np.array(t["from"], I64), np.array(t["xs"], I64)], np.array(t["expected"], I64))
+    t = v["issue137"]
+    a = np.arange(1, t["size"] + 1, dtype=I64)
+    exp = np.array(t["expected"], I64)
+    add("issue137", Q.issue137(), [8 - (a % 17), a // 8], [exp[:, 0].copy(), exp[:, 1].copy()])
+    return out
+
+
+def same(a, b, exact=True, rtol=0.0, atol=0.0):
+    """Structural comparison of results: nested pairs of arrays / lists of leaf arrays."""
+    if isinstance(a, (tuple, list)):
+        return isinstance(b, (tuple, list)) and len(a) == len(b) and all(
+            same(x, y, exact, rtol, atol) for x, y in zip(a, b))
+    a, b = np.asarray(a), np.asarray(b)
+    if a.shape != b.shape:
+        return False
+    if exact:
+        return bool(np.array_equal(a, b, equal_nan=True)) if a.dtype.kind == "f" else bool(np.array_equal(a, b))
+    return bool(np.allclose(a, b, rtol=rtol, atol=atol, equal_nan=True))
+
+
+# ------------------------------------------------------------------------------------------
+# random cases shaped like the reference's property tests (Test/NoFib/Prelude/*.hs): small
+# extents, every rank, empty dimensions, neutral and non-neutral seeds, non-commutative
+# operators, all boundary kinds.  (id, program, args, tolerance): tolerance None = bit-exact.
+
+NPT = {"i8": np.int8, "i16": np.int16, "i32": np.int32, "i64": np.int64, "u8": np.uint8, "u16": np.uint16,
+       "u32": np.uint32, "u64": np.uint64, "f16": np.float16, "f32": np.float32, "f64": np.float64}
+
+
+def _rand(rng, ty, shape, lo=-1000, hi=1000):
+    if ty in A.FLOATING:
+        return rng.uniform(-4, 4, shape).astype(NPT[ty])
+    if ty[0] == "u":
+        lo = 0
+    info = np.iinfo(NPT[ty])
+    return rng.integers(max(lo, info.min), min(hi, info.max), shape, endpoint=True).astype(NPT[ty])
+
+
+SHAPES = {1: [(0,), (1,), (63,), (300,), (5000,)], 2: [(3, 0), (0, 4), (5, 10), (17, 129), (2, 4100)],
+          3: [(2, 3, 0), (3, 4, 50), (2, 2, 700)]}
+
+
+def parity_cases():
+    rng = np.random.default_rng(2024)
+    out = []
+    add = lambda *c: out.append(c)
+    # ---- fold (Prelude/Fold.hs:42-121)
+    for rank, shapes in SHAPES.items():
+        for shp in shapes:
+            for ty in (A.i32, A.i64):
+                x = _rand(rng, ty, shp)
+                add("fold_sum_%s_%s" % (ty, shp), P.fold_sum(ty, rank, 0), [x], None)
+                add("fold_sum_seed_%s_%s" % (ty, shp), P.fold_sum(ty, rank, 42), [x], None)
+                if shp[-1] > 0:
+                    add("fold1_min_%s_%s" % (ty, shp), P.fold1_op(A.min_, ty, rank), [x], None)
+                    add("fold1_max_%s_%s" % (ty, shp), P.fold1_op(A.max_, ty, rank), [x], None)
+            if shp[-1] > 0:
+                add("fold_mss_%s" % (shp,), Q.mss(A.Int, rank), [_rand(rng, A.i64, shp, -100, 100)], None)
+            xf = _rand(rng, A.f32, shp)
+            add("fold_sum_f32_%s" % (shp,), P.fold_sum(A.f32, rank, 0), [xf], 1e-4 * 4 * max(1, shp[-1]))
+    # ---- scans (Prelude/Scan.hs:47-469)
+    for rank, shapes in SHAPES.items():
+        for shp in shapes:
+            x = _rand(rng, A.i64, shp)
+            pr = [_rand(rng, A.i64, shp), _rand(rng, A.i64, shp)]
+            for d in "lr":
+                add("scan_%s_seed_%s" % (d, shp), P.scan_sum(d, A.i64, rank, 7), [x], None)
+                add("scan'_%s_%s" % (d, shp), P.scan_prime_sum(d, A.i64, rank, 0), [x], None)
+                add("scan_interval_%s_%s" % (d, shp), Q.interval_scan(d, "scan", A.Int, rank), [pr], None)
+                add("scan'_interval_%s_%s" % (d, shp), Q.interval_scan(d, "scan'", A.Int, rank), [pr], None)
+                if shp[-1] > 0:
+                    add("scan1_%s_%s" % (d, shp), P.scan1_sum(d, A.i64, rank), [x], None)
+                    add("scan1_interval_%s_%s" % (d, shp), Q.interval_scan(d, "scan1", A.Int, rank), [pr], None)
+        xf = _rand(rng, A.f32, shapes[-1]) + np.float32(4)
+        add("scanl1_f32_%s" % (shapes[-1],), P.scanl1_sum(A.f32, rank), [xf], 1e-4 * 8 * shapes[-1][-1])
+    # ---- foldSeg (Prelude/Fold.hs:102-121): both descriptor types, empty segments, outer rows
+    for ity in (A.i32, A.i64):
+        for shp, nseg in [((0,), 3), ((200,), 1), ((5000,), 64), ((3, 700), 9), ((2, 5, 300), 4), ((9000,), 2500)]:
+            n = shp[-1]
+            cuts = np.sort(rng.integers(0, n + 1, nseg - 1)) if nseg > 1 else np.array([], np.int64)
+            lens = np.diff(np.concatenate([[0], cuts, [n]])).astype(NPT[ity])
+            if nseg > 2:
+                lens[-1] = max(0, int(lens[-1]) - 3)     # leave a few trailing elements in no segment
+            v = _rand(rng, A.i32, shp)
+            add("foldseg_%s_%s_%d" % (ity, shp, nseg), P.foldseg_sum(A.i32, ity, len(shp), 5), [v, lens], None)
+    # ---- permute (Prelude/Permute.hs:46-146): (+) with collisions and drops, every rank pair
+    for sr, dr in [(1, 1), (2, 1), (1, 2), (3, 2), (2, 3)]:
+        sshape = {1: (400,), 2: (13, 31), 3: (4, 5, 21)}[sr]
+        dshape = {1: (37,), 2: (5, 7), 3: (2, 3, 4)}[dr]
+        nd = int(np.prod(dshape))
+        to = rng.integers(-nd // 4, nd, int(np.prod(sshape))).astype(np.int64)  # negatives are dropped
+        for ty in (A.i32, A.i64, A.f32):
+            xs = _rand(rng, ty, sshape, -20, 20)
+            if ty == A.f32:
+                xs = np.round(xs * 4) / 4     # sums of quarters are exact in any order
+            add("permute_add_%s_%d_%d" % (ty, sr, dr), Q.accumulate(ty, sr, dr), [xs, to, _rand(rng, ty, dshape, -5, 5)
+                if ty != A.f32 else np.zeros(dshape, np.float32)], None)
+    # ---- backpermute (Prelude/Backpermute.hs)
+    add("transpose_33x17", Q.transpose(A.i32), [_rand(rng, A.i32, (33, 17))], None)
+    add("gather", Q.gather(A.f32), [rng.integers(0, 100, 257).astype(np.int64), _rand(rng, A.f32, (100,))], None)
+    # ---- stencil (Prelude/Stencil.hs:48-290): 1D/2D/3D, widths 3..9, all five boundary kinds
+    for widths, shp in [([3], (1,)), ([3], (50,)), ([5], (64,)), ([7], (9,)), ([9], (300,)), ([3, 3], (1, 1)),
+                        ([3, 3], (17, 40)), ([5, 5], (9, 11)), ([3, 5], (30, 70)), ([7, 7], (8, 8)),
+                        ([3, 3, 3], (5, 6, 7)), ([3, 3, 3], (2, 1, 9))]:
+        for bname in ("clamp", "mirror", "wrap", "constant", "function"):
+            if bname == "mirror" and any(s < (w // 2) + 1 for w, s in zip(widths, shp)):
+                continue    # mirror needs extent > halo, or the remapped index is still outside
+            if bname == "wrap" and any(s < w // 2 for w, s in zip(widths, shp)):
+                continue
+            b = {"constant": A.constant(A.i64, -3), "function": Q.boundary_function(A.i64, len(shp))}.get(bname, bname)
+            add("stencil_%s_%s_%s" % ("x".join(map(str, widths)), shp, bname),
+                Q.stencil_weighted(A.i64, widths, b), [_rand(rng, A.i64, shp, -9, 9)], None)
+    g = rng.uniform(0, 1, (37, 53)).astype(np.float32)
+    add("jacobi_37x53", P.jacobi_step(), [g], None)
+    add("stencil2_clamp_const", Q.stencil2_sum(A.f32, "clamp", A.constant(A.f32, 0.5)),
+        [g, rng.uniform(0, 1, (40, 50)).astype(np.float32)], None)
+    # ---- the benchmark programs at small size
+    add("dotp_1000", P.dotp(), [_rand(rng, A.f32, (1000,)), _rand(rng, A.f32, (900,))], 1e-4 * 16 * 900)
+    add("histogram_zipf", P.histogram(97), [rng.integers(0, 97, 3000).astype(np.int32)], None)
+    add("map_affine", P.map_affine(), [_rand(rng, A.f32, (1234,))], None)
+    return out

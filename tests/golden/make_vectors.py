@@ -1,0 +1,94 @@
+"""Writes tests/golden/vectors.json: known-answer vectors the reference's own doctests and
+regression tests hold for the hot path (inputs and expected outputs only -- data, no
+code).  Short vectors are transcribed here with the file:line they come from; the long
+expected vector of Issue137 is read out of the reference's test file, which is why this
+script needs the reference tree (default /root/reference) and is run in the build
+container only.  The parity tests read the committed JSON and never the reference.
+
+Usage: python tests/golden/make_vectors.py [/path/to/reference]
+"""
+from __future__ import annotations
+
+import json
+import os
+import re
+import sys
+
+REF = sys.argv[1] if len(sys.argv) > 1 else "/root/reference"
+SRC = os.path.join(REF, "src", "Data", "Array", "Accelerate")
+OUT = os.path.join(os.path.dirname(os.path.abspath(__file__)), "vectors.json")
+
+iota5x10 = [list(range(r * 10, r * 10 + 10)) for r in range(5)]
+iota4x10 = [list(range(r * 10, r * 10 + 10)) for r in range(4)]
+
+V = {}
+
+# Language.hs:473-483  fold (+) 42 over the rows of a 5x10 iota matrix
+V["fold_sum_seed42"] = {"cite": "Language.hs:473-483", "mat": iota5x10, "expected": [87, 187, 287, 387, 487]}
+# Language.hs:516-518  maximum segment sum (non-commutative fold1 over 4-tuples)
+V["mss"] = {"cite": "Language.hs:491-518", "vec": [-2, 1, -3, 4, -1, 2, 1, -5, 4, 0], "expected": 6}
+# Language.hs:595-605  scanl
+V["scanl_vec"] = {"cite": "Language.hs:595-597", "vec": list(range(10)), "seed": 10,
+                  "expected": [10, 10, 11, 13, 16, 20, 25, 31, 38, 46, 55]}
+V["scanl_mat"] = {"cite": "Language.hs:599-605", "mat": iota4x10, "seed": 0, "expected": [
+    [0, 0, 1, 3, 6, 10, 15, 21, 28, 36, 45],
+    [0, 10, 21, 33, 46, 60, 75, 91, 108, 126, 145],
+    [0, 20, 41, 63, 86, 110, 135, 161, 188, 216, 245],
+    [0, 30, 61, 93, 126, 160, 195, 231, 268, 306, 345]]}
+# Language.hs:623-639  scanl'
+V["scanl_prime_vec"] = {"cite": "Language.hs:623-628", "vec": list(range(10)), "seed": 0,
+                        "expected": [0, 0, 1, 3, 6, 10, 15, 21, 28, 36], "expected_sum": 45}
+V["scanl_prime_mat"] = {"cite": "Language.hs:630-639", "mat": iota4x10, "seed": 0, "expected": [
+    [0, 0, 1, 3, 6, 10, 15, 21, 28, 36],
+    [0, 10, 21, 33, 46, 60, 75, 91, 108, 126],
+    [0, 20, 41, 63, 86, 110, 135, 161, 188, 216],
+    [0, 30, 61, 93, 126, 160, 195, 231, 268, 306]], "expected_sum": [45, 145, 245, 345]}
+# Language.hs:653-659  scanl1
+V["scanl1_mat"] = {"cite": "Language.hs:653-659", "mat": iota4x10, "expected": [
+    [0, 1, 3, 6, 10, 15, 21, 28, 36, 45],
+    [10, 21, 33, 46, 60, 75, 91, 108, 126, 145],
+    [20, 41, 63, 86, 110, 135, 161, 188, 216, 245],
+    [30, 61, 93, 126, 160, 195, 231, 268, 306, 345]]}
+# Test/NoFib/Misc/Scanl1.hs:32-39  257x31 scanl1 (+) of [1..] with a closed form
+V["misc_scanl1"] = {"cite": "Test/NoFib/Misc/Scanl1.hs:32-39", "rows": 257, "cols": 31,
+                    "closed_form": "out[i][j] = sum [1+i*cols .. 1+i*cols+j]"}
+# Prelude.hs:689-708  foldSeg with an empty segment
+V["foldseg_doctest"] = {"cite": "Prelude.hs:689-708", "mat": iota5x10, "seg": [1, 4, 0, 3], "expected": [
+    [0, 10, 0, 18], [10, 50, 0, 48], [20, 90, 0, 78], [30, 130, 0, 108], [40, 170, 0, 138]]}
+# Language.hs:716-728  histogram via permute (+)
+V["histogram_doctest"] = {"cite": "Language.hs:716-728",
+                          "keys": [0, 0, 1, 2, 1, 1, 2, 4, 8, 3, 4, 9, 8, 3, 2, 5, 5, 3, 1, 2], "bins": 10,
+                          "expected": [2, 4, 4, 3, 2, 2, 0, 0, 2, 1]}
+# Language.hs:734-749  identity matrix via permute const (source rank 1, destination rank 2)
+V["identity_permute"] = {"cite": "Language.hs:734-749", "n": 5,
+                         "expected": [[1 if i == j else 0 for j in range(5)] for i in range(5)]}
+# Language.hs:821-842  transpose via backpermute
+V["transpose_backpermute"] = {"cite": "Language.hs:821-842", "mat": iota5x10,
+                              "expected": [[r * 10 + c for r in range(5)] for c in range(10)]}
+# Test/NoFib/Issues/Issue228.hs:30-46  non-commutative pair monoid, fold with seed (1,0) and fold1
+V["issue228"] = {"cite": "Test/NoFib/Issues/Issue228.hs:30-46", "fst": [1, 0, 1], "snd": [1, 0, 1],
+                 "seed": [1, 0], "expected": [0, 1]}
+# Test/NoFib/Issues/Issue362.hs:38-71  scanl1 over 4- and 5-tuples
+V["issue362"] = {"cite": "Test/NoFib/Issues/Issue362.hs:38-71", "vec": list(range(10)),
+                 "expected": [0, 1, 3, 6, 10, 15, 21, 28, 36, 45]}
+# Test/NoFib/Issues/Issue185.hs:44-97  scatter / gather
+V["issue185_A"] = {"cite": "Test/NoFib/Issues/Issue185.hs:44-52", "to": [1, 3, 7, 2, 5, 8],
+                   "xs": [1, 9, 6, 4, 4, 2, 5], "over": [0] * 9, "expected": [0, 1, 4, 9, 0, 4, 0, 6, 2]}
+V["issue185_B"] = {"cite": "Test/NoFib/Issues/Issue185.hs:55-63", "to": [1, 3, 7, 2, 5, 8],
+                   "xs": [1, 9, 6], "over": [0] * 9, "expected": [0, 1, 0, 9, 0, 0, 0, 6, 0]}
+V["issue185_E"] = {"cite": "Test/NoFib/Issues/Issue185.hs:96-103", "from": [1, 3, 7, 2, 5, 3],
+                   "xs": [1, 9, 6, 4, 4, 2, 0, 1, 2], "expected": [9, 4, 1, 6, 2, 4]}
+
+# Test/NoFib/Issues/Issue137.hs:33-59  permute with a min-merge combiner over pairs:
+# inputs are closed forms, the 384-entry expected vector is read from the reference's file
+text = open(os.path.join(SRC, "Test", "NoFib", "Issues", "Issue137.hs")).read()
+m = re.search(r"ref1 = fromList \(Z:\.384\) \[(.*?)\]\s*\n", text, re.S)
+pairs = [[int(a), int(b)] for a, b in re.findall(r"\((-?\d+),(-?\d+)\)", m.group(1))]
+assert len(pairs) == 384
+V["issue137"] = {"cite": "Test/NoFib/Issues/Issue137.hs:33-59", "size": 3000, "bins": 384, "inf": 10000,
+                 "values": "abs (8 - (a mod 17)) for a in 1..size", "targets": "a div 8 for a in 1..size",
+                 "expected": pairs}
+
+with open(OUT, "w") as f:
+    json.dump(V, f, indent=1, sort_keys=True)
+print("wrote", OUT, len(V), "vectors")

@@ -1,0 +1,241 @@
+"""Fused terms for the programs the reference's test-suite runs (Test/NoFib/**), written
+with the builder the way Trafo.Fusion would hand them to a backend.  Shared by the CPU
+tests (oracle vs. golden vectors) and the GPU tests (HIP backend vs. oracle)."""
+from __future__ import annotations
+
+from accelerate_amd import ir as A
+
+Int = A.Int
+
+
+def binop(op, ty):
+    return A.lam([ty, ty], lambda x, y: op(ty, x, y))
+
+
+def fold_op(op, ty, rank, z=None):
+    return A.alam([A.tarray(rank, ty)],
+                  lambda xs: A.fold(binop(op, ty), None if z is None else A.const(ty, z), xs))
+
+
+# -- maximum segment sum: fold1 of a non-commutative operator over 4-tuples (Language.hs:491-518)
+def mss(ty=Int, rank=1):
+    t4 = A.ttup(ty, ty, ty, ty)
+
+    def f(x, y):
+        mssx, misx, mcsx, tsx = A.untup(x)
+        mssy, misy, mcsy, tsy = A.untup(y)
+        mx = lambda a, b: A.max_(ty, a, b)
+        return A.tup(mx(mssx, mx(mssy, A.add(ty, mcsx, misy))),
+                     mx(misx, A.add(ty, tsx, misy)),
+                     mx(mcsy, A.add(ty, mcsx, tsy)),
+                     A.add(ty, tsx, tsy))
+
+    def g(x):
+        return A.let(ty, A.max_(ty, x, A.const(ty, 0)), lambda y: A.tup(y, y, y, x))
+
+    def first(v):
+        return A.untup(v)[0]
+
+    # map fst . fold1 f . map g : the inner map fuses into the fold as a Delayed operand, the
+    # outer map is a separate node over the fold's result
+    def body(xs):
+        sht = A.tshape(rank)
+        dl = A.delayed(A.tarray(rank, t4), A.shape(xs),
+                       A.lam([sht], lambda ix: A.let(ty, A.index(xs, A.vexp(ix)), g)),
+                       A.lam([Int], lambda i: A.let(ty, A.linearindex(xs, i), g)))
+        return A.map_(ty, A.lam([t4], first), A.fold(A.lam([t4, t4], f), None, dl))
+
+    return A.alam([A.tarray(rank, ty)], body)
+
+
+# -- Issue228: fold / fold1 with the non-commutative pair monoid merge
+def issue228(seeded):
+    t2 = A.ttup(Int, Int)
+
+    def merge(l, r):
+        onl, lenl = A.untup(l)
+        onr, lenr = A.untup(r)
+        return A.tup(A.mul(Int, onl, onr), A.add(Int, A.mul(Int, onl, lenr), lenl))
+
+    z = A.tup(A.constI(1), A.constI(0)) if seeded else None
+    return A.alam([A.tarray(1, t2)], lambda xs: A.fold(A.lam([t2, t2], merge), z, xs))
+
+
+# -- Issue362: scanl1 of component-wise (+) over k-tuples
+def tuple_scanl1(k, direction="l"):
+    tk = A.ttup(*([Int] * k))
+
+    def f(x, y):
+        return A.tup(*[A.add(Int, a, b) for a, b in zip(A.untup(x), A.untup(y))])
+
+    return A.alam([A.tarray(1, tk)], lambda xs: A.scan(direction, A.lam([tk, tk], f), None, xs))
+
+
+# -- interval monoid of the scan tests (Test/NoFib/Prelude/Scan.hs:745-771): non-commutative
+#    iappend (One x y) (One a b) = One x b with Elem = pair; here the "take leftmost first,
+#    rightmost second" monoid over pairs, identity-free (used with scan*1 and seeded variants)
+def interval_scan(direction, kind, ty=Int, rank=1):
+    t2 = A.ttup(ty, ty)
+
+    def f(x, y):
+        a, _ = A.untup(x)
+        _, d = A.untup(y)
+        return A.tup(a, d)
+
+    fn = A.lam([t2, t2], f)
+    z = A.tup(A.const(ty, -7), A.const(ty, 9))
+    if kind == "scan1":
+        return A.alam([A.tarray(rank, t2)], lambda xs: A.scan(direction, fn, None, xs))
+    if kind == "scan":
+        return A.alam([A.tarray(rank, t2)], lambda xs: A.scan(direction, fn, z, xs))
+    return A.alam([A.tarray(rank, t2)], lambda xs: A.scan_(direction, fn, z, xs))
+
+
+# -- permute const: identity matrix (Language.hs:734-749)
+def identity_permute(ty=Int):
+    sh1, sh2 = A.tshape(1), A.tshape(2)
+
+    def body(n_arr):
+        n = A.index(n_arr, A.nil)
+        return A.permute(
+            A.lam([ty, A.wild(ty)], lambda x, _: x),
+            A.generate(A.tarray(2, ty), A.sh(n, n), A.lam([sh2], lambda ix: A.const(ty, 0))),
+            A.lam([sh1], lambda ix: A.just(A.sh(A.untup(ix)[0], A.untup(ix)[0]))),
+            A.delayed(A.tarray(1, ty), A.sh(n), A.lam([sh1], lambda ix: A.const(ty, 1)),
+                      A.lam([Int], lambda i: A.const(ty, 1))))
+
+    return A.alam([A.tarray(0, Int)], body)
+
+
+# -- scatter to defaults input = permute const defaults (\ix -> Just (to!ix)) input'
+#    with input' = backpermute (shape to `intersect` shape input) id input  (Prelude.hs scatter)
+def scatter(ty=Int):
+    sh1 = A.tshape(1)
+
+    def body(to, over, xs):
+        ext = A.let(sh1, A.shape(to), lambda s1: A.let(sh1, A.shape(xs), lambda s0: A.sh(
+            A.min_(Int, A.untup(s1)[0], A.untup(s0)[0]))))
+        src = A.delayed(A.tarray(1, ty), ext, A.lam([sh1], lambda ix: A.index(xs, A.vexp(ix))),
+                        A.lam([Int], lambda i: A.linearindex(xs, i)))
+        return A.permute(A.lam([ty, A.wild(ty)], lambda x, _: x), over,
+                         A.lam([sh1], lambda ix: A.just(A.sh(A.index(to, A.vexp(ix))))), src)
+
+    return A.alam([A.tarray(1, Int), A.tarray(1, ty), A.tarray(1, ty)], body)
+
+
+# -- accumulate: permute (+) into defaults with an optional drop (Nothing) for negative targets
+def accumulate(ty, src_rank, dst_rank):
+    shs, shd = A.tshape(src_rank), A.tshape(dst_rank)
+
+    def body(xs, to, defaults):
+        def p(ix):
+            lin = A.toindex(src_rank, A.shape(xs), A.vexp(ix))
+            t = A.linearindex(to, lin)
+            return A.let(Int, t, lambda tv: A.cond(
+                A.lt(Int, tv, A.constI(0)), A.nothing(shd),
+                A.just(A.fromindex(dst_rank, A.shape(defaults), tv))))
+        return A.permute(binop(A.add, ty), defaults, A.lam([shs], p), xs)
+
+    return A.alam([A.tarray(src_rank, ty), A.tarray(1, Int), A.tarray(dst_rank, ty)], body)
+
+
+# -- Issue137: permute with a min-merge combiner over pairs (CAS-free path: per-cell locks)
+def issue137():
+    t2 = A.ttup(Int, Int)
+    sh1 = A.tshape(1)
+    inf = A.constI(10000)
+
+    def comb(a12, b12):
+        a1, a2 = A.untup(a12)
+        b1, b2 = A.untup(b12)
+        return A.cond(A.lte(Int, a1, b1), A.tup(a1, A.min_(Int, a2, b1)), A.tup(b1, A.min_(Int, b2, a1)))
+
+    def body(interm, ms):
+        src = A.delayed(A.tarray(1, t2), A.shape(interm),
+                        A.lam([sh1], lambda ix: A.tup(A.abs_(Int, A.index(interm, A.vexp(ix))), inf)),
+                        A.lam([Int], lambda i: A.tup(A.abs_(Int, A.linearindex(interm, i)), inf)))
+        return A.permute(A.lam([t2, t2], comb),
+                         A.generate(A.tarray(1, t2), A.sh(384), A.lam([sh1], lambda ix: A.tup(inf, inf))),
+                         A.lam([sh1], lambda ix: A.just(A.sh(A.index(ms, A.vexp(ix))))), src)
+
+    return A.alam([A.tarray(1, Int), A.tarray(1, Int)], body)
+
+
+# -- backpermute: transpose (Language.hs:821-842) and gather (Issue185 E)
+def transpose(ty=Int):
+    sh2 = A.tshape(2)
+
+    def swap(v):
+        y, x = A.untup(v)
+        return A.sh(x, y)
+
+    return A.alam([A.tarray(2, ty)], lambda m: A.backpermute(
+        2, A.let(sh2, A.shape(m), swap), A.lam([sh2], swap), m))
+
+
+def gather(ty=Int):
+    sh1 = A.tshape(1)
+    return A.alam([A.tarray(1, Int), A.tarray(1, ty)], lambda frm, xs: A.backpermute(
+        1, A.shape(frm), A.lam([sh1], lambda ix: A.sh(A.index(frm, A.vexp(ix)))), xs))
+
+
+# -- stencils: weighted sum of all taps with distinct weights, any rank / width / boundary
+def stencil_weighted(ty, widths, boundary):
+    """widths: stencil width per dimension, outermost first (each 3, 5, 7 or 9)."""
+    rank = len(widths)
+
+    def pattern(d):
+        if d == rank - 1:
+            return A.sunit(widths[d], ty)
+        return A.stup(*[pattern(d + 1) for _ in range(widths[d])])
+
+    sr = pattern(0)
+    counter = [0]
+
+    def weigh(v, d):
+        parts = A.untup(v)
+        if d == rank - 1:
+            terms = []
+            for t in parts:
+                counter[0] += 1
+                terms.append(A.mul(ty, A.const(ty, counter[0]), t))
+        else:
+            terms = [weigh(p, d + 1) for p in parts]
+        acc = terms[0]
+        for t in terms[1:]:
+            acc = A.add(ty, acc, t)
+        return acc
+
+    def f(st):
+        counter[0] = 0
+        return weigh(st, 0)
+
+    return A.alam([A.tarray(rank, ty)],
+                  lambda g: A.stencil(sr, ty, A.lam([A.stencil_type(sr)], f), boundary, g))
+
+
+def boundary_function(ty, rank):
+    """Function boundary: value depends on the (out-of-bounds) index."""
+    sht = A.tshape(rank)
+
+    def g(ix):
+        acc = A.constI(100)
+        for c in A.untup(ix):
+            acc = A.add(Int, A.mul(Int, acc, A.constI(3)), c)
+        return A.fromintegral(Int, ty, acc)
+
+    return A.function(A.lam([sht], g))
+
+
+def stencil2_sum(ty, b1, b2):
+    sr = A.stup(A.sunit(3, ty), A.sunit(3, ty), A.sunit(3, ty))
+
+    def f(s1, s2):
+        a = A.untup(A.untup(s1)[1])  # middle row of the first stencil
+        b = A.untup(s2)              # middle column of the second
+        top, mid, bot = (A.untup(r)[1] for r in b)
+        return A.add(ty, A.add(ty, A.add(ty, a[0], a[2]), A.mul(ty, A.const(ty, 2), mid)), A.sub(ty, top, bot))
+
+    st = A.stencil_type(sr)
+    return A.alam([A.tarray(2, ty), A.tarray(2, ty)],
+                  lambda x, y: A.stencil2(sr, sr, ty, A.lam([st, st], f), b1, x, b2, y))

@@ -1,0 +1,136 @@
+"""Parity of the HIP backend with the oracle, through the C ABI, on a real MI355X.
+
+Bar: bit-exact for every integer / index result and for Float32 code without a reduction
+(map, stencil); Float32 reductions and scans within |gpu - ref| <= 1e-4 * sum |x_i| per
+output element (the tolerance the benchmark definition states), written at each case.
+"""
+import numpy as np
+import pytest
+
+from accelerate_amd import hip
+from accelerate_amd import ir as A
+from accelerate_amd import programs as P
+from accelerate_amd import workloads as W
+from oracle import c as OC
+from oracle import interp as O
+
+from . import progs as Q
+from .cases import golden_cases, parity_cases, same
+
+pytestmark = pytest.mark.gpu
+
+GOLDEN = golden_cases()
+PARITY = parity_cases()
+
+
+def test_native_library_is_what_runs(gpu_ctx):
+    # the shared library is loaded and a device context exists: no eager / CPU path can answer
+    assert hip.lib() is not None and gpu_ctx.mem_info()[0] > 100 << 30
+
+
+@pytest.mark.parametrize("case", GOLDEN, ids=[c[0] for c in GOLDEN])
+def test_reference_known_answers(gpu_ctx, case):
+    _, prog, args, expected = case
+    assert same(gpu_ctx.compile(prog)(*args), expected)
+
+
+@pytest.mark.parametrize("case", PARITY, ids=[c[0] for c in PARITY])
+def test_random_cases_match_oracle(gpu_ctx, case):
+    _, prog, args, tol = case
+    got = gpu_ctx.compile(prog)(*args)
+    exp = O.run_n(prog.text(), *args)
+    if tol is None:
+        assert same(got, exp)
+    else:
+        assert same(got, exp, exact=False, atol=tol)
+
+
+# ---- the five benchmark configurations at the size the oracle's C loops handle in seconds ----
+
+def test_dotp_2pow24(gpu_ctx):
+    n = 1 << 24
+    x, y = W.uniform_f32(n, 1), W.uniform_f32(n, 2)
+    got = gpu_ctx.compile(P.dotp())(x, y)
+    exact = np.dot(x.astype(np.float64), y.astype(np.float64))
+    bound = 1e-4 * np.sum(np.abs(x.astype(np.float64) * y))    # 1e-4 * sum |x_i * y_i|
+    assert abs(float(got) - exact) <= bound
+    assert abs(float(OC.dotp_f32(x, y)) - exact) <= bound      # the sequential reference meets the same bound
+
+
+def test_scanl1_int64_2pow28_bit_exact(gpu_ctx):
+    n = 1 << 28
+    x = W.uniform_int(n, 3)
+    got = gpu_ctx.compile(P.scanl1_sum(A.i64))(x)
+    ref = OC.scanl1_i64(x)
+    assert np.array_equal(got, ref)
+    # size-independent properties: first difference restores the input, last element is the total
+    assert got[0] == x[0] and np.array_equal(np.diff(got), x[1:]) and got[-1] == x.sum()
+
+
+def test_scanl1_float32_2pow28_within_tolerance(gpu_ctx):
+    n = 1 << 28
+    x = W.uniform_f32(n, 4, 0.0, 1.0)
+    got = gpu_ctx.compile(P.scanl1_sum(A.f32))(x)
+    exact = np.cumsum(x, dtype=np.float64)                      # = sum_{k<=i} |x_k| since x >= 0
+    assert np.all(np.abs(got - exact) <= 1e-4 * exact + 1e-30)
+    assert np.all(np.diff(got[:: 1 << 16]) >= 0)                # monotone for non-negative input
+
+
+def test_foldseg_2pow27_bit_exact(gpu_ctx):
+    nseg, total = 1 << 20, 1 << 27
+    lens, vals = W.segment_lengths(nseg, total, 5), W.uniform_int(total, 6, dtype=np.int32)
+    got = gpu_ctx.compile(P.foldseg_sum())(vals, lens)
+    assert np.array_equal(got, OC.foldseg_i32(vals, lens))
+    assert got.sum(dtype=np.int64) & 0xFFFFFFFF == int(vals.sum(dtype=np.int64)) & 0xFFFFFFFF   # sum of sums
+    assert np.all(got[lens == 0] == 0)
+
+
+def test_histogram_2pow26_bit_exact(gpu_ctx):
+    n, nbins = 1 << 26, 1 << 16
+    keys = W.zipf_keys(n, nbins, 7)
+    got = gpu_ctx.compile(P.histogram(nbins))(keys)
+    assert np.array_equal(got, OC.histogram_i32(keys, nbins))
+    assert got.sum(dtype=np.int64) == n and np.array_equal(got, np.bincount(keys, minlength=nbins))
+
+
+def test_jacobi_8192_bit_equal(gpu_ctx):
+    g = W.uniform_f32(8192 * 8192, 8, 0.0, 1.0).reshape(8192, 8192)
+    step = gpu_ctx.compile(P.jacobi_step())
+    d = gpu_ctx.to_device(g, A.tarray(2, A.f32))
+    for _ in range(3):
+        d = step.execute(d)
+    got = d.to_host()
+    assert np.array_equal(got, OC.jacobi_f32(g, 3))             # no reduction, no contraction: bit-equal
+    assert got.min() >= g.min() and got.max() <= g.max()        # averaging never leaves the input's range
+
+
+def test_jacobi_100_iterations_small_grid_bit_equal(gpu_ctx):
+    g = W.uniform_f32(96 * 160, 9, 0.0, 1.0).reshape(96, 160)
+    step = gpu_ctx.compile(P.jacobi_step())
+    d = gpu_ctx.to_device(g, A.tarray(2, A.f32))
+    for _ in range(100):
+        d = step.execute(d)
+    assert np.array_equal(d.to_host(), OC.jacobi_f32(g, 100))
+
+
+# ---- error conventions (Error.hs:33-62) -------------------------------------------------------
+
+def test_fold1_of_empty_is_a_bounds_error(gpu_ctx):
+    with pytest.raises(hip.AccError) as e:
+        gpu_ctx.compile(P.fold1_op(A.add, A.i32, 2))(np.zeros((3, 0), np.int32))
+    assert e.value.code == 4 and "empty array" in str(e.value)
+
+
+def test_empty_segment_descriptor_is_a_bounds_error(gpu_ctx):
+    prog = A.alam([A.tarray(1, A.i32), A.tarray(1, A.i32)], lambda v, offs: A.foldseg(
+        A.i32, Q.binop(A.add, A.i32), A.const(A.i32, 0), v, offs))
+    with pytest.raises(hip.AccError) as e:
+        gpu_ctx.compile(prog)(np.zeros(3, np.int32), np.zeros(0, np.int32))
+    assert e.value.code == 4
+
+
+def test_wrong_argument_type_is_rejected(gpu_ctx):
+    run = gpu_ctx.compile(P.fold_sum(A.i32, 2, 0))
+    wrong = gpu_ctx.to_device(np.zeros((2, 2), np.float32), A.tarray(2, A.f32))
+    with pytest.raises(hip.AccError):
+        run.execute(wrong)

@@ -1,0 +1,48 @@
+"""Every program the GPU suite runs is first generated and compiled for gfx950 here, with no
+GPU: this catches code-generation errors on the CPU and leaves the code objects in the
+in-tree kernel cache that travels to the GPU box.  The oracle is run on the same programs
+so that a case the oracle cannot evaluate fails here and not on the GPU box."""
+import pytest
+
+from oracle import interp as O
+
+from .cases import parity_cases
+from .runtime_cases import jacobi_awhile, runtime_cases
+from .scalar_cases import scalar_cases
+
+
+def _compile_all(cc_ctx, named_programs):
+    seen = set()
+    for cid, prog in named_programs:
+        text = prog.text()
+        if text in seen:
+            continue
+        seen.add(text)
+        try:
+            assert cc_ctx.compile(prog).num_kernels >= 0
+        except Exception as e:  # name the program that failed
+            pytest.fail("%s: %s" % (cid, e))
+
+
+def test_all_parity_programs_compile(cc_ctx):
+    _compile_all(cc_ctx, [(c[0], c[1]) for c in parity_cases()])
+
+
+def test_all_scalar_programs_compile_and_oracle_evaluates_them(cc_ctx):
+    cases = scalar_cases()
+    _compile_all(cc_ctx, [(c[0], c[1]) for c in cases])
+    for cid, prog, args, _ in cases:
+        try:
+            O.run_n(prog.text(), *args)
+        except Exception as e:
+            pytest.fail("oracle on %s: %r" % (cid, e))
+
+
+def test_all_runtime_programs_compile_and_oracle_evaluates_them(cc_ctx):
+    cases = runtime_cases()
+    _compile_all(cc_ctx, [(c[0], c[1]) for c in cases] + [("jacobi_awhile", jacobi_awhile(20))])
+    for cid, prog, args, uses in cases:
+        try:
+            O.run_n(prog.text(), *args, uses=[O.to_arr(u, t) for u, t in uses])
+        except Exception as e:
+            pytest.fail("oracle on %s: %r" % (cid, e))
