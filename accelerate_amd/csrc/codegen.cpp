@@ -1130,8 +1130,12 @@ KernelSource Codegen::permute(const Sx& f, const ArrayR& dst, const Sx& p, const
     u += "      Elt r_ = combine(env, x, y_);\n      " + B + " new_ = __builtin_bit_cast(" + B + ", r_.c0);\n";
     u += "      if (__hip_atomic_compare_exchange_strong(a_, &old_, new_, __ATOMIC_RELAXED, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)) break;\n    }\n";
   } else {
-    u += "    u32* lk_ = locks + j;\n    bool done_ = false;\n    while (!done_) {\n";
-    u += "      if (__hip_atomic_exchange(lk_, 1u, __ATOMIC_ACQUIRE, __HIP_MEMORY_SCOPE_AGENT) == 0u) {\n        Elt y_;\n";
+    // The loop runs until every lane of the wave is done (wave-uniform exit through the
+    // ballot).  With a per-lane exit the compiler may move the critical section behind the
+    // loop, where a lane that won the lock waits for the lanes still spinning on it: two
+    // lanes of one wave with the same destination then never finish.
+    u += "    u32* lk_ = locks + j;\n    bool done_ = false;\n    while (__ballot(!done_) != 0ull) {\n";
+    u += "      if (!done_ && __hip_atomic_exchange(lk_, 1u, __ATOMIC_ACQUIRE, __HIP_MEMORY_SCOPE_AGENT) == 0u) {\n        Elt y_;\n";
     for (size_t k = 0; k < leaves.size(); ++k)
       u += "        y_.c" + std::to_string(k) + " = __hip_atomic_load(&out.o" + std::to_string(k) + "[j], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);\n";
     u += "        Elt r_ = combine(env, x, y_);\n";

@@ -162,7 +162,7 @@ class Context:
         parts = list(data) if isinstance(data, (list, tuple)) else [data]
         if len(parts) != len(lv):
             raise ValueError("one numpy array per scalar leaf of the element type")
-        parts = [np.ascontiguousarray(p, dtype=NP[t]) for p, t in zip(parts, lv)]
+        parts = [np.asarray(p, dtype=NP[t], order="C") for p, t in zip(parts, lv)]  # keeps rank 0
         shape = parts[0].shape if parts else ()
         if len(shape) != rank:
             raise ValueError("array of rank %d passed where rank %d is declared" % (len(shape), rank))

@@ -1,0 +1,161 @@
+#!/usr/bin/env python3
+"""Benchmark of the MI355X Accelerate backend on its headline workload.
+
+One step = one application of the prepared program `runN (scanl1 (+))` to a device-resident
+Int64 vector of 2^28 elements (one launch of the single-pass scan kernel), through the C
+ABI.  Prints one JSON line.  The other four configurations and the 2^28 fold / map are
+timed once each and reported under "skeletons" in the same line (skip with --quick).
+
+  python bench.py [--gpus 1] [--steps K] [--warmup W] [--quick] [--no-cpu]
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0   # MI355X HBM3E, published peak
+
+
+def log(*a):
+    print(*a, file=sys.stderr, flush=True)
+
+
+def time_program(ctx, run, args, steps, warmup):
+    """Returns (wall ms per step, event ms per step) over exactly `steps` applications."""
+    for _ in range(warmup):
+        res = run.execute(*args)
+    ctx.sync()
+    e0 = ctx.event()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        res = run.execute(*args)
+    e1 = ctx.event()
+    ctx.sync()
+    wall = (time.perf_counter() - t0) * 1e3 / steps
+    ev = e0.elapsed_ms(e1) / steps
+    del res
+    return wall, ev
+
+
+def entry(name, n, nbytes, ev_ms):
+    gbs = nbytes / ev_ms / 1e6
+    return {"workload": name, "elements": n, "algorithmic_bytes": nbytes, "us": round(ev_ms * 1e3, 2),
+            "gelem_per_s": round(n / ev_ms / 1e6, 2), "gb_per_s": round(gbs, 1), "frac_of_hbm_peak": round(gbs / HBM_PEAK_GBS, 4)}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--quick", action="store_true", help="headline workload only")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
+    a = ap.parse_args()
+    if a.gpus != 1:
+        sys.exit("bench.py: this backend runs on one GPU per process and has no multi-GPU path; "
+                 "run with --gpus 1 (the per-GPU figure is the whole-job figure)")
+
+    from accelerate_amd import hip, ir as A, programs as P, workloads as W
+    ctx = hip.Context(0)   # fails loudly without the HIP library or a GPU: there is no fallback
+
+    # ---- headline: scanl1 (+) on Int64, n = 2^28 -------------------------------------------
+    n = 1 << 28
+    log("generating 2^28 Int64 input ...")
+    x = W.uniform_int(n, 20240601)
+    run = ctx.compile(P.scanl1_sum(A.i64))
+    dx = ctx.to_device(x, A.tarray(1, A.i64))
+    wall, ev = time_program(ctx, run, [dx], a.steps, a.warmup)
+    alg_bytes = 16 * n          # 8 B read + 8 B written per element
+    achieved = alg_bytes / ev / 1e6
+    # cheap integrity check of the timed path: last element equals the total
+    last = run.execute(dx).to_host()[-1]
+    assert int(last) == int(x.sum()), "scan result does not match the input's total"
+
+    cpu = None
+    if not a.no_cpu:
+        from oracle import c as OC
+        reps = 3
+        OC.scanl1_i64(x[: 1 << 20])
+        t0 = time.perf_counter()
+        for _ in range(reps):
+            ref = OC.scanl1_i64(x)
+        dt = (time.perf_counter() - t0) / reps
+        assert int(ref[-1]) == int(last)
+        cpu = {"value": round(n / dt / 1e9, 4), "unit": "Gelem/s", "cores": 1, "kind": "port",
+               "sample": "full workload (2^28 Int64), %d repetitions of oracle/configs.c oracle_scanl1_i64, "
+                         "sequential as the reference interpreter's loop" % reps}
+        del ref
+    del dx
+
+    out = {
+        "metric": "Gelem/s + HBM GB/s (% peak) per skeleton: fold, scan, foldSeg, permute, stencil",
+        "value": round(n / wall / 1e6, 3), "unit": "Gelem/s", "n_gpus": 1, "steps": a.steps, "warmup": a.warmup,
+        "ms_per_step": round(wall, 5), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "int64", "data": "synthetic",
+        "config": {"workload": "scanl1 (+) on an Int64 vector, n=2^28, uniform integers in [-1000,1000]",
+                   "program": "Scan LeftToRight (+) Nothing (Manifest (Avar a0))", "kernel": "acc_scan"},
+        "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None},
+        "cpu_baseline": cpu,
+    }
+
+    # ---- the other configurations, once each ------------------------------------------------
+    if not a.quick:
+        sk = []
+        k, w = max(5, a.steps // 2), 3
+        x32 = W.uniform_f32(n, 11, 0.0, 1.0)
+        d = ctx.to_device(x32, A.tarray(1, A.f32))
+        _, ev = time_program(ctx, ctx.compile(P.scanl1_sum(A.f32)), [d], k, w)
+        sk.append(entry("scanl1 (+) Float32 n=2^28", n, 8 * n, ev))
+        _, ev = time_program(ctx, ctx.compile(P.map_affine()), [d], k, w)
+        sk.append(entry("map (\\x -> 2*x+1) Float32 n=2^28", n, 8 * n, ev))
+        y32 = W.uniform_f32(n, 12)
+        d2 = ctx.to_device(y32, A.tarray(1, A.f32))
+        dot = ctx.compile(P.dotp())
+        _, ev = time_program(ctx, dot, [d, d2], k, w)
+        sk.append(entry("dotp Float32 n=2^28", n, 8 * n, ev))
+        del d, d2
+        m = 1 << 24
+        da, db = ctx.to_device(x32[:m], A.tarray(1, A.f32)), ctx.to_device(y32[:m], A.tarray(1, A.f32))
+        _, ev = time_program(ctx, dot, [da, db], 50, 10)
+        sk.append(entry("dotp Float32 n=2^24 (fits the last-level cache)", m, 8 * m, ev))
+        del da, db, x32, y32
+        nseg, total = 1 << 20, 1 << 27
+        dv = ctx.to_device(W.uniform_int(total, 13, dtype=np.int32), A.tarray(1, A.i32))
+        dl = ctx.to_device(W.segment_lengths(nseg, total, 14), A.tarray(1, A.i32))
+        _, ev = time_program(ctx, ctx.compile(P.foldseg_sum()), [dv, dl], k, w)
+        sk.append(entry("foldSeg (+) 0 Int32, 2^27 values / 2^20 segments (offsets scan included)",
+                        total, 4 * total + 4 * (nseg + 1) + 4 * nseg + 8 * nseg + 4, ev))
+        del dv, dl
+        nk, nb = 1 << 26, 1 << 16
+        dk = ctx.to_device(W.zipf_keys(nk, nb, 15), A.tarray(1, A.i32))
+        _, ev = time_program(ctx, ctx.compile(P.histogram(nb)), [dk], 3, 1)
+        sk.append(entry("histogram: permute (+) of 2^26 Zipf(1.1) keys into 2^16 Int32 bins", nk, 4 * nk + 8 * nb, ev))
+        del dk
+        side = 8192
+        dg = ctx.to_device(W.uniform_f32(side * side, 16, 0.0, 1.0).reshape(side, side), A.tarray(2, A.f32))
+        step = ctx.compile(P.jacobi_step())
+        ctx.sync()
+        e0 = ctx.event()
+        g = dg
+        for _ in range(100):
+            g = step.execute(g)
+        e1 = ctx.event()
+        e1.sync()
+        ev = e0.elapsed_ms(e1) / 100
+        sk.append(entry("Jacobi 3x3 cross, clamp, 8192x8192 Float32, per iteration of 100", side * side, 8 * side * side, ev))
+        out["skeletons"] = sk
+
+    print(json.dumps(out), flush=True)
+
+
+if __name__ == "__main__":
+    main()

@@ -36,15 +36,18 @@ def test_awhile_jacobi_counts_iterations(gpu_ctx):
 def test_pool_reuses_blocks_and_counts_bytes(gpu_ctx):
     ctx = gpu_ctx
     before_hits, before_alloc = ctx.stat("pool_hits"), ctx.stat("bytes_allocated_remote")
-    p = ctx.malloc(5000)
-    assert p and ctx.stat("bytes_allocated_remote") - before_alloc == 5120   # rounded up to 1 KiB chunks
+    ctx.purge()                                     # start from empty free lists
+    before_hits, before_alloc = ctx.stat("pool_hits"), ctx.stat("bytes_allocated_remote")
+    p = ctx.malloc(7777777)
+    rounded = (7777777 + 1023) // 1024 * 1024       # requests are rounded up to 1 KiB chunks
+    assert p and ctx.stat("bytes_allocated_remote") - before_alloc == rounded
     ctx.free(p)
-    q = ctx.malloc(4100)                                                     # same size class: reused
+    q = ctx.malloc(rounded - 5)                     # same size class: the freed block comes back
     assert q == p and ctx.stat("pool_hits") == before_hits + 1
     ctx.free(q)
-    ctx.purge()
     evicted = ctx.stat("bytes_evicted_from_remote")
-    assert evicted >= 5120
+    ctx.purge()
+    assert ctx.stat("bytes_evicted_from_remote") - evicted == rounded
     total, avail = ctx.mem_info()
     assert 0 < avail <= total
 
