@@ -881,6 +881,20 @@ static int flaggedWords(const std::vector<ST>& leaves) {
   return ((off + align - 1) / align * align + 3) / 4;
 }
 
+// bytes of elements a lane holds in a scan tile (tuning knob: ACCHIP_SCAN_BYTES)
+static int scanBytesPerLane() {
+  const char* e = std::getenv("ACCHIP_SCAN_BYTES");
+  int v = e ? std::atoi(e) : 128;
+  return v >= 16 && v <= 512 ? v : 128;
+}
+
+// threads per workgroup of the scan-family kernels (tuning knob: ACCHIP_SCAN_BLOCK)
+static int scanBlock() {
+  const char* e = std::getenv("ACCHIP_SCAN_BLOCK");
+  int v = e ? std::atoi(e) : 1024;
+  return (v == 256 || v == 512 || v == 1024) ? v : 1024;
+}
+
 KernelSource Codegen::foldSeg(const Sx& f, const Sx* seed, const Operand& src, const Operand& seg, ST segType) {
   const TypeP elt = src.r.elt;
   std::string body;
@@ -927,9 +941,11 @@ KernelSource Codegen::foldSeg(const Sx& f, const Sx* seed, const Operand& src, c
   for (auto& kv : used_)
     if (kv.second.name != seg.slot) tmpOrder.push_back(kv.second);
   int vec = vecFor(leaves, tmpOrder);
-  int g = std::max(1, std::min(8, 128 / std::max(1, vec * eltBytes)));
+  int g = std::max(1, std::min(8, scanBytesPerLane() / std::max(1, vec * eltBytes)));
   body += "  static constexpr int G = " + std::to_string(g) + ";\n";
+  body += "#define ACC_SCAN_BLOCK " + std::to_string(scanBlock()) + "\n";
   KernelSource ks = finish(body, elt, leaves, "scan.hpp+foldseg.hpp", vec);
+  ks.block = scanBlock();
   ks.group = g;
   ks.words = flaggedWords(leaves);
   return ks;
@@ -979,9 +995,11 @@ KernelSource Codegen::scan(const Sx& f, const Sx* seed, const Operand& src, bool
   std::vector<ArraySlot> tmpOrder;
   for (auto& kv : used_) tmpOrder.push_back(kv.second);
   int vec = vecFor(leaves, tmpOrder);
-  int g = std::max(1, std::min(8, 128 / std::max(1, vec * std::max(1, eltBytes))));
+  int g = std::max(1, std::min(16, scanBytesPerLane() / std::max(1, vec * std::max(1, eltBytes))));
   body += "  static constexpr int G = " + std::to_string(g) + ";\n";
+  body += "#define ACC_SCAN_BLOCK " + std::to_string(scanBlock()) + "\n";
   KernelSource ks = finish(body, elt, leaves, "scan.hpp+scan_kernel.hpp", vec);
+  ks.block = scanBlock();
   ks.group = g;
   ks.words = structWords(leaves);
   return ks;

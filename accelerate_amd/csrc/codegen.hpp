@@ -52,6 +52,7 @@ struct KernelSource {
   int vec = 1;                        // Spec::V
   int group = 1;                      // Spec::G (scan: groups per wave)
   int words = 1;                      // 32-bit words of Spec::Elt (scan descriptors)
+  int block = 256;                    // threads per workgroup of the main kernel
   bool commutative = false;
   std::string permuteMode;            // permute only: "atomic", "cas", "lock", "store"
 };

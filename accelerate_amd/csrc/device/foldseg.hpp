@@ -83,7 +83,7 @@ acc_foldseg_partition(Spec::Env env, Spec::Out out, FoldSegParams p) {
   p.part[t] = row * sp1 + lo;
 }
 
-extern "C" __global__ void __launch_bounds__(ACC_BLOCK)
+extern "C" __global__ void __launch_bounds__(ACC_SCAN_BLOCK)
 acc_foldseg(Spec::Env env, Spec::Out out, FoldSegParams p) {
   typedef Spec S;
   typedef AccSegSpec<Spec> SS;
@@ -95,9 +95,9 @@ acc_foldseg(Spec::Env env, Spec::Out out, FoldSegParams p) {
   const i64 tlo = tile * (i64)C::TILE;
   const i64 sp1 = p.nseg + 1;
   const i64 j0 = p.part[tile], j1 = p.part[tile + 1];
-  for (int i = threadIdx.x; i <= C::TILE; i += ACC_BLOCK) sh_first[i] = NONE;
+  for (int i = threadIdx.x; i <= C::TILE; i += ACC_SCAN_BLOCK) sh_first[i] = NONE;
   __syncthreads();
-  for (i64 j = j0 + threadIdx.x; j < j1; j += ACC_BLOCK) {
+  for (i64 j = j0 + threadIdx.x; j < j1; j += ACC_SCAN_BLOCK) {
     const i64 row = j / sp1, s = j - row * sp1;
     const i64 o = S::seg_at(env, s);
     const i64 rel = row * p.n + o - tlo;

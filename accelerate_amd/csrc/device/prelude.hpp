@@ -80,12 +80,52 @@ template <class S> ACC_DEV typename S::Elt acc_wave_reduce(const typename S::Env
   return v;
 }
 
-// Ordered inclusive scan across the lanes of a wave (valid lanes must form a prefix).
-template <class S> ACC_DEV typename S::Elt acc_wave_scan(const typename S::Env& env, typename S::Elt v, int lane) {
+// Data-parallel-primitive moves (VALU, no LDS traffic).  Controls of the gfx9 family:
+// row_shr:n = 0x110 + n (shift right by n inside each row of 16 lanes), wave_shr:1 = 0x138
+// (whole wave shifted by one lane), row_bcast:15 = 0x142 (lane 15 of each row to the next
+// row), row_bcast:31 = 0x143 (lane 31 to rows 2 and 3).  Lanes without a source, or in
+// rows the row mask disables, keep their own value.
+template <int CTRL, int ROW_MASK, class T> ACC_DEV T acc_dpp(const T& v) {
+  u32 w[AccWords<T>::N];
+  acc_to_words(v, w);
 #pragma unroll
-  for (int d = 1; d < ACC_WAVE; d <<= 1) {
-    typename S::Elt o = acc_shfl_up(v, d);
-    if (lane >= d) v = S::combine(env, o, v);
+  for (int k = 0; k < AccWords<T>::N; ++k)
+    w[k] = (u32)__builtin_amdgcn_update_dpp((int)w[k], (int)w[k], CTRL, ROW_MASK, 0xf, false);
+  return acc_from_words<T>(w);
+}
+
+// value held by lane `src` (wave-uniform) of the wave
+template <class T> ACC_DEV T acc_readlane(const T& v, int src) {
+  u32 w[AccWords<T>::N];
+  acc_to_words(v, w);
+  const int s = __builtin_amdgcn_readfirstlane(src);
+#pragma unroll
+  for (int k = 0; k < AccWords<T>::N; ++k) w[k] = (u32)__builtin_amdgcn_readlane((int)w[k], s);
+  return acc_from_words<T>(w);
+}
+
+// Ordered inclusive scan across the lanes of a wave (valid lanes must form a prefix):
+// four shifts inside the rows of 16 lanes, then the row totals are handed to the next row
+// and the half totals to the upper half.  Operands stay in lane order, so the operator need
+// only be associative.
+template <class S> ACC_DEV typename S::Elt acc_wave_scan(const typename S::Env& env, typename S::Elt v, int lane) {
+  typedef typename S::Elt Elt;
+  const int rl = lane & 15;
+#define ACC_SCAN_STEP(CTRL, ROWS, COND)             \
+  {                                                 \
+    Elt o_ = acc_dpp<CTRL, ROWS>(v);                \
+    Elt r_ = S::combine(env, o_, v);                \
+    if (COND) v = r_;                               \
   }
+  ACC_SCAN_STEP(0x111, 0xf, rl >= 1)
+  ACC_SCAN_STEP(0x112, 0xf, rl >= 2)
+  ACC_SCAN_STEP(0x114, 0xf, rl >= 4)
+  ACC_SCAN_STEP(0x118, 0xf, rl >= 8)
+  ACC_SCAN_STEP(0x142, 0xa, (lane & 16) != 0)
+  ACC_SCAN_STEP(0x143, 0xc, lane >= 32)
+#undef ACC_SCAN_STEP
   return v;
 }
+
+// value of the previous lane (lane 0 keeps its own)
+template <class T> ACC_DEV T acc_prev_lane(const T& v) { return acc_dpp<0x138, 0xf>(v); }

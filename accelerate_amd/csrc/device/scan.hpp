@@ -13,7 +13,8 @@
 //                            tot[row] = val[n-1], or z when n = 0
 // (entry u lives at position u for left scans and at the mirrored position for right scans).
 //
-// Tile layout: a tile is ACC_WAVES * G * 64 * V consecutive elements of one row.  Wave w
+// Tile layout: a workgroup has 16 waves (1024 threads) and a tile is 16 * G * 64 * V
+// consecutive elements of one row.  Wave w
 // owns G consecutive groups; in a group, lane l owns V consecutive elements, so every
 // load and store of a wave is one coalesced run of 64 * V elements (128 bits per lane for
 // plain arrays).  Order of work: lane-local scan, ordered wave scan per group, chain of
@@ -21,9 +22,15 @@
 // from its predecessors by look-back.
 //
 // Look-back: tiles take their number from an atomic ticket, so a tile only ever waits for
-// tiles that have already started.  Each tile publishes its aggregate, looks back over
-// windows of 64 predecessors with one lane per predecessor, and publishes its inclusive
-// prefix.  A published value is cut into 32-bit words, each stored with a relaxed
+// tiles that have already started.  Each tile publishes its aggregate, looks back, and
+// publishes its inclusive prefix.  One round trip to a predecessor's descriptor costs on
+// the order of a microsecond on this part (device-scope loads cross the XCDs), and the
+// prefix can only advance along the row by (descriptors inspected per round trip) per
+// round trip.  Large tiles (1024 threads x 128 bytes) keep the number of tiles, and with it
+// the number of round trips on the critical path, small; with one workgroup resident per
+// CU the nearest inclusive prefix is a few dozen tiles away, so one wave polling a window of
+// 64 predecessors (one lane each) resolves it in one round trip.  ACC_SCAN_LBWAVES waves can
+// poll further windows in parallel; measured on MI355X more polling only costs.  A published value is cut into 32-bit words, each stored with a relaxed
 // device-scope 64-bit atomic next to the launch's epoch: a word is valid exactly when its
 // upper half equals the epoch, so no fence or initialisation pass is needed, values of
 // any size can be exchanged, and descriptors left by earlier launches read as "not yet".
@@ -32,11 +39,19 @@ struct ScanParams {
   i64 rows;
   i64 n;            // extent of the innermost dimension
   i64 tpr;          // tiles per row (>= 1)
-  u64* desc;        // [rows * tpr][2][W] words: aggregate, inclusive prefix
+  u64* desc;        // [rows * tpr][W] descriptor words
   u64* ticket;      // monotonically increasing counter shared by all launches of a context
   u64 ticket_base;  // value of the counter when this launch starts
-  u64 epoch;        // tag of this launch, never 0
+  u64 epoch;        // tag of this launch, 1 .. 2^30 - 1
 };
+
+#ifndef ACC_SCAN_BLOCK
+#define ACC_SCAN_BLOCK 1024  // threads per workgroup; the generated code may set another size
+#endif
+#define ACC_SCAN_WAVES (ACC_SCAN_BLOCK / ACC_WAVE)
+#ifndef ACC_SCAN_MINWAVES
+#define ACC_SCAN_MINWAVES 4  // waves per SIMD the register allocation must leave room for
+#endif
 
 template <class S> struct AccScanCfg {
   enum {
@@ -44,29 +59,47 @@ template <class S> struct AccScanCfg {
     G = S::G,
     W = AccWords<typename S::Elt>::N,
     GROUP = ACC_WAVE * V,
-    TILE = ACC_WAVES * G * GROUP
+    TILE = ACC_SCAN_WAVES * G * GROUP
   };
 };
 
-template <class E> ACC_DEV void acc_publish(u64* slot, const E& v, u64 epoch) {
+// Descriptor words.  A tile owns W 64-bit words; word k carries the k-th 32-bit word of the
+// published value in its lower half and (epoch << 2 | state) in its upper half, state 1 =
+// the tile's aggregate, 2 = its inclusive prefix (which overwrites the aggregate).  A read
+// is valid when all W words carry the same tag of this launch.
+#ifndef ACC_SCAN_LBWAVES
+#define ACC_SCAN_LBWAVES 1   // waves of the workgroup that poll predecessors (64 each)
+#endif
+#ifndef ACC_SCAN_SLEEP
+#define ACC_SCAN_SLEEP 16    // s_sleep argument between two polls of the same window
+#endif
+
+template <class E> ACC_DEV void acc_publish(u64* slot, const E& v, u64 epoch, u64 state) {
   u32 w[AccWords<E>::N];
   acc_to_words(v, w);
+  const u64 tag = ((epoch << 2) | state) << 32;
 #pragma unroll
   for (int k = 0; k < AccWords<E>::N; ++k)
-    __hip_atomic_store(slot + k, (epoch << 32) | (u64)w[k], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    __hip_atomic_store(slot + k, tag | (u64)w[k], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
-template <class E> ACC_DEV bool acc_try_read(const u64* slot, E& v, u64 epoch) {
+// 0: nothing valid yet, 1: aggregate, 2: inclusive prefix
+template <class E> ACC_DEV int acc_try_read(const u64* slot, E& v, u64 epoch) {
   u32 w[AccWords<E>::N];
-  bool ok = true;
+  u64 tag0 = 0;
+  bool same = true;
 #pragma unroll
   for (int k = 0; k < AccWords<E>::N; ++k) {
     u64 x = __hip_atomic_load(slot + k, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    ok = ok && ((x >> 32) == epoch);
+    if (k == 0) tag0 = x >> 32;
+    same = same && ((x >> 32) == tag0);
     w[k] = (u32)x;
   }
-  if (ok) v = acc_from_words<E>(w);
-  return ok;
+  if (!same || (tag0 >> 2) != epoch) return 0;
+  const int st = (int)(tag0 & 3);
+  if (st != 1 && st != 2) return 0;
+  v = acc_from_words<E>(w);
+  return st;
 }
 
 // a (+) b where either side may be absent
@@ -79,60 +112,96 @@ ACC_DEV bool acc_join(const typename S::Env& env, bool ha, const typename S::Elt
   return ha || hb;
 }
 
-// Exclusive prefix of tile `tile` (> 0) of a row whose descriptors start at `rowDesc`;
-// run by all lanes of one wave, result valid in lane 0.
+// One wave resolves the window of 64 predecessors ending at tile index `look` (lane 0
+// looks at `look`, lane l at look - l).  It polls until it sees, from the nearest
+// predecessor outwards, only aggregates up to the first predecessor that ends the walk (an
+// inclusive prefix, or the start of the row), or 64 aggregates.  On return lane 0 holds in
+// `r` the ordered combination of the `nv` values found (nv may be 0) and `terminal` says
+// whether the walk ends inside this window.
 template <class S>
-ACC_DEV bool acc_lookback(const typename S::Env& env, const u64* rowDesc, i64 tile, u64 epoch, typename S::Elt& excl) {
+ACC_DEV void acc_window(const typename S::Env& env, const u64* rowDesc, i64 look, u64 epoch, typename S::Elt& r,
+                        int& nv, bool& terminal) {
   typedef typename S::Elt Elt;
   const int W = AccScanCfg<S>::W;
   const int lane = acc_lane();
+  const i64 idx = look - lane;
+  int st;  // 0 not yet, 1 aggregate, 2 inclusive prefix, 3 before the row
+  Elt val;
+  int first;
+  for (;;) {
+    st = idx < 0 ? 3 : acc_try_read<Elt>(rowDesc + idx * W, val, epoch);
+    const u64 mEnd = __ballot(st >= 2);
+    const u64 mInv = __ballot(st == 0);
+    first = mEnd ? __builtin_ctzll(mEnd) : ACC_WAVE;
+    const u64 need = first >= 63 ? ~0ull : ((2ull << first) - 1);
+    if ((mInv & need) == 0) break;
+    __builtin_amdgcn_s_sleep(ACC_SCAN_SLEEP);
+  }
+  nv = ACC_WAVE;
+  terminal = first < ACC_WAVE;
+  if (terminal) {
+    const int stEnd = __shfl(st, first, ACC_WAVE);
+    if (stEnd == 3) {
+      if (S::kSeeded) {
+        if (lane == first) val = S::seed(env);
+        nv = first + 1;
+      } else {
+        nv = first;
+      }
+    } else {
+      nv = first + 1;
+    }
+  }
+  // earlier tiles sit in higher lanes: fold them in from the left
+  r = val;
+#pragma unroll
+  for (int d = 1; d < ACC_WAVE; d <<= 1) {
+    Elt o = acc_shfl_down(r, d);
+    if (lane + d < nv) r = S::combine(env, o, r);
+  }
+}
+
+// Exclusive prefix of tile `tile` (> 0) of a row whose descriptors start at `rowDesc`.
+// Called by all threads of the workgroup; the result is valid in thread 0.
+template <class S>
+ACC_DEV bool acc_lookback(const typename S::Env& env, const u64* rowDesc, i64 tile, u64 epoch, typename S::Elt& excl) {
+  typedef typename S::Elt Elt;
+  enum { LB = ACC_SCAN_LBWAVES < ACC_SCAN_WAVES ? ACC_SCAN_LBWAVES : ACC_SCAN_WAVES };
+  __shared__ Elt sh_win[LB];
+  __shared__ int sh_nv[LB];
+  __shared__ int sh_term[LB];
+  __shared__ int sh_done;
+  const int w = acc_wave();
   bool have = false;
   Elt running;
   i64 look = tile - 1;
   for (;;) {
-    const i64 idx = look - lane;  // lane 0 looks at the nearest predecessor
-    int st;                       // 0 not yet, 1 aggregate, 2 inclusive prefix, 3 before the row
-    Elt val;
-    int first;
-    for (;;) {
-      st = 0;
-      if (idx < 0) st = 3;
-      else if (acc_try_read<Elt>(rowDesc + (idx * 2 + 1) * W, val, epoch)) st = 2;
-      else if (acc_try_read<Elt>(rowDesc + (idx * 2 + 0) * W, val, epoch)) st = 1;
-      const u64 mEnd = __ballot(st >= 2);
-      const u64 mInv = __ballot(st == 0);
-      first = mEnd ? __builtin_ctzll(mEnd) : ACC_WAVE;
-      const u64 need = first >= 63 ? ~0ull : ((2ull << first) - 1);
-      if ((mInv & need) == 0) break;
-      __builtin_amdgcn_s_sleep(1);
-    }
-    int nv = ACC_WAVE;
-    if (first < ACC_WAVE) {
-      const int stEnd = __shfl(st, first, ACC_WAVE);
-      if (stEnd == 3) {
-        if (S::kSeeded) {
-          if (lane == first) val = S::seed(env);
-          nv = first + 1;
-        } else {
-          nv = first;
-        }
-      } else {
-        nv = first + 1;
+    if (w < LB) {
+      Elt r;
+      int nv;
+      bool term;
+      acc_window<S>(env, rowDesc, look - (i64)w * ACC_WAVE, epoch, r, nv, term);
+      if (acc_lane() == 0) {
+        sh_win[w] = r;
+        sh_nv[w] = nv;
+        sh_term[w] = term ? 1 : 0;
       }
     }
-    // earlier tiles sit in higher lanes: fold them in from the left
-    Elt r = val;
-#pragma unroll
-    for (int d = 1; d < ACC_WAVE; d <<= 1) {
-      Elt o = acc_shfl_down(r, d);
-      if (lane + d < nv) r = S::combine(env, o, r);
+    __syncthreads();
+    if (threadIdx.x == 0) {
+      int done = 0;
+      for (int k = 0; k < LB && !done; ++k) {  // nearest window first
+        if (sh_nv[k] > 0) {
+          running = have ? S::combine(env, sh_win[k], running) : sh_win[k];
+          have = true;
+        }
+        done = sh_term[k];
+      }
+      sh_done = done;
     }
-    if (nv > 0) {
-      running = have ? S::combine(env, r, running) : r;
-      have = true;
-    }
-    if (first < ACC_WAVE) break;
-    look -= ACC_WAVE;
+    __syncthreads();
+    if (sh_done) break;
+    look -= (i64)LB * ACC_WAVE;
   }
   excl = running;
   return have;
@@ -141,14 +210,14 @@ ACC_DEV bool acc_lookback(const typename S::Env& env, const u64* rowDesc, i64 ti
 // One tile of a scan over a sequence of n elements: load(t) yields element t, store(t, y)
 // receives val[t] (the inclusive combination up to t, seed included when S::kSeeded).
 // `desc` holds the descriptors of this sequence's tiles.  Called by all threads of the
-// workgroup.
+// workgroup (ACC_SCAN_BLOCK threads).
 template <class S, class Load, class Store>
 ACC_DEV void acc_scan_tile(const typename S::Env& env, u64* desc, i64 tiles, i64 tile, i64 n, u64 epoch,
                            const Load& load, const Store& store) {
   typedef typename S::Elt Elt;
   typedef AccScanCfg<S> C;
   const int V = C::V, G = C::G, W = C::W;
-  __shared__ Elt sh_wave[ACC_WAVES];
+  __shared__ Elt sh_wave[ACC_SCAN_WAVES];   // wave totals, then inclusive prefixes of the wave totals
   __shared__ Elt sh_excl;
   __shared__ int sh_has_excl;
   const int lane = acc_lane(), w = acc_wave();
@@ -156,39 +225,60 @@ ACC_DEV void acc_scan_tile(const typename S::Env& env, u64* desc, i64 tiles, i64
   const i64 wlo = tlo + (i64)w * G * C::GROUP;
 
   // load + lane-local scan; trailing invalid slots repeat the last valid value so that
-  // x[g][V-1] is always the lane's total
+  // x[g][V-1] is always the lane's total.  A tile that lies completely inside the sequence
+  // takes the branch without bounds tests, which lets the V consecutive accesses of a lane
+  // become one wide request.
   Elt x[C::G][C::V];
+  const bool full = tlo + (i64)C::TILE <= n;
+  if (full) {
 #pragma unroll
-  for (int g = 0; g < G; ++g) {
-    const i64 t0 = wlo + ((i64)g * ACC_WAVE + lane) * V;
+    for (int g = 0; g < G; ++g) {
+      const i64 t0 = wlo + ((i64)g * ACC_WAVE + lane) * V;
+      Elt e[C::V];
 #pragma unroll
-    for (int k = 0; k < V; ++k) {
-      const i64 t = t0 + k;
-      if (t < n) {
-        Elt e = load(t);
-        x[g][k] = k == 0 ? e : S::combine(env, x[g][k - 1], e);
-      } else if (k > 0) {
-        x[g][k] = x[g][k - 1];
+      for (int k = 0; k < V; ++k) e[k] = load(t0 + k);
+      x[g][0] = e[0];
+#pragma unroll
+      for (int k = 1; k < V; ++k) x[g][k] = S::combine(env, x[g][k - 1], e[k]);
+    }
+  } else {
+#pragma unroll
+    for (int g = 0; g < G; ++g) {
+      const i64 t0 = wlo + ((i64)g * ACC_WAVE + lane) * V;
+#pragma unroll
+      for (int k = 0; k < V; ++k) {
+        const i64 t = t0 + k;
+        if (t < n) {
+          Elt e = load(t);
+          x[g][k] = k == 0 ? e : S::combine(env, x[g][k - 1], e);
+        } else if (k > 0) {
+          x[g][k] = x[g][k - 1];
+        }
       }
     }
   }
 
-  // wave scan per group, then chain the groups of this wave
-  Elt lanePre[C::G];   // exclusive prefix of the lane inside its group (lane > 0)
-  Elt groupPre[C::G];  // exclusive prefix of the group inside its wave
-  bool hasGroupPre[C::G];
+  // Wave scan per group, chained over the groups of this wave; the prefix inside the wave
+  // is applied to the elements at once, so that only x stays live across the look-back.
   Elt waveTot;
   bool hasWaveTot = false;
 #pragma unroll
   for (int g = 0; g < G; ++g) {
     i64 cnt = n - (wlo + (i64)g * C::GROUP);
     cnt = cnt < 0 ? 0 : (cnt > C::GROUP ? C::GROUP : cnt);
+#ifdef ACC_X_NOWAVESCAN
+    Elt ts = x[g][V - 1];
+#else
     Elt ts = acc_wave_scan<S>(env, x[g][V - 1], lane);
-    lanePre[g] = acc_shfl_up(ts, 1);
+#endif
+    Elt lanePre = acc_prev_lane(ts);  // exclusive prefix of the lane inside its group (lane > 0)
     const int last = cnt > 0 ? (int)((cnt - 1) / V) : 0;
-    Elt gt = acc_shfl(ts, last);
-    groupPre[g] = waveTot;
-    hasGroupPre[g] = hasWaveTot;
+    Elt gt = acc_readlane(ts, last);
+    Elt pre;
+    if (acc_join<S>(env, hasWaveTot, waveTot, lane > 0, lanePre, pre)) {
+#pragma unroll
+      for (int k = 0; k < V; ++k) x[g][k] = S::combine(env, pre, x[g][k]);
+    }
     if (cnt > 0) {
       waveTot = hasWaveTot ? S::combine(env, waveTot, gt) : gt;
       hasWaveTot = true;
@@ -201,70 +291,71 @@ ACC_DEV void acc_scan_tile(const typename S::Env& env, u64* desc, i64 tiles, i64
   const i64 tcnt = n - tlo;  // elements from the tile's start to the end (may exceed TILE)
   const i64 perWave = (i64)G * C::GROUP;
   i64 wd = tcnt <= 0 ? 0 : (tcnt + perWave - 1) / perWave;
-  const int wavesWithData = wd > ACC_WAVES ? ACC_WAVES : (int)wd;
-  Elt wavePre;
-  bool hasWavePre = false;
-#pragma unroll
-  for (int k = 0; k < ACC_WAVES; ++k) {
-    if (k < w && k < wavesWithData) {
-      wavePre = hasWavePre ? S::combine(env, wavePre, sh_wave[k]) : sh_wave[k];
-      hasWavePre = true;
-    }
-  }
+  const int wavesWithData = wd > ACC_SCAN_WAVES ? ACC_SCAN_WAVES : (int)wd;
+  const bool successors = tile + 1 < tiles;
 
+  // the first wave scans the wave totals (ordered) and publishes the tile's aggregate
   if (w == 0) {
-    Elt agg;
-    bool hasAgg = false;
-#pragma unroll
-    for (int k = 0; k < ACC_WAVES; ++k) {
-      if (k < wavesWithData) {
-        agg = hasAgg ? S::combine(env, agg, sh_wave[k]) : sh_wave[k];
-        hasAgg = true;
-      }
+    Elt t = sh_wave[lane < ACC_SCAN_WAVES ? lane : 0];
+    t = acc_wave_scan<S>(env, t, lane);
+    if (lane < ACC_SCAN_WAVES) sh_wave[lane] = t;
+    if (lane == wavesWithData - 1 && tile > 0 && successors) acc_publish<Elt>(desc + tile * W, t, epoch, 1);
+  }
+  __syncthreads();
+
+  Elt excl;
+  bool hasExcl = false;
+#ifdef ACC_X_NOLOOKBACK
+  if (true) {
+#else
+  if (tile == 0) {
+#endif
+    if (S::kSeeded) {
+      excl = S::seed(env);
+      hasExcl = true;
     }
-    const bool successors = tile + 1 < tiles;
-    Elt excl;
-    bool hasExcl = false;
-    if (tile == 0) {
-      if (S::kSeeded) {
-        excl = S::seed(env);
-        hasExcl = true;
-      }
-    } else {
-      if (lane == 0 && successors && hasAgg) acc_publish<Elt>(desc + (tile * 2 + 0) * W, agg, epoch);
-      hasExcl = acc_lookback<S>(env, desc, tile, epoch, excl);
+  } else {
+    hasExcl = acc_lookback<S>(env, desc, tile, epoch, excl);  // valid in thread 0
+  }
+  if (threadIdx.x == 0) {
+    if (successors && wavesWithData > 0) {
+      Elt inc;
+      acc_join<S>(env, hasExcl, excl, true, sh_wave[wavesWithData - 1], inc);
+      acc_publish<Elt>(desc + tile * W, inc, epoch, 2);
     }
-    if (lane == 0) {
-      if (successors && hasAgg) {
-        Elt inc;
-        acc_join<S>(env, hasExcl, excl, hasAgg, agg, inc);
-        acc_publish<Elt>(desc + (tile * 2 + 1) * W, inc, epoch);
-      }
-      sh_excl = excl;
-      sh_has_excl = hasExcl ? 1 : 0;
-    }
+    sh_excl = excl;
+    sh_has_excl = hasExcl ? 1 : 0;
   }
   __syncthreads();
 
   // prefix of everything before this wave
   Elt base;
+  const bool hasWavePre = w > 0 && w <= wavesWithData;
+  Elt wavePre = sh_wave[w > 0 ? w - 1 : 0];
   bool hasBase = acc_join<S>(env, sh_has_excl != 0, sh_excl, hasWavePre, wavePre, base);
 #pragma unroll
   for (int g = 0; g < G; ++g) {
-    Elt gb;
-    bool hasGb = acc_join<S>(env, hasBase, base, hasGroupPre[g], groupPre[g], gb);
-    Elt lp;
-    bool hasLp = acc_join<S>(env, hasGb, gb, lane > 0, lanePre[g], lp);
     const i64 t0 = wlo + ((i64)g * ACC_WAVE + lane) * V;
+    if (full) {
+      Elt y[C::V];
 #pragma unroll
-    for (int k = 0; k < V; ++k) {
-      const i64 t = t0 + k;
-      if (t < n) store(t, hasLp ? S::combine(env, lp, x[g][k]) : x[g][k]);
+      for (int k = 0; k < V; ++k) y[k] = hasBase ? S::combine(env, base, x[g][k]) : x[g][k];
+#pragma unroll
+      for (int k = 0; k < V; ++k) store(t0 + k, y[k]);
+    } else {
+#pragma unroll
+      for (int k = 0; k < V; ++k) {
+        const i64 t = t0 + k;
+        if (t < n) store(t, hasBase ? S::combine(env, base, x[g][k]) : x[g][k]);
+      }
     }
   }
 }
 
 ACC_DEV i64 acc_take_ticket(u64* ticket, u64 base) {
+#ifdef ACC_X_NOTICKET
+  return (i64)blockIdx.x;
+#endif
   __shared__ i64 sh_tile;
   if (threadIdx.x == 0)
     sh_tile = (i64)(__hip_atomic_fetch_add(ticket, 1ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) - base);

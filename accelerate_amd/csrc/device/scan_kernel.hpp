@@ -1,7 +1,7 @@
 // Entry point of the scan skeleton: one workgroup per tile, tiles numbered by ticket in
 // row-major (row, tile-in-row) order; the tile machinery lives in scan.hpp.
 
-extern "C" __global__ void __launch_bounds__(ACC_BLOCK)
+extern "C" __global__ void __launch_bounds__(ACC_SCAN_BLOCK, ACC_SCAN_MINWAVES)
 acc_scan(Spec::Env env, Spec::Out out, Spec::Out tot, ScanParams p) {
   typedef Spec S;
   typedef S::Elt Elt;
@@ -13,7 +13,7 @@ acc_scan(Spec::Env env, Spec::Out out, Spec::Out tot, ScanParams p) {
   const i64 inBase = row * n;
   const i64 m = S::kKind == 1 ? n + 1 : n;  // entries per output row
   const i64 outBase = row * m;
-  u64* rowDesc = p.desc + (u64)row * (u64)p.tpr * 2 * W;
+  u64* rowDesc = p.desc + (u64)row * (u64)p.tpr * W;
 
   auto load = [&](i64 t) -> Elt { return S::in_linear(env, inBase + (S::kRight ? n - 1 - t : t)); };
   auto store = [&](i64 t, const Elt& y) {

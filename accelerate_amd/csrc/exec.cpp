@@ -913,7 +913,7 @@ AValP Program::eval(const Sx& n, AEnv& aenv) {
     DArrayP out = alloc(plan.ty->r, oshape);
     if (rows == 0 || nseg == 0) return avArr(out);
     const KernelSource& m = plan.k->meta;
-    const int64_t tile = (int64_t)4 * m.group * 64 * m.vec;
+    const int64_t tile = (int64_t)m.block * m.group * m.vec;
     const int64_t total = rows * len;
     const int64_t tiles = std::max<int64_t>(1, (total + tile - 1) / tile);
     if (tiles > 0x7ffffff0LL) throw Error("foldSeg: too many tiles for one launch");
@@ -921,7 +921,7 @@ AValP Program::eval(const Sx& n, AEnv& aenv) {
     pr.rank = 1;
     pr.elt = tScalar(ST::I64);
     DArrayP part = alloc(pr, {tiles + 1});
-    Context::ScanState& st = ctx_.scanState((size_t)tiles * 2 * m.words * sizeof(uint64_t));
+    Context::ScanState& st = ctx_.scanState((size_t)tiles * m.words * sizeof(uint64_t));
     std::vector<uint64_t> args = packArgs(m, aenv, temps, {});
     packOut(args, *out);
     args.push_back((uint64_t)rows);
@@ -935,7 +935,7 @@ AValP Program::eval(const Sx& n, AEnv& aenv) {
     args.push_back((uint64_t)st.ticketBase);
     args.push_back((uint64_t)st.epoch);
     ctx_.launch(plan.k, "acc_foldseg_partition", (unsigned)((tiles + 1 + 255) / 256), 256, args);
-    ctx_.launch(plan.k, "acc_foldseg", (unsigned)tiles, 256, args);
+    ctx_.launch(plan.k, "acc_foldseg", (unsigned)tiles, (unsigned)m.block, args);
     st.ticketBase += (uint64_t)tiles;
     return avArr(out);
   }
@@ -958,11 +958,11 @@ AValP Program::eval(const Sx& n, AEnv& aenv) {
     AValP result = prime ? avPair(avArr(out), avArr(tot)) : avArr(out);
     if (rows == 0 || (kind == 0 && len == 0)) return result;
     const KernelSource& m = plan.k->meta;
-    const int64_t tile = (int64_t)4 * m.group * 64 * m.vec;
+    const int64_t tile = (int64_t)m.block * m.group * m.vec;
     const int64_t tpr = std::max<int64_t>(1, (len + tile - 1) / tile);
     const int64_t tiles = rows * tpr;
     if (tiles > 0x7fffffffLL) throw Error("scan: too many tiles for one launch");
-    Context::ScanState& st = ctx_.scanState((size_t)tiles * 2 * m.words * sizeof(uint64_t));
+    Context::ScanState& st = ctx_.scanState((size_t)tiles * m.words * sizeof(uint64_t));
     std::vector<uint64_t> args = packArgs(m, aenv, temps, {});
     packOut(args, *out);
     packOut(args, *tot);
@@ -973,7 +973,7 @@ AValP Program::eval(const Sx& n, AEnv& aenv) {
     args.push_back((uint64_t)(uintptr_t)st.ticket);
     args.push_back((uint64_t)st.ticketBase);
     args.push_back((uint64_t)st.epoch);
-    ctx_.launch(plan.k, "acc_scan", (unsigned)tiles, 256, args);
+    ctx_.launch(plan.k, "acc_scan", (unsigned)tiles, (unsigned)m.block, args);
     st.ticketBase += (uint64_t)tiles;
     return result;
   }

@@ -221,7 +221,7 @@ Context::ScanState& Context::scanState(size_t descBytes) {
     scan_.descBytes = n;
     scan_.epoch = 0;
   }
-  if (++scan_.epoch == 0) {  // wrapped: stale flags could alias, start over from a clean slate
+  if (++scan_.epoch >= (1u << 30)) {  // wrapped: stale tags could alias, start over from a clean slate
     hipCheck(hipMemsetAsync(scan_.desc, 0, scan_.descBytes, stream_), "hipMemsetAsync");
     scan_.epoch = 1;
   }
@@ -270,7 +270,32 @@ static std::string compileHipRTC(const std::string& source, std::string& log) {
   return code;
 }
 
-KernelP Context::kernel(const KernelSource& ks) {
+// Extra preprocessor definitions for generated kernels (tuning experiments):
+// ACCHIP_DEFINES="NAME=VALUE NAME2" becomes #define lines in front of the source, and so
+// takes part in the cache key.
+static std::string definesPrefix() {
+  const char* d = std::getenv("ACCHIP_DEFINES");
+  std::string out;
+  if (!d) return out;
+  std::string tok;
+  for (const char* p = d;; ++p) {
+    if (*p == ' ' || *p == '\0') {
+      if (!tok.empty()) {
+        size_t eq = tok.find('=');
+        out += "#define " + (eq == std::string::npos ? tok : tok.substr(0, eq) + " " + tok.substr(eq + 1)) + "\n";
+        tok.clear();
+      }
+      if (!*p) break;
+    } else {
+      tok += *p;
+    }
+  }
+  return out;
+}
+
+KernelP Context::kernel(const KernelSource& ks0) {
+  KernelSource ks = ks0;
+  ks.source = definesPrefix() + ks0.source;
   std::string keyText = ks.source;
   for (int i = 0; i < kNumCompileOptions; ++i) keyText += std::string("\n//opt ") + kCompileOptions[i];
   int major = 0, minor = 0;
