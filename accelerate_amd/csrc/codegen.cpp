@@ -1132,6 +1132,7 @@ KernelSource Codegen::permute(const Sx& f, const ArrayR& dst, const Sx& p, const
            (op == "add" ? (st != ST::F16) : (op != "mul" && stIsInt(st))))
     mode = "atomic";
   else if (wide) mode = "cas";
+  std::string lds;
   std::string u = "  ACC_DEV void update(const Env& env, const Out& out, i64 j, const Elt& x, u32* locks) {\n";
   if (mode == "store") {
     u += "    Elt y_{};\n    store(out, j, combine(env, x, y_));\n";
@@ -1140,6 +1141,22 @@ KernelSource Codegen::permute(const Sx& f, const ArrayR& dst, const Sx& p, const
                    : op == "max" ? "__hip_atomic_fetch_max" : op == "band" ? "__hip_atomic_fetch_and"
                    : op == "bor" ? "__hip_atomic_fetch_or" : "__hip_atomic_fetch_xor";
     u += "    (void)" + fn + "(&out.o0[j], x.c0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);\n";
+    // pieces of the LDS-privatised variant (permute.hpp): identity, LDS and global updates
+    std::string T = stName(st), idv;
+    if (op == "add" || op == "bor" || op == "bxor") idv = "(" + T + ")0";
+    else if (op == "band") idv = "(" + T + ")~(" + T + ")0";
+    else {
+      int bits = stBits(st);
+      unsigned long long mx = stIsSigned(st) ? ((1ULL << (bits - 1)) - 1) : (bits == 64 ? ~0ULL : ((1ULL << bits) - 1));
+      unsigned long long mn = stIsSigned(st) ? (1ULL << (bits - 1)) : 0ULL;
+      char buf[64];
+      snprintf(buf, sizeof buf, "(%s)0x%llxULL", T.c_str(), op == "min" ? mx : mn);
+      idv = buf;
+    }
+    lds = "#define ACC_PERMUTE_LDS 1\n  typedef " + T + " Prim;\n";
+    lds += "  ACC_DEV Prim identity() { return " + idv + "; }\n";
+    lds += "  ACC_DEV void lds_update(Prim* p, const Elt& x) { (void)" + fn + "(p, x.c0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP); }\n";
+    lds += "  ACC_DEV void global_update(const Out& out, i64 j, Prim v) { (void)" + fn + "(&out.o0[j], v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); }\n";
   } else if (mode == "cas") {
     std::string B = stSize(leaves[0]) == 4 ? "u32" : "u64", T = stName(leaves[0]);
     u += "    " + B + "* a_ = (" + B + "*)&out.o0[j];\n";
@@ -1161,7 +1178,7 @@ KernelSource Codegen::permute(const Sx& f, const ArrayR& dst, const Sx& p, const
       u += "        __hip_atomic_store(&out.o" + std::to_string(k) + "[j], r_.c" + std::to_string(k) + ", __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);\n";
     u += "        __hip_atomic_store(lk_, 0u, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_AGENT);\n        done_ = true;\n      }\n    }\n";
   }
-  u += "  }\n";
+  u += "  }\n" + lds;
   // update() uses store()/combine(): it must come after them, and finish() appends load/store
   // last, so emit our own forward-safe copies by placing update in a trailing block
   KernelSource ks = finish(body + "//@UPDATE@\n", elt, leaves, "permute.hpp", 1);

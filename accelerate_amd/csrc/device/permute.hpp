@@ -30,3 +30,66 @@ acc_permute(Spec::Env env, Spec::Out out, PermuteParams p) {
     }
   }
 }
+
+#ifdef ACC_PERMUTE_LDS
+// Privatised variant for combination functions that are a single hardware atomic (+, min,
+// max, and, or, xor on a 32/64-bit scalar) and destinations of at most a few LDS-fuls.
+// Contended destinations (a histogram over skewed keys) serialise in the memory-side atomic
+// units; here a workgroup first combines its share of the sources into a private copy of one
+// destination range held in LDS (LDS atomics), then adds what it found to the real
+// destination with one global atomic per touched element.
+//
+// The destination is cut into `nparts` ranges of `part` elements (part <= ACC_PERMUTE_PART,
+// 128 KiB of LDS).  The sources are cut into `groups` chunks; workgroup b serves chunk
+// (b / (8 * nparts)) * 8 + b % 8 and range (b / 8) % nparts: workgroups are dealt to the 8
+// XCDs round-robin, so the nparts workgroups that read the same chunk run on the same XCD
+// and share its L2 -- the sources come from HBM once.
+#define ACC_PERMUTE_LDS_BLOCK 1024
+#define ACC_PERMUTE_PART (131072 / (int)sizeof(Spec::Prim))
+
+struct PermuteLdsParams {
+  i64 n;       // number of source elements
+  i64 chunk;   // sources per chunk (multiple of 4)
+  i64 nparts;  // destination ranges
+  i64 part;    // elements per range
+  i64 dst_n;   // destination elements
+};
+
+extern "C" __global__ void __launch_bounds__(ACC_PERMUTE_LDS_BLOCK)
+acc_permute_lds(Spec::Env env, Spec::Out out, PermuteLdsParams p) {
+  typedef Spec S;
+  typedef S::Prim Prim;
+  __shared__ Prim priv[ACC_PERMUTE_PART];
+  const i64 b = (i64)blockIdx.x;
+  const i64 range = (b / 8) % p.nparts;
+  const i64 chunkId = (b / (8 * p.nparts)) * 8 + (b % 8);
+  const i64 lo = range * p.part;
+  const i64 hi = lo + p.part < p.dst_n ? lo + p.part : p.dst_n;
+  const Prim id = S::identity();
+  for (int i = threadIdx.x; i < (int)(hi - lo); i += ACC_PERMUTE_LDS_BLOCK) priv[i] = id;
+  __syncthreads();
+  const i64 begin = chunkId * p.chunk;
+  const i64 end = begin + p.chunk < p.n ? begin + p.chunk : p.n;
+  for (i64 i0 = begin + (i64)threadIdx.x * 4; i0 < end; i0 += (i64)ACC_PERMUTE_LDS_BLOCK * 4) {
+    if (i0 + 4 <= end) {
+      i64 j[4];
+      bool ok[4];
+#pragma unroll
+      for (int k = 0; k < 4; ++k) ok[k] = S::target(env, i0 + k, j[k]);
+#pragma unroll
+      for (int k = 0; k < 4; ++k)
+        if (ok[k] && j[k] >= lo && j[k] < hi) S::lds_update(&priv[j[k] - lo], S::in_linear(env, i0 + k));
+    } else {
+      for (i64 i = i0; i < end; ++i) {
+        i64 j;
+        if (S::target(env, i, j) && j >= lo && j < hi) S::lds_update(&priv[j - lo], S::in_linear(env, i));
+      }
+    }
+  }
+  __syncthreads();
+  for (int i = threadIdx.x; i < (int)(hi - lo); i += ACC_PERMUTE_LDS_BLOCK) {
+    const Prim v = priv[i];
+    if (v != id) S::global_update(out, lo + i, v);
+  }
+}
+#endif

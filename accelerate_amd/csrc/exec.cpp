@@ -880,6 +880,22 @@ AValP Program::eval(const Sx& n, AEnv& aenv) {
     }
     std::vector<uint64_t> args = packArgs(plan.k->meta, aenv, temps, out->shape);
     packOut(args, *out);
+    // Many sources into a destination of a few LDS-fuls with a hardware-atomic combination:
+    // combine in workgroup-private LDS copies first (see permute.hpp).
+    const int64_t partMax = 131072 / stSize(plan.k->meta.outLeaves.empty() ? ST::I32 : plan.k->meta.outLeaves[0]);
+    if (plan.mode == "atomic" && cnt >= (1 << 20) && out->size() <= 8 * partMax) {
+      const int64_t nparts = (out->size() + partMax - 1) / partMax;
+      const int64_t part = (out->size() + nparts - 1) / nparts;
+      const int64_t groups = 256;
+      int64_t chunk = ((cnt + groups - 1) / groups + 3) / 4 * 4;
+      args.push_back((uint64_t)cnt);
+      args.push_back((uint64_t)chunk);
+      args.push_back((uint64_t)nparts);
+      args.push_back((uint64_t)part);
+      args.push_back((uint64_t)out->size());
+      ctx_.launch(plan.k, "acc_permute_lds", (unsigned)(groups * nparts), 1024, args);
+      return avArr(out);
+    }
     args.push_back((uint64_t)cnt);
     args.push_back(locks ? (uint64_t)(uintptr_t)locks->bufs[0]->p : 0);
     int64_t grid = std::min<int64_t>((cnt + 255) / 256, 256 * 32);

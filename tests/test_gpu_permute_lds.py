@@ -1,0 +1,55 @@
+"""The LDS-privatised permute path (many sources, small destination, hardware-atomic
+combination) against numpy's unbuffered ufunc.at, which applies the updates one by one in
+source order exactly like permuteOp (Interpreter.hs:585-624).  Integer results bit-exact;
+the Float32 case sums multiples of 1/4, which are exact in any order."""
+import numpy as np
+import pytest
+
+from accelerate_amd import ir as A
+
+from . import progs as Q
+
+N = (1 << 20) + 12345        # above the threshold that selects the privatised kernel
+
+
+def lds_programs():
+    """(id, program, numpy dtype, ufunc, destination size)"""
+    out = []
+    for ty, dt in ((A.i32, np.int32), (A.i64, np.int64), (A.f32, np.float32)):
+        for dst in (100, 40000, 70000):     # 1 range, 2 ranges (4-byte), up to 5 ranges (8-byte)
+            out.append(("add_%s_%d" % (ty, dst), Q.accumulate(ty, 1, 1), dt, np.add, dst))
+    for name, op, uf in (("min", A.min_, np.minimum), ("max", A.max_, np.maximum), ("bxor", A.bxor, np.bitwise_xor)):
+        out.append(("%s_i32_5000" % name, _combine_prog(op, A.i32), np.int32, uf, 5000))
+    return out
+
+
+def _combine_prog(op, ty):
+    sh1 = A.tshape(1)
+    return A.alam([A.tarray(1, ty), A.tarray(1, A.Int), A.tarray(1, ty)], lambda xs, to, dfl: A.permute(
+        Q.binop(op, ty), dfl,
+        A.lam([sh1], lambda ix: A.let(A.Int, A.index(to, A.vexp(ix)), lambda t: A.cond(
+            A.lt(A.Int, t, A.constI(0)), A.nothing(sh1), A.just(A.sh(t))))), xs))
+
+
+CASES = lds_programs()
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("case", CASES, ids=[c[0] for c in CASES])
+def test_privatised_permute_matches_sequential_updates(gpu_ctx, case):
+    _, prog, dt, uf, dst = case
+    rng = np.random.default_rng(dst)
+    # skewed targets (hot destinations) and some dropped sources (negative target)
+    to = np.minimum((rng.pareto(1.1, N) * 3).astype(np.int64), dst - 1)
+    to[rng.random(N) < 0.05] = -1
+    if dt == np.float32:
+        xs = (rng.integers(-8, 9, N) / 4).astype(dt)
+        dfl = (rng.integers(-8, 9, dst) / 4).astype(dt)
+    else:
+        xs = rng.integers(-1000, 1000, N).astype(dt)
+        dfl = rng.integers(-1000, 1000, dst).astype(dt)
+    got = gpu_ctx.compile(prog)(xs, to, dfl)
+    ref = dfl.copy()
+    keep = to >= 0
+    uf.at(ref, to[keep], xs[keep])
+    assert np.array_equal(got, ref)

@@ -25,7 +25,8 @@ def _compile_all(cc_ctx, named_programs):
 
 
 def test_all_parity_programs_compile(cc_ctx):
-    _compile_all(cc_ctx, [(c[0], c[1]) for c in parity_cases()])
+    from .test_gpu_permute_lds import lds_programs
+    _compile_all(cc_ctx, [(c[0], c[1]) for c in parity_cases()] + [(c[0], c[1]) for c in lds_programs()])
 
 
 def test_all_scalar_programs_compile_and_oracle_evaluates_them(cc_ctx):
