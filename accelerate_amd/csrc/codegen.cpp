@@ -1301,6 +1301,130 @@ KernelSource Codegen::stencil(const std::vector<Sx>& patterns, const TypeP& outE
   return finish(body, outElt, typeLeaves(outElt), "map.hpp", 0);
 }
 
+// rows of results per stencil tile (tuning knob: ACCHIP_STENCIL_H; multiple of 4)
+int stencilTileH() {
+  const char* e = std::getenv("ACCHIP_STENCIL_H");
+  int v = e ? std::atoi(e) : 32;
+  return (v == 8 || v == 16 || v == 32 || v == 64) ? v : 32;
+}
+
+KernelSource Codegen::stencil2d(const Sx& pattern, const TypeP& outElt, const Sx& f, const Sx& bnd,
+                                const Operand& src) {
+  const TypeP srcElt = src.r.elt;
+  auto sleaves = typeLeaves(srcElt);
+  const std::string kind = bnd.atom ? bnd.s : bnd.head();
+  if (kind != "clamp" && kind != "mirror" && kind != "wrap" && kind != "constant" && kind != "function")
+    throw Error("unknown stencil boundary '" + kind + "'");
+  if (pattern.head().compare(0, 3, "tup") != 0) throw Error("stencil2d: pattern is not of rank 2");
+  const int hy = stencilWidth(pattern) / 2;
+  int hx = 0;
+  for (size_t r = 1; r < pattern.size(); ++r) hx = std::max(hx, stencilWidth(pattern.at(r)) / 2);
+  const int tileH = stencilTileH();
+  const int pw = 64 + 2 * hx, ph = tileH + 2 * hy;
+  std::string body;
+  body += "#define ACC_ST_H " + std::to_string(tileH) + "\n";
+  body += "  static constexpr int HY = " + std::to_string(hy) + ";\n  static constexpr int HX = " + std::to_string(hx) + ";\n";
+  body += "  struct SrcElt {\n" + leafDecls(sleaves, "c", false, false) + "  };\n  struct Tile {\n";
+  for (size_t k = 0; k < sleaves.size(); ++k)
+    body += std::string("    ") + stName(sleaves[k]) + " c" + std::to_string(k) + "[" + std::to_string(pw * ph) + "];\n";
+  body += "  };\n  ACC_DEV void stage(Tile& t, int idx, const SrcElt& v) {\n";
+  for (size_t k = 0; k < sleaves.size(); ++k)
+    body += "    t.c" + std::to_string(k) + "[idx] = v.c" + std::to_string(k) + ";\n";
+  body += "  }\n";
+  auto retSrc = [&](const ValP& v, Emit& em) {
+    auto lv = leavesOf(v);
+    em.line("SrcElt r_;");
+    for (size_t k = 0; k < lv.size(); ++k) em.line("r_.c" + std::to_string(k) + " = " + lv[k]->ex + ";");
+    em.line("return r_;");
+  };
+  auto idx2 = [](const std::string& y, const std::string& x) {
+    return vPair(vPair(vUnit(), vLeaf(ST::I64, y)), vLeaf(ST::I64, x));
+  };
+  {
+    Emit em;
+    em.ind = 4;
+    ValP v = operandIndex(src, idx2("y", "x"), em);
+    if (!typeEq(valType(v), srcElt)) throw Error("stencil: fused producer does not return the element type");
+    retSrc(v, em);
+    body += fnHead("SrcElt", "src_in", "const Env& env, i64 y, i64 x") + em.code + "  }\n";
+  }
+  {
+    // bounded (Interpreter.hs:797-839) at an index that may lie outside on either side
+    Emit em;
+    em.ind = 4;
+    std::vector<std::string> dims;
+    shapeDims(operandShape(src, em), dims);
+    const char* raw[2] = {"y", "x"};
+    std::string idx[2], inside;
+    for (int d = 0; d < 2; ++d) {
+      const std::string j = raw[d], sz = dims[d];
+      if (kind == "clamp") idx[d] = bindLeaf(ST::I64, "(" + j + " < 0) ? (i64)0 : ((" + j + " >= " + sz + ") ? " + sz + " - 1 : " + j + ")", em)->ex;
+      else if (kind == "mirror") idx[d] = bindLeaf(ST::I64, "(" + j + " < 0) ? -" + j + " : ((" + j + " >= " + sz + ") ? " + sz + " - (" + j + " - " + sz + " + 2) : " + j + ")", em)->ex;
+      else if (kind == "wrap") idx[d] = bindLeaf(ST::I64, "(" + j + " < 0) ? " + sz + " + " + j + " : ((" + j + " >= " + sz + ") ? " + j + " - " + sz + " : " + j + ")", em)->ex;
+      else {
+        idx[d] = j;
+        inside += std::string(inside.empty() ? "" : " && ") + "(" + j + " >= 0) && (" + j + " < " + sz + ")";
+      }
+    }
+    if (kind == "constant" || kind == "function") {
+      Emit ei, eo;
+      ei.ind = eo.ind = em.ind + 2;
+      ValP vin = operandIndex(src, idx2(idx[0], idx[1]), ei);
+      ValP vout = kind == "constant" ? exp(bnd.at(1), {}, eo) : applyFun(bnd.at(1), {idx2("y", "x")}, {}, eo);
+      if (!typeEq(valType(vin), valType(vout))) throw Error("stencil: boundary value does not have the element type");
+      ValP res = declareVars(valType(vin), em);
+      em.line("if (" + inside + ") {");
+      em.code += ei.code;
+      em.ind += 2;
+      assign(res, vin, em);
+      em.ind -= 2;
+      em.line("} else {");
+      em.code += eo.code;
+      em.ind += 2;
+      assign(res, vout, em);
+      em.ind -= 2;
+      em.line("}");
+      retSrc(res, em);
+    } else {
+      retSrc(operandIndex(src, idx2(idx[0], idx[1]), em), em);
+    }
+    body += fnHead("SrcElt", "src_at", "const Env& env, i64 y, i64 x") + em.code + "  }\n";
+  }
+  {
+    // the stencil function over taps read from the staged tile; c is the focus inside the tile
+    Emit em;
+    em.ind = 4;
+    const int k0 = stencilWidth(pattern) / 2;
+    ValP arg = vUnit();
+    for (int dy = -k0; dy <= k0; ++dy) {
+      const Sx& row = pattern.at(1 + dy + k0);
+      if (row.head().compare(0, 4, "unit") != 0) throw Error("stencil2d: pattern is not of rank 2");
+      const int k1 = stencilWidth(row) / 2;
+      ValP rv = vUnit();
+      for (int dx = -k1; dx <= k1; ++dx) {
+        int leaf = 0;
+        struct R {
+          static ValP go(Codegen& cg, const TypeP& t, int& leaf, const std::string& at, Emit& em) {
+            if (t->k == Type::Unit) return vUnit();
+            if (t->k == Type::Scalar) return cg.bindLeaf(t->st, "t.c" + std::to_string(leaf++) + "[" + at + "]", em);
+            ValP a = go(cg, t->a, leaf, at, em);
+            return vPair(a, go(cg, t->b, leaf, at, em));
+          }
+        };
+        std::string at = "c + (" + std::to_string(dy * pw + dx) + ")";
+        rv = vPair(rv, R::go(*this, srcElt, leaf, at, em));
+      }
+      arg = vPair(arg, rv);
+    }
+    ValP r = applyFun(f, {arg}, {}, em);
+    if (!typeEq(valType(r), outElt)) throw Error("stencil: function result does not match the declared element type");
+    body += fnHead("Elt", "apply", "const Env& env, const Tile& t, int c, i64 gy, i64 gx") + returnElt(r, em) + "  }\n";
+  }
+  KernelSource ks = finish(body, outElt, typeLeaves(outElt), "stencil2d.hpp", 1);
+  ks.group = tileH;
+  return ks;
+}
+
 KernelSource Codegen::scalarKernel(const Sx& e) {
   Emit em;
   em.ind = 4;

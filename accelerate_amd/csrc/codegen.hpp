@@ -75,6 +75,8 @@ class Codegen {
   KernelSource permute(const Sx& f, const ArrayR& dst, const Sx& p, const Operand& src);
   KernelSource stencil(const std::vector<Sx>& patterns, const TypeP& outElt, const Sx& f,
                        const std::vector<Sx>& boundaries, const std::vector<Operand>& srcs);
+  // rank-2 single-source stencil through LDS halo tiles
+  KernelSource stencil2d(const Sx& pattern, const TypeP& outElt, const Sx& f, const Sx& boundary, const Operand& src);
   KernelSource scalarKernel(const Sx& exp);  // evaluates a closed Exp with one thread
 
   // type of a closed scalar expression / result of a function, without emitting code

@@ -529,7 +529,12 @@ ATyP Program::prepare(const Sx& n, TEnv& tenv) {
       srcs.push_back(operandOf(n.at(8), cg, tenv, plan));
       if (srcs[0].r.rank != srcs[1].r.rank) throw Error("stencil2: operands of different rank");
     }
-    plan.k = ctx_.kernel(cg.stencil(pats, outElt, *f, bnds, srcs));
+    if (!two && srcs[0].r.rank == 2) {
+      plan.k = ctx_.kernel(cg.stencil2d(pats[0], outElt, *f, bnds[0], srcs[0]));
+      plan.mode = "lds2d";
+    } else {
+      plan.k = ctx_.kernel(cg.stencil(pats, outElt, *f, bnds, srcs));
+    }
     ArrayR r;
     r.rank = srcs[0].r.rank;
     r.elt = outElt;
@@ -912,6 +917,19 @@ AValP Program::eval(const Sx& n, AEnv& aenv) {
       for (size_t k = 0; k < ext.size(); ++k) ext[k] = std::min(ext[k], e2[k]);
     }
     DArrayP out = alloc(plan.ty->r, ext);
+    if (plan.mode == "lds2d") {
+      if (out->size() == 0) return avArr(out);
+      const int64_t th = plan.k->meta.group;  // rows per tile chosen by the code generator
+      const int64_t tilesY = (ext[0] + th - 1) / th, tilesX = (ext[1] + 63) / 64;
+      if (tilesX * tilesY > 0x7fffffffLL) throw Error("stencil: too many tiles for one launch");
+      std::vector<uint64_t> args = packArgs(plan.k->meta, aenv, temps, ext);
+      packOut(args, *out);
+      args.push_back((uint64_t)ext[0]);
+      args.push_back((uint64_t)ext[1]);
+      args.push_back((uint64_t)tilesX);
+      ctx_.launch(plan.k, "acc_stencil2d", (unsigned)(tilesX * tilesY), 256, args);
+      return avArr(out);
+    }
     launchMap(plan.k, aenv, temps, *out);
     return avArr(out);
   }
