@@ -943,11 +943,19 @@ KernelSource Codegen::foldSeg(const Sx& f, const Sx* seed, const Operand& src, c
   for (auto& kv : used_)
     if (kv.second.name != seg.slot) tmpOrder.push_back(kv.second);
   int vec = vecFor(leaves, tmpOrder);
-  int g = std::max(1, std::min(8, scanBytesPerLane() / std::max(1, vec * eltBytes)));
+  // tile size of the segmented fold: its own knob (ACCHIP_FOLDSEG_BYTES), the tile also pays
+  // for an LDS word per element
+  const char* fe = std::getenv("ACCHIP_FOLDSEG_BYTES");
+  int fbytes = fe ? std::atoi(fe) : 128;
+  if (fbytes < 16 || fbytes > 512) fbytes = 128;
+  int g = std::max(1, std::min(8, fbytes / std::max(1, vec * eltBytes)));
   body += "  static constexpr int G = " + std::to_string(g) + ";\n";
-  body += "#define ACC_SCAN_BLOCK " + std::to_string(scanBlock()) + "\n";
+  const char* fb = std::getenv("ACCHIP_FOLDSEG_BLOCK");
+  int fblock = fb ? std::atoi(fb) : 1024;
+  if (fblock != 256 && fblock != 512 && fblock != 1024) fblock = 1024;
+  body += "#define ACC_SCAN_BLOCK " + std::to_string(fblock) + "\n";
   KernelSource ks = finish(body, elt, leaves, "scan.hpp+foldseg.hpp", vec);
-  ks.block = scanBlock();
+  ks.block = fblock;
   ks.group = g;
   ks.words = flaggedWords(leaves);
   return ks;
@@ -960,6 +968,7 @@ KernelSource Codegen::scan(const Sx& f, const Sx* seed, const Operand& src, bool
   body += std::string("  static constexpr bool kSeeded = ") + (seed ? "true" : "false") + ";\n";
   body += std::string("  static constexpr bool kRight = ") + (right ? "true" : "false") + ";\n";
   body += "  static constexpr int kKind = " + std::to_string(kind) + ";\n";
+  body += "  ACC_DEV bool stops(const Elt&) { return false; }\n";
   auto leaves = typeLeaves(elt);
   int eltBytes = 0;
   for (ST s : leaves) eltBytes += stSize(s);

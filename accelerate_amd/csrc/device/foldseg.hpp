@@ -55,6 +55,9 @@ template <class S> struct AccSegSpec {
     Elt r{};
     return r;
   }
+  // an aggregate that contains a segment head hides everything before it: the look-back
+  // of a later tile may stop there
+  ACC_DEV bool stops(const Elt& a) { return a.f != 0; }
 };
 
 extern "C" __global__ void __launch_bounds__(ACC_BLOCK)
@@ -98,7 +101,7 @@ acc_foldseg(Spec::Env env, Spec::Out out, FoldSegParams p) {
   for (int i = threadIdx.x; i <= C::TILE; i += ACC_SCAN_BLOCK) sh_first[i] = NONE;
   __syncthreads();
   for (i64 j = j0 + threadIdx.x; j < j1; j += ACC_SCAN_BLOCK) {
-    const i64 row = j / sp1, s = j - row * sp1;
+    const i64 row = p.rows == 1 ? 0 : acc_quot(j, sp1), s = j - row * sp1;
     const i64 o = S::seg_at(env, s);
     const i64 rel = row * p.n + o - tlo;
     if (rel >= 0 && rel <= C::TILE) atomicMin(&sh_first[rel], (int)(j - j0));
@@ -121,7 +124,7 @@ acc_foldseg(Spec::Env env, Spec::Out out, FoldSegParams p) {
     const int nxt = sh_first[t - tlo + 1];
     if (nxt == NONE) return;
     const i64 j = j0 + nxt;
-    const i64 row = j / sp1, s = j - row * sp1;
+    const i64 row = p.rows == 1 ? 0 : acc_quot(j, sp1), s = j - row * sp1;
     if (s == 0) return;  // what precedes a row's first boundary belongs to no segment
     S::store(out, row * p.nseg + s - 1, S::kSeeded ? S::combine(env, S::seed(env), y.v) : y.v);
   };

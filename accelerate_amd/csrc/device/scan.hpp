@@ -130,6 +130,7 @@ ACC_DEV void acc_window(const typename S::Env& env, const u64* rowDesc, i64 look
   int first;
   for (;;) {
     st = idx < 0 ? 3 : acc_try_read<Elt>(rowDesc + idx * W, val, epoch);
+    if (st == 1 && S::stops(val)) st = 2;  // nothing before this aggregate can matter
     const u64 mEnd = __ballot(st >= 2);
     const u64 mInv = __ballot(st == 0);
     first = mEnd ? __builtin_ctzll(mEnd) : ACC_WAVE;
