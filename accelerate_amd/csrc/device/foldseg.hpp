@@ -86,19 +86,52 @@ acc_foldseg_partition(Spec::Env env, Spec::Out out, FoldSegParams p) {
   p.part[t] = row * sp1 + lo;
 }
 
+// One tile.  A lane owns, per group, a run of V consecutive elements and reduces it in
+// order, starting afresh at every head.  A segment end whose segment began inside the run
+// is written at once; the first end of a run that has seen no head yet still lacks what
+// precedes the run, and is kept as the run's pending end (at most one per run).  The runs'
+// aggregates (head seen, value since the last head) go through the ordered wave scan and
+// the wave totals through LDS, exactly as in a plain scan, but only pending ends receive
+// the prefix: a prefix that contains a head closes them inside the wave, the others wait
+// for the tile's exclusive prefix from the look-back.
 extern "C" __global__ void __launch_bounds__(ACC_SCAN_BLOCK)
 acc_foldseg(Spec::Env env, Spec::Out out, FoldSegParams p) {
   typedef Spec S;
   typedef AccSegSpec<Spec> SS;
   typedef AccScanCfg<SS> C;
+  typedef SS::Elt P;
+  const int V = C::V, G = C::G, W = C::W;
   const int NONE = 0x7fffffff;
-  __shared__ int sh_first[C::TILE + 1];
+  __shared__ __attribute__((aligned(16))) int sh_first[C::TILE + 4];
+  __shared__ P sh_wave[ACC_SCAN_WAVES];
+  __shared__ P sh_excl;
+  __shared__ int sh_has_excl;
 
   const i64 tile = acc_take_ticket(p.ticket, p.ticket_base);
   const i64 tlo = tile * (i64)C::TILE;
   const i64 sp1 = p.nseg + 1;
   const i64 j0 = p.part[tile], j1 = p.part[tile + 1];
-  for (int i = threadIdx.x; i <= C::TILE; i += ACC_SCAN_BLOCK) sh_first[i] = NONE;
+  const int lane = acc_lane(), w = acc_wave();
+  const i64 n = p.total;
+  const i64 wlo = tlo + (i64)w * G * C::GROUP;
+  const bool full = tlo + (i64)C::TILE <= n;
+  // all loads of the tile are issued first: they depend on nothing but the tile number, and
+  // could not be moved past the stores further down
+  S::Elt x[C::G][C::V];
+#pragma unroll
+  for (int g = 0; g < G; ++g) {
+    const i64 t0 = wlo + ((i64)g * ACC_WAVE + lane) * V;
+    if (full) {
+#pragma unroll
+      for (int k = 0; k < V; ++k) x[g][k] = S::in_linear(env, t0 + k);
+    } else {
+#pragma unroll
+      for (int k = 0; k < V; ++k)
+        if (t0 + k < n) x[g][k] = S::in_linear(env, t0 + k);
+    }
+  }
+  for (int i = threadIdx.x; i < C::TILE / 4 + 1; i += ACC_SCAN_BLOCK)
+    reinterpret_cast<int4*>(sh_first)[i] = make_int4(NONE, NONE, NONE, NONE);
   __syncthreads();
   for (i64 j = j0 + threadIdx.x; j < j1; j += ACC_SCAN_BLOCK) {
     const i64 row = p.rows == 1 ? 0 : acc_quot(j, sp1), s = j - row * sp1;
@@ -114,19 +147,108 @@ acc_foldseg(Spec::Env env, Spec::Out out, FoldSegParams p) {
   }
   __syncthreads();
 
-  auto load = [&](i64 t) -> SS::Elt {
-    SS::Elt e;
-    e.v = S::in_linear(env, t);
-    e.f = sh_first[t - tlo] != NONE ? 1u : 0u;
-    return e;
-  };
-  auto store = [&](i64 t, const SS::Elt& y) {
-    const int nxt = sh_first[t - tlo + 1];
-    if (nxt == NONE) return;
-    const i64 j = j0 + nxt;
+  // the segment that ends where boundary j0 + idx sits
+  auto emit = [&](int idx, const S::Elt& v) {
+    const i64 j = j0 + idx;
     const i64 row = p.rows == 1 ? 0 : acc_quot(j, sp1), s = j - row * sp1;
     if (s == 0) return;  // what precedes a row's first boundary belongs to no segment
-    S::store(out, row * p.nseg + s - 1, S::kSeeded ? S::combine(env, S::seed(env), y.v) : y.v);
+    S::store(out, row * p.nseg + s - 1, S::kSeeded ? S::combine(env, S::seed(env), v) : v);
   };
-  acc_scan_tile<SS>(env, p.desc, p.tiles, tile, p.total, p.epoch, load, store);
+
+  P waveTot;
+  bool hasWaveTot = false;
+  S::Elt pendVal[C::G];
+  int pendIdx[C::G];
+#pragma unroll
+  for (int g = 0; g < G; ++g) {
+    const i64 t0 = wlo + ((i64)g * ACC_WAVE + lane) * V;
+    const int rel0 = (int)(t0 - tlo);
+    int m[C::V + 1];
+#pragma unroll
+    for (int k = 0; k <= V; ++k) m[k] = sh_first[rel0 + k];
+    i64 c = n - t0;
+    c = c < 0 ? 0 : (c > V ? V : c);
+    const S::Elt* e = x[g];
+    P a{};
+    bool has = false;
+    pendIdx[g] = NONE;
+#pragma unroll
+    for (int k = 0; k < V; ++k) {
+      if (full || k < c) {
+        if (m[k] != NONE) {
+          a.v = e[k];
+          a.f = 1u;
+        } else {
+          a.v = has ? S::combine(env, a.v, e[k]) : e[k];
+        }
+        has = true;
+        if (m[k + 1] != NONE) {
+          if (a.f) {
+            emit(m[k + 1], a.v);
+          } else {
+            pendVal[g] = a.v;
+            pendIdx[g] = m[k + 1];
+          }
+        }
+      }
+    }
+
+    i64 cnt = n - (wlo + (i64)g * C::GROUP);
+    cnt = cnt < 0 ? 0 : (cnt > C::GROUP ? C::GROUP : cnt);
+    P ts = acc_wave_scan<SS>(env, a, lane);
+    P lanePre = acc_prev_lane(ts);  // exclusive prefix of the run inside its group (lane > 0)
+    const int last = cnt > 0 ? (int)((cnt - 1) / V) : 0;
+    P gt = acc_readlane(ts, last);
+    P pre;
+    if (acc_join<SS>(env, hasWaveTot, waveTot, lane > 0, lanePre, pre) && pendIdx[g] != NONE) {
+      pendVal[g] = S::combine(env, pre.v, pendVal[g]);
+      if (pre.f) {
+        emit(pendIdx[g], pendVal[g]);
+        pendIdx[g] = NONE;
+      }
+    }
+    if (cnt > 0) {
+      waveTot = hasWaveTot ? SS::combine(env, waveTot, gt) : gt;
+      hasWaveTot = true;
+    }
+  }
+  if (lane == 0) sh_wave[w] = waveTot;
+  __syncthreads();
+
+  // a wave has data only if all earlier waves are full, so validity follows from counts
+  const i64 tcnt = n - tlo;
+  const i64 perWave = (i64)G * C::GROUP;
+  i64 wd = tcnt <= 0 ? 0 : (tcnt + perWave - 1) / perWave;
+  const int wavesWithData = wd > ACC_SCAN_WAVES ? ACC_SCAN_WAVES : (int)wd;
+  const bool successors = tile + 1 < p.tiles;
+  if (w == 0) {
+    P t = sh_wave[lane < ACC_SCAN_WAVES ? lane : 0];
+    t = acc_wave_scan<SS>(env, t, lane);
+    if (lane < ACC_SCAN_WAVES) sh_wave[lane] = t;
+    if (lane == wavesWithData - 1 && tile > 0 && successors) acc_publish<P>(p.desc + tile * W, t, p.epoch, 1);
+  }
+  __syncthreads();
+
+  P excl;
+  bool hasExcl = false;
+  if (tile > 0) hasExcl = acc_lookback<SS>(env, p.desc, tile, p.epoch, excl);  // valid in thread 0
+  if (threadIdx.x == 0) {
+    if (successors && wavesWithData > 0) {
+      P inc;
+      acc_join<SS>(env, hasExcl, excl, true, sh_wave[wavesWithData - 1], inc);
+      acc_publish<P>(p.desc + tile * W, inc, p.epoch, 2);
+    }
+    sh_excl = excl;
+    sh_has_excl = hasExcl ? 1 : 0;
+  }
+  __syncthreads();
+
+  // ends still pending have seen no head since the start of the tile
+  P base;
+  const bool hasWavePre = w > 0 && w <= wavesWithData;
+  P wavePre = sh_wave[w > 0 ? w - 1 : 0];
+  const bool hasBase = acc_join<SS>(env, sh_has_excl != 0, sh_excl, hasWavePre, wavePre, base);
+#pragma unroll
+  for (int g = 0; g < G; ++g)
+    if (pendIdx[g] != NONE) emit(pendIdx[g], hasBase ? S::combine(env, base.v, pendVal[g]) : pendVal[g]);
 }
