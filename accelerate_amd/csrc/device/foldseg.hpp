@@ -27,10 +27,9 @@ struct FoldSegParams {
   i64 total;   // rows * n
   i64 tiles;   // >= 1
   i64* part;   // [tiles + 1]: boundaries before each tile border; part[tiles] = rows * (S + 1)
-  u64* desc;
-  u64* ticket;
-  u64 ticket_base;
-  u64 epoch;
+  void* carry;    // [tiles] (head seen, value since the last head) of each tile
+  void* pend;     // [tiles] value of the tile's one segment end that precedes all its heads
+  i64* pend_at;   // [tiles] boundary number of that end, or -1
 };
 
 template <class S> struct AccSegSpec {
@@ -100,14 +99,14 @@ acc_foldseg(Spec::Env env, Spec::Out out, FoldSegParams p) {
   typedef AccSegSpec<Spec> SS;
   typedef AccScanCfg<SS> C;
   typedef SS::Elt P;
-  const int V = C::V, G = C::G, W = C::W;
+  const int V = C::V, G = C::G;
   const int NONE = 0x7fffffff;
   __shared__ __attribute__((aligned(16))) int sh_first[C::TILE + 4];
   __shared__ P sh_wave[ACC_SCAN_WAVES];
-  __shared__ P sh_excl;
-  __shared__ int sh_has_excl;
+  __shared__ S::Elt sh_pend;
+  __shared__ int sh_pend_at;
 
-  const i64 tile = acc_take_ticket(p.ticket, p.ticket_base);
+  const i64 tile = blockIdx.x;
   const i64 tlo = tile * (i64)C::TILE;
   const i64 sp1 = p.nseg + 1;
   const i64 j0 = p.part[tile], j1 = p.part[tile + 1];
@@ -213,6 +212,7 @@ acc_foldseg(Spec::Env env, Spec::Out out, FoldSegParams p) {
     }
   }
   if (lane == 0) sh_wave[w] = waveTot;
+  if (threadIdx.x == 0) sh_pend_at = NONE;
   __syncthreads();
 
   // a wave has data only if all earlier waves are full, so validity follows from counts
@@ -220,35 +220,77 @@ acc_foldseg(Spec::Env env, Spec::Out out, FoldSegParams p) {
   const i64 perWave = (i64)G * C::GROUP;
   i64 wd = tcnt <= 0 ? 0 : (tcnt + perWave - 1) / perWave;
   const int wavesWithData = wd > ACC_SCAN_WAVES ? ACC_SCAN_WAVES : (int)wd;
-  const bool successors = tile + 1 < p.tiles;
   if (w == 0) {
     P t = sh_wave[lane < ACC_SCAN_WAVES ? lane : 0];
     t = acc_wave_scan<SS>(env, t, lane);
     if (lane < ACC_SCAN_WAVES) sh_wave[lane] = t;
-    if (lane == wavesWithData - 1 && tile > 0 && successors) acc_publish<P>(p.desc + tile * W, t, p.epoch, 1);
+    if (lane == wavesWithData - 1) reinterpret_cast<P*>(p.carry)[tile] = t;
   }
   __syncthreads();
 
-  P excl;
-  bool hasExcl = false;
-  if (tile > 0) hasExcl = acc_lookback<SS>(env, p.desc, tile, p.epoch, excl);  // valid in thread 0
-  if (threadIdx.x == 0) {
-    if (successors && wavesWithData > 0) {
-      P inc;
-      acc_join<SS>(env, hasExcl, excl, true, sh_wave[wavesWithData - 1], inc);
-      acc_publish<P>(p.desc + tile * W, inc, p.epoch, 2);
-    }
-    sh_excl = excl;
-    sh_has_excl = hasExcl ? 1 : 0;
-  }
-  __syncthreads();
-
-  // ends still pending have seen no head since the start of the tile
-  P base;
+  // an end still pending has seen no head since the start of its wave; if none of the
+  // earlier waves has one either it is the tile's pending end (there is at most one)
   const bool hasWavePre = w > 0 && w <= wavesWithData;
-  P wavePre = sh_wave[w > 0 ? w - 1 : 0];
-  const bool hasBase = acc_join<SS>(env, sh_has_excl != 0, sh_excl, hasWavePre, wavePre, base);
+  const P wavePre = sh_wave[w > 0 ? w - 1 : 0];
 #pragma unroll
-  for (int g = 0; g < G; ++g)
-    if (pendIdx[g] != NONE) emit(pendIdx[g], hasBase ? S::combine(env, base.v, pendVal[g]) : pendVal[g]);
+  for (int g = 0; g < G; ++g) {
+    if (pendIdx[g] != NONE) {
+      const S::Elt v = hasWavePre ? S::combine(env, wavePre.v, pendVal[g]) : pendVal[g];
+      if (hasWavePre && wavePre.f) {
+        emit(pendIdx[g], v);
+      } else {
+        sh_pend_at = pendIdx[g];
+        sh_pend = v;
+      }
+    }
+  }
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    p.pend_at[tile] = sh_pend_at == NONE ? (i64)-1 : j0 + sh_pend_at;
+    if (sh_pend_at != NONE) reinterpret_cast<P*>(p.pend)[tile].v = sh_pend;
+  }
+}
+
+// One wave per tile that has a pending end: walk back over the carries of the preceding
+// tiles, 64 at a time, up to the nearest tile that contains a head (or the start of the
+// stream), combine them in order and complete the end.
+extern "C" __global__ void __launch_bounds__(ACC_BLOCK)
+acc_foldseg_fixup(Spec::Env env, Spec::Out out, FoldSegParams p) {
+  typedef Spec S;
+  typedef AccSegSpec<Spec> SS;
+  typedef SS::Elt P;
+  const int lane = acc_lane();
+  const i64 tile = (i64)blockIdx.x * (ACC_BLOCK / ACC_WAVE) + acc_wave();
+  if (tile >= p.tiles) return;
+  const i64 j = p.pend_at[tile];
+  if (j < 0) return;
+  const P* carry = reinterpret_cast<const P*>(p.carry);
+  S::Elt v = reinterpret_cast<const P*>(p.pend)[tile].v;
+  bool have = false;
+  S::Elt run;
+  for (i64 look = tile - 1; look >= 0; look -= ACC_WAVE) {
+    const i64 idx = look - lane;
+    P c{};
+    if (idx >= 0) c = carry[idx];
+    const u64 mHead = __ballot(idx >= 0 && c.f != 0);
+    const int first = mHead ? __builtin_ctzll(mHead) : ACC_WAVE;
+    const int nvalid = look + 1 < ACC_WAVE ? (int)(look + 1) : ACC_WAVE;
+    const int nv = first < ACC_WAVE ? first + 1 : nvalid;
+    // earlier tiles sit in higher lanes: fold them in from the left
+    S::Elt r = c.v;
+#pragma unroll
+    for (int d = 1; d < ACC_WAVE; d <<= 1) {
+      S::Elt o = acc_shfl_down(r, d);
+      if (lane + d < nv) r = S::combine(env, o, r);
+    }
+    run = have ? S::combine(env, r, run) : r;
+    have = true;
+    if (first < ACC_WAVE) break;
+  }
+  if (lane != 0) return;
+  if (have) v = S::combine(env, run, v);
+  const i64 sp1 = p.nseg + 1;
+  const i64 row = p.rows == 1 ? 0 : acc_quot(j, sp1), s = j - row * sp1;
+  if (s == 0) return;  // what precedes a row's first boundary belongs to no segment
+  S::store(out, row * p.nseg + s - 1, S::kSeeded ? S::combine(env, S::seed(env), v) : v);
 }

@@ -955,7 +955,9 @@ AValP Program::eval(const Sx& n, AEnv& aenv) {
     pr.rank = 1;
     pr.elt = tScalar(ST::I64);
     DArrayP part = alloc(pr, {tiles + 1});
-    Context::ScanState& st = ctx_.scanState((size_t)tiles * m.words * sizeof(uint64_t));
+    // per tile: its carry and its pending end, both (value, head flag) records of m.words words
+    const int64_t recs = (tiles * (int64_t)m.words * 4 + 7) / 8;
+    DArrayP carry = alloc(pr, {recs}), pend = alloc(pr, {recs}), pendAt = alloc(pr, {tiles});
     std::vector<uint64_t> args = packArgs(m, aenv, temps, {});
     packOut(args, *out);
     args.push_back((uint64_t)rows);
@@ -964,13 +966,12 @@ AValP Program::eval(const Sx& n, AEnv& aenv) {
     args.push_back((uint64_t)total);
     args.push_back((uint64_t)tiles);
     args.push_back((uint64_t)(uintptr_t)part->bufs[0]->p);
-    args.push_back((uint64_t)(uintptr_t)st.desc);
-    args.push_back((uint64_t)(uintptr_t)st.ticket);
-    args.push_back((uint64_t)st.ticketBase);
-    args.push_back((uint64_t)st.epoch);
+    args.push_back((uint64_t)(uintptr_t)carry->bufs[0]->p);
+    args.push_back((uint64_t)(uintptr_t)pend->bufs[0]->p);
+    args.push_back((uint64_t)(uintptr_t)pendAt->bufs[0]->p);
     ctx_.launch(plan.k, "acc_foldseg_partition", (unsigned)((tiles + 1 + 255) / 256), 256, args);
     ctx_.launch(plan.k, "acc_foldseg", (unsigned)tiles, (unsigned)m.block, args);
-    st.ticketBase += (uint64_t)tiles;
+    ctx_.launch(plan.k, "acc_foldseg_fixup", (unsigned)((tiles + 3) / 4), 256, args);
     return avArr(out);
   }
   if (h == "scan" || h == "scan'") {
