@@ -92,20 +92,20 @@ acc_foldseg_partition(Spec::Env env, Spec::Out out, FoldSegParams p) {
 // aggregates (head seen, value since the last head) go through the ordered wave scan and
 // the wave totals through LDS, exactly as in a plain scan, but only pending ends receive
 // the prefix: a prefix that contains a head closes them inside the wave, the others wait
-// for the tile's exclusive prefix from the look-back.
-extern "C" __global__ void __launch_bounds__(ACC_SCAN_BLOCK)
-acc_foldseg(Spec::Env env, Spec::Out out, FoldSegParams p) {
+// for what the earlier waves of the tile contribute; the one end of a tile that no head of
+// the tile precedes is left to the fix-up kernel together with the tile's carry.
+//
+// ONE_ROW: the stream is a single row, so boundary j is segment boundary j of that row and
+// no division is needed.  FULL: the tile lies completely inside the stream.
+template <bool ONE_ROW, bool FULL>
+ACC_DEV void acc_foldseg_tile(const Spec::Env& env, const Spec::Out& out, const FoldSegParams& p, int* sh_first,
+                              AccSegSpec<Spec>::Elt* sh_wave, Spec::Elt& sh_pend, int& sh_pend_at) {
   typedef Spec S;
   typedef AccSegSpec<Spec> SS;
   typedef AccScanCfg<SS> C;
   typedef SS::Elt P;
   const int V = C::V, G = C::G;
   const int NONE = 0x7fffffff;
-  __shared__ __attribute__((aligned(16))) int sh_first[C::TILE + 4];
-  __shared__ P sh_wave[ACC_SCAN_WAVES];
-  __shared__ S::Elt sh_pend;
-  __shared__ int sh_pend_at;
-
   const i64 tile = blockIdx.x;
   const i64 tlo = tile * (i64)C::TILE;
   const i64 sp1 = p.nseg + 1;
@@ -113,14 +113,13 @@ acc_foldseg(Spec::Env env, Spec::Out out, FoldSegParams p) {
   const int lane = acc_lane(), w = acc_wave();
   const i64 n = p.total;
   const i64 wlo = tlo + (i64)w * G * C::GROUP;
-  const bool full = tlo + (i64)C::TILE <= n;
   // all loads of the tile are issued first: they depend on nothing but the tile number, and
   // could not be moved past the stores further down
   S::Elt x[C::G][C::V];
 #pragma unroll
   for (int g = 0; g < G; ++g) {
     const i64 t0 = wlo + ((i64)g * ACC_WAVE + lane) * V;
-    if (full) {
+    if (FULL) {
 #pragma unroll
       for (int k = 0; k < V; ++k) x[g][k] = S::in_linear(env, t0 + k);
     } else {
@@ -133,7 +132,7 @@ acc_foldseg(Spec::Env env, Spec::Out out, FoldSegParams p) {
     reinterpret_cast<int4*>(sh_first)[i] = make_int4(NONE, NONE, NONE, NONE);
   __syncthreads();
   for (i64 j = j0 + threadIdx.x; j < j1; j += ACC_SCAN_BLOCK) {
-    const i64 row = p.rows == 1 ? 0 : acc_quot(j, sp1), s = j - row * sp1;
+    const i64 row = ONE_ROW ? 0 : acc_quot(j, sp1), s = j - row * sp1;
     const i64 o = S::seg_at(env, s);
     const i64 rel = row * p.n + o - tlo;
     if (rel >= 0 && rel <= C::TILE) atomicMin(&sh_first[rel], (int)(j - j0));
@@ -141,7 +140,7 @@ acc_foldseg(Spec::Env env, Spec::Out out, FoldSegParams p) {
   }
   if (threadIdx.x == 0 && tile + 1 < p.tiles && j1 < p.rows * sp1) {
     // a boundary sitting exactly on this tile's upper border belongs to the next tile
-    const i64 row = j1 / sp1, s = j1 - row * sp1;
+    const i64 row = ONE_ROW ? 0 : j1 / sp1, s = j1 - row * sp1;
     if (row * p.n + S::seg_at(env, s) - tlo == C::TILE) sh_first[C::TILE] = (int)(j1 - j0);
   }
   __syncthreads();
@@ -149,7 +148,7 @@ acc_foldseg(Spec::Env env, Spec::Out out, FoldSegParams p) {
   // the segment that ends where boundary j0 + idx sits
   auto emit = [&](int idx, const S::Elt& v) {
     const i64 j = j0 + idx;
-    const i64 row = p.rows == 1 ? 0 : acc_quot(j, sp1), s = j - row * sp1;
+    const i64 row = ONE_ROW ? 0 : acc_quot(j, sp1), s = j - row * sp1;
     if (s == 0) return;  // what precedes a row's first boundary belongs to no segment
     S::store(out, row * p.nseg + s - 1, S::kSeeded ? S::combine(env, S::seed(env), v) : v);
   };
@@ -173,7 +172,7 @@ acc_foldseg(Spec::Env env, Spec::Out out, FoldSegParams p) {
     pendIdx[g] = NONE;
 #pragma unroll
     for (int k = 0; k < V; ++k) {
-      if (full || k < c) {
+      if (FULL || k < c) {
         if (m[k] != NONE) {
           a.v = e[k];
           a.f = 1u;
@@ -248,6 +247,24 @@ acc_foldseg(Spec::Env env, Spec::Out out, FoldSegParams p) {
   if (threadIdx.x == 0) {
     p.pend_at[tile] = sh_pend_at == NONE ? (i64)-1 : j0 + sh_pend_at;
     if (sh_pend_at != NONE) reinterpret_cast<P*>(p.pend)[tile].v = sh_pend;
+  }
+}
+
+extern "C" __global__ void __launch_bounds__(ACC_SCAN_BLOCK)
+acc_foldseg(Spec::Env env, Spec::Out out, FoldSegParams p) {
+  typedef AccScanCfg<AccSegSpec<Spec>> C;
+  // sh_first[q]: first boundary (relative to the tile's first) at position q of the tile
+  __shared__ __attribute__((aligned(16))) int sh_first[C::TILE + 4];
+  __shared__ AccSegSpec<Spec>::Elt sh_wave[ACC_SCAN_WAVES];
+  __shared__ Spec::Elt sh_pend;
+  __shared__ int sh_pend_at;
+  const bool full = ((i64)blockIdx.x + 1) * (i64)C::TILE <= p.total;
+  if (p.rows == 1) {
+    if (full) acc_foldseg_tile<true, true>(env, out, p, sh_first, sh_wave, sh_pend, sh_pend_at);
+    else acc_foldseg_tile<true, false>(env, out, p, sh_first, sh_wave, sh_pend, sh_pend_at);
+  } else {
+    if (full) acc_foldseg_tile<false, true>(env, out, p, sh_first, sh_wave, sh_pend, sh_pend_at);
+    else acc_foldseg_tile<false, false>(env, out, p, sh_first, sh_wave, sh_pend, sh_pend_at);
   }
 }
 
