@@ -30,6 +30,15 @@ ACC_DEV i64 acc_rem(i64 a, i64 b) {
   return a % b;
 }
 
+// Workgroups are handed to the 8 XCDs (each with its own L2) round-robin by workgroup
+// number.  This renumbering gives every XCD one contiguous range of the nb work items, so
+// that neighbouring items, which share cache lines at their borders, meet in the same L2.
+ACC_DEV i64 acc_xcd_contiguous(i64 b, i64 nb) {
+  const i64 q = nb >> 3, r = nb & 7;
+  const i64 xcd = b & 7, k = b >> 3;
+  return xcd * q + (xcd < r ? xcd : r) + k;
+}
+
 ACC_DEV int acc_lane() { return (int)(threadIdx.x & (ACC_WAVE - 1)); }
 ACC_DEV int acc_wave() { return (int)(threadIdx.x / ACC_WAVE); }
 

@@ -920,14 +920,23 @@ AValP Program::eval(const Sx& n, AEnv& aenv) {
     if (plan.mode == "lds2d") {
       if (out->size() == 0) return avArr(out);
       const int64_t th = plan.k->meta.group;  // rows per tile chosen by the code generator
-      const int64_t tilesY = (ext[0] + th - 1) / th, tilesX = (ext[1] + 63) / 64;
+      const int64_t tw = plan.k->meta.words;  // and columns per tile
+      const int64_t tilesY = (ext[0] + th - 1) / th, tilesX = (ext[1] + tw - 1) / tw;
       if (tilesX * tilesY > 0x7fffffffLL) throw Error("stencil: too many tiles for one launch");
       std::vector<uint64_t> args = packArgs(plan.k->meta, aenv, temps, ext);
       packOut(args, *out);
       args.push_back((uint64_t)ext[0]);
       args.push_back((uint64_t)ext[1]);
       args.push_back((uint64_t)tilesX);
-      ctx_.launch(plan.k, "acc_stencil2d", (unsigned)(tilesX * tilesY), 256, args);
+      args.push_back((uint64_t)tilesY);
+      // a workgroup chains up to 4 tiles down a column (measured best of 1..16) as long as
+      // the grid still fills the device twice over
+      const char* ce = std::getenv("ACCHIP_STENCIL_CHAIN");
+      int64_t chain = ce ? std::atoll(ce) : std::min<int64_t>(4, (tilesX * tilesY) / 512);
+      chain = std::max<int64_t>(1, std::min(chain, tilesY));
+      args.push_back((uint64_t)chain);
+      const int64_t chunksY = (tilesY + chain - 1) / chain;
+      ctx_.launch(plan.k, "acc_stencil2d", (unsigned)(tilesX * chunksY), 256, args);
       return avArr(out);
     }
     launchMap(plan.k, aenv, temps, *out);

@@ -115,6 +115,20 @@ def test_jacobi_100_iterations_small_grid_bit_equal(gpu_ctx):
 
 # ---- error conventions (Error.hs:33-62) -------------------------------------------------------
 
+@pytest.mark.parametrize("chain", [2, 3, 7])
+@pytest.mark.parametrize("bname", ["clamp", "mirror", "wrap", "constant", "function"])
+def test_stencil_tile_chains_match_oracle(gpu_ctx, monkeypatch, bname, chain):
+    # a workgroup that walks down several tiles of a column (forced here; by default only
+    # large arrays do that), on extents that leave ragged tiles at the right and bottom edge
+    monkeypatch.setenv("ACCHIP_STENCIL_CHAIN", str(chain))
+    rng = np.random.default_rng(1000 + chain)
+    b = {"constant": A.constant(A.i64, -3), "function": Q.boundary_function(A.i64, 2)}.get(bname, bname)
+    for widths, shp in [([3, 3], (150, 70)), ([5, 3], (97, 130)), ([3, 5], (33, 64))]:
+        prog = Q.stencil_weighted(A.i64, widths, b)
+        x = rng.integers(-9, 10, shp).astype(np.int64)
+        assert same(gpu_ctx.compile(prog)(x), O.run_n(prog.text(), x))
+
+
 def test_fold1_of_empty_is_a_bounds_error(gpu_ctx):
     with pytest.raises(hip.AccError) as e:
         gpu_ctx.compile(P.fold1_op(A.add, A.i32, 2))(np.zeros((3, 0), np.int32))
