@@ -59,30 +59,31 @@ template <class S> struct AccSegSpec {
   ACC_DEV bool stops(const Elt& a) { return a.f != 0; }
 };
 
+// part[t] = number of boundaries that lie before position t * TILE of the stream.  One
+// thread per boundary j: the borders t * TILE in (position of boundary j-1, position of
+// boundary j] have exactly j boundaries before them.  The offsets are read once, coalesced,
+// and no thread waits for a chain of dependent loads as a search per border would.
 extern "C" __global__ void __launch_bounds__(ACC_BLOCK)
 acc_foldseg_partition(Spec::Env env, Spec::Out out, FoldSegParams p) {
   typedef AccScanCfg<AccSegSpec<Spec>> C;
-  const i64 t = (i64)blockIdx.x * ACC_BLOCK + threadIdx.x;
-  if (t > p.tiles) return;
   const i64 sp1 = p.nseg + 1;
-  if (t == p.tiles) {
-    p.part[t] = p.rows * sp1;
-    return;
+  const i64 nb = p.rows * sp1;
+  const i64 j = (i64)blockIdx.x * ACC_BLOCK + threadIdx.x;
+  if (j >= nb) return;
+  const i64 row = p.rows == 1 ? 0 : acc_quot(j, sp1), s = j - row * sp1;
+  const i64 pos = row * p.n + Spec::seg_at(env, s);
+  i64 lo = 0;  // first border after the previous boundary
+  if (j > 0) {
+    const i64 prev = s > 0 ? row * p.n + Spec::seg_at(env, s - 1) : (row - 1) * p.n + Spec::seg_at(env, p.nseg);
+    lo = prev < 0 ? 0 : prev / (i64)C::TILE + 1;
   }
-  if (p.n <= 0) {
-    p.part[t] = 0;
-    return;
+  i64 hi = pos < 0 ? -1 : pos / (i64)C::TILE;  // last border not after this boundary
+  if (hi > p.tiles - 1) hi = p.tiles - 1;
+  for (i64 t = lo; t <= hi; ++t) p.part[t] = j;
+  if (j == nb - 1) {
+    for (i64 t = (hi < lo - 1 ? lo - 1 : hi) + 1; t < p.tiles; ++t) p.part[t] = nb;
+    p.part[p.tiles] = nb;
   }
-  const i64 pos = t * (i64)C::TILE;
-  const i64 row = pos / p.n;
-  const i64 within = pos - row * p.n;
-  i64 lo = 0, hi = sp1;  // first s with offs[s] >= within
-  while (lo < hi) {
-    const i64 mid = (lo + hi) >> 1;
-    if (Spec::seg_at(env, mid) < within) lo = mid + 1;
-    else hi = mid;
-  }
-  p.part[t] = row * sp1 + lo;
 }
 
 // One tile.  A lane owns, per group, a run of V consecutive elements and reduces it in
@@ -109,7 +110,11 @@ ACC_DEV void acc_foldseg_tile(const Spec::Env& env, const Spec::Out& out, const 
   const i64 tile = blockIdx.x;
   const i64 tlo = tile * (i64)C::TILE;
   const i64 sp1 = p.nseg + 1;
-  const i64 j0 = p.part[tile], j1 = p.part[tile + 1];
+  // (clamped: offsets that do not ascend leave entries of part unwritten)
+  const i64 nb = p.rows * sp1;
+  i64 j0 = p.part[tile], j1 = p.part[tile + 1];
+  j0 = j0 < 0 ? 0 : (j0 > nb ? nb : j0);
+  j1 = j1 < j0 ? j0 : (j1 > nb ? nb : j1);
   const int lane = acc_lane(), w = acc_wave();
   const i64 n = p.total;
   const i64 wlo = tlo + (i64)w * G * C::GROUP;
