@@ -966,7 +966,7 @@ KernelSource Codegen::foldSeg(const Sx& f, const Sx* seed, const Operand& src, c
   return ks;
 }
 
-KernelSource Codegen::scan(const Sx& f, const Sx* seed, const Operand& src, bool right, int kind) {
+KernelSource Codegen::scan(const Sx& f, const Sx* seed, const Operand& src, bool right, int kind, bool small) {
   const TypeP elt = src.r.elt;
   if (kind != 0 && !seed) throw Error("scan: this variant needs a seed");
   std::string body;
@@ -1011,11 +1011,23 @@ KernelSource Codegen::scan(const Sx& f, const Sx* seed, const Operand& src, bool
   std::vector<ArraySlot> tmpOrder;
   for (auto& kv : used_) tmpOrder.push_back(kv.second);
   int vec = vecFor(leaves, tmpOrder);
+  // Large tiles keep the number of look-back steps on the critical path small, but a row of
+  // a few tiles cannot fill 256 CUs and a row shorter than a tile leaves most of a large
+  // workgroup idle: short rows get 256-thread workgroups with 128 bytes per lane (one row
+  // of 2^20 Int32: 8 us against 15 us with the large tiles; the large tiles win from 2^23 on).
   int g = std::max(1, std::min(16, scanBytesPerLane() / std::max(1, vec * std::max(1, eltBytes))));
+  const int block = small ? 256 : scanBlock();
+  if (small) {
+    const char* sb = std::getenv("ACCHIP_SCAN_SMALL_BYTES");
+    const char* sl = std::getenv("ACCHIP_SCAN_SMALL_LB");
+    const int bytes = sb ? std::atoi(sb) : 128;
+    g = std::max(1, std::min(16, bytes / std::max(1, vec * std::max(1, eltBytes))));
+    body += "#define ACC_SCAN_LBWAVES " + std::to_string(sl ? std::max(1, std::min(4, std::atoi(sl))) : 1) + "\n";
+  }
   body += "  static constexpr int G = " + std::to_string(g) + ";\n";
-  body += "#define ACC_SCAN_BLOCK " + std::to_string(scanBlock()) + "\n";
+  body += "#define ACC_SCAN_BLOCK " + std::to_string(block) + "\n";
   KernelSource ks = finish(body, elt, leaves, "scan.hpp+scan_kernel.hpp", vec);
-  ks.block = scanBlock();
+  ks.block = block;
   ks.group = g;
   ks.words = structWords(leaves);
   return ks;

@@ -70,7 +70,8 @@ class Codegen {
   KernelSource generate(const ArrayR& out, const Sx& f);
   KernelSource backpermute(int outRank, const Sx& p, const Sx* f, const TypeP& outElt, const Operand& src);
   // kind 0: scanl1/scanr1, 1: scanl/scanr, 2: scanl'/scanr' (seed required for 1 and 2)
-  KernelSource scan(const Sx& f, const Sx* seed, const Operand& src, bool right, int kind);
+  // small: the variant for short rows (256-thread workgroups)
+  KernelSource scan(const Sx& f, const Sx* seed, const Operand& src, bool right, int kind, bool small = false);
   KernelSource foldSeg(const Sx& f, const Sx* seed, const Operand& src, const Operand& seg, ST segType);
   KernelSource permute(const Sx& f, const ArrayR& dst, const Sx& p, const Operand& src);
   KernelSource stencil(const std::vector<Sx>& patterns, const TypeP& outElt, const Sx& f,

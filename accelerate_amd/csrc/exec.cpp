@@ -558,6 +558,13 @@ ATyP Program::prepare(const Sx& n, TEnv& tenv) {
     const Sx* z = prime ? &n.at(3) : seedOf(n.at(3));
     int kind = prime ? 2 : (z ? 1 : 0);
     plan.k = ctx_.kernel(cg.scan(n.at(2), z, src, dir == "r", kind));
+    {
+      // the same scan with small tiles, chosen at launch for short rows
+      Codegen cgs(aenvOf(tenv));
+      Plan scratch;
+      Operand srcS = operandOf(n.at(4), cgs, tenv, scratch);
+      plan.k2 = ctx_.kernel(cgs.scan(n.at(2), z, srcS, dir == "r", kind, true));
+    }
     if (prime) {
       ArrayR tr = src.r;
       tr.rank -= 1;
@@ -1003,7 +1010,21 @@ AValP Program::eval(const Sx& n, AEnv& aenv) {
     for (int64_t d : outer) rows *= std::max<int64_t>(d, 0);
     AValP result = prime ? avPair(avArr(out), avArr(tot)) : avArr(out);
     if (rows == 0 || (kind == 0 && len == 0)) return result;
-    const KernelSource& m = plan.k->meta;
+    // large tiles when they fill the device, small ones otherwise
+    const KernelSource& big = plan.k->meta;
+    const int64_t bigTile = (int64_t)big.block * big.group * big.vec;
+    bool small = false;
+    if (plan.k2) {
+      const KernelSource& sm = plan.k2->meta;
+      const int64_t smallTile = (int64_t)sm.block * sm.group * sm.vec;
+      small = rows * ((len + bigTile - 1) / bigTile) < 128 || len <= 2 * smallTile;
+    }
+    if (const char* v = std::getenv("ACCHIP_SCAN_TILES")) {  // "large" / "small": override, for tests
+      if (std::string(v) == "large") small = false;
+      if (std::string(v) == "small" && plan.k2) small = true;
+    }
+    const KernelP& kern = small ? plan.k2 : plan.k;
+    const KernelSource& m = kern->meta;
     const int64_t tile = (int64_t)m.block * m.group * m.vec;
     const int64_t tpr = std::max<int64_t>(1, (len + tile - 1) / tile);
     const int64_t tiles = rows * tpr;
@@ -1019,7 +1040,7 @@ AValP Program::eval(const Sx& n, AEnv& aenv) {
     args.push_back((uint64_t)(uintptr_t)st.ticket);
     args.push_back((uint64_t)st.ticketBase);
     args.push_back((uint64_t)st.epoch);
-    ctx_.launch(plan.k, "acc_scan", (unsigned)tiles, (unsigned)m.block, args);
+    ctx_.launch(kern, "acc_scan", (unsigned)tiles, (unsigned)m.block, args);
     st.ticketBase += (uint64_t)tiles;
     return result;
   }

@@ -45,6 +45,25 @@ def test_random_cases_match_oracle(gpu_ctx, case):
         assert same(got, exp, exact=False, atol=tol)
 
 
+SCANS = [(c, g) for cs, g in ((GOLDEN, True), (PARITY, False)) for c in cs if "scan" in c[0] or "foldseg" in c[0]]
+
+
+@pytest.mark.parametrize("tiles", ["large", "small"])
+@pytest.mark.parametrize("case", SCANS, ids=[c[0][0] for c in SCANS])
+def test_scans_with_either_tile_size(gpu_ctx, monkeypatch, case, tiles):
+    # rows this short take the small-tile kernel by default; both variants must agree with
+    # the reference's known answers and with the oracle on every case
+    monkeypatch.setenv("ACCHIP_SCAN_TILES", tiles)
+    (_, prog, args, last), golden = case
+    got = gpu_ctx.compile(prog)(*args)
+    if golden:
+        assert same(got, last)
+    elif last is None:
+        assert same(got, O.run_n(prog.text(), *args))
+    else:
+        assert same(got, O.run_n(prog.text(), *args), exact=False, atol=last)
+
+
 # ---- the five benchmark configurations at the size the oracle's C loops handle in seconds ----
 
 def test_dotp_2pow24(gpu_ctx):
