@@ -39,12 +39,20 @@ acc_permute(Spec::Env env, Spec::Out out, PermuteParams p) {
 // destination range held in LDS (LDS atomics), then adds what it found to the real
 // destination with one global atomic per touched element.
 //
+// Measured on 2^26 keys into 2^16 Int32 bins (two ranges): streaming the keys alone takes
+// 45 us, the LDS atomics add 40 us whether the keys are uniform or Zipf-distributed, adding
+// the private copies to the destination 12 us; sorted keys or a single key serialise in the
+// LDS atomic unit (440 us).
+//
 // The destination is cut into `nparts` ranges of `part` elements (part <= ACC_PERMUTE_PART,
 // 128 KiB of LDS).  The sources are cut into `groups` chunks; workgroup b serves chunk
 // (b / (8 * nparts)) * 8 + b % 8 and range (b / 8) % nparts: workgroups are dealt to the 8
 // XCDs round-robin, so the nparts workgroups that read the same chunk run on the same XCD
 // and share its L2 -- the sources come from HBM once.
 #define ACC_PERMUTE_LDS_BLOCK 1024
+#ifndef ACC_PERMUTE_UNROLL
+#define ACC_PERMUTE_UNROLL 4
+#endif
 #define ACC_PERMUTE_PART (131072 / (int)sizeof(Spec::Prim))
 
 struct PermuteLdsParams {
@@ -70,17 +78,29 @@ acc_permute_lds(Spec::Env env, Spec::Out out, PermuteLdsParams p) {
   __syncthreads();
   const i64 begin = chunkId * p.chunk;
   const i64 end = begin + p.chunk < p.n ? begin + p.chunk : p.n;
-  for (i64 i0 = begin + (i64)threadIdx.x * 4; i0 < end; i0 += (i64)ACC_PERMUTE_LDS_BLOCK * 4) {
-    if (i0 + 4 <= end) {
-      i64 j[4];
-      bool ok[4];
+  // ACC_PERMUTE_UNROLL groups of 4 consecutive sources per thread and step: all targets of
+  // a step are computed (their loads issued) before the first update, which keeps enough
+  // loads in flight for a single resident workgroup per CU to stream at HBM speed
+  const i64 step = (i64)ACC_PERMUTE_LDS_BLOCK * 4 * ACC_PERMUTE_UNROLL;
+  for (i64 base = begin; base < end; base += step) {
+    if (base + step <= end) {
+      i64 j[ACC_PERMUTE_UNROLL][4];
+      bool ok[ACC_PERMUTE_UNROLL][4];
 #pragma unroll
-      for (int k = 0; k < 4; ++k) ok[k] = S::target(env, i0 + k, j[k]);
+      for (int g = 0; g < ACC_PERMUTE_UNROLL; ++g) {
+        const i64 i0 = base + ((i64)g * ACC_PERMUTE_LDS_BLOCK + threadIdx.x) * 4;
 #pragma unroll
-      for (int k = 0; k < 4; ++k)
-        if (ok[k] && j[k] >= lo && j[k] < hi) S::lds_update(&priv[j[k] - lo], S::in_linear(env, i0 + k));
+        for (int k = 0; k < 4; ++k) ok[g][k] = S::target(env, i0 + k, j[g][k]);
+      }
+#pragma unroll
+      for (int g = 0; g < ACC_PERMUTE_UNROLL; ++g) {
+        const i64 i0 = base + ((i64)g * ACC_PERMUTE_LDS_BLOCK + threadIdx.x) * 4;
+#pragma unroll
+        for (int k = 0; k < 4; ++k)
+          if (ok[g][k] && j[g][k] >= lo && j[g][k] < hi) S::lds_update(&priv[j[g][k] - lo], S::in_linear(env, i0 + k));
+      }
     } else {
-      for (i64 i = i0; i < end; ++i) {
+      for (i64 i = base + threadIdx.x; i < end; i += ACC_PERMUTE_LDS_BLOCK) {
         i64 j;
         if (S::target(env, i, j) && j >= lo && j < hi) S::lds_update(&priv[j - lo], S::in_linear(env, i));
       }

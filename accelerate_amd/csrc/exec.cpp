@@ -898,7 +898,11 @@ AValP Program::eval(const Sx& n, AEnv& aenv) {
     if (plan.mode == "atomic" && cnt >= (1 << 20) && out->size() <= 8 * partMax) {
       const int64_t nparts = (out->size() + partMax - 1) / partMax;
       const int64_t part = (out->size() + nparts - 1) / nparts;
-      const int64_t groups = 256;
+      // one workgroup per CU in total (each holds 128 KiB of LDS): fewer, longer workgroups
+      // mean fewer private copies to add into the destination at the end
+      const char* ge = std::getenv("ACCHIP_PERMUTE_GROUPS");
+      int64_t groups = ge ? std::atoll(ge) : 256 / nparts;
+      groups = std::max<int64_t>(8, groups / 8 * 8);
       int64_t chunk = ((cnt + groups - 1) / groups + 3) / 4 * 4;
       args.push_back((uint64_t)cnt);
       args.push_back((uint64_t)chunk);
