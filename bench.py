@@ -22,6 +22,11 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0   # MI355X HBM3E, published peak
+# HBM bytes one launch of the headline kernel moves, from the rocprofv3 FETCH_SIZE and
+# WRITE_SIZE passes over this same program (profiles/acc_scan_scanl1_int64_2p28.md: 2.0047 GiB
+# read + 2.0016 GiB written, counters scaled by a copy kernel of known size); a counter pass
+# cannot run inside the timed process, so the figure is carried here.
+SCAN_TRAFFIC_BYTES = 4301803417
 
 
 def log(*a):
@@ -103,7 +108,7 @@ def main():
         "config": {"workload": "scanl1 (+) on an Int64 vector, n=2^28, uniform integers in [-1000,1000]",
                    "program": "Scan LeftToRight (+) Nothing (Manifest (Avar a0))", "kernel": "acc_scan"},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None},
+                     "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": SCAN_TRAFFIC_BYTES},
         "cpu_baseline": cpu,
     }
 
