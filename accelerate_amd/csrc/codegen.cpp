@@ -850,8 +850,21 @@ KernelSource Codegen::fold(const Sx& f, const Sx* seed, const Operand& src) {
     if (!typeEq(valType(v), elt)) throw Error("fold: fused producer does not return the element type");
     body += fnHead("Elt", "in_linear", "const Env& env, i64 i") + returnElt(v, em) + "  }\n";
   }
-  KernelSource ks = finish(body, elt, typeLeaves(elt), "fold.hpp", 0);
+  // geometry of the kernel for many short rows (acc_fold_rows): 256 threads, about 64 bytes
+  // of (value, flag) pairs per lane
+  auto leaves = typeLeaves(elt);
+  int eltBytes = 4;
+  for (ST st : leaves) eltBytes += stSize(st);
+  std::vector<ArraySlot> tmpOrder;
+  for (auto& kv : used_) tmpOrder.push_back(kv.second);
+  const int vec = vecFor(leaves, tmpOrder);
+  const int g = std::max(1, std::min(8, 64 / std::max(1, vec * eltBytes)));
+  body += "  static constexpr int G = " + std::to_string(g) + ";\n";
+  body += "#define ACC_SCAN_BLOCK 256\n";
+  KernelSource ks = finish(body, elt, leaves, "scan.hpp+fold.hpp", vec);
   ks.commutative = comm;
+  ks.group = g;
+  ks.block = 256;
   return ks;
 }
 

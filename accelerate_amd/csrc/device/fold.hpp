@@ -169,3 +169,31 @@ acc_fold_final(Spec::Env env, Spec::Out out, Spec::Out tmp, FoldParams p) {
   bool have = acc_fold_block<S>(env, src, row * p.bpr, 0, p.bpr, r);
   acc_fold_finish<S>(env, out, row, have, r);
 }
+
+// Rows of at most half a tile of the scan machinery: a workgroup reduces rpt whole rows at
+// once as a scan of (head flag, value) pairs over the row-major stream (acc_rows_tile); the
+// lane that holds the last element of a row writes the row's result.  One workgroup per row
+// would leave all but a few lanes idle.
+struct FoldRowsParams {
+  i64 rows;
+  i64 n;    // 1 <= n, rpt * n <= TILE
+  i64 rpt;  // rows per workgroup
+};
+
+extern "C" __global__ void __launch_bounds__(ACC_SCAN_BLOCK)
+acc_fold_rows(Spec::Env env, Spec::Out out, Spec::Out tmp, FoldRowsParams p) {
+  typedef Spec S;
+  typedef S::Elt Elt;
+  const i64 row0 = (i64)blockIdx.x * p.rpt;
+  const i64 nrows = p.rows - row0 < p.rpt ? p.rows - row0 : p.rpt;
+  const int n = (int)p.n;
+  auto load = [&](int idx, int r, int t) -> Elt {
+    Elt v = S::in_linear(env, row0 * p.n + idx);
+    if (S::kSeeded && t == 0) v = S::combine(env, S::seed(env), v);
+    return v;
+  };
+  auto store = [&](int idx, int r, int t, const Elt& y) {
+    if (t == n - 1) S::store(out, row0 + r, y);
+  };
+  acc_rows_tile<S>(env, (int)(nrows * p.n), n, load, store);
+}

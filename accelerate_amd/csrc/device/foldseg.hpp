@@ -32,33 +32,6 @@ struct FoldSegParams {
   i64* pend_at;   // [tiles] boundary number of that end, or -1
 };
 
-template <class S> struct AccSegSpec {
-  typedef typename S::Env Env;
-  struct Elt {
-    typename S::Elt v;
-    u32 f;
-  };
-  enum { V = S::V, G = S::G };
-  static constexpr bool kSeeded = false;  // z is applied when a segment's value is written
-  ACC_DEV Elt combine(const Env& env, const Elt& a, const Elt& b) {
-    Elt r;
-    if (b.f) {
-      r = b;
-    } else {
-      r.v = S::combine(env, a.v, b.v);
-      r.f = a.f;
-    }
-    return r;
-  }
-  ACC_DEV Elt seed(const Env&) {
-    Elt r{};
-    return r;
-  }
-  // an aggregate that contains a segment head hides everything before it: the look-back
-  // of a later tile may stop there
-  ACC_DEV bool stops(const Elt& a) { return a.f != 0; }
-};
-
 // part[t] = number of boundaries that lie before position t * TILE of the stream.  One
 // thread per boundary j: the borders t * TILE in (position of boundary j-1, position of
 // boundary j] have exactly j boundaries before them.  The offsets are read once, coalesced,

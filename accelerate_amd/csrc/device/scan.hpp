@@ -353,6 +353,127 @@ ACC_DEV void acc_scan_tile(const typename S::Env& env, u64* desc, i64 tiles, i64
   }
 }
 
+// Values paired with a head flag: the scan of such pairs under
+//     (fa, a) (+) (fb, b) = fb ? (1, b) : (fa, a (+) b)
+// restarts at every head and is associative whenever (+) is.
+template <class S> struct AccSegSpec {
+  typedef typename S::Env Env;
+  struct Elt {
+    typename S::Elt v;
+    u32 f;
+  };
+  enum { V = S::V, G = S::G };
+  static constexpr bool kSeeded = false;  // z is applied when a segment's value is written
+  ACC_DEV Elt combine(const Env& env, const Elt& a, const Elt& b) {
+    Elt r;
+    if (b.f) {
+      r = b;
+    } else {
+      r.v = S::combine(env, a.v, b.v);
+      r.f = a.f;
+    }
+    return r;
+  }
+  ACC_DEV Elt seed(const Env&) {
+    Elt r{};
+    return r;
+  }
+  // an aggregate that contains a segment head hides everything before it: the look-back
+  // of a later tile may stop there
+  ACC_DEV bool stops(const Elt& a) { return a.f != 0; }
+};
+
+// Many rows shorter than a tile: a workgroup takes `cnt` consecutive elements of the
+// row-major stream that are a whole number of rows of n elements (cnt <= TILE) and scans
+// them as (head flag, value) pairs with a head at the start of every row, so that no lane
+// idles however short the rows are and nothing is exchanged between workgroups.
+// load(idx, r, t) yields the element at stream position idx of the tile = row r of the
+// tile, traversal position t; store(idx, r, t, y) receives the running combination of
+// row r up to t.  Called by all threads of the workgroup.
+template <class S, class Load, class Store>
+ACC_DEV void acc_rows_tile(const typename S::Env& env, int cnt, int n, const Load& load, const Store& store) {
+  typedef AccSegSpec<S> SS;
+  typedef typename SS::Elt P;
+  typedef AccScanCfg<S> C;
+  const int V = C::V, G = C::G;
+  __shared__ P sh_wave[ACC_SCAN_WAVES];
+  const int lane = acc_lane(), w = acc_wave();
+  const int wlo = w * G * C::GROUP;
+  P x[C::G][C::V];
+  int r0[C::G], t0[C::G];
+#pragma unroll
+  for (int g = 0; g < G; ++g) {
+    const int idx0 = wlo + (g * ACC_WAVE + lane) * V;
+    int r = idx0 / n, t = idx0 - r * n;
+    r0[g] = r;
+    t0[g] = t;
+#pragma unroll
+    for (int k = 0; k < V; ++k) {
+      if (idx0 + k < cnt) {
+        P e;
+        e.v = load(idx0 + k, r, t);
+        e.f = t == 0 ? 1u : 0u;
+        x[g][k] = k == 0 ? e : SS::combine(env, x[g][k - 1], e);
+      } else if (k > 0) {
+        x[g][k] = x[g][k - 1];
+      }
+      if (++t == n) {
+        t = 0;
+        ++r;
+      }
+    }
+  }
+  P waveTot;
+  bool hasWaveTot = false;
+#pragma unroll
+  for (int g = 0; g < G; ++g) {
+    int c = cnt - (wlo + g * C::GROUP);
+    c = c < 0 ? 0 : (c > C::GROUP ? C::GROUP : c);
+    P ts = acc_wave_scan<SS>(env, x[g][V - 1], lane);
+    P lanePre = acc_prev_lane(ts);
+    const int last = c > 0 ? (c - 1) / V : 0;
+    P gt = acc_readlane(ts, last);
+    P pre;
+    if (acc_join<SS>(env, hasWaveTot, waveTot, lane > 0, lanePre, pre)) {
+#pragma unroll
+      for (int k = 0; k < V; ++k) x[g][k] = SS::combine(env, pre, x[g][k]);
+    }
+    if (c > 0) {
+      waveTot = hasWaveTot ? SS::combine(env, waveTot, gt) : gt;
+      hasWaveTot = true;
+    }
+  }
+  if (lane == 0) sh_wave[w] = waveTot;
+  __syncthreads();
+  const int perWave = G * C::GROUP;
+  int wavesWithData = (cnt + perWave - 1) / perWave;
+  if (wavesWithData > ACC_SCAN_WAVES) wavesWithData = ACC_SCAN_WAVES;
+  if (w == 0) {
+    P t = sh_wave[lane < ACC_SCAN_WAVES ? lane : 0];
+    t = acc_wave_scan<SS>(env, t, lane);
+    if (lane < ACC_SCAN_WAVES) sh_wave[lane] = t;
+  }
+  __syncthreads();
+  const bool hasBase = w > 0 && w <= wavesWithData;
+  const P base = sh_wave[w > 0 ? w - 1 : 0];
+#pragma unroll
+  for (int g = 0; g < G; ++g) {
+    const int idx0 = wlo + (g * ACC_WAVE + lane) * V;
+    int r = r0[g], t = t0[g];
+#pragma unroll
+    for (int k = 0; k < V; ++k) {
+      if (idx0 + k < cnt) {
+        const P y = hasBase ? SS::combine(env, base, x[g][k]) : x[g][k];
+        store(idx0 + k, r, t, y.v);
+      }
+      if (++t == n) {
+        t = 0;
+        ++r;
+      }
+    }
+  }
+}
+
 ACC_DEV i64 acc_take_ticket(u64* ticket, u64 base) {
 #ifdef ACC_X_NOTICKET
   return (i64)blockIdx.x;

@@ -33,3 +33,38 @@ acc_scan(Spec::Env env, Spec::Out out, Spec::Out tot, ScanParams p) {
     else S::store(out, outBase + (S::kRight ? m - 1 : 0), z);
   }
 }
+
+// Rows of at most half a tile: a workgroup scans rpt whole rows at once (acc_rows_tile).
+struct ScanRowsParams {
+  i64 rows;
+  i64 n;    // 1 <= n, rpt * n <= TILE
+  i64 rpt;  // rows per workgroup
+};
+
+extern "C" __global__ void __launch_bounds__(ACC_SCAN_BLOCK, ACC_SCAN_MINWAVES)
+acc_scan_rows(Spec::Env env, Spec::Out out, Spec::Out tot, ScanRowsParams p) {
+  typedef Spec S;
+  typedef S::Elt Elt;
+  const i64 row0 = (i64)blockIdx.x * p.rpt;
+  const i64 nrows = p.rows - row0 < p.rpt ? p.rows - row0 : p.rpt;
+  const int n = (int)p.n;
+  const i64 m = S::kKind == 1 ? p.n + 1 : p.n;  // entries per output row
+  auto load = [&](int idx, int r, int t) -> Elt {
+    Elt v = S::in_linear(env, S::kRight ? (row0 + r) * p.n + (n - 1 - t) : row0 * p.n + idx);
+    if (S::kSeeded && t == 0) v = S::combine(env, S::seed(env), v);
+    return v;
+  };
+  auto store = [&](int idx, int r, int t, const Elt& y) {
+    const i64 row = row0 + r;
+    if (S::kKind == 0) {
+      S::store(out, S::kRight ? row * p.n + (n - 1 - t) : row0 * p.n + idx, y);
+    } else {
+      const i64 outBase = row * m;
+      if (t == 0) S::store(out, outBase + (S::kRight ? m - 1 : 0), S::seed(env));
+      const i64 u = (i64)t + 1;
+      if (S::kKind == 2 && u == p.n) S::store(tot, row, y);
+      else S::store(out, outBase + (S::kRight ? m - 1 - u : u), y);
+    }
+  };
+  acc_rows_tile<S>(env, (int)(nrows * p.n), n, load, store);
+}

@@ -835,6 +835,28 @@ AValP Program::eval(const Sx& n, AEnv& aenv) {
     DArrayP out = alloc(plan.ty->r, ext);
     int64_t rows = out->size();
     if (rows == 0) return avArr(out);
+    {
+      // many short rows: several whole rows per workgroup (acc_fold_rows)
+      const KernelSource& m = plan.k->meta;
+      const int64_t rowsTile = (int64_t)m.block * m.group * m.vec;
+      const char* fr = std::getenv("ACCHIP_FOLD_ROWS");  // "0" / "1": override, for tests
+      bool useRows = len >= 1 && rows >= 64 && 4 * len <= rowsTile;
+      if (fr && fr[0] == '0') useRows = false;
+      if (fr && fr[0] == '1') useRows = len >= 1 && len <= rowsTile;
+      if (useRows) {
+        const int64_t rpt = rowsTile / len;
+        const int64_t groups = (rows + rpt - 1) / rpt;
+        if (groups > 0x7fffffffLL) throw Error("fold: too many rows for one launch");
+        std::vector<uint64_t> args = packArgs(m, aenv, temps, {});
+        packOut(args, *out);
+        packOut(args, *out);
+        args.push_back((uint64_t)rows);
+        args.push_back((uint64_t)len);
+        args.push_back((uint64_t)rpt);
+        ctx_.launch(plan.k, "acc_fold_rows", (unsigned)groups, (unsigned)m.block, args);
+        return avArr(out);
+      }
+    }
     // geometry: enough workgroups to fill the chip, each with at least a few tiles of work
     const int64_t tile = (int64_t)4 * 64 * plan.k->meta.vec;
     const int64_t target = 2048;
@@ -1026,6 +1048,26 @@ AValP Program::eval(const Sx& n, AEnv& aenv) {
     if (const char* v = std::getenv("ACCHIP_SCAN_TILES")) {  // "large" / "small": override, for tests
       if (std::string(v) == "large") small = false;
       if (std::string(v) == "small" && plan.k2) small = true;
+    }
+    if (plan.k2 && len >= 1) {
+      // many short rows: several whole rows per workgroup (acc_scan_rows)
+      const KernelSource& sm = plan.k2->meta;
+      const int64_t rowsTile = (int64_t)sm.block * sm.group * sm.vec;
+      const char* v = std::getenv("ACCHIP_SCAN_TILES");
+      const bool forced = v && std::string(v) == "rows";
+      if ((forced && len <= rowsTile) || (!v && rows >= 2 && 2 * len <= rowsTile)) {
+        const int64_t rpt = rowsTile / len;
+        const int64_t groups = (rows + rpt - 1) / rpt;
+        if (groups > 0x7fffffffLL) throw Error("scan: too many rows for one launch");
+        std::vector<uint64_t> args = packArgs(sm, aenv, temps, {});
+        packOut(args, *out);
+        packOut(args, *tot);
+        args.push_back((uint64_t)rows);
+        args.push_back((uint64_t)len);
+        args.push_back((uint64_t)rpt);
+        ctx_.launch(plan.k2, "acc_scan_rows", (unsigned)groups, (unsigned)sm.block, args);
+        return result;
+      }
     }
     const KernelP& kern = small ? plan.k2 : plan.k;
     const KernelSource& m = kern->meta;

@@ -102,8 +102,9 @@ def _rand(rng, ty, shape, lo=-1000, hi=1000):
     return rng.integers(max(lo, info.min), min(hi, info.max), shape, endpoint=True).astype(NPT[ty])
 
 
-SHAPES = {1: [(0,), (1,), (63,), (300,), (5000,)], 2: [(3, 0), (0, 4), (5, 10), (17, 129), (2, 4100)],
-          3: [(2, 3, 0), (3, 4, 50), (2, 2, 700)]}
+SHAPES = {1: [(0,), (1,), (63,), (300,), (5000,)],
+          2: [(3, 0), (0, 4), (5, 10), (17, 129), (2, 4100), (900, 7), (150, 33), (3000, 1)],
+          3: [(2, 3, 0), (3, 4, 50), (2, 2, 700), (30, 20, 3)]}
 
 
 def parity_cases():

@@ -48,12 +48,32 @@ def test_random_cases_match_oracle(gpu_ctx, case):
 SCANS = [(c, g) for cs, g in ((GOLDEN, True), (PARITY, False)) for c in cs if "scan" in c[0] or "foldseg" in c[0]]
 
 
-@pytest.mark.parametrize("tiles", ["large", "small"])
+@pytest.mark.parametrize("tiles", ["large", "small", "rows"])
 @pytest.mark.parametrize("case", SCANS, ids=[c[0][0] for c in SCANS])
 def test_scans_with_either_tile_size(gpu_ctx, monkeypatch, case, tiles):
-    # rows this short take the small-tile kernel by default; both variants must agree with
-    # the reference's known answers and with the oracle on every case
+    # rows this short take the small-tile kernel or, several rows per workgroup, the rows
+    # kernel by default; every variant must agree with the reference's known answers and with
+    # the oracle on every case ("rows" falls back to tiles where a row exceeds a tile)
     monkeypatch.setenv("ACCHIP_SCAN_TILES", tiles)
+    (_, prog, args, last), golden = case
+    got = gpu_ctx.compile(prog)(*args)
+    if golden:
+        assert same(got, last)
+    elif last is None:
+        assert same(got, O.run_n(prog.text(), *args))
+    else:
+        assert same(got, O.run_n(prog.text(), *args), exact=False, atol=last)
+
+
+FOLDS = [(c, g) for cs, g in ((GOLDEN, True), (PARITY, False)) for c in cs
+         if c[0].startswith(("fold", "dotp", "mss", "issue228")) and "foldseg" not in c[0]]
+
+
+@pytest.mark.parametrize("rows_kernel", ["0", "1"])
+@pytest.mark.parametrize("case", FOLDS, ids=[c[0][0] for c in FOLDS])
+def test_folds_with_and_without_the_rows_kernel(gpu_ctx, monkeypatch, case, rows_kernel):
+    # short rows are reduced several per workgroup; both paths must give the same answers
+    monkeypatch.setenv("ACCHIP_FOLD_ROWS", rows_kernel)
     (_, prog, args, last), golden = case
     got = gpu_ctx.compile(prog)(*args)
     if golden:
