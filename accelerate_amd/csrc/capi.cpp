@@ -8,21 +8,23 @@
 
 using namespace acchip;
 
+// Handles may be released in any order, also after acchip_shutdown: programs, arrays and
+// events each hold a reference to the context, which goes away with the last of them.
 struct acchip_ctx {
-  Context ctx;
-  explicit acchip_ctx(int device) : ctx(device) {}
+  std::shared_ptr<Context> ctx;
+  explicit acchip_ctx(int device) : ctx(std::make_shared<Context>(device)) {}
 };
 struct acchip_program {
-  acchip_ctx* owner;
+  std::shared_ptr<Context> keep;  // declared first: destroyed after prog
   Program prog;
-  acchip_program(acchip_ctx* c, const char* t, size_t n) : owner(c), prog(c->ctx, t, n) {}
+  acchip_program(acchip_ctx* c, const char* t, size_t n) : keep(c->ctx), prog(*c->ctx, t, n) {}
 };
 struct acchip_array {
   AValP v;
   std::string eltText;
 };
 struct acchip_event {
-  acchip_ctx* owner;
+  std::shared_ptr<Context> keep;
   hipEvent_t ev;
 };
 
@@ -72,46 +74,46 @@ void acchip_shutdown(acchip_ctx* ctx) { delete ctx; }
 
 int acchip_mem_info(acchip_ctx* ctx, size_t* total, size_t* available) {
   ACCHIP_TRY
-  ctx->ctx.memInfo(total, available);
+  ctx->ctx->memInfo(total, available);
   return ACCHIP_OK;
   ACCHIP_END
 }
 
 void* acchip_malloc(acchip_ctx* ctx, size_t bytes) {
   try {
-    return ctx->ctx.malloc(bytes);
+    return ctx->ctx->malloc(bytes);
   } catch (...) {
     return nullptr;
   }
 }
 void acchip_free(acchip_ctx* ctx, void* p) {
   try {
-    ctx->ctx.free(p);
+    ctx->ctx->free(p);
   } catch (...) {
   }
 }
 void acchip_purge(acchip_ctx* ctx) {
   try {
-    ctx->ctx.purge();
+    ctx->ctx->purge();
   } catch (...) {
   }
 }
 
 int acchip_poke(acchip_ctx* ctx, void* devptr, const void* host, size_t bytes) {
   ACCHIP_TRY
-  ctx->ctx.poke(devptr, host, bytes);
+  ctx->ctx->poke(devptr, host, bytes);
   return ACCHIP_OK;
   ACCHIP_END
 }
 int acchip_peek(acchip_ctx* ctx, void* host, const void* devptr, size_t bytes) {
   ACCHIP_TRY
-  ctx->ctx.peek(host, devptr, bytes);
+  ctx->ctx->peek(host, devptr, bytes);
   return ACCHIP_OK;
   ACCHIP_END
 }
 
 long long acchip_stat(acchip_ctx* ctx, const char* name) {
-  Stats& s = ctx->ctx.stats;
+  Stats& s = ctx->ctx->stats;
   std::string n = name ? name : "";
   if (n == "bytes_allocated_remote") return s.bytesAllocated;
   if (n == "bytes_copied_to_remote") return s.bytesCopiedToRemote;
@@ -130,10 +132,10 @@ long long acchip_stat(acchip_ctx* ctx, const char* name) {
 
 int acchip_event_record(acchip_ctx* ctx, acchip_event** out) {
   ACCHIP_TRY
-  if (!ctx->ctx.hasDevice()) throw Error("no device");
-  auto* e = new acchip_event{ctx, nullptr};
+  if (!ctx->ctx->hasDevice()) throw Error("no device");
+  auto* e = new acchip_event{ctx->ctx, nullptr};
   hipError_t r = hipEventCreate(&e->ev);
-  if (r == hipSuccess) r = hipEventRecord(e->ev, ctx->ctx.stream());
+  if (r == hipSuccess) r = hipEventRecord(e->ev, ctx->ctx->stream());
   if (r != hipSuccess) {
     delete e;
     hipCheck(r, "hipEventRecord");
@@ -172,7 +174,7 @@ void acchip_event_destroy(acchip_event* ev) {
 }
 int acchip_sync(acchip_ctx* ctx) {
   ACCHIP_TRY
-  ctx->ctx.sync();
+  ctx->ctx->sync();
   return ACCHIP_OK;
   ACCHIP_END
 }
@@ -205,7 +207,7 @@ int acchip_array_wrap(acchip_ctx* ctx, int rank, const int64_t* shape, const cha
   int64_t n = d->size();
   for (int i = 0; i < n_buffers; ++i) {
     auto b = std::make_shared<Buffer>();
-    b->ctx = &ctx->ctx;
+    b->ctx = ctx->ctx;
     b->p = buffers[i];
     b->bytes = (size_t)n * stSize(leaves[i]);
     b->owned = false;
@@ -222,14 +224,14 @@ int acchip_array_wrap(acchip_ctx* ctx, int rank, const int64_t* shape, const cha
 
 int acchip_array_new(acchip_ctx* ctx, int rank, const int64_t* shape, const char* elt_type, acchip_array** out) {
   ACCHIP_TRY
-  if (!ctx->ctx.hasDevice()) throw Error("no device");
+  if (!ctx->ctx->hasDevice()) throw Error("no device");
   DArrayP d = describe(rank, shape, elt_type);
   int64_t n = d->size();
   for (ST st : typeLeaves(d->r.elt)) {
     auto b = std::make_shared<Buffer>();
-    b->ctx = &ctx->ctx;
+    b->ctx = ctx->ctx;
     b->bytes = (size_t)n * stSize(st);
-    b->p = ctx->ctx.malloc(b->bytes);
+    b->p = ctx->ctx->malloc(b->bytes);
     if (!b->p) throw Error("Remote memory exhausted");
     b->owned = true;
     d->bufs.push_back(b);
@@ -316,8 +318,8 @@ int acchip_sha3_256(const void* data, size_t length, uint8_t digest[32]) {
 int acchip_execute(acchip_ctx* ctx, acchip_program* p, acchip_array* const* args, int n_args,
                    acchip_array* const* uses, int n_uses, acchip_array** result) {
   ACCHIP_TRY
-  if (!ctx->ctx.hasDevice()) throw Error("no device");
-  if (p->owner != ctx) throw Error("program was compiled in a different context");
+  if (!ctx->ctx->hasDevice()) throw Error("no device");
+  if (p->keep != ctx->ctx) throw Error("program was compiled in a different context");
   std::vector<AValP> av;
   for (int i = 0; i < n_args; ++i) av.push_back(args[i]->v);
   std::vector<DArrayP> uv;

@@ -3,22 +3,20 @@
 // segment yields z.  The node receives offsets (Prelude.hs:710-717), not lengths.
 //
 // Load balance does not depend on segment lengths: the rows are laid end to end into one
-// stream of rows*n elements which is cut into equal tiles, exactly as for a scan, and a
-// tile computes a segmented inclusive scan of its elements, i.e. a scan of (head flag,
-// value) pairs under
+// stream of rows*n elements which is cut into equal tiles, and a tile reduces its elements
+// as (head flag, value) pairs under
 //     (fa, a) (+) (fb, b) = fb ? (1, b) : (fa, a (+) b)
-// which is associative whenever (+) is.  Segments that cross tile borders get their
-// carry through the same decoupled look-back as a plain scan.  The value of a segment is
-// the scan value at its last element; it is written by the lane that holds that element.
+// which is associative whenever (+) is.  Tiles do not wait for each other: a tile leaves its
+// carry (head seen, value since the last head) and the one segment end that no head of the
+// tile precedes; acc_foldseg_fixup completes those ends from the carries of the tiles before.
 //
 // Boundaries: row r contributes S+1 boundaries at stream positions r*n + offs[s],
 // s = 0..S (S segments per row).  Boundary number j = r*(S+1) + s starts segment (r, s)
 // when s < S; what lies between boundary (r, S) and boundary (r+1, 0) belongs to no
-// segment and is discarded.  A partition kernel finds, for every tile border, how many
-// boundaries lie before it (binary search in the offsets), so a tile knows which
-// boundaries fall inside it and marks them in LDS: sh_first[p] = first boundary at
-// position p of the tile.  Empty segments are recognised while marking (two equal
-// consecutive offsets) and get z directly.
+// segment and is discarded.  acc_foldseg_partition finds, for every tile border, how many
+// boundaries lie before it, so a tile knows which boundaries fall inside it and marks them
+// in LDS: sh_first[p] = first boundary at position p of the tile.  Empty segments (two equal
+// consecutive offsets) get z from the partition kernel.
 
 struct FoldSegParams {
   i64 rows;
@@ -36,27 +34,47 @@ struct FoldSegParams {
 // thread per boundary j: the borders t * TILE in (position of boundary j-1, position of
 // boundary j] have exactly j boundaries before them.  The offsets are read once, coalesced,
 // and no thread waits for a chain of dependent loads as a search per border would.
+// A range of more than a few borders (a segment that spans many tiles, the tail behind the
+// last boundary) is filled by the whole wave, 64 borders a step.
+ACC_DEV void acc_fill_borders(i64* part, bool valid, i64 lo, i64 hi, i64 value) {
+  const int lane = acc_lane();
+  const bool big = valid && hi - lo >= 4;
+  if (valid && !big)
+    for (i64 t = lo; t <= hi; ++t) part[t] = value;
+  u64 m = __ballot(big);
+  while (m) {
+    const int src = __builtin_ctzll(m);
+    m &= m - 1;
+    const i64 l = acc_shfl(lo, src), h = acc_shfl(hi, src), v = acc_shfl(value, src);
+    for (i64 t = l + lane; t <= h; t += ACC_WAVE) part[t] = v;
+  }
+}
+
 extern "C" __global__ void __launch_bounds__(ACC_BLOCK)
 acc_foldseg_partition(Spec::Env env, Spec::Out out, FoldSegParams p) {
   typedef AccScanCfg<AccSegSpec<Spec>> C;
   const i64 sp1 = p.nseg + 1;
   const i64 nb = p.rows * sp1;
   const i64 j = (i64)blockIdx.x * ACC_BLOCK + threadIdx.x;
-  if (j >= nb) return;
-  const i64 row = p.rows == 1 ? 0 : acc_quot(j, sp1), s = j - row * sp1;
-  const i64 pos = row * p.n + Spec::seg_at(env, s);
-  i64 lo = 0;  // first border after the previous boundary
-  if (j > 0) {
-    const i64 prev = s > 0 ? row * p.n + Spec::seg_at(env, s - 1) : (row - 1) * p.n + Spec::seg_at(env, p.nseg);
-    lo = prev < 0 ? 0 : prev / (i64)C::TILE + 1;
+  const bool valid = j < nb;
+  i64 lo = 0, hi = -1;  // borders in (previous boundary, this boundary]
+  if (valid) {
+    const i64 row = p.rows == 1 ? 0 : acc_quot(j, sp1), s = j - row * sp1;
+    const i64 pos = row * p.n + Spec::seg_at(env, s);
+    if (j > 0) {
+      const i64 prev = s > 0 ? row * p.n + Spec::seg_at(env, s - 1) : (row - 1) * p.n + Spec::seg_at(env, p.nseg);
+      lo = prev < 0 ? 0 : prev / (i64)C::TILE + 1;
+      // an empty segment yields z; it is written here, where every boundary has a thread of its own
+      if (Spec::kSeeded && s > 0 && prev == pos) Spec::store(out, row * p.nseg + s - 1, Spec::seed(env));
+    }
+    hi = pos < 0 ? -1 : pos / (i64)C::TILE;
+    if (hi > p.tiles - 1) hi = p.tiles - 1;
   }
-  i64 hi = pos < 0 ? -1 : pos / (i64)C::TILE;  // last border not after this boundary
-  if (hi > p.tiles - 1) hi = p.tiles - 1;
-  for (i64 t = lo; t <= hi; ++t) p.part[t] = j;
-  if (j == nb - 1) {
-    for (i64 t = (hi < lo - 1 ? lo - 1 : hi) + 1; t < p.tiles; ++t) p.part[t] = nb;
-    p.part[p.tiles] = nb;
-  }
+  acc_fill_borders(p.part, valid, lo, hi, j);
+  // the borders behind the last boundary, and the end marker
+  const bool last = valid && j == nb - 1;
+  acc_fill_borders(p.part, last, (hi < lo - 1 ? lo - 1 : hi) + 1, p.tiles - 1, nb);
+  if (last) p.part[p.tiles] = nb;
 }
 
 // One tile.  A lane owns, per group, a run of V consecutive elements and reduces it in
@@ -109,12 +127,48 @@ ACC_DEV void acc_foldseg_tile(const Spec::Env& env, const Spec::Out& out, const 
   for (int i = threadIdx.x; i < C::TILE / 4 + 1; i += ACC_SCAN_BLOCK)
     reinterpret_cast<int4*>(sh_first)[i] = make_int4(NONE, NONE, NONE, NONE);
   __syncthreads();
-  for (i64 j = j0 + threadIdx.x; j < j1; j += ACC_SCAN_BLOCK) {
-    const i64 row = ONE_ROW ? 0 : acc_quot(j, sp1), s = j - row * sp1;
-    const i64 o = S::seg_at(env, s);
-    const i64 rel = row * p.n + o - tlo;
-    if (rel >= 0 && rel <= C::TILE) atomicMin(&sh_first[rel], (int)(j - j0));
-    if (S::kSeeded && s < p.nseg && S::seg_at(env, s + 1) == o) S::store(out, row * p.nseg + s, S::seed(env));
+  // Boundaries are marked four per thread and step so that their offsets are loaded
+  // together.  A boundary at the same position as its predecessor in the row (an empty
+  // segment before it) is not the first at its position and is skipped: a run of empty
+  // segments would otherwise serialise in one LDS word.
+  const bool crowded = j1 - j0 > 4 * (i64)C::TILE;
+  if (crowded) {
+    // far more boundaries than positions (long runs of empty segments): every position
+    // looks for its first boundary by binary search instead
+    for (int q = threadIdx.x; q <= C::TILE; q += ACC_SCAN_BLOCK) {
+      auto position = [&](i64 j) {
+        const i64 row = ONE_ROW ? 0 : acc_quot(j, sp1);
+        return row * p.n + S::seg_at(env, j - row * sp1);
+      };
+      i64 a = j0, b = j1;  // first boundary at a position >= tlo + q
+      while (a < b) {
+        const i64 mid = (a + b) >> 1;
+        if (position(mid) < tlo + q) a = mid + 1;
+        else b = mid;
+      }
+      if (a < j1 && position(a) == tlo + q) sh_first[q] = (int)(a - j0);
+    }
+  }
+  for (i64 jb = j0; jb < j1 && !crowded; jb += (i64)ACC_SCAN_BLOCK * 4) {
+    i64 row[4], sg[4], o[4], before[4];
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      const i64 j = jb + (i64)u * ACC_SCAN_BLOCK + threadIdx.x;
+      if (j < j1) {
+        row[u] = ONE_ROW ? 0 : acc_quot(j, sp1);
+        sg[u] = j - row[u] * sp1;
+        o[u] = S::seg_at(env, sg[u]);
+        before[u] = sg[u] > 0 ? S::seg_at(env, sg[u] - 1) : -1;
+      }
+    }
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      const i64 j = jb + (i64)u * ACC_SCAN_BLOCK + threadIdx.x;
+      if (j < j1 && o[u] != before[u]) {
+        const i64 rel = row[u] * p.n + o[u] - tlo;
+        if (rel >= 0 && rel <= C::TILE) atomicMin(&sh_first[rel], (int)(j - j0));
+      }
+    }
   }
   if (threadIdx.x == 0 && tile + 1 < p.tiles && j1 < p.rows * sp1) {
     // a boundary sitting exactly on this tile's upper border belongs to the next tile
@@ -247,8 +301,8 @@ acc_foldseg(Spec::Env env, Spec::Out out, FoldSegParams p) {
 }
 
 // One wave per tile that has a pending end: walk back over the carries of the preceding
-// tiles, 64 at a time, up to the nearest tile that contains a head (or the start of the
-// stream), combine them in order and complete the end.
+// tiles, a window of 64 at a time, up to the nearest tile that contains a head (or the
+// start of the stream), combine them in order and complete the end.
 extern "C" __global__ void __launch_bounds__(ACC_BLOCK)
 acc_foldseg_fixup(Spec::Env env, Spec::Out out, FoldSegParams p) {
   typedef Spec S;
@@ -263,10 +317,9 @@ acc_foldseg_fixup(Spec::Env env, Spec::Out out, FoldSegParams p) {
   S::Elt v = reinterpret_cast<const P*>(p.pend)[tile].v;
   bool have = false;
   S::Elt run;
-  for (i64 look = tile - 1; look >= 0; look -= ACC_WAVE) {
+  // one window of 64 carries: returns true when the walk ends in it
+  auto window = [&](i64 look, const P& c) {
     const i64 idx = look - lane;
-    P c{};
-    if (idx >= 0) c = carry[idx];
     const u64 mHead = __ballot(idx >= 0 && c.f != 0);
     const int first = mHead ? __builtin_ctzll(mHead) : ACC_WAVE;
     const int nvalid = look + 1 < ACC_WAVE ? (int)(look + 1) : ACC_WAVE;
@@ -280,7 +333,35 @@ acc_foldseg_fixup(Spec::Env env, Spec::Out out, FoldSegParams p) {
     }
     run = have ? S::combine(env, r, run) : r;
     have = true;
-    if (first < ACC_WAVE) break;
+    return first < ACC_WAVE;
+  };
+  // The nearest window usually ends the walk.  A segment that spans many tiles is walked
+  // eight windows at a time, their loads issued together: one memory round trip per 512
+  // tiles instead of one per 64.
+  enum { U = 8 };
+  i64 look = tile - 1;
+  bool done = look < 0;
+  if (!done) {
+    P c{};
+    if (look - lane >= 0) c = carry[look - lane];
+    done = window(look, c);
+    look -= ACC_WAVE;
+  }
+  while (!done && look >= 0) {
+    P c[U];
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const i64 idx = look - (i64)u * ACC_WAVE - lane;
+      c[u] = P{};
+      if (idx >= 0) c[u] = carry[idx];
+    }
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      if (!done && look >= 0) {
+        done = window(look, c[u]);
+        look -= ACC_WAVE;
+      }
+    }
   }
   if (lane != 0) return;
   if (have) v = S::combine(env, run, v);

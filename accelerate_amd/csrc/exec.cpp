@@ -586,7 +586,7 @@ DArrayP Program::alloc(const ArrayR& r, const std::vector<int64_t>& shape) {
   int64_t n = a->size();
   for (ST st : typeLeaves(r.elt)) {
     auto b = std::make_shared<Buffer>();
-    b->ctx = &ctx_;
+    b->ctx = ctx_.shared_from_this();
     b->bytes = (size_t)n * stSize(st);
     b->p = ctx_.malloc(b->bytes);
     if (!b->p) throw Error("Remote memory exhausted");  // Array/Remote/LRU.hs:258-303

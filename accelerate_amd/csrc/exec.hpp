@@ -12,7 +12,7 @@
 namespace acchip {
 
 struct Buffer {
-  Context* ctx = nullptr;
+  std::shared_ptr<Context> ctx;  // keeps the pool alive until the block has gone back to it
   void* p = nullptr;
   size_t bytes = 0;
   bool owned = false;

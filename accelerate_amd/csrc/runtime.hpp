@@ -30,7 +30,9 @@ struct Stats {
       kernelsCompiled{0}, kernelsFromDisk{0}, kernelsFromMemory{0}, launches{0}, poolHits{0}, poolMisses{0};
 };
 
-class Context {
+// Always owned by a std::shared_ptr: device buffers, programs and events keep their
+// context alive, so handles may be released in any order (finalisers run in any order).
+class Context : public std::enable_shared_from_this<Context> {
  public:
   // device < 0: a context that can generate and compile code but owns no GPU
   explicit Context(int device);

@@ -89,3 +89,13 @@ def test_errors_are_reported_not_thrown(cc_ctx):
         ok.execute(hip.DeviceArray(cc_ctx, C.c_void_p()), hip.DeviceArray(cc_ctx, C.c_void_p()))
     assert e.value.code == 2                     # ACCHIP_NO_DEVICE: nothing falls back to the CPU
     assert cc_ctx.malloc(1024) is None           # mallocRemote without a device: NULL, no abort
+
+
+def test_program_may_outlive_its_context():
+    # finalisers run in any order: a program released after acchip_shutdown must not touch
+    # freed memory (the context lives until its last handle is gone)
+    ctx = hip.Context(-1)
+    prog = ctx.compile(P.dotp())
+    assert prog.num_kernels >= 1
+    ctx.close()
+    del prog

@@ -124,6 +124,32 @@ def test_foldseg_2pow27_bit_exact(gpu_ctx):
     assert np.all(got[lens == 0] == 0)
 
 
+@pytest.mark.parametrize("shape", ["one giant segment", "giants and dwarfs", "runs of empty segments",
+                                   "empty segments at the end", "single elements"])
+def test_foldseg_segment_shapes_bit_exact(gpu_ctx, shape):
+    # segments that span hundreds of tiles (the carries of many tiles are chained), tiles
+    # with far more boundaries than elements (runs of empty segments), and length-1 segments
+    rng = np.random.default_rng(77)
+    total = 1 << 23
+    if shape == "one giant segment":
+        lens = np.array([total], np.int32)
+    elif shape == "giants and dwarfs":
+        lens = np.array([5, 3_000_000, 0, 1, total - 3_000_006 - 700_001, 700_001], np.int32)
+    elif shape == "runs of empty segments":
+        total = 1 << 16
+        lens = np.concatenate([[40000], np.zeros(50_000, np.int32), [20000], np.zeros(70_000, np.int32),
+                               [total - 60000 - 7, 7], np.zeros(3, np.int32)]).astype(np.int32)
+    elif shape == "empty segments at the end":
+        total = 1 << 18
+        lens = np.concatenate([np.full(total // 64, 64, np.int32), np.zeros(100_000, np.int32)])
+    else:
+        total = 1 << 20
+        lens = np.ones(total, np.int32)
+    vals = rng.integers(-1000, 1000, total).astype(np.int32)
+    got = gpu_ctx.compile(P.foldseg_sum())(vals, lens)
+    assert np.array_equal(got, OC.foldseg_i32(vals, lens))
+
+
 def test_histogram_2pow26_bit_exact(gpu_ctx):
     n, nbins = 1 << 26, 1 << 16
     keys = W.zipf_keys(n, nbins, 7)

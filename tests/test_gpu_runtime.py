@@ -3,6 +3,7 @@ manager behind the C ABI, on the GPU."""
 import numpy as np
 import pytest
 
+from accelerate_amd import hip
 from accelerate_amd import ir as A
 from accelerate_amd import programs as P
 from oracle import c as OC
@@ -77,3 +78,20 @@ def test_results_stay_on_the_device_between_calls(gpu_ctx):
         d = step.execute(d)
     assert gpu_ctx.stat("bytes_copied_from_remote") == copied
     assert np.all(d.to_host() == 63.0)      # x -> 2x+1 five times from 1
+
+
+def test_handles_may_be_released_after_shutdown():
+    # arrays, results, events and programs released after acchip_shutdown, in any order
+    ctx = hip.Context(0)
+    run = ctx.compile(P.map_affine())
+    x = np.arange(1000, dtype=np.float32)
+    dx = ctx.to_device(x, A.tarray(1, A.f32))
+    res = run.execute(dx)
+    ev = ctx.event()
+    host = res.to_host()
+    ctx.close()
+    del dx
+    del run
+    del ev
+    del res
+    assert np.array_equal(host, 2 * x + 1)
