@@ -33,7 +33,9 @@ struct Stencil2dParams {
 
 // A workgroup walks down `chain` tiles of one column of tiles.  The loads of the next tile
 // are issued before the current tile is computed from LDS, so that a workgroup has global
-// loads in flight all the time instead of only at its start.  INSIDE: every tile of the
+// loads in flight all the time instead of only at its start.  (Two tiles ahead was measured
+// too: 106 us against 98 us per 8192 x 8192 sweep; the second set of staging registers
+// costs a wave per SIMD and the waits still drain both sets together.)  INSIDE: every tile of the
 // chain lies, with its halo, completely inside the array, and no boundary code is needed;
 // the two cases are separate loops so that each has exactly one way of loading.
 template <bool INSIDE>
