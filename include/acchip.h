@@ -48,6 +48,9 @@ const char* acchip_last_error(void);
  * creates a compile-only context.  Replaces the implicit global state of the reference
  * interpreter; a compiling backend creates this once per process. */
 int acchip_init(int device, acchip_ctx** out);
+/* Gives up the caller's handle.  Arrays, programs and events made in the context keep it
+ * alive and may be released afterwards, in any order (GHC finalisers run in any order,
+ * Array/Remote/Table.hs:116-121); the device resources go with the last of them. */
 void acchip_shutdown(acchip_ctx* ctx);
 
 /* totalRemoteMem / availableRemoteMem of class RemoteMemory (Array/Remote/Class.hs:47-73). */
