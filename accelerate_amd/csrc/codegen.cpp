@@ -1239,31 +1239,137 @@ static int stencilWidth(const Sx& sr) {
   throw Error("malformed stencil pattern " + sr.str());
 }
 
+// halo of a stencil pattern per dimension (outermost first)
+static void stencilHalo(const Sx& sr, int dim, std::vector<int>& halo) {
+  const int w = stencilWidth(sr);
+  if ((int)halo.size() <= dim) halo.resize(dim + 1, 0);
+  halo[dim] = std::max(halo[dim], w / 2);
+  if (sr.head().compare(0, 4, "unit") != 0)
+    for (size_t r = 1; r < sr.size(); ++r) stencilHalo(sr.at(r), dim + 1, halo);
+}
+
 KernelSource Codegen::stencil(const std::vector<Sx>& patterns, const TypeP& outElt, const Sx& f,
                               const std::vector<Sx>& boundaries, const std::vector<Operand>& srcs) {
   Emit em;
   em.ind = 4;
   const int rank = srcs.at(0).r.rank;
+  if (rank < 1) throw Error("stencil: rank must be at least 1");
   declareOut(used_, rank);
   ArraySlot o = used_.at("out");
-  ValP focus = fromIndex(rank, shapeOf(o), "i", em);
-  std::vector<std::string> fx;
-  shapeDims(focus, fx);
+  // the focus arrives as a multi-dimensional index: the skeleton splits the linear index
+  // of a thread's first result once and steps to the following results by increments
+  std::vector<std::string> fx(rank);
+  for (int d = 0; d < rank; ++d) fx[d] = "ix[" + std::to_string(d) + "]";
+  std::string indexFns;
+  {
+    Emit ef;
+    ef.ind = 4;
+    ValP ix0 = fromIndex(rank, shapeOf(o), "i", ef);
+    std::vector<std::string> c;
+    shapeDims(ix0, c);
+    for (int d = 0; d < rank; ++d) ef.line("ix[" + std::to_string(d) + "] = " + c[d] + ";");
+    indexFns += fnHead("void", "from_index", "const Env& env, i64 i, i64* ix") + ef.code + "  }\n";
+    std::vector<std::string> od;
+    shapeDims(shapeOf(o), od);
+    Emit en;
+    en.ind = 4;
+    for (int d = rank - 1; d >= 1; --d) {
+      en.line("if (++ix[" + std::to_string(d) + "] < " + od[d] + ") return;");
+      en.line("ix[" + std::to_string(d) + "] = 0;");
+    }
+    en.line("++ix[0];");
+    indexFns += fnHead("void", "next_index", "const Env& env, i64* ix") + en.code + "  }\n";
+  }
 
+  // stencilAccess (Interpreter.hs:670-794): the outermost tuple walks the left-most
+  // dimension, offsets -k..+k left to right
+  struct Rec {
+    static ValP go(const Sx& sr, int dim, int rank, std::vector<int>& off,
+                   const std::function<ValP(const std::vector<int>&)>& access) {
+      int w = stencilWidth(sr), k = w / 2;
+      bool unit = sr.head().compare(0, 4, "unit") == 0;
+      if (unit != (dim == rank - 1)) throw Error("stencil pattern does not match the array rank");
+      if (!unit && (int)sr.size() != w + 1) throw Error("malformed stencil pattern " + sr.str());
+      ValP v = vUnit();
+      for (int d = -k; d <= k; ++d) {
+        off[dim] = d;
+        v = vPair(v, unit ? access(off) : go(sr.at(1 + d + k), dim + 1, rank, off, access));
+      }
+      off[dim] = 0;
+      return v;
+    }
+  };
+  auto mk = [&](const std::vector<std::string>& c) {
+    ValP v = vUnit();
+    for (int d = 0; d < rank; ++d) v = vPair(v, vLeaf(ST::I64, c[d]));
+    return v;
+  };
+
+  // extents of the sources, and the condition under which no tap of this focus leaves them
+  std::vector<std::vector<std::string>> dimsOf(srcs.size());
+  std::string interior;
+  for (size_t a = 0; a < srcs.size(); ++a) {
+    const std::string kind = boundaries[a].atom ? boundaries[a].s : boundaries[a].head();
+    if (kind != "clamp" && kind != "mirror" && kind != "wrap" && kind != "constant" && kind != "function")
+      throw Error("unknown stencil boundary '" + kind + "'");
+    ValP sh = operandShape(srcs[a], em);
+    shapeDims(sh, dimsOf[a]);
+    std::vector<int> halo;
+    stencilHalo(patterns[a], 0, halo);
+    if ((int)halo.size() != rank) throw Error("stencil pattern does not match the array rank");
+    for (int d = 0; d < rank; ++d) {
+      if (halo[d] == 0) continue;
+      interior += (interior.empty() ? "" : " && ") + std::string("(") + fx[d] + " >= (i64)" + std::to_string(halo[d]) +
+                  ") && (" + fx[d] + " + (i64)" + std::to_string(halo[d]) + " < " + dimsOf[a][d] + ")";
+    }
+  }
+
+  // Away from the borders (almost every focus of a large array) no tap needs the boundary
+  // condition: a stencil over one array reads at constant distances from the focus' linear
+  // index, which costs one addition per tap instead of an index computation per tap.
+  Emit ei;
+  ei.ind = em.ind + 2;
+  ValP ri;
+  {
+    std::vector<std::string> stride(rank);
+    if (srcs.size() == 1) {
+      std::string acc = "(i64)1";
+      for (int d = rank - 1; d >= 0; --d) {
+        stride[d] = acc;
+        if (d > 0) acc = bindLeaf(ST::I64, acc + " * " + dimsOf[0][d], em)->ex;
+      }
+    }
+    std::vector<ValP> args;
+    for (size_t a = 0; a < srcs.size(); ++a) {
+      auto access = [&](const std::vector<int>& off) -> ValP {
+        if (srcs.size() == 1) {
+          std::string lin = "i";
+          for (int d = 0; d < rank; ++d)
+            if (off[d] != 0) lin += " + (i64)" + std::to_string(off[d]) + " * " + stride[d];
+          return operandLinear(srcs[a], bindLeaf(ST::I64, lin, ei)->ex, ei);
+        }
+        std::vector<std::string> raw(rank);
+        for (int d = 0; d < rank; ++d)
+          raw[d] = off[d] == 0 ? fx[d] : bindLeaf(ST::I64, fx[d] + " + (i64)" + std::to_string(off[d]), ei)->ex;
+        return operandIndex(srcs[a], mk(raw), ei);
+      };
+      std::vector<int> off(rank, 0);
+      args.push_back(Rec::go(patterns[a], 0, rank, off, access));
+    }
+    ri = applyFun(f, args, {}, ei);
+  }
+
+  // At the borders: bounded (Interpreter.hs:797-839) decides every tap
+  Emit eb;
+  eb.ind = em.ind + 2;
   std::vector<ValP> stencilArgs;
   for (size_t a = 0; a < srcs.size(); ++a) {
     const Operand& src = srcs[a];
     const Sx& bnd = boundaries[a];
     const std::string kind = bnd.atom ? bnd.s : bnd.head();
-    if (kind != "clamp" && kind != "mirror" && kind != "wrap" && kind != "constant" && kind != "function")
-      throw Error("unknown stencil boundary '" + kind + "'");
-    std::vector<std::string> dims;
-    {
-      ValP sh = operandShape(src, em);
-      shapeDims(sh, dims);
-    }
-    // bounded (Interpreter.hs:797-839): value of the source at focus + off
+    const std::vector<std::string>& dims = dimsOf[a];
     auto access = [&](const std::vector<int>& off) -> ValP {
+      Emit& em = eb;
       std::vector<std::string> raw(rank), idx(rank);
       std::string inside;
       for (int d = 0; d < rank; ++d) {
@@ -1288,21 +1394,16 @@ KernelSource Codegen::stencil(const std::vector<Sx>& patterns, const TypeP& outE
           inside += (inside.empty() ? "" : " && ") + (off[d] < 0 ? "(" + j + " >= 0)" : "(" + j + " < " + sz + ")");
         }
       }
-      auto mk = [&](const std::vector<std::string>& c) {
-        ValP v = vUnit();
-        for (int d = 0; d < rank; ++d) v = vPair(v, vLeaf(ST::I64, c[d]));
-        return v;
-      };
       if ((kind != "constant" && kind != "function") || inside.empty()) return operandIndex(src, mk(idx), em);
       // Constant / Function: the whole index decides (no per-dimension remapping)
-      Emit ei, eo;
-      ei.ind = eo.ind = em.ind + 2;
-      ValP vin = operandIndex(src, mk(idx), ei);
+      Emit ein, eo;
+      ein.ind = eo.ind = em.ind + 2;
+      ValP vin = operandIndex(src, mk(idx), ein);
       ValP vout = kind == "constant" ? exp(bnd.at(1), {}, eo) : applyFun(bnd.at(1), {mk(raw)}, {}, eo);
       if (!typeEq(valType(vin), valType(vout))) throw Error("stencil: boundary value does not have the element type");
       ValP res = declareVars(valType(vin), em);
       em.line("if (" + inside + ") {");
-      em.code += ei.code;
+      em.code += ein.code;
       em.ind += 2;
       assign(res, vin, em);
       em.ind -= 2;
@@ -1314,31 +1415,33 @@ KernelSource Codegen::stencil(const std::vector<Sx>& patterns, const TypeP& outE
       em.line("}");
       return res;
     };
-    // stencilAccess (Interpreter.hs:670-794): the outermost tuple walks the left-most
-    // dimension, offsets -k..+k left to right
-    struct Rec {
-      static ValP go(const Sx& sr, int dim, int rank, std::vector<int>& off,
-                     const std::function<ValP(const std::vector<int>&)>& access) {
-        int w = stencilWidth(sr), k = w / 2;
-        bool unit = sr.head().compare(0, 4, "unit") == 0;
-        if (unit != (dim == rank - 1)) throw Error("stencil pattern does not match the array rank");
-        if (!unit && (int)sr.size() != w + 1) throw Error("malformed stencil pattern " + sr.str());
-        ValP v = vUnit();
-        for (int d = -k; d <= k; ++d) {
-          off[dim] = d;
-          v = vPair(v, unit ? access(off) : go(sr.at(1 + d + k), dim + 1, rank, off, access));
-        }
-        off[dim] = 0;
-        return v;
-      }
-    };
-    if (rank < 1) throw Error("stencil: rank must be at least 1");
     std::vector<int> off(rank, 0);
     stencilArgs.push_back(Rec::go(patterns[a], 0, rank, off, access));
   }
-  ValP r = applyFun(f, stencilArgs, {}, em);
-  if (!typeEq(valType(r), outElt)) throw Error("stencil: function result does not match the declared element type");
-  std::string body = fnHead("Elt", "produce", "const Env& env, i64 i") + returnElt(r, em) + "  }\n";
+  ValP rb = applyFun(f, stencilArgs, {}, eb);
+  if (!typeEq(valType(rb), outElt) || !typeEq(valType(ri), outElt))
+    throw Error("stencil: function result does not match the declared element type");
+
+  ValP r = rb;
+  if (interior.empty()) {
+    em.code += eb.code;  // no halo at all: nothing can leave the array (eb was emitted one level deeper)
+  } else {
+    r = declareVars(outElt, em);
+    em.line("if (" + interior + ") {");
+    em.code += ei.code;
+    em.ind += 2;
+    assign(r, ri, em);
+    em.ind -= 2;
+    em.line("} else {");
+    em.code += eb.code;
+    em.ind += 2;
+    assign(r, rb, em);
+    em.ind -= 2;
+    em.line("}");
+  }
+  std::string body = indexFns + fnHead("Elt", "produce_at", "const Env& env, i64 i, const i64* ix") + returnElt(r, em) + "  }\n";
+  body += "  static constexpr int kRank = " + std::to_string(rank) + ";\n#define ACC_MAP_INDEXED 1\n";
+  if (rank >= 2) body += "#define ACC_MAP_XCD 1\n";
   return finish(body, outElt, typeLeaves(outElt), "map.hpp", 0);
 }
 
@@ -1478,6 +1581,136 @@ KernelSource Codegen::stencil2d(const Sx& pattern, const TypeP& outElt, const Sx
   KernelSource ks = finish(body, outElt, typeLeaves(outElt), "stencil2d.hpp", 1);
   ks.group = tileH;
   ks.words = tileW;
+  return ks;
+}
+
+// Rank-3 stencils: tiles of ACC_ST_H x ACC_ST_W results in (y, x) that march along z with a
+// ring of 2*HZ+1 staged planes in LDS (stencil3d.hpp).  Same generated members as for rank 2,
+// with a z coordinate; apply() receives the LDS offsets of the planes z-HZ .. z+HZ.
+KernelSource Codegen::stencil3d(const Sx& pattern, const TypeP& outElt, const Sx& f, const Sx& bnd,
+                                const Operand& src) {
+  const TypeP srcElt = src.r.elt;
+  auto sleaves = typeLeaves(srcElt);
+  const std::string kind = bnd.atom ? bnd.s : bnd.head();
+  if (kind != "clamp" && kind != "mirror" && kind != "wrap" && kind != "constant" && kind != "function")
+    throw Error("unknown stencil boundary '" + kind + "'");
+  std::vector<int> halo;
+  stencilHalo(pattern, 0, halo);
+  if (halo.size() != 3) throw Error("stencil3d: pattern is not of rank 3");
+  const int hz = halo[0], hy = halo[1], hx = halo[2];
+  const int tileH = stencilTileH(hy), tileW = stencilTileW();
+  const int pw = tileW + 2 * hx, ph = tileH + 2 * hy, np = 2 * hz + 1;
+  std::string body;
+  body += "#define ACC_ST_H " + std::to_string(tileH) + "\n";
+  body += "#define ACC_ST_W " + std::to_string(tileW) + "\n";
+  body += "  static constexpr int HZ = " + std::to_string(hz) + ";\n  static constexpr int HY = " + std::to_string(hy) +
+          ";\n  static constexpr int HX = " + std::to_string(hx) + ";\n";
+  body += "  struct SrcElt {\n" + leafDecls(sleaves, "c", false, false) + "  };\n  struct Tile {\n";
+  for (size_t k = 0; k < sleaves.size(); ++k)
+    body += std::string("    ") + stName(sleaves[k]) + " c" + std::to_string(k) + "[" + std::to_string(np * pw * ph) + "];\n";
+  body += "  };\n  ACC_DEV void stage(Tile& t, int idx, const SrcElt& v) {\n";
+  for (size_t k = 0; k < sleaves.size(); ++k)
+    body += "    t.c" + std::to_string(k) + "[idx] = v.c" + std::to_string(k) + ";\n";
+  body += "  }\n";
+  auto retSrc = [&](const ValP& v, Emit& em) {
+    auto lv = leavesOf(v);
+    em.line("SrcElt r_;");
+    for (size_t k = 0; k < lv.size(); ++k) em.line("r_.c" + std::to_string(k) + " = " + lv[k]->ex + ";");
+    em.line("return r_;");
+  };
+  auto idx3 = [](const std::string& z, const std::string& y, const std::string& x) {
+    return vPair(vPair(vPair(vUnit(), vLeaf(ST::I64, z)), vLeaf(ST::I64, y)), vLeaf(ST::I64, x));
+  };
+  {
+    Emit em;
+    em.ind = 4;
+    ValP v = operandIndex(src, idx3("z", "y", "x"), em);
+    if (!typeEq(valType(v), srcElt)) throw Error("stencil: fused producer does not return the element type");
+    retSrc(v, em);
+    body += fnHead("SrcElt", "src_in", "const Env& env, i64 z, i64 y, i64 x") + em.code + "  }\n";
+  }
+  {
+    // bounded (Interpreter.hs:797-839) at an index that may lie outside on either side
+    Emit em;
+    em.ind = 4;
+    std::vector<std::string> dims;
+    shapeDims(operandShape(src, em), dims);
+    const char* raw[3] = {"z", "y", "x"};
+    std::string idx[3], inside;
+    for (int d = 0; d < 3; ++d) {
+      const std::string j = raw[d], sz = dims[d];
+      if (kind == "clamp") idx[d] = bindLeaf(ST::I64, "(" + j + " < 0) ? (i64)0 : ((" + j + " >= " + sz + ") ? " + sz + " - 1 : " + j + ")", em)->ex;
+      else if (kind == "mirror") idx[d] = bindLeaf(ST::I64, "(" + j + " < 0) ? -" + j + " : ((" + j + " >= " + sz + ") ? " + sz + " - (" + j + " - " + sz + " + 2) : " + j + ")", em)->ex;
+      else if (kind == "wrap") idx[d] = bindLeaf(ST::I64, "(" + j + " < 0) ? " + sz + " + " + j + " : ((" + j + " >= " + sz + ") ? " + j + " - " + sz + " : " + j + ")", em)->ex;
+      else {
+        idx[d] = j;
+        inside += std::string(inside.empty() ? "" : " && ") + "(" + j + " >= 0) && (" + j + " < " + sz + ")";
+      }
+    }
+    if (kind == "constant" || kind == "function") {
+      Emit ei, eo;
+      ei.ind = eo.ind = em.ind + 2;
+      ValP vin = operandIndex(src, idx3(idx[0], idx[1], idx[2]), ei);
+      ValP vout = kind == "constant" ? exp(bnd.at(1), {}, eo) : applyFun(bnd.at(1), {idx3("z", "y", "x")}, {}, eo);
+      if (!typeEq(valType(vin), valType(vout))) throw Error("stencil: boundary value does not have the element type");
+      ValP res = declareVars(valType(vin), em);
+      em.line("if (" + inside + ") {");
+      em.code += ei.code;
+      em.ind += 2;
+      assign(res, vin, em);
+      em.ind -= 2;
+      em.line("} else {");
+      em.code += eo.code;
+      em.ind += 2;
+      assign(res, vout, em);
+      em.ind -= 2;
+      em.line("}");
+      retSrc(res, em);
+    } else {
+      retSrc(operandIndex(src, idx3(idx[0], idx[1], idx[2]), em), em);
+    }
+    body += fnHead("SrcElt", "src_at", "const Env& env, i64 z, i64 y, i64 x") + em.code + "  }\n";
+  }
+  {
+    // the stencil function over taps read from the staged planes; c is the focus inside a
+    // plane, pl[dz + HZ] the LDS offset of plane z + dz
+    Emit em;
+    em.ind = 4;
+    ValP arg = vUnit();
+    for (int dz = -hz; dz <= hz; ++dz) {
+      const Sx& plane = pattern.at(1 + dz + hz);
+      const int k1 = stencilWidth(plane) / 2;
+      ValP pv = vUnit();
+      for (int dy = -k1; dy <= k1; ++dy) {
+        const Sx& row = plane.at(1 + dy + k1);
+        if (row.head().compare(0, 4, "unit") != 0) throw Error("stencil3d: pattern is not of rank 3");
+        const int k2 = stencilWidth(row) / 2;
+        ValP rv = vUnit();
+        for (int dx = -k2; dx <= k2; ++dx) {
+          int leaf = 0;
+          struct R {
+            static ValP go(Codegen& cg, const TypeP& t, int& leaf, const std::string& at, Emit& em) {
+              if (t->k == Type::Unit) return vUnit();
+              if (t->k == Type::Scalar) return cg.bindLeaf(t->st, "t.c" + std::to_string(leaf++) + "[" + at + "]", em);
+              ValP a = go(cg, t->a, leaf, at, em);
+              return vPair(a, go(cg, t->b, leaf, at, em));
+            }
+          };
+          std::string at = "pl[" + std::to_string(dz + hz) + "] + c + (" + std::to_string(dy * pw + dx) + ")";
+          rv = vPair(rv, R::go(*this, srcElt, leaf, at, em));
+        }
+        pv = vPair(pv, rv);
+      }
+      arg = vPair(arg, pv);
+    }
+    ValP r = applyFun(f, {arg}, {}, em);
+    if (!typeEq(valType(r), outElt)) throw Error("stencil: function result does not match the declared element type");
+    body += fnHead("Elt", "apply", "const Env& env, const Tile& t, const int* pl, int c") + returnElt(r, em) + "  }\n";
+  }
+  KernelSource ks = finish(body, outElt, typeLeaves(outElt), "stencil3d.hpp", 1);
+  ks.group = tileH;
+  ks.words = tileW;
+  ks.block = np;  // planes in the ring
   return ks;
 }
 

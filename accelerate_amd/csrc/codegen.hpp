@@ -78,6 +78,7 @@ class Codegen {
                        const std::vector<Sx>& boundaries, const std::vector<Operand>& srcs);
   // rank-2 single-source stencil through LDS halo tiles
   KernelSource stencil2d(const Sx& pattern, const TypeP& outElt, const Sx& f, const Sx& boundary, const Operand& src);
+  KernelSource stencil3d(const Sx& pattern, const TypeP& outElt, const Sx& f, const Sx& boundary, const Operand& src);
   KernelSource scalarKernel(const Sx& exp);  // evaluates a closed Exp with one thread
 
   // type of a closed scalar expression / result of a function, without emitting code

@@ -532,6 +532,9 @@ ATyP Program::prepare(const Sx& n, TEnv& tenv) {
     if (!two && srcs[0].r.rank == 2) {
       plan.k = ctx_.kernel(cg.stencil2d(pats[0], outElt, *f, bnds[0], srcs[0]));
       plan.mode = "lds2d";
+    } else if (!two && srcs[0].r.rank == 3 && !std::getenv("ACCHIP_STENCIL_NO3D")) {
+      plan.k = ctx_.kernel(cg.stencil3d(pats[0], outElt, *f, bnds[0], srcs[0]));
+      plan.mode = "lds3d";
     } else {
       plan.k = ctx_.kernel(cg.stencil(pats, outElt, *f, bnds, srcs));
     }
@@ -970,6 +973,27 @@ AValP Program::eval(const Sx& n, AEnv& aenv) {
       args.push_back((uint64_t)chain);
       const int64_t chunksY = (tilesY + chain - 1) / chain;
       ctx_.launch(plan.k, "acc_stencil2d", (unsigned)(tilesX * chunksY), 256, args);
+      return avArr(out);
+    }
+    if (plan.mode == "lds3d") {
+      if (out->size() == 0) return avArr(out);
+      const int64_t th = plan.k->meta.group, tw = plan.k->meta.words;
+      const int64_t tilesY = (ext[1] + th - 1) / th, tilesX = (ext[2] + tw - 1) / tw;
+      // planes per workgroup: long enough to amortise the 2*HZ planes staged before the first
+      // result, short enough that the grid fills the device
+      const char* ce = std::getenv("ACCHIP_STENCIL_CHAIN");
+      int64_t chain = ce ? std::atoll(ce) : 32;
+      while (!ce && chain > 4 && tilesX * tilesY * ((ext[0] + chain - 1) / chain) < 2048) chain /= 2;
+      chain = std::max<int64_t>(1, std::min(chain, ext[0]));
+      const int64_t chunksZ = (ext[0] + chain - 1) / chain;
+      if (tilesX * tilesY * chunksZ > 0x7fffffffLL) throw Error("stencil: too many tiles for one launch");
+      std::vector<uint64_t> args = packArgs(plan.k->meta, aenv, temps, ext);
+      packOut(args, *out);
+      for (int k = 0; k < 3; ++k) args.push_back((uint64_t)ext[k]);
+      args.push_back((uint64_t)tilesX);
+      args.push_back((uint64_t)tilesY);
+      args.push_back((uint64_t)chain);
+      ctx_.launch(plan.k, "acc_stencil3d", (unsigned)(tilesX * tilesY * chunksZ), 256, args);
       return avArr(out);
     }
     launchMap(plan.k, aenv, temps, *out);

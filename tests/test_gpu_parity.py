@@ -194,6 +194,34 @@ def test_stencil_tile_chains_match_oracle(gpu_ctx, monkeypatch, bname, chain):
         assert same(gpu_ctx.compile(prog)(x), O.run_n(prog.text(), x))
 
 
+@pytest.mark.parametrize("chain", [1, 3, 32])
+@pytest.mark.parametrize("bname", ["clamp", "mirror", "wrap", "constant", "function"])
+def test_stencil3d_plane_ring_matches_oracle(gpu_ctx, monkeypatch, bname, chain):
+    # rank 3: columns that march along z over a ring of planes in LDS; chains shorter than,
+    # equal to and longer than the array, ragged columns at the y and x edges
+    monkeypatch.setenv("ACCHIP_STENCIL_CHAIN", str(chain))
+    rng = np.random.default_rng(2000 + chain)
+    b = {"constant": A.constant(A.i64, -3), "function": Q.boundary_function(A.i64, 3)}.get(bname, bname)
+    for widths, shp in [([3, 3, 3], (7, 19, 150)), ([5, 3, 3], (9, 8, 128)), ([3, 5, 7], (4, 30, 40))]:
+        prog = Q.stencil_weighted(A.i64, widths, b)
+        x = rng.integers(-9, 10, shp).astype(np.int64)
+        assert same(gpu_ctx.compile(prog)(x), O.run_n(prog.text(), x))
+
+
+def test_stencil3d_direct_evaluation_matches_oracle(monkeypatch):
+    # the direct (one thread per result) evaluation that ranks other than 2 and 3 use, forced
+    # here for rank 3
+    monkeypatch.setenv("ACCHIP_STENCIL_NO3D", "1")
+    ctx = hip.Context(0)
+    rng = np.random.default_rng(31)
+    for bname in ("clamp", "wrap", "constant"):
+        b = {"constant": A.constant(A.i64, -3)}.get(bname, bname)
+        prog = Q.stencil_weighted(A.i64, [3, 3, 3], b)
+        x = rng.integers(-9, 10, (6, 7, 70)).astype(np.int64)
+        assert same(ctx.compile(prog)(x), O.run_n(prog.text(), x))
+    ctx.close()
+
+
 def test_fold1_of_empty_is_a_bounds_error(gpu_ctx):
     with pytest.raises(hip.AccError) as e:
         gpu_ctx.compile(P.fold1_op(A.add, A.i32, 2))(np.zeros((3, 0), np.int32))
