@@ -57,3 +57,44 @@ acc_map(Spec::Env env, Spec::Out out, MapParams p) {
   }
 #endif
 }
+
+// The same over two-dimensional tiles of the result: a workgroup produces 32 rows x 8*V
+// columns of the (outer dimensions flattened) x (innermost dimension) view, 8 lanes a row.
+// For producers that permute indices (Backpermute, Transform): when the source is walked
+// along another dimension than the result -- a transposition -- the 32 rows of a tile use
+// whole cache lines of the source, where 256*V consecutive results would use four bytes of
+// each line they touch.
+struct MapTiledParams {
+  i64 h, w;     // rows (outer extents multiplied) and columns (innermost extent)
+  i64 tilesX;   // tiles per row of tiles
+};
+
+extern "C" __global__ void __launch_bounds__(ACC_BLOCK)
+acc_map_tiled(Spec::Env env, Spec::Out out, MapTiledParams p) {
+  typedef Spec S;
+  const int V = S::V;
+  const i64 b = (i64)blockIdx.x;
+  const i64 ty = b / p.tilesX, tx = b - ty * p.tilesX;
+  const i64 row = ty * (ACC_BLOCK / 8) + threadIdx.x / 8;
+  const i64 x0 = (tx * 8 + (threadIdx.x & 7)) * V;
+  if (row >= p.h || x0 >= p.w) return;
+  const i64 i0 = row * p.w + x0;
+#ifdef ACC_MAP_INDEXED
+  i64 ix[S::kRank];
+  S::from_index(env, i0, ix);
+  for (int k = 0; k < V && x0 + k < p.w; ++k) {
+    S::store(out, i0 + k, S::produce_at(env, i0 + k, ix));
+    S::next_index(env, ix);
+  }
+#else
+  if (x0 + V <= p.w) {
+    S::Elt r[S::V];
+#pragma unroll
+    for (int k = 0; k < V; ++k) r[k] = S::produce(env, i0 + k);
+#pragma unroll
+    for (int k = 0; k < V; ++k) S::store(out, i0 + k, r[k]);
+  } else {
+    for (int k = 0; k < V && x0 + k < p.w; ++k) S::store(out, i0 + k, S::produce(env, i0 + k));
+  }
+#endif
+}

@@ -807,6 +807,59 @@ AValP Program::eval(const Sx& n, AEnv& aenv) {
     std::vector<DArrayP> temps = evalTemps(plan.temps, aenv);
     const ArrayR& r = plan.ty->r;
     DArrayP out = alloc(r, hostShape(n.at(2), aenv, plan, r.rank));
+    // index-permuting producers of rank >= 2 go over two-dimensional tiles of the result
+    // (acc_map_tiled): a transposition then uses whole cache lines of its source
+    const int64_t w = r.rank >= 2 ? out->shape.back() : 0;
+    const int64_t cols = 8 * (int64_t)plan.k->meta.vec;
+    const char* te = std::getenv("ACCHIP_MAP_TILED");  // "0" / "1": override, for tests
+    bool tiled = h != "generate" && r.rank >= 2 && w >= cols && out->size() / w >= 32;
+    if (tiled && !te) {
+      // Tiles pay off only when neighbouring results read far-apart sources.  Where the index
+      // function is pure index arithmetic it is evaluated here at two neighbouring result
+      // indices; one that reads index arrays (a gather) keeps the linear order.
+      tiled = false;
+      const Sx& perm = n.at(3);
+      if (perm.is("lam") && hostSupported(perm.at(2))) {
+        size_t cur = 0;
+        const std::vector<int64_t> sext = operandExtent(n.at(h == "transform" ? 5 : 4), aenv, plan, temps, cur);
+        auto sourceAt = [&](const std::vector<int64_t>& ix) {
+          HValP v = hvUnit();
+          for (int64_t c : ix) v = hvPair(v, hvInt(ST::I64, c));
+          std::vector<HValP> env;
+          hPush(perm.at(1), v, env);
+          std::vector<int64_t> sx;
+          hDims(hostEval(perm.at(2), env, aenv), sx);
+          if (sx.size() != sext.size()) throw Error("backpermute: index function does not return a source index");
+          int64_t lin = 0;
+          for (size_t k = 0; k < sx.size(); ++k) lin = lin * sext[k] + sx[k];
+          return lin;
+        };
+        std::vector<int64_t> a;
+        for (int64_t dim : out->shape) a.push_back(dim / 2);
+        std::vector<int64_t> b = a;
+        b.back() += b.back() + 1 < out->shape.back() ? 1 : -1;
+        try {
+          const int64_t step = sourceAt(b) - sourceAt(a);
+          tiled = step > 1 || step < -1;
+        } catch (const Error&) {
+          tiled = false;  // the probe is only a hint
+        }
+      }
+    }
+    if (te && te[0] == '0') tiled = false;
+    if (te && te[0] == '1') tiled = h != "generate" && r.rank >= 2 && out->size() > 0;
+    if (tiled) {
+      const int64_t rows = out->size() / w;
+      const int64_t tilesX = (w + cols - 1) / cols, tilesY = (rows + 31) / 32;
+      if (tilesX * tilesY > 0x7fffffffLL) throw Error("too many tiles for one launch");
+      std::vector<uint64_t> args = packArgs(plan.k->meta, aenv, temps, out->shape);
+      packOut(args, *out);
+      args.push_back((uint64_t)rows);
+      args.push_back((uint64_t)w);
+      args.push_back((uint64_t)tilesX);
+      ctx_.launch(plan.k, "acc_map_tiled", (unsigned)(tilesX * tilesY), 256, args);
+      return avArr(out);
+    }
     launchMap(plan.k, aenv, temps, *out);
     return avArr(out);
   }

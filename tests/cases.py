@@ -186,3 +186,17 @@ def parity_cases():
     add("histogram_zipf", P.histogram(97), [rng.integers(0, 97, 3000).astype(np.int32)], None)
     add("map_affine", P.map_affine(), [_rand(rng, A.f32, (1234,))], None)
     return out
+
+
+def gpu_only_programs():
+    """Programs that only GPU tests run (larger inputs, forced kernel variants): compiled by
+    the CPU suite too, so that their code objects travel in the kernel cache."""
+    out = []
+    for bname in ("clamp", "mirror", "wrap", "constant", "function"):
+        for rank, widths_list in ((2, ([3, 3], [5, 3], [3, 5])), (3, ([3, 3, 3], [5, 3, 3], [3, 5, 7]))):
+            b = {"constant": A.constant(A.i64, -3), "function": Q.boundary_function(A.i64, rank)}.get(bname, bname)
+            for widths in widths_list:
+                out.append(("stencil_%s_%s" % (widths, bname), Q.stencil_weighted(A.i64, widths, b)))
+    out.append(("transpose_i32", Q.transpose(A.i32)))
+    out.append(("transpose_i64", Q.transpose(A.i64)))
+    return out

@@ -222,6 +222,22 @@ def test_stencil3d_direct_evaluation_matches_oracle(monkeypatch):
     ctx.close()
 
 
+@pytest.mark.parametrize("tiled", ["0", "1", None])
+def test_transposes_with_and_without_tiles(gpu_ctx, monkeypatch, tiled):
+    # index-permuting producers go over 32 x 8V tiles of the result when it is large enough;
+    # forced on and off here, ragged tiles included
+    if tiled is None:
+        monkeypatch.delenv("ACCHIP_MAP_TILED", raising=False)
+    else:
+        monkeypatch.setenv("ACCHIP_MAP_TILED", tiled)
+    rng = np.random.default_rng(5)
+    for ty, npt in ((A.i32, np.int32), (A.i64, np.int64)):
+        run = gpu_ctx.compile(Q.transpose(ty))
+        for shp in [(33, 17), (100, 300), (64, 64), (5, 1000), (1, 1), (257, 3), (1000, 513)]:
+            x = rng.integers(-1000, 1000, shp).astype(npt)
+            assert np.array_equal(run(x), x.T)
+
+
 def test_fold1_of_empty_is_a_bounds_error(gpu_ctx):
     with pytest.raises(hip.AccError) as e:
         gpu_ctx.compile(P.fold1_op(A.add, A.i32, 2))(np.zeros((3, 0), np.int32))

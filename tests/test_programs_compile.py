@@ -6,7 +6,7 @@ import pytest
 
 from oracle import interp as O
 
-from .cases import parity_cases
+from .cases import gpu_only_programs, parity_cases
 from .runtime_cases import jacobi_awhile, runtime_cases
 from .scalar_cases import scalar_cases
 
@@ -26,7 +26,8 @@ def _compile_all(cc_ctx, named_programs):
 
 def test_all_parity_programs_compile(cc_ctx):
     from .test_gpu_permute_lds import lds_programs
-    _compile_all(cc_ctx, [(c[0], c[1]) for c in parity_cases()] + [(c[0], c[1]) for c in lds_programs()])
+    _compile_all(cc_ctx, [(c[0], c[1]) for c in parity_cases()] + [(c[0], c[1]) for c in lds_programs()] +
+                 gpu_only_programs())
 
 
 def test_all_scalar_programs_compile_and_oracle_evaluates_them(cc_ctx):
