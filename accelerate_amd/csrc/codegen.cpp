@@ -959,18 +959,19 @@ KernelSource Codegen::foldSeg(const Sx& f, const Sx* seed, const Operand& src, c
   // Geometry of the segmented fold, with its own knobs: a lane's run is two 128-bit loads
   // long (ACCHIP_FOLDSEG_VECMUL), which halves the number of wave scans per element; a lane
   // holds ACCHIP_FOLDSEG_BYTES of (value, flag) pairs; workgroups of ACCHIP_FOLDSEG_BLOCK
-  // threads (smaller ones lose less at the barriers).  The tile also pays for an LDS word
-  // per element.
+  // threads (smaller ones lose less at the barriers).  The tile also pays for 2 bytes of LDS
+  // per element.  Measured on 2^27 Int32 values in 2^20 segments, whole pipeline: 256
+  // threads x 256 B 136 us, 256 x 128 B 154, 512 x 256 B 157, 512 x 128 B 150, 1024 x 256 B 173.
   const char* vm = std::getenv("ACCHIP_FOLDSEG_VECMUL");
   vec *= vm ? std::max(1, std::min(4, std::atoi(vm))) : 2;
   const char* fe = std::getenv("ACCHIP_FOLDSEG_BYTES");
-  int fbytes = fe ? std::atoi(fe) : 128;
-  if (fbytes < 16 || fbytes > 512) fbytes = 128;
+  int fbytes = fe ? std::atoi(fe) : 256;
+  if (fbytes < 16 || fbytes > 512) fbytes = 256;
   int g = std::max(1, std::min(8, fbytes / std::max(1, vec * eltBytes)));
   body += "  static constexpr int G = " + std::to_string(g) + ";\n";
   const char* fb = std::getenv("ACCHIP_FOLDSEG_BLOCK");
-  int fblock = fb ? std::atoi(fb) : 512;
-  if (fblock != 256 && fblock != 512 && fblock != 1024) fblock = 512;
+  int fblock = fb ? std::atoi(fb) : 256;
+  if (fblock != 256 && fblock != 512 && fblock != 1024) fblock = 256;
   body += "#define ACC_SCAN_BLOCK " + std::to_string(fblock) + "\n";
   KernelSource ks = finish(body, elt, leaves, "scan.hpp+foldseg.hpp", vec);
   ks.block = fblock;

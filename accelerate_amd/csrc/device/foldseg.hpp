@@ -90,14 +90,17 @@ acc_foldseg_partition(Spec::Env env, Spec::Out out, FoldSegParams p) {
 // ONE_ROW: the stream is a single row, so boundary j is segment boundary j of that row and
 // no division is needed.  FULL: the tile lies completely inside the stream.
 template <bool ONE_ROW, bool FULL>
-ACC_DEV void acc_foldseg_tile(const Spec::Env& env, const Spec::Out& out, const FoldSegParams& p, int* sh_first,
+ACC_DEV void acc_foldseg_tile(const Spec::Env& env, const Spec::Out& out, const FoldSegParams& p, unsigned short* sh_first,
                               AccSegSpec<Spec>::Elt* sh_wave, Spec::Elt& sh_pend, int& sh_pend_at) {
   typedef Spec S;
   typedef AccSegSpec<Spec> SS;
   typedef AccScanCfg<SS> C;
   typedef SS::Elt P;
   const int V = C::V, G = C::G;
-  const int NONE = 0x7fffffff;
+  // marks are 16 bits: the boundary number relative to the tile's first, NONE, or LOOKUP
+  // (a boundary sits here, its number must be searched: crowded tiles only)
+  const int NONE = 0xffff, LOOKUP = 0xfffe;
+  const int NOPEND = 0x7fffffff;
   const i64 tile = blockIdx.x;
   const i64 tlo = tile * (i64)C::TILE;
   const i64 sp1 = p.nseg + 1;
@@ -124,59 +127,79 @@ ACC_DEV void acc_foldseg_tile(const Spec::Env& env, const Spec::Out& out, const 
         if (t0 + k < n) x[g][k] = S::in_linear(env, t0 + k);
     }
   }
-  for (int i = threadIdx.x; i < C::TILE / 4 + 1; i += ACC_SCAN_BLOCK)
-    reinterpret_cast<int4*>(sh_first)[i] = make_int4(NONE, NONE, NONE, NONE);
-  __syncthreads();
   // Boundaries are marked four per thread and step so that their offsets are loaded
-  // together.  A boundary at the same position as its predecessor in the row (an empty
-  // segment before it) is not the first at its position and is skipped: a run of empty
-  // segments would otherwise serialise in one LDS word.
-  const bool crowded = j1 - j0 > 4 * (i64)C::TILE;
+  // together; the loads of the first step are issued before the marks are cleared, so that
+  // they travel while the workgroup waits at the barrier.  A boundary at the same position
+  // as its predecessor (an empty segment before it, or the previous row's last boundary) is
+  // not the first at its position and is skipped, so every mark has exactly one writer.  The first boundary of the next tile is looked at too: it may sit exactly on this
+  // tile's upper border, where it ends a segment of this tile.
+  const bool crowded = j1 - j0 > (4 * (i64)C::TILE < 65000 ? 4 * (i64)C::TILE : 65000);
+  const i64 jend = tile + 1 < p.tiles && j1 < nb ? j1 + 1 : j1;
+  i64 row[4], sg[4], o[4], before[4];
+  auto loadBatch = [&](i64 jb) {
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      const i64 j = jb + (i64)u * ACC_SCAN_BLOCK + threadIdx.x;
+      if (j < jend) {
+        row[u] = ONE_ROW ? 0 : acc_quot(j, sp1);
+        sg[u] = j - row[u] * sp1;
+        o[u] = S::seg_at(env, sg[u]);
+        // position of the boundary before it, relative to this row's start
+        before[u] = sg[u] > 0 ? S::seg_at(env, sg[u] - 1) : (row[u] > 0 ? S::seg_at(env, p.nseg) - p.n : -1);
+      }
+    }
+  };
+  auto markBatch = [&](i64 jb) {
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      const i64 j = jb + (i64)u * ACC_SCAN_BLOCK + threadIdx.x;
+      if (j < jend && o[u] != before[u]) {
+        const i64 rel = row[u] * p.n + o[u] - tlo;
+        if (rel >= 0 && rel <= C::TILE) sh_first[rel] = (unsigned short)(j - j0);  // the only writer of this mark
+      }
+    }
+  };
+  if (!crowded) loadBatch(j0);
+  for (int i = threadIdx.x; i < C::TILE / 8 + 1; i += ACC_SCAN_BLOCK)
+    reinterpret_cast<int4*>(sh_first)[i] = make_int4(-1, -1, -1, -1);
+  __syncthreads();
   if (crowded) {
     // far more boundaries than positions (long runs of empty segments): every position
     // looks for its first boundary by binary search instead
+    auto position = [&](i64 j) {
+      const i64 r = ONE_ROW ? 0 : acc_quot(j, sp1);
+      return r * p.n + S::seg_at(env, j - r * sp1);
+    };
     for (int q = threadIdx.x; q <= C::TILE; q += ACC_SCAN_BLOCK) {
-      auto position = [&](i64 j) {
-        const i64 row = ONE_ROW ? 0 : acc_quot(j, sp1);
-        return row * p.n + S::seg_at(env, j - row * sp1);
-      };
-      i64 a = j0, b = j1;  // first boundary at a position >= tlo + q
+      i64 a = j0, b = jend;  // first boundary at a position >= tlo + q
       while (a < b) {
         const i64 mid = (a + b) >> 1;
         if (position(mid) < tlo + q) a = mid + 1;
         else b = mid;
       }
-      if (a < j1 && position(a) == tlo + q) sh_first[q] = (int)(a - j0);
+      if (a < jend && position(a) == tlo + q) sh_first[q] = (unsigned short)LOOKUP;
     }
-  }
-  for (i64 jb = j0; jb < j1 && !crowded; jb += (i64)ACC_SCAN_BLOCK * 4) {
-    i64 row[4], sg[4], o[4], before[4];
-#pragma unroll
-    for (int u = 0; u < 4; ++u) {
-      const i64 j = jb + (i64)u * ACC_SCAN_BLOCK + threadIdx.x;
-      if (j < j1) {
-        row[u] = ONE_ROW ? 0 : acc_quot(j, sp1);
-        sg[u] = j - row[u] * sp1;
-        o[u] = S::seg_at(env, sg[u]);
-        before[u] = sg[u] > 0 ? S::seg_at(env, sg[u] - 1) : -1;
-      }
+  } else {
+    markBatch(j0);
+    for (i64 jb = j0 + (i64)ACC_SCAN_BLOCK * 4; jb < jend; jb += (i64)ACC_SCAN_BLOCK * 4) {
+      loadBatch(jb);
+      markBatch(jb);
     }
-#pragma unroll
-    for (int u = 0; u < 4; ++u) {
-      const i64 j = jb + (i64)u * ACC_SCAN_BLOCK + threadIdx.x;
-      if (j < j1 && o[u] != before[u]) {
-        const i64 rel = row[u] * p.n + o[u] - tlo;
-        if (rel >= 0 && rel <= C::TILE) atomicMin(&sh_first[rel], (int)(j - j0));
-      }
-    }
-  }
-  if (threadIdx.x == 0 && tile + 1 < p.tiles && j1 < p.rows * sp1) {
-    // a boundary sitting exactly on this tile's upper border belongs to the next tile
-    const i64 row = ONE_ROW ? 0 : j1 / sp1, s = j1 - row * sp1;
-    if (row * p.n + S::seg_at(env, s) - tlo == C::TILE) sh_first[C::TILE] = (int)(j1 - j0);
   }
   __syncthreads();
 
+  // boundary number (relative to j0) behind the mark found at position pos of the stream
+  auto resolve = [&](int mark, i64 pos) -> int {
+    if (mark != LOOKUP) return mark;
+    i64 a = j0, b = j1 + 1 < nb ? j1 + 1 : nb;
+    while (a < b) {
+      const i64 mid = (a + b) >> 1;
+      const i64 r = ONE_ROW ? 0 : acc_quot(mid, sp1);
+      if (r * p.n + S::seg_at(env, mid - r * sp1) < pos) a = mid + 1;
+      else b = mid;
+    }
+    return (int)(a - j0);
+  };
   // the segment that ends where boundary j0 + idx sits
   auto emit = [&](int idx, const S::Elt& v) {
     const i64 j = j0 + idx;
@@ -201,7 +224,7 @@ ACC_DEV void acc_foldseg_tile(const Spec::Env& env, const Spec::Out& out, const 
     const S::Elt* e = x[g];
     P a{};
     bool has = false;
-    pendIdx[g] = NONE;
+    pendIdx[g] = NOPEND;
 #pragma unroll
     for (int k = 0; k < V; ++k) {
       if (FULL || k < c) {
@@ -213,11 +236,12 @@ ACC_DEV void acc_foldseg_tile(const Spec::Env& env, const Spec::Out& out, const 
         }
         has = true;
         if (m[k + 1] != NONE) {
+          const int idx = resolve(m[k + 1], t0 + k + 1);
           if (a.f) {
-            emit(m[k + 1], a.v);
+            emit(idx, a.v);
           } else {
             pendVal[g] = a.v;
-            pendIdx[g] = m[k + 1];
+            pendIdx[g] = idx;
           }
         }
       }
@@ -230,11 +254,11 @@ ACC_DEV void acc_foldseg_tile(const Spec::Env& env, const Spec::Out& out, const 
     const int last = cnt > 0 ? (int)((cnt - 1) / V) : 0;
     P gt = acc_readlane(ts, last);
     P pre;
-    if (acc_join<SS>(env, hasWaveTot, waveTot, lane > 0, lanePre, pre) && pendIdx[g] != NONE) {
+    if (acc_join<SS>(env, hasWaveTot, waveTot, lane > 0, lanePre, pre) && pendIdx[g] != NOPEND) {
       pendVal[g] = S::combine(env, pre.v, pendVal[g]);
       if (pre.f) {
         emit(pendIdx[g], pendVal[g]);
-        pendIdx[g] = NONE;
+        pendIdx[g] = NOPEND;
       }
     }
     if (cnt > 0) {
@@ -243,7 +267,7 @@ ACC_DEV void acc_foldseg_tile(const Spec::Env& env, const Spec::Out& out, const 
     }
   }
   if (lane == 0) sh_wave[w] = waveTot;
-  if (threadIdx.x == 0) sh_pend_at = NONE;
+  if (threadIdx.x == 0) sh_pend_at = NOPEND;
   __syncthreads();
 
   // a wave has data only if all earlier waves are full, so validity follows from counts
@@ -265,7 +289,7 @@ ACC_DEV void acc_foldseg_tile(const Spec::Env& env, const Spec::Out& out, const 
   const P wavePre = sh_wave[w > 0 ? w - 1 : 0];
 #pragma unroll
   for (int g = 0; g < G; ++g) {
-    if (pendIdx[g] != NONE) {
+    if (pendIdx[g] != NOPEND) {
       const S::Elt v = hasWavePre ? S::combine(env, wavePre.v, pendVal[g]) : pendVal[g];
       if (hasWavePre && wavePre.f) {
         emit(pendIdx[g], v);
@@ -277,8 +301,8 @@ ACC_DEV void acc_foldseg_tile(const Spec::Env& env, const Spec::Out& out, const 
   }
   __syncthreads();
   if (threadIdx.x == 0) {
-    p.pend_at[tile] = sh_pend_at == NONE ? (i64)-1 : j0 + sh_pend_at;
-    if (sh_pend_at != NONE) reinterpret_cast<P*>(p.pend)[tile].v = sh_pend;
+    p.pend_at[tile] = sh_pend_at == NOPEND ? (i64)-1 : j0 + sh_pend_at;
+    if (sh_pend_at != NOPEND) reinterpret_cast<P*>(p.pend)[tile].v = sh_pend;
   }
 }
 
@@ -286,7 +310,7 @@ extern "C" __global__ void __launch_bounds__(ACC_SCAN_BLOCK)
 acc_foldseg(Spec::Env env, Spec::Out out, FoldSegParams p) {
   typedef AccScanCfg<AccSegSpec<Spec>> C;
   // sh_first[q]: first boundary (relative to the tile's first) at position q of the tile
-  __shared__ __attribute__((aligned(16))) int sh_first[C::TILE + 4];
+  __shared__ __attribute__((aligned(16))) unsigned short sh_first[C::TILE + 8];
   __shared__ AccSegSpec<Spec>::Elt sh_wave[ACC_SCAN_WAVES];
   __shared__ Spec::Elt sh_pend;
   __shared__ int sh_pend_at;
