@@ -194,18 +194,22 @@ def test_stencil_tile_chains_match_oracle(gpu_ctx, monkeypatch, bname, chain):
         assert same(gpu_ctx.compile(prog)(x), O.run_n(prog.text(), x))
 
 
+_ORACLE_3D = {}
+
+
 @pytest.mark.parametrize("chain", [1, 3, 32])
 @pytest.mark.parametrize("bname", ["clamp", "mirror", "wrap", "constant", "function"])
 def test_stencil3d_plane_ring_matches_oracle(gpu_ctx, monkeypatch, bname, chain):
     # rank 3: columns that march along z over a ring of planes in LDS; chains shorter than,
     # equal to and longer than the array, ragged columns at the y and x edges
     monkeypatch.setenv("ACCHIP_STENCIL_CHAIN", str(chain))
-    rng = np.random.default_rng(2000 + chain)
     b = {"constant": A.constant(A.i64, -3), "function": Q.boundary_function(A.i64, 3)}.get(bname, bname)
-    for widths, shp in [([3, 3, 3], (7, 19, 150)), ([5, 3, 3], (9, 8, 128)), ([3, 5, 7], (4, 30, 40))]:
+    for n, (widths, shp) in enumerate([([3, 3, 3], (7, 11, 140)), ([5, 3, 3], (6, 8, 128)), ([3, 5, 7], (4, 19, 30))]):
         prog = Q.stencil_weighted(A.i64, widths, b)
-        x = rng.integers(-9, 10, shp).astype(np.int64)
-        assert same(gpu_ctx.compile(prog)(x), O.run_n(prog.text(), x))
+        x = np.random.default_rng(2000 + n).integers(-9, 10, shp).astype(np.int64)
+        if (bname, n) not in _ORACLE_3D:     # the same for every chain length
+            _ORACLE_3D[(bname, n)] = O.run_n(prog.text(), x)
+        assert same(gpu_ctx.compile(prog)(x), _ORACLE_3D[(bname, n)])
 
 
 def test_stencil3d_direct_evaluation_matches_oracle(monkeypatch):
