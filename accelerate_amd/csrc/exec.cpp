@@ -915,7 +915,8 @@ AValP Program::eval(const Sx& n, AEnv& aenv) {
     }
     // geometry: enough workgroups to fill the chip, each with at least a few tiles of work
     const int64_t tile = (int64_t)4 * 64 * plan.k->meta.vec;
-    const int64_t target = 2048;
+    const char* ft = std::getenv("ACCHIP_FOLD_TARGET");  // workgroups aimed at (tuning knob)
+    const int64_t target = ft ? std::max<int64_t>(1, std::atoll(ft)) : 2048;
     int64_t bpr = 1;
     if (rows < target && len > 8 * tile)
       bpr = std::min((target + rows - 1) / rows, (len + 8 * tile - 1) / (8 * tile));
