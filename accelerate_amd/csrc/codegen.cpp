@@ -1446,12 +1446,10 @@ KernelSource Codegen::stencil(const std::vector<Sx>& patterns, const TypeP& outE
   return finish(body, outElt, typeLeaves(outElt), "map.hpp", 0);
 }
 
-// Results per stencil tile: 128 columns x 8 rows (16 rows when the halo is wider than one
-// row, to keep the share of halo rows down).  Workgroups chain several tiles down a column
-// and prefetch the next one, so small tiles cost no occupancy and keep more independent
-// loads in flight; measured on the 8192 x 8192 Jacobi sweep (us per sweep, chains of 4):
-// 64x32 118, 64x16 106, 128x16 104, 128x8 98, 256x8 98.
-// Tuning knobs: ACCHIP_STENCIL_H, ACCHIP_STENCIL_W.
+// Results per stencil tile: 256 columns x 8 rows (16 rows when the halo is wider than one
+// row, to keep the share of halo rows down).  Measured on the 8192 x 8192 Jacobi sweep (us
+// per sweep, one tile per workgroup): 256x8 92, 128x16 94, 256x16 94, 64x16 97, 128x32 99,
+// 128x8 100.  Tuning knobs: ACCHIP_STENCIL_H, ACCHIP_STENCIL_W.
 int stencilTileH(int hy) {
   const char* e = std::getenv("ACCHIP_STENCIL_H");
   const int dflt = hy <= 1 ? 8 : 16;
@@ -1461,8 +1459,8 @@ int stencilTileH(int hy) {
 
 int stencilTileW() {
   const char* e = std::getenv("ACCHIP_STENCIL_W");
-  int v = e ? std::atoi(e) : 128;
-  return (v == 64 || v == 128 || v == 256) ? v : 128;
+  int v = e ? std::atoi(e) : 256;
+  return (v == 64 || v == 128 || v == 256) ? v : 256;
 }
 
 KernelSource Codegen::stencil2d(const Sx& pattern, const TypeP& outElt, const Sx& f, const Sx& bnd,
@@ -1478,14 +1476,15 @@ KernelSource Codegen::stencil2d(const Sx& pattern, const TypeP& outElt, const Sx
   for (size_t r = 1; r < pattern.size(); ++r) hx = std::max(hx, stencilWidth(pattern.at(r)) / 2);
   const int tileH = stencilTileH(hy);
   const int tileW = stencilTileW();
-  const int pw = tileW + 2 * hx, ph = tileH + 2 * hy;
+  const int hxp = (hx + 3) / 4 * 4;  // halo columns padded so that result columns stay 16-byte aligned in LDS
+  const int pw = tileW + 2 * hxp, ph = tileH + 2 * hy;
   std::string body;
   body += "#define ACC_ST_H " + std::to_string(tileH) + "\n";
   body += "#define ACC_ST_W " + std::to_string(tileW) + "\n";
-  body += "  static constexpr int HY = " + std::to_string(hy) + ";\n  static constexpr int HX = " + std::to_string(hx) + ";\n";
+  body += "  static constexpr int HY = " + std::to_string(hy) + ";\n  static constexpr int HX = " + std::to_string(hx) + ";\n  static constexpr int HXP = " + std::to_string(hxp) + ";\n";
   body += "  struct SrcElt {\n" + leafDecls(sleaves, "c", false, false) + "  };\n  struct Tile {\n";
   for (size_t k = 0; k < sleaves.size(); ++k)
-    body += std::string("    ") + stName(sleaves[k]) + " c" + std::to_string(k) + "[" + std::to_string(pw * ph) + "];\n";
+    body += std::string("    __attribute__((aligned(16))) ") + stName(sleaves[k]) + " c" + std::to_string(k) + "[" + std::to_string(pw * ph) + "];\n";
   body += "  };\n  ACC_DEV void stage(Tile& t, int idx, const SrcElt& v) {\n";
   for (size_t k = 0; k < sleaves.size(); ++k)
     body += "    t.c" + std::to_string(k) + "[idx] = v.c" + std::to_string(k) + ";\n";

@@ -1019,10 +1019,11 @@ AValP Program::eval(const Sx& n, AEnv& aenv) {
       args.push_back((uint64_t)ext[1]);
       args.push_back((uint64_t)tilesX);
       args.push_back((uint64_t)tilesY);
-      // a workgroup chains up to 4 tiles down a column (measured best of 1..16) as long as
-      // the grid still fills the device twice over
+      // a workgroup can chain several tiles down a column, prefetching the next one; with
+      // 128-bit staging one tile per workgroup measured best (92 us against 103 / 107 us for
+      // chains of 2 / 4 on the 8192 x 8192 Jacobi sweep), so chains are only a knob
       const char* ce = std::getenv("ACCHIP_STENCIL_CHAIN");
-      int64_t chain = ce ? std::atoll(ce) : std::min<int64_t>(4, (tilesX * tilesY) / 512);
+      int64_t chain = ce ? std::atoll(ce) : 1;
       chain = std::max<int64_t>(1, std::min(chain, tilesY));
       args.push_back((uint64_t)chain);
       const int64_t chunksY = (tilesY + chain - 1) / chain;
