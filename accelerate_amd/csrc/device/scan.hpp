@@ -407,19 +407,37 @@ ACC_DEV void acc_rows_tile(const typename S::Env& env, int cnt, int n, const Loa
     int r = idx0 / n, t = idx0 - r * n;
     r0[g] = r;
     t0[g] = t;
+    if (wlo + (g + 1) * C::GROUP <= cnt) {
+      // the whole group lies inside (wave-uniform): no tests, so that the V loads of a lane
+      // can become one wide request
+      P e[C::V];
 #pragma unroll
-    for (int k = 0; k < V; ++k) {
-      if (idx0 + k < cnt) {
-        P e;
-        e.v = load(idx0 + k, r, t);
-        e.f = t == 0 ? 1u : 0u;
-        x[g][k] = k == 0 ? e : SS::combine(env, x[g][k - 1], e);
-      } else if (k > 0) {
-        x[g][k] = x[g][k - 1];
+      for (int k = 0; k < V; ++k) {
+        e[k].v = load(idx0 + k, r, t);
+        e[k].f = t == 0 ? 1u : 0u;
+        if (++t == n) {
+          t = 0;
+          ++r;
+        }
       }
-      if (++t == n) {
-        t = 0;
-        ++r;
+      x[g][0] = e[0];
+#pragma unroll
+      for (int k = 1; k < V; ++k) x[g][k] = SS::combine(env, x[g][k - 1], e[k]);
+    } else {
+#pragma unroll
+      for (int k = 0; k < V; ++k) {
+        if (idx0 + k < cnt) {
+          P e;
+          e.v = load(idx0 + k, r, t);
+          e.f = t == 0 ? 1u : 0u;
+          x[g][k] = k == 0 ? e : SS::combine(env, x[g][k - 1], e);
+        } else if (k > 0) {
+          x[g][k] = x[g][k - 1];
+        }
+        if (++t == n) {
+          t = 0;
+          ++r;
+        }
       }
     }
   }
@@ -460,15 +478,29 @@ ACC_DEV void acc_rows_tile(const typename S::Env& env, int cnt, int n, const Loa
   for (int g = 0; g < G; ++g) {
     const int idx0 = wlo + (g * ACC_WAVE + lane) * V;
     int r = r0[g], t = t0[g];
+    if (wlo + (g + 1) * C::GROUP <= cnt) {
+      typename S::Elt y[C::V];
 #pragma unroll
-    for (int k = 0; k < V; ++k) {
-      if (idx0 + k < cnt) {
-        const P y = hasBase ? SS::combine(env, base, x[g][k]) : x[g][k];
-        store(idx0 + k, r, t, y.v);
+      for (int k = 0; k < V; ++k) y[k] = (hasBase ? SS::combine(env, base, x[g][k]) : x[g][k]).v;
+#pragma unroll
+      for (int k = 0; k < V; ++k) {
+        store(idx0 + k, r, t, y[k]);
+        if (++t == n) {
+          t = 0;
+          ++r;
+        }
       }
-      if (++t == n) {
-        t = 0;
-        ++r;
+    } else {
+#pragma unroll
+      for (int k = 0; k < V; ++k) {
+        if (idx0 + k < cnt) {
+          const P y = hasBase ? SS::combine(env, base, x[g][k]) : x[g][k];
+          store(idx0 + k, r, t, y.v);
+        }
+        if (++t == n) {
+          t = 0;
+          ++r;
+        }
       }
     }
   }
