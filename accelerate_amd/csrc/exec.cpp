@@ -119,24 +119,30 @@ static bool hostPrimOk(const std::string& n) {
   return false;
 }
 
-// structural test: can hostEval handle this term without touching array contents?
-static bool hostSupported(const Sx& e) {
+// thrown by hostEval when it needs the contents of an array the host does not know
+struct HostUnknown {};
+
+// structural test: can hostEval handle this term without touching array contents?  With
+// `scalars`, reading a rank-0 array is allowed too (it succeeds at run time when the host
+// knows that array's value).
+static bool hostSupported(const Sx& e, bool scalars = false) {
   if (e.isAtom("nil")) return true;
   if (e.atom) return false;
   const std::string& h = e.head();
   if (h == "var" || h == "shape") return true;
+  if (scalars && (h == "index" || h == "linearindex")) return hostSupported(e.at(2), true);
   if (h == "const") return isST(e.at(1)) && !stIsFloat(parseST(e.at(1)));
-  if (h == "let") return hostSupported(e.at(2)) && hostSupported(e.at(3));
-  if (h == "pair") return hostSupported(e.at(1)) && hostSupported(e.at(2));
-  if (h == "cond") return hostSupported(e.at(1)) && hostSupported(e.at(2)) && hostSupported(e.at(3));
-  if (h == "toindex" || h == "fromindex") return hostSupported(e.at(2)) && hostSupported(e.at(3));
-  if (h == "indexslice" || h == "indexfull") return hostSupported(e.at(2)) && hostSupported(e.at(3));
-  if (h == "shapesize") return hostSupported(e.at(2));
+  if (h == "let") return hostSupported(e.at(2), scalars) && hostSupported(e.at(3), scalars);
+  if (h == "pair") return hostSupported(e.at(1), scalars) && hostSupported(e.at(2), scalars);
+  if (h == "cond") return hostSupported(e.at(1), scalars) && hostSupported(e.at(2), scalars) && hostSupported(e.at(3), scalars);
+  if (h == "toindex" || h == "fromindex") return hostSupported(e.at(2), scalars) && hostSupported(e.at(3), scalars);
+  if (h == "indexslice" || h == "indexfull") return hostSupported(e.at(2), scalars) && hostSupported(e.at(3), scalars);
+  if (h == "shapesize") return hostSupported(e.at(2), scalars);
   if (h == "prim") {
     if (!hostPrimOk(e.at(1).s)) return false;
     for (size_t k = 2; k + 1 < e.size(); ++k)
       if (!isST(e.at(k)) || stIsFloat(parseST(e.at(k)))) return false;
-    return hostSupported(e.at(e.size() - 1));
+    return hostSupported(e.at(e.size() - 1), scalars);
   }
   return false;
 }
@@ -193,6 +199,14 @@ static HValP hostEval(const Sx& e, std::vector<HValP> env, const std::vector<DAr
     size_t ix = (size_t)e.at(1).asInt();
     if (ix >= aenv.size()) throw Error("host evaluation: array variable out of range");
     return hShape(aenv[aenv.size() - 1 - ix]->shape);
+  }
+  if (h == "index" || h == "linearindex") {
+    size_t ix = (size_t)e.at(1).asInt();
+    if (ix >= aenv.size()) throw Error("host evaluation: array variable out of range");
+    const DArrayP& a = aenv[aenv.size() - 1 - ix];
+    if (!a->hostKnown) throw HostUnknown();
+    auto leaves = typeLeaves(a->r.elt);
+    return hvInt(leaves.at(0), a->hostValue);
   }
   if (h == "const") {
     ST st = parseST(e.at(1));
@@ -634,6 +648,12 @@ std::vector<uint64_t> Program::packArgs(const KernelSource& ks, const AEnv& aenv
 HValP Program::hostExp(const Sx& e, const AEnv& aenv, const Plan& plan) {
   auto it = plan.scalarKernels.find(&e);
   if (it == plan.scalarKernels.end()) return hostEval(e, {}, aenv);
+  if (hostSupported(e, true)) {
+    try {
+      return hostEval(e, {}, aenv);  // only reads scalars the host knows
+    } catch (const HostUnknown&) {
+    }
+  }
   // one-thread kernel, then read the leaves back
   const KernelP& k = it->second;
   ArrayR r;
@@ -773,7 +793,8 @@ AValP Program::eval(const Sx& n, AEnv& aenv) {
       AValP p = evalFun(n.at(1), aenv, {x});
       if (p->k != AVal::Arr || p->arr->bufs.size() != 1) throw Error("awhile: predicate must be a scalar boolean array");
       unsigned char flag = 0;
-      ctx_.peek(&flag, p->arr->bufs[0]->p, 1);
+      if (p->arr->hostKnown) flag = p->arr->hostValue != 0;  // no round trip to the device
+      else ctx_.peek(&flag, p->arr->bufs[0]->p, 1);
       if (!flag) break;
       x = evalFun(n.at(2), aenv, {x});
     }
@@ -791,6 +812,17 @@ AValP Program::eval(const Sx& n, AEnv& aenv) {
   if (h == "unit") {
     DArrayP out = alloc(plan.ty->r, {});
     launchMap(plan.k, aenv, {}, *out);
+    // the host follows integral scalars made of index arithmetic and other such scalars
+    if (plan.ty->r.elt->k == Type::Scalar && !stIsFloat(plan.ty->r.elt->st) && hostSupported(n.at(2), true)) {
+      try {
+        HValP v = hostEval(n.at(2), {}, aenv);
+        if (v->k == HVal::Leaf) {
+          out->hostKnown = true;
+          out->hostValue = wrapTo(plan.ty->r.elt->st, v->i);
+        }
+      } catch (const HostUnknown&) {
+      }
+    }
     return avArr(out);
   }
   if (h == "reshape") {

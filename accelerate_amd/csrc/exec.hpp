@@ -28,6 +28,11 @@ struct DArray {
   ArrayR r;
   std::vector<int64_t> shape;
   std::vector<BufferP> bufs;
+  // A rank-0 array of one integral leaf whose value the host computed alongside the device
+  // (`unit e` with e made of index arithmetic and such arrays): loop counters and flags of
+  // awhile / acond are then read here instead of from the device.
+  bool hostKnown = false;
+  int64_t hostValue = 0;
   int64_t size() const {
     int64_t n = 1;
     for (int64_t d : shape) n = d <= 0 ? 0 : n * d;
