@@ -618,6 +618,34 @@ void Program::packOut(std::vector<uint64_t>& args, const DArray& a) {
   for (auto& b : a.bufs) args.push_back((uint64_t)(uintptr_t)b->p);
 }
 
+// A scalar the host computed (`unit` of index arithmetic) reaches the device only when
+// something there reads it: a kernel that takes the array, a copy, or the caller.
+void Program::materialize(DArray& a) {
+  if (!a.hostKnown || a.onDevice) return;
+  auto leaves = typeLeaves(a.r.elt);
+  void* p = a.bufs.at(0)->p;
+  const uint64_t v = (uint64_t)a.hostValue;
+  hipStream_t st = ctx_.stream();
+  switch (stSize(leaves.at(0))) {
+    case 1: hipCheck(hipMemsetD8Async(p, (unsigned char)v, 1, st), "hipMemsetD8Async"); break;
+    case 2: hipCheck(hipMemsetD16Async(p, (unsigned short)v, 1, st), "hipMemsetD16Async"); break;
+    case 4: hipCheck(hipMemsetD32Async(p, (int)(uint32_t)v, 1, st), "hipMemsetD32Async"); break;
+    default:
+      hipCheck(hipMemsetD32Async(p, (int)(uint32_t)v, 1, st), "hipMemsetD32Async");
+      hipCheck(hipMemsetD32Async(static_cast<char*>(p) + 4, (int)(uint32_t)(v >> 32), 1, st), "hipMemsetD32Async");
+  }
+  a.onDevice = true;
+}
+
+void Program::materializeAll(const AValP& v) {
+  if (!v) return;
+  if (v->k == AVal::Arr) materialize(*v->arr);
+  else if (v->k == AVal::Pair) {
+    materializeAll(v->a);
+    materializeAll(v->b);
+  }
+}
+
 std::vector<uint64_t> Program::packArgs(const KernelSource& ks, const AEnv& aenv, const std::vector<DArrayP>& temps,
                                         const std::vector<int64_t>& outShape) {
   std::vector<uint64_t> args;
@@ -639,6 +667,7 @@ std::vector<uint64_t> Program::packArgs(const KernelSource& ks, const AEnv& aenv
     if (a->r.rank != s.r.rank || !typeEq(a->r.elt, s.r.elt))
       throw Error("array bound to " + s.name + " does not have the type the program declares (rank " +
                   std::to_string(s.r.rank) + ", " + typeStr(s.r.elt) + ")");
+    materialize(*a);
     for (auto& b : a->bufs) args.push_back((uint64_t)(uintptr_t)b->p);
     for (int64_t d : a->shape) args.push_back((uint64_t)d);
   }
@@ -755,7 +784,9 @@ AValP Program::run(const std::vector<AValP>& args, const std::vector<DArrayP>& u
   uses_ = &uses;
   AEnv aenv;
   for (size_t i = 0; i < args.size(); ++i) pushVals(lams_[i]->at(1), args[i], aenv);
-  return eval(*body_, aenv);
+  AValP r = eval(*body_, aenv);
+  materializeAll(r);  // what the caller gets is on the device
+  return r;
 }
 
 AValP Program::eval(const Sx& n, AEnv& aenv) {
@@ -811,18 +842,21 @@ AValP Program::eval(const Sx& n, AEnv& aenv) {
 
   if (h == "unit") {
     DArrayP out = alloc(plan.ty->r, {});
-    launchMap(plan.k, aenv, {}, *out);
-    // the host follows integral scalars made of index arithmetic and other such scalars
+    // the host follows integral scalars made of index arithmetic and other such scalars; the
+    // device copy is written only if something reads it there (materialize)
     if (plan.ty->r.elt->k == Type::Scalar && !stIsFloat(plan.ty->r.elt->st) && hostSupported(n.at(2), true)) {
       try {
         HValP v = hostEval(n.at(2), {}, aenv);
         if (v->k == HVal::Leaf) {
           out->hostKnown = true;
           out->hostValue = wrapTo(plan.ty->r.elt->st, v->i);
+          out->onDevice = false;
+          return avArr(out);
         }
       } catch (const HostUnknown&) {
       }
     }
+    launchMap(plan.k, aenv, {}, *out);
     return avArr(out);
   }
   if (h == "reshape") {
@@ -978,6 +1012,7 @@ AValP Program::eval(const Sx& n, AEnv& aenv) {
     // a fresh array nobody else can see and is updated in place (Trafo/Fusion.hs:559-566)
     AValP dv = eval(n.at(2), aenv);
     if (dv->k != AVal::Arr) throw Error("permute: defaults must be a single array");
+    materialize(*dv->arr);
     DArrayP out = dv->arr;
     static const char* fresh[] = {"generate", "map", "zipwith", "transform", "backpermute", "fold", "foldseg",
                                   "scan", "permute", "stencil", "stencil2", "unit"};

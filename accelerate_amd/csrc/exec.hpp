@@ -33,6 +33,7 @@ struct DArray {
   // awhile / acond are then read here instead of from the device.
   bool hostKnown = false;
   int64_t hostValue = 0;
+  bool onDevice = true;  // false: the buffer has not been written yet (Program::materialize)
   int64_t size() const {
     int64_t n = 1;
     for (int64_t d : shape) n = d <= 0 ? 0 : n * d;
@@ -116,6 +117,9 @@ class Program {
   std::vector<int64_t> operandExtent(const Sx& o, const AEnv& aenv, const Plan& plan, const std::vector<DArrayP>& temps,
                                      size_t& tempCursor);
   DArrayP alloc(const ArrayR& r, const std::vector<int64_t>& shape);
+  // write a host-known scalar to its device buffer if that has not happened yet
+  void materialize(DArray& a);
+  void materializeAll(const AValP& v);
   std::vector<uint64_t> packArgs(const KernelSource& ks, const AEnv& aenv, const std::vector<DArrayP>& temps,
                                  const std::vector<int64_t>& outShape);
   static void packOut(std::vector<uint64_t>& args, const DArray& a);

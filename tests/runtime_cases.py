@@ -61,6 +61,21 @@ def runtime_cases():
     add("acond_true", A.alam([V(Int), V(Int)], cond_prog), [x, y], [])
     add("acond_false", A.alam([V(Int), V(Int)], cond_prog), [y, x], [])
 
+    # a scalar the host can follow (unit of index arithmetic): returned as a result, read by a
+    # kernel, fed into another such scalar, and deciding an acond
+    def host_scalars(xs):
+        n = A.untup_shape(xs)[0]
+        S0 = A.tarray(0, Int)
+        k = A.unit_(Int, A.add(Int, A.mul(Int, n, A.constI(3)), A.constI(-7)))
+        return A.alet(S0, k, lambda kv: A.alet(
+            S0, A.unit_(Int, A.sub(Int, A.index(kv, A.nil), A.constI(1000))), lambda k2: A.apair(
+                A.apair(kv, k2),
+                A.acond(A.gt(Int, A.index(k2, A.nil), A.constI(0)),
+                        A.map_(Int, A.lam([Int], lambda v: A.add(Int, v, A.index(kv, A.nil))), xs),
+                        A.map_(Int, A.lam([Int], lambda v: A.sub(Int, v, A.index(k2, A.nil))), xs)))))
+    add("host_scalars_big", A.alam([V(Int)], host_scalars), [x], [])
+    add("host_scalars_small", A.alam([V(Int)], host_scalars), [x[:20]], [])
+
     # acond whose predicate reads array contents (evaluated by a one-thread kernel)
     def cond_data(xs):
         first = A.index(xs, A.sh(0))
