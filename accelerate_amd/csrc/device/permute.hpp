@@ -42,7 +42,8 @@ acc_permute(Spec::Env env, Spec::Out out, PermuteParams p) {
 // Measured on 2^26 keys into 2^16 Int32 bins (two ranges): streaming the keys alone takes
 // 45 us, the LDS atomics add 40 us whether the keys are uniform or Zipf-distributed, adding
 // the private copies to the destination 12 us; sorted keys or a single key serialise in the
-// LDS atomic unit (440 us).
+// LDS atomic unit (440 us).  Issuing the key loads of the next step before the LDS updates of
+// the current one changed nothing (101 us against 100 us).
 //
 // The destination is cut into `nparts` ranges of `part` elements (part <= ACC_PERMUTE_PART,
 // 128 KiB of LDS).  The sources are cut into `groups` chunks; workgroup b serves chunk
