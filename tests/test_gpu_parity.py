@@ -242,6 +242,25 @@ def test_transposes_with_and_without_tiles(gpu_ctx, monkeypatch, tiled):
             assert np.array_equal(run(x), x.T)
 
 
+def test_more_than_2_pow_31_elements(gpu_ctx):
+    # linear indices beyond 32 bits: a map, a fold and a scan over 2^31 + 1000 Word8 elements
+    n = (1 << 31) + 1000
+    x = np.arange(n, dtype=np.uint32).astype(np.uint8)
+    x[-3:] = (7, 11, 13)
+    dx = gpu_ctx.to_device(x, A.tarray(1, A.u8))
+    inc = gpu_ctx.compile(A.alam([A.tarray(1, A.u8)], lambda xs: A.map_(
+        A.u8, A.lam([A.u8], lambda v: A.add(A.u8, v, A.const(A.u8, 1))), xs)))
+    got = inc.execute(dx).to_host()
+    assert got.shape == (n,) and np.array_equal(got[-1000:], x[-1000:] + np.uint8(1)) and np.array_equal(got[:1000], x[:1000] + np.uint8(1))
+    assert np.array_equal(got[1 << 31 : (1 << 31) + 8], x[1 << 31 : (1 << 31) + 8] + np.uint8(1))
+    del got
+    total = gpu_ctx.compile(P.fold_sum(A.u8, 1, 0)).execute(dx).to_host()
+    assert int(total) == int(x.sum(dtype=np.uint64) & 0xFF)
+    run = gpu_ctx.compile(P.scanl1_sum(A.u8)).execute(dx).to_host()
+    assert run[-1] == total and np.array_equal(run[:4096], np.cumsum(x[:4096], dtype=np.uint8))
+    assert np.array_equal(np.diff(run[-5000:]).astype(np.uint8), x[-4999:])
+
+
 def test_fold1_of_empty_is_a_bounds_error(gpu_ctx):
     with pytest.raises(hip.AccError) as e:
         gpu_ctx.compile(P.fold1_op(A.add, A.i32, 2))(np.zeros((3, 0), np.int32))
