@@ -45,8 +45,6 @@ Context::Context(int device) : device_(device) {
     forceRecomp = f.find("force-recomp") != std::string::npos;
   }
   if (device_ >= 0) {
-    if (std::getenv("ACCHIP_SPIN")) (void)hipSetDeviceFlags(hipDeviceScheduleSpin);
-    (void)hipGetLastError();
     hipCheck(hipSetDevice(device_), "hipSetDevice");
     hipCheck(hipStreamCreateWithFlags(&stream_, hipStreamNonBlocking), "hipStreamCreate");
   }
