@@ -181,6 +181,20 @@ def parity_cases():
     add("jacobi_37x53", P.jacobi_step(), [g], None)
     add("stencil2_clamp_const", Q.stencil2_sum(A.f32, "clamp", A.constant(A.f32, 0.5)),
         [g, rng.uniform(0, 1, (40, 50)).astype(np.float32)], None)
+    # ---- whole programs (Test/NoFib/Spectral: SMVM, RadixSort; Prelude/Filter.hs)
+    for nrows, ncols in ((40, 30), (700, 500)):
+        segd = rng.integers(0, 7, nrows).astype(np.int64)
+        nnz = int(segd.sum())
+        inds = rng.integers(0, ncols, nnz).astype(np.int64)
+        add("smvm_i64_%d" % nrows, Q.smvm(A.i64),
+            [segd, inds, _rand(rng, A.i64, (nnz,), -9, 9), _rand(rng, A.i64, (ncols,), -9, 9)], None)
+        add("smvm_f32_%d" % nrows, Q.smvm(A.f32),
+            [segd, inds, _rand(rng, A.f32, (nnz,)), _rand(rng, A.f32, (ncols,))], 1e-4 * 16 * 7)
+    for n in (0, 1, 300, 5000):
+        add("filter_positive_%d" % n, Q.filter_positive(), [_rand(rng, A.i64, (n,), -50, 50)], None)
+    add("filter_none_pass", Q.filter_positive(), [-np.abs(_rand(rng, A.i64, (200,), -50, 50)) - 1], None)
+    add("radix_4_passes", Q.radix_passes(4), [rng.integers(0, 16, 500).astype(np.int64)], None)
+    add("radix_6_passes", Q.radix_passes(6), [rng.integers(0, 64, 3000).astype(np.int64)], None)
     # ---- the benchmark programs at small size
     add("dotp_1000", P.dotp(), [_rand(rng, A.f32, (1000,)), _rand(rng, A.f32, (900,))], 1e-4 * 16 * 900)
     add("histogram_zipf", P.histogram(97), [rng.integers(0, 97, 3000).astype(np.int32)], None)

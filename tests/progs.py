@@ -239,3 +239,85 @@ def stencil2_sum(ty, b1, b2):
     st = A.stencil_type(sr)
     return A.alam([A.tarray(2, ty), A.tarray(2, ty)],
                   lambda x, y: A.stencil2(sr, sr, ty, A.lam([st, st], f), b1, x, b2, y))
+
+
+# -- whole programs in the shape the reference's nofib "spectral" group has them ------------
+
+def smvm(ty):
+    """Spectral/SMVM.hs: foldSeg (+) 0 (zipWith (*) vals (gather inds vec)) segd -- the product
+    and the gather are fused into the segmented fold's source; the offsets scan is let-bound."""
+    sh1 = A.tshape(1)
+
+    def body(segd, inds, vals, vec):
+        def at(ix):
+            return A.mul(ty, A.index(vals, A.vexp(ix)), A.index(vec, A.sh(A.index(inds, A.vexp(ix)))))
+
+        def at_lin(i):
+            return A.mul(ty, A.linearindex(vals, i), A.index(vec, A.sh(A.linearindex(inds, i))))
+
+        src = A.delayed(A.tarray(1, ty), A.shape(vals), A.lam([sh1], at), A.lam([Int], at_lin))
+        return A.alet(A.tarray(1, Int), A.scan("l", binop(A.add, Int), A.constI(0), segd),
+                      lambda offs: A.foldseg(Int, binop(A.add, ty), A.const(ty, 0), src, offs))
+
+    return A.alam([A.tarray(1, Int), A.tarray(1, Int), A.tarray(1, ty), A.tarray(1, ty)], body)
+
+
+def filter_positive(ty=Int):
+    """filter (> 0) (Prelude.hs filter): keep-flags, an exclusive scan for the targets and
+    the count, a result whose extent is read from the count, a permute that drops the rest."""
+    sh1 = A.tshape(1)
+    V1, S0 = A.tarray(1, Int), A.tarray(0, Int)
+
+    def body(xs):
+        flags = A.map_(Int, A.lam([ty], lambda x: A.cond(A.gt(ty, x, A.const(ty, 0)), A.constI(1), A.constI(0))), xs)
+
+        def with_flags(fl):
+            def with_scan(st):
+                targets, total = st
+                return A.permute(
+                    A.lam([ty, A.wild(ty)], lambda x, _: x),
+                    A.generate(A.tarray(1, ty), A.sh(A.index(total, A.nil)), A.lam([sh1], lambda ix: A.const(ty, 0))),
+                    A.lam([sh1], lambda ix: A.cond(A.eq(Int, A.index(fl, A.vexp(ix)), A.constI(0)), A.nothing(sh1),
+                                                   A.just(A.sh(A.index(targets, A.vexp(ix)))))),
+                    xs)
+            return A.alet(A.tpair(V1, S0), A.scan_("l", binop(A.add, Int), A.constI(0), fl), with_scan)
+        return A.alet(V1, flags, with_flags)
+
+    return A.alam([A.tarray(1, ty)], body)
+
+
+def radix_passes(bits):
+    """Spectral/RadixSort.hs, `bits` least-significant-bit passes over Int keys: per pass two
+    exclusive scans give the zero-bit keys' and the one-bit keys' places, a permute moves them."""
+    sh1 = A.tshape(1)
+    V1, S0 = A.tarray(1, Int), A.tarray(0, Int)
+
+    def one_pass(keys, b, rest):
+        def bit(k):
+            return A.band(Int, A.shr(Int, k, A.constI(b)), A.constI(1))
+        ones = A.map_(Int, A.lam([Int], bit), keys)
+        zeros = A.map_(Int, A.lam([Int], lambda k: A.sub(Int, A.constI(1), bit(k))), keys)
+
+        def with_zeros(zs):
+            zpos, nz = zs
+
+            def with_ones(os_):
+                opos, _ = os_
+
+                def dest(ix):
+                    k = A.index(keys, A.vexp(ix))
+                    return A.just(A.sh(A.cond(A.eq(Int, bit(k), A.constI(0)), A.index(zpos, A.vexp(ix)),
+                                              A.add(Int, A.index(nz, A.nil), A.index(opos, A.vexp(ix))))))
+                moved = A.permute(A.lam([Int, A.wild(Int)], lambda x, _: x),
+                                  A.generate(V1, A.shape(keys), A.lam([sh1], lambda ix: A.constI(0))),
+                                  A.lam([sh1], dest), keys)
+                return A.alet(V1, moved, rest)
+            return A.alet(A.tpair(V1, S0), A.scan_("l", binop(A.add, Int), A.constI(0), ones), with_ones)
+        return A.alet(A.tpair(V1, S0), A.scan_("l", binop(A.add, Int), A.constI(0), zeros), with_zeros)
+
+    def build(keys, b):
+        if b == bits:
+            return keys
+        return one_pass(keys, b, lambda moved: build(moved, b + 1))
+
+    return A.alam([V1], lambda keys: build(keys, 0))

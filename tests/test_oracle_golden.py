@@ -257,3 +257,21 @@ def test_workload_generators_are_seeded_and_shaped():
     keys = W.zipf_keys(100000, 1 << 10, 4)
     h = np.bincount(keys, minlength=1 << 10)
     assert h[0] == h.max() and 0.1 < h[0] / 100000 < 0.25   # 1/H(1024, 1.1) is about 0.17
+
+
+def test_oracle_on_whole_programs_against_numpy():
+    # SMVM, filter and LSD radix sort as the reference's nofib states them, against what numpy
+    # gives for the same inputs: pins the oracle on compositions of scan, permute and foldSeg
+    from . import progs as Q
+    rng = np.random.default_rng(11)
+    segd = rng.integers(0, 6, 40).astype(np.int64)
+    nnz = int(segd.sum())
+    inds, vals = rng.integers(0, 30, nnz).astype(np.int64), rng.integers(-9, 9, nnz).astype(np.int64)
+    vec = rng.integers(-9, 9, 30).astype(np.int64)
+    off = np.concatenate([[0], np.cumsum(segd)])
+    ref = np.array([(vals[off[i]:off[i + 1]] * vec[inds[off[i]:off[i + 1]]]).sum() for i in range(40)])
+    assert np.array_equal(O.run_n(Q.smvm(A.i64).text(), segd, inds, vals, vec), ref)
+    x = rng.integers(-50, 50, 300).astype(np.int64)
+    assert np.array_equal(O.run_n(Q.filter_positive().text(), x), x[x > 0])
+    k = rng.integers(0, 16, 500).astype(np.int64)
+    assert np.array_equal(O.run_n(Q.radix_passes(4).text(), k), np.sort(k, kind="stable"))
