@@ -1040,6 +1040,14 @@ KernelSource Codegen::scan(const Sx& f, const Sx* seed, const Operand& src, bool
   }
   body += "  static constexpr int G = " + std::to_string(g) + ";\n";
   body += "#define ACC_SCAN_BLOCK " + std::to_string(block) + "\n";
+  {
+    // prefixes of the lane totals by raking through LDS, when the totals of a workgroup fit
+    int sz = 0, al = 1;
+    structLayout(leaves, sz, al);
+    const long rake = (long)(block / 64) * (64 * (g + 1) + 1) * sz;
+    const char* re = std::getenv("ACCHIP_SCAN_RAKE");
+    if (g > 1 && rake <= 112 * 1024 && !(re && re[0] == '0')) body += "#define ACC_SCAN_RAKE 1\n";
+  }
   KernelSource ks = finish(body, elt, leaves, "scan.hpp+scan_kernel.hpp", vec);
   ks.block = block;
   ks.group = g;

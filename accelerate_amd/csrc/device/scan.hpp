@@ -259,10 +259,67 @@ ACC_DEV void acc_scan_tile(const typename S::Env& env, u64* desc, i64 tiles, i64
     }
   }
 
-  // Wave scan per group, chained over the groups of this wave; the prefix inside the wave
-  // is applied to the elements at once, so that only x stays live across the look-back.
   Elt waveTot;
   bool hasWaveTot = false;
+#ifdef ACC_SCAN_RAKE
+  // Prefixes of the 64 * G lane totals of this wave (in the order group, lane) by raking: the
+  // totals go to the wave's stretch of LDS, every lane scans G consecutive ones serially, one
+  // ordered wave scan joins the 64 chunks, and every lane reads the exclusive prefix of each of
+  // its G totals back.  One wave scan per tile instead of G: the G wave scans were most of
+  // the vector instructions of the kernel.  A chunk takes G + 1 slots so that the lanes' reads
+  // of their chunks spread over the banks.
+  {
+    __shared__ Elt sh_rake[ACC_SCAN_WAVES][ACC_WAVE * (C::G + 1) + 1];
+    Elt* mine = sh_rake[w];
+    i64 wcnt = n - wlo;  // elements of the sequence from this wave's start on
+    wcnt = wcnt < 0 ? 0 : (wcnt > (i64)G * C::GROUP ? (i64)G * C::GROUP : wcnt);
+    const int entries = (int)((wcnt + V - 1) / V);  // lane totals that hold data; they come first
+#pragma unroll
+    for (int g = 0; g < G; ++g) {
+      const int e = g * ACC_WAVE + lane;
+      mine[(e / G) * (G + 1) + e % G] = x[g][V - 1];
+    }
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    Elt c[C::G];
+#pragma unroll
+    for (int j = 0; j < G; ++j) c[j] = mine[lane * (G + 1) + j];
+#pragma unroll
+    for (int j = 1; j < G; ++j) c[j] = S::combine(env, c[j - 1], c[j]);  // inclusive inside the chunk
+    Elt ts = acc_wave_scan<S>(env, c[G - 1], lane);
+    Elt chunkPre = acc_prev_lane(ts);  // everything before this lane's chunk (lane > 0)
+    // the wave's total is the inclusive value of the last total that holds data
+    if (entries > 0 && (entries - 1) / G == lane) {
+      const int jl = (entries - 1) % G;
+      Elt t = c[0];
+#pragma unroll
+      for (int j = 1; j < G; ++j)
+        if (j == jl) t = c[j];
+      mine[ACC_WAVE * (G + 1)] = lane > 0 ? S::combine(env, chunkPre, t) : t;
+    }
+    // exclusive prefixes go back in place (entry 0 of the wave has none)
+    if (lane > 0) mine[lane * (G + 1)] = chunkPre;
+#pragma unroll
+    for (int j = 1; j < G; ++j) mine[lane * (G + 1) + j] = lane > 0 ? S::combine(env, chunkPre, c[j - 1]) : c[j - 1];
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+#pragma unroll
+    for (int g = 0; g < G; ++g) {
+      const int e = g * ACC_WAVE + lane;
+      if (e > 0) {
+        const Elt pre = mine[(e / G) * (G + 1) + e % G];
+#pragma unroll
+        for (int k = 0; k < V; ++k) x[g][k] = S::combine(env, pre, x[g][k]);
+      }
+    }
+    hasWaveTot = entries > 0;
+    if (hasWaveTot) waveTot = mine[ACC_WAVE * (G + 1)];
+  }
+#else
+  // Wave scan per group, chained over the groups of this wave; the prefix inside the wave
+  // is applied to the elements at once, so that only x stays live across the look-back.
 #pragma unroll
   for (int g = 0; g < G; ++g) {
     i64 cnt = n - (wlo + (i64)g * C::GROUP);
@@ -285,6 +342,7 @@ ACC_DEV void acc_scan_tile(const typename S::Env& env, u64* desc, i64 tiles, i64
       hasWaveTot = true;
     }
   }
+#endif
   if (lane == 0) sh_wave[w] = waveTot;
   __syncthreads();
 
