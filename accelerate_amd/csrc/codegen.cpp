@@ -817,6 +817,8 @@ static std::string fnHead(const char* ret, const char* name, const char* params)
   return std::string("  ACC_DEV ") + ret + " " + name + "(" + params + ") {\n";
 }
 
+static void structLayout(const std::vector<ST>& leaves, int& size, int& align);
+
 KernelSource Codegen::fold(const Sx& f, const Sx* seed, const Operand& src) {
   const TypeP elt = src.r.elt;
   std::string body;
@@ -861,6 +863,13 @@ KernelSource Codegen::fold(const Sx& f, const Sx* seed, const Operand& src) {
   const int g = std::max(1, std::min(8, 64 / std::max(1, vec * eltBytes)));
   body += "  static constexpr int G = " + std::to_string(g) + ";\n";
   body += "#define ACC_SCAN_BLOCK 256\n";
+  {
+    int sz = 0, al = 1;
+    std::vector<ST> flagged = leaves;
+    flagged.push_back(ST::U32);
+    structLayout(flagged, sz, al);
+    if (g > 1 && 4L * (64 * (g + 1) + 1) * sz <= 64 * 1024) body += "#define ACC_ROWS_RAKE 1\n";
+  }
   KernelSource ks = finish(body, elt, leaves, "scan.hpp+fold.hpp", vec);
   ks.commutative = comm;
   ks.group = g;
@@ -1047,6 +1056,12 @@ KernelSource Codegen::scan(const Sx& f, const Sx* seed, const Operand& src, bool
     const long rake = (long)(block / 64) * (64 * (g + 1) + 1) * sz;
     const char* re = std::getenv("ACCHIP_SCAN_RAKE");
     if (g > 1 && rake <= 112 * 1024 && !(re && re[0] == '0')) body += "#define ACC_SCAN_RAKE 1\n";
+    // the same for the rows kernel, whose values carry a head flag (only the 256-thread variant runs it)
+    std::vector<ST> flagged = leaves;
+    flagged.push_back(ST::U32);
+    structLayout(flagged, sz, al);
+    if (small && g > 1 && (long)(block / 64) * (64 * (g + 1) + 1) * sz <= 64 * 1024 && !(re && re[0] == '0'))
+      body += "#define ACC_ROWS_RAKE 1\n";
   }
   KernelSource ks = finish(body, elt, leaves, "scan.hpp+scan_kernel.hpp", vec);
   ks.block = block;

@@ -91,7 +91,7 @@ acc_foldseg_partition(Spec::Env env, Spec::Out out, FoldSegParams p) {
 // no division is needed.  FULL: the tile lies completely inside the stream.
 template <bool ONE_ROW, bool FULL>
 ACC_DEV void acc_foldseg_tile(const Spec::Env& env, const Spec::Out& out, const FoldSegParams& p, unsigned short* sh_first,
-                              AccSegSpec<Spec>::Elt* sh_wave, Spec::Elt& sh_pend, int& sh_pend_at) {
+                              AccSegSpec<Spec>::Elt* sh_wave, AccSegSpec<Spec>::Elt* sh_rake, Spec::Elt& sh_pend, int& sh_pend_at) {
   typedef Spec S;
   typedef AccSegSpec<Spec> SS;
   typedef AccScanCfg<SS> C;
@@ -212,6 +212,7 @@ ACC_DEV void acc_foldseg_tile(const Spec::Env& env, const Spec::Out& out, const 
   bool hasWaveTot = false;
   S::Elt pendVal[C::G];
   int pendIdx[C::G];
+  P agg[C::G];
 #pragma unroll
   for (int g = 0; g < G; ++g) {
     const i64 t0 = wlo + ((i64)g * ACC_WAVE + lane) * V;
@@ -247,23 +248,26 @@ ACC_DEV void acc_foldseg_tile(const Spec::Env& env, const Spec::Out& out, const 
       }
     }
 
-    i64 cnt = n - (wlo + (i64)g * C::GROUP);
-    cnt = cnt < 0 ? 0 : (cnt > C::GROUP ? C::GROUP : cnt);
-    P ts = acc_wave_scan<SS>(env, a, lane);
-    P lanePre = acc_prev_lane(ts);  // exclusive prefix of the run inside its group (lane > 0)
-    const int last = cnt > 0 ? (int)((cnt - 1) / V) : 0;
-    P gt = acc_readlane(ts, last);
-    P pre;
-    if (acc_join<SS>(env, hasWaveTot, waveTot, lane > 0, lanePre, pre) && pendIdx[g] != NOPEND) {
-      pendVal[g] = S::combine(env, pre.v, pendVal[g]);
-      if (pre.f) {
-        emit(pendIdx[g], pendVal[g]);
-        pendIdx[g] = NOPEND;
+    agg[g] = a;
+  }
+  // exclusive prefixes of the runs' aggregates inside the wave, by raking (acc_rake); a prefix
+  // that contains a head closes a pending end here
+  {
+    i64 wcnt = n - wlo;
+    wcnt = wcnt < 0 ? 0 : (wcnt > (i64)G * C::GROUP ? (i64)G * C::GROUP : wcnt);
+    const int entries = (int)((wcnt + V - 1) / V);
+    P pre[C::G];
+    acc_rake<SS, C::G>(env, sh_rake + w * (ACC_WAVE * (C::G + 1) + 1), agg, lane, entries, pre, waveTot);
+    hasWaveTot = entries > 0;
+#pragma unroll
+    for (int g = 0; g < G; ++g) {
+      if (g * ACC_WAVE + lane > 0 && pendIdx[g] != NOPEND) {
+        pendVal[g] = S::combine(env, pre[g].v, pendVal[g]);
+        if (pre[g].f) {
+          emit(pendIdx[g], pendVal[g]);
+          pendIdx[g] = NOPEND;
+        }
       }
-    }
-    if (cnt > 0) {
-      waveTot = hasWaveTot ? SS::combine(env, waveTot, gt) : gt;
-      hasWaveTot = true;
     }
   }
   if (lane == 0) sh_wave[w] = waveTot;
@@ -312,15 +316,16 @@ acc_foldseg(Spec::Env env, Spec::Out out, FoldSegParams p) {
   // sh_first[q]: first boundary (relative to the tile's first) at position q of the tile
   __shared__ __attribute__((aligned(16))) unsigned short sh_first[C::TILE + 8];
   __shared__ AccSegSpec<Spec>::Elt sh_wave[ACC_SCAN_WAVES];
+  __shared__ AccSegSpec<Spec>::Elt sh_rake[ACC_SCAN_WAVES * (ACC_WAVE * (C::G + 1) + 1)];
   __shared__ Spec::Elt sh_pend;
   __shared__ int sh_pend_at;
   const bool full = ((i64)blockIdx.x + 1) * (i64)C::TILE <= p.total;
   if (p.rows == 1) {
-    if (full) acc_foldseg_tile<true, true>(env, out, p, sh_first, sh_wave, sh_pend, sh_pend_at);
-    else acc_foldseg_tile<true, false>(env, out, p, sh_first, sh_wave, sh_pend, sh_pend_at);
+    if (full) acc_foldseg_tile<true, true>(env, out, p, sh_first, sh_wave, sh_rake, sh_pend, sh_pend_at);
+    else acc_foldseg_tile<true, false>(env, out, p, sh_first, sh_wave, sh_rake, sh_pend, sh_pend_at);
   } else {
-    if (full) acc_foldseg_tile<false, true>(env, out, p, sh_first, sh_wave, sh_pend, sh_pend_at);
-    else acc_foldseg_tile<false, false>(env, out, p, sh_first, sh_wave, sh_pend, sh_pend_at);
+    if (full) acc_foldseg_tile<false, true>(env, out, p, sh_first, sh_wave, sh_rake, sh_pend, sh_pend_at);
+    else acc_foldseg_tile<false, false>(env, out, p, sh_first, sh_wave, sh_rake, sh_pend, sh_pend_at);
   }
 }
 

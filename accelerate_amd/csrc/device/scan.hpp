@@ -208,6 +208,57 @@ ACC_DEV bool acc_lookback(const typename S::Env& env, const u64* rowDesc, i64 ti
   return have;
 }
 
+// Exclusive prefixes of the 64 * G values t[g] that the lanes of a wave hold, taken in the
+// order (g, lane), by raking: the values go to the wave's stretch of LDS (`mine`, room for
+// 64 * (G + 1) + 1 elements), every lane scans G consecutive ones serially, one ordered wave
+// scan joins the 64 chunks, and every lane reads the prefix of each of its values back.  One
+// wave scan instead of G, which were most of the vector instructions of these kernels.  A
+// chunk takes G + 1 slots so that the lanes' reads of their chunks spread over the banks.
+// Only the first `entries` values (in that order) hold data.  pre[g] is undefined for the
+// very first value (g = 0 in lane 0); total is their combination, valid when entries > 0.
+template <class S, int G>
+ACC_DEV void acc_rake(const typename S::Env& env, typename S::Elt* mine, const typename S::Elt (&t)[G], int lane,
+                      int entries, typename S::Elt (&pre)[G], typename S::Elt& total) {
+  typedef typename S::Elt Elt;
+#pragma unroll
+  for (int g = 0; g < G; ++g) {
+    const int e = g * ACC_WAVE + lane;
+    mine[(e / G) * (G + 1) + e % G] = t[g];
+  }
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+  __builtin_amdgcn_wave_barrier();
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+  Elt c[G];
+#pragma unroll
+  for (int j = 0; j < G; ++j) c[j] = mine[lane * (G + 1) + j];
+#pragma unroll
+  for (int j = 1; j < G; ++j) c[j] = S::combine(env, c[j - 1], c[j]);  // inclusive inside the chunk
+  Elt ts = acc_wave_scan<S>(env, c[G - 1], lane);
+  Elt chunkPre = acc_prev_lane(ts);  // everything before this lane's chunk (lane > 0)
+  // the total is the inclusive value of the last value that holds data
+  if (entries > 0 && (entries - 1) / G == lane) {
+    const int jl = (entries - 1) % G;
+    Elt v = c[0];
+#pragma unroll
+    for (int j = 1; j < G; ++j)
+      if (j == jl) v = c[j];
+    mine[ACC_WAVE * (G + 1)] = lane > 0 ? S::combine(env, chunkPre, v) : v;
+  }
+  // exclusive prefixes go back in place
+  if (lane > 0) mine[lane * (G + 1)] = chunkPre;
+#pragma unroll
+  for (int j = 1; j < G; ++j) mine[lane * (G + 1) + j] = lane > 0 ? S::combine(env, chunkPre, c[j - 1]) : c[j - 1];
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+  __builtin_amdgcn_wave_barrier();
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+#pragma unroll
+  for (int g = 0; g < G; ++g) {
+    const int e = g * ACC_WAVE + lane;
+    if (e > 0) pre[g] = mine[(e / G) * (G + 1) + e % G];
+  }
+  if (entries > 0) total = mine[ACC_WAVE * (G + 1)];
+}
+
 // One tile of a scan over a sequence of n elements: load(t) yields element t, store(t, y)
 // receives val[t] (the inclusive combination up to t, seed included when S::kSeeded).
 // `desc` holds the descriptors of this sequence's tiles.  Called by all threads of the
@@ -262,60 +313,25 @@ ACC_DEV void acc_scan_tile(const typename S::Env& env, u64* desc, i64 tiles, i64
   Elt waveTot;
   bool hasWaveTot = false;
 #ifdef ACC_SCAN_RAKE
-  // Prefixes of the 64 * G lane totals of this wave (in the order group, lane) by raking: the
-  // totals go to the wave's stretch of LDS, every lane scans G consecutive ones serially, one
-  // ordered wave scan joins the 64 chunks, and every lane reads the exclusive prefix of each of
-  // its G totals back.  One wave scan per tile instead of G: the G wave scans were most of
-  // the vector instructions of the kernel.  A chunk takes G + 1 slots so that the lanes' reads
-  // of their chunks spread over the banks.
+  // prefixes of the lane totals by raking (acc_rake), applied to the elements at once, so
+  // that only x stays live across the look-back
   {
     __shared__ Elt sh_rake[ACC_SCAN_WAVES][ACC_WAVE * (C::G + 1) + 1];
-    Elt* mine = sh_rake[w];
     i64 wcnt = n - wlo;  // elements of the sequence from this wave's start on
     wcnt = wcnt < 0 ? 0 : (wcnt > (i64)G * C::GROUP ? (i64)G * C::GROUP : wcnt);
     const int entries = (int)((wcnt + V - 1) / V);  // lane totals that hold data; they come first
+    Elt tl[C::G], pre[C::G];
+#pragma unroll
+    for (int g = 0; g < G; ++g) tl[g] = x[g][V - 1];
+    acc_rake<S, C::G>(env, sh_rake[w], tl, lane, entries, pre, waveTot);
 #pragma unroll
     for (int g = 0; g < G; ++g) {
-      const int e = g * ACC_WAVE + lane;
-      mine[(e / G) * (G + 1) + e % G] = x[g][V - 1];
-    }
-    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-    __builtin_amdgcn_wave_barrier();
-    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-    Elt c[C::G];
+      if (g * ACC_WAVE + lane > 0) {
 #pragma unroll
-    for (int j = 0; j < G; ++j) c[j] = mine[lane * (G + 1) + j];
-#pragma unroll
-    for (int j = 1; j < G; ++j) c[j] = S::combine(env, c[j - 1], c[j]);  // inclusive inside the chunk
-    Elt ts = acc_wave_scan<S>(env, c[G - 1], lane);
-    Elt chunkPre = acc_prev_lane(ts);  // everything before this lane's chunk (lane > 0)
-    // the wave's total is the inclusive value of the last total that holds data
-    if (entries > 0 && (entries - 1) / G == lane) {
-      const int jl = (entries - 1) % G;
-      Elt t = c[0];
-#pragma unroll
-      for (int j = 1; j < G; ++j)
-        if (j == jl) t = c[j];
-      mine[ACC_WAVE * (G + 1)] = lane > 0 ? S::combine(env, chunkPre, t) : t;
-    }
-    // exclusive prefixes go back in place (entry 0 of the wave has none)
-    if (lane > 0) mine[lane * (G + 1)] = chunkPre;
-#pragma unroll
-    for (int j = 1; j < G; ++j) mine[lane * (G + 1) + j] = lane > 0 ? S::combine(env, chunkPre, c[j - 1]) : c[j - 1];
-    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-    __builtin_amdgcn_wave_barrier();
-    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-#pragma unroll
-    for (int g = 0; g < G; ++g) {
-      const int e = g * ACC_WAVE + lane;
-      if (e > 0) {
-        const Elt pre = mine[(e / G) * (G + 1) + e % G];
-#pragma unroll
-        for (int k = 0; k < V; ++k) x[g][k] = S::combine(env, pre, x[g][k]);
+        for (int k = 0; k < V; ++k) x[g][k] = S::combine(env, pre[g], x[g][k]);
       }
     }
     hasWaveTot = entries > 0;
-    if (hasWaveTot) waveTot = mine[ACC_WAVE * (G + 1)];
   }
 #else
   // Wave scan per group, chained over the groups of this wave; the prefix inside the wave
@@ -501,24 +517,48 @@ ACC_DEV void acc_rows_tile(const typename S::Env& env, int cnt, int n, const Loa
   }
   P waveTot;
   bool hasWaveTot = false;
+#ifdef ACC_ROWS_RAKE
+  {
+    // prefixes of the lane totals by raking (acc_rake)
+    __shared__ P sh_rake[ACC_SCAN_WAVES][ACC_WAVE * (C::G + 1) + 1];
+    int wcnt = cnt - wlo;
+    wcnt = wcnt < 0 ? 0 : (wcnt > G * C::GROUP ? G * C::GROUP : wcnt);
+    const int entries = (wcnt + V - 1) / V;
+    P tl[C::G], pre[C::G];
 #pragma unroll
-  for (int g = 0; g < G; ++g) {
-    int c = cnt - (wlo + g * C::GROUP);
-    c = c < 0 ? 0 : (c > C::GROUP ? C::GROUP : c);
-    P ts = acc_wave_scan<SS>(env, x[g][V - 1], lane);
-    P lanePre = acc_prev_lane(ts);
-    const int last = c > 0 ? (c - 1) / V : 0;
-    P gt = acc_readlane(ts, last);
-    P pre;
-    if (acc_join<SS>(env, hasWaveTot, waveTot, lane > 0, lanePre, pre)) {
+    for (int g = 0; g < G; ++g) tl[g] = x[g][V - 1];
+    acc_rake<SS, C::G>(env, sh_rake[w], tl, lane, entries, pre, waveTot);
 #pragma unroll
-      for (int k = 0; k < V; ++k) x[g][k] = SS::combine(env, pre, x[g][k]);
+    for (int g = 0; g < G; ++g) {
+      if (g * ACC_WAVE + lane > 0) {
+#pragma unroll
+        for (int k = 0; k < V; ++k) x[g][k] = SS::combine(env, pre[g], x[g][k]);
+      }
     }
-    if (c > 0) {
-      waveTot = hasWaveTot ? SS::combine(env, waveTot, gt) : gt;
-      hasWaveTot = true;
+    hasWaveTot = entries > 0;
+  }
+#else
+  {
+#pragma unroll
+    for (int g = 0; g < G; ++g) {
+      int c = cnt - (wlo + g * C::GROUP);
+      c = c < 0 ? 0 : (c > C::GROUP ? C::GROUP : c);
+      P ts = acc_wave_scan<SS>(env, x[g][V - 1], lane);
+      P lanePre = acc_prev_lane(ts);
+      const int last = c > 0 ? (c - 1) / V : 0;
+      P gt = acc_readlane(ts, last);
+      P pre;
+      if (acc_join<SS>(env, hasWaveTot, waveTot, lane > 0, lanePre, pre)) {
+#pragma unroll
+        for (int k = 0; k < V; ++k) x[g][k] = SS::combine(env, pre, x[g][k]);
+      }
+      if (c > 0) {
+        waveTot = hasWaveTot ? SS::combine(env, waveTot, gt) : gt;
+        hasWaveTot = true;
+      }
     }
   }
+#endif
   if (lane == 0) sh_wave[w] = waveTot;
   __syncthreads();
   const int perWave = G * C::GROUP;
