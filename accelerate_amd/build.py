@@ -48,7 +48,7 @@ def build(verbose=True):
            "-D__HIP_PLATFORM_AMD__", "-I" + os.path.join(rocm, "include"),
            "-o", LIB] + [os.path.join(CSRC, s) for s in HOST_SOURCES] + [
                gen, "-L" + os.path.join(rocm, "lib"), "-Wl,-rpath," + os.path.join(rocm, "lib"),
-               "-lamdhip64", "-lhiprtc", "-ldl"]
+               "-lamdhip64", "-lhiprtc", "-pthread", "-ldl"]
     if verbose:
         print(" ".join(cmd), flush=True)
     subprocess.run(cmd, check=True)

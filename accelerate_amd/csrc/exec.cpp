@@ -343,6 +343,13 @@ Program::Program(Context& ctx, const char* text, size_t len) : ctx_(ctx) {
   }
   body_ = f;
   resultType = prepare(*body_, tenv);
+  // the kernels were handed to the compiler as they were generated; collect them (and what the
+  // compiler had to say) before the program is handed out
+  for (auto& kv : plans_) {
+    ctx_.wait(kv.second.k);
+    ctx_.wait(kv.second.k2);
+    for (auto& sk : kv.second.scalarKernels) ctx_.wait(sk.second);
+  }
 }
 
 std::vector<ArrayR> Program::aenvOf(const TEnv& tenv) {

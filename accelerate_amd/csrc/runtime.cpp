@@ -51,6 +51,12 @@ Context::Context(int device) : device_(device) {
 }
 
 Context::~Context() {
+  for (auto& kv : kernels_) {
+    try {
+      wait(kv.second);  // a worker may still be writing into the kernel
+    } catch (...) {
+    }
+  }
   if (device_ < 0) return;
   (void)hipSetDevice(device_);
   (void)hipStreamSynchronize(stream_);
@@ -293,6 +299,33 @@ static std::string definesPrefix() {
   return out;
 }
 
+// limits the hipRTC compilations that run at the same time
+namespace {
+std::mutex g_slotMu;
+std::condition_variable g_slotCv;
+int g_slotsFree = -1;
+struct CompileSlot {
+  CompileSlot() {
+    std::unique_lock<std::mutex> l(g_slotMu);
+    if (g_slotsFree < 0) {
+      long n = sysconf(_SC_NPROCESSORS_ONLN);
+      const char* e = std::getenv("ACCHIP_COMPILE_JOBS");
+      if (e) n = std::atol(e);
+      g_slotsFree = (int)std::max<long>(1, std::min<long>(n, 16));
+    }
+    g_slotCv.wait(l, [] { return g_slotsFree > 0; });
+    --g_slotsFree;
+  }
+  ~CompileSlot() {
+    {
+      std::lock_guard<std::mutex> l(g_slotMu);
+      ++g_slotsFree;
+    }
+    g_slotCv.notify_one();
+  }
+};
+}  // namespace
+
 KernelP Context::kernel(const KernelSource& ks0) {
   KernelSource ks = ks0;
   ks.source = definesPrefix() + ks0.source;
@@ -319,20 +352,32 @@ KernelP Context::kernel(const KernelSource& ks0) {
   if (!forceRecomp && readFile(path, k->code) && !k->code.empty()) {
     stats.kernelsFromDisk++;
   } else {
-    std::string log;
-    k->code = compileHipRTC(ks.source, log);
-    if (dumpCC && !log.empty()) fprintf(stderr, "[acchip] hipRTC log:\n%s\n", log.c_str());
+    // compile on a worker thread, at most as many at once as there are cores
     stats.kernelsCompiled++;
-    ::mkdir(cacheDir.c_str(), 0777);
-    writeFile(path, k->code);
+    const bool dump = dumpCC;
+    const std::string dir = cacheDir;
+    Kernel* raw = k.get();  // kept alive by kernels_ until the context goes, which waits
+    k->ready = std::async(std::launch::async, [raw, src = ks.source, path, dir, dump]() {
+                 CompileSlot slot;
+                 std::string log;
+                 raw->code = compileHipRTC(src, log);
+                 if (dump && !log.empty()) fprintf(stderr, "[acchip] hipRTC log:\n%s\n", log.c_str());
+                 ::mkdir(dir.c_str(), 0777);
+                 writeFile(path, raw->code);
+               }).share();
   }
   std::lock_guard<std::mutex> g(mu_);
   auto ins = kernels_.emplace(hash, k);
   return ins.first->second;
 }
 
+void Context::wait(const KernelP& k) {
+  if (k && k->ready.valid()) k->ready.get();
+}
+
 void Context::ensureLoaded(const KernelP& k) {
   if (k->module) return;
+  wait(k);
   if (device_ < 0) throw Error("this context has no device: programs can be compiled but not executed");
   hipCheck(hipModuleLoadData(&k->module, k->code.data()), "hipModuleLoadData");
 }

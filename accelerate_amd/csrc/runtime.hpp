@@ -4,6 +4,8 @@
 #include <hip/hip_runtime.h>
 
 #include <atomic>
+#include <condition_variable>
+#include <future>
 #include <map>
 #include <memory>
 #include <mutex>
@@ -17,7 +19,8 @@ namespace acchip {
 
 struct Kernel {
   std::string hash;
-  std::string code;                 // code object (hsaco)
+  std::shared_future<void> ready;   // compilation in flight (valid only when hipRTC had to run)
+  std::string code;                 // code object (hsaco), complete once `ready` is
   hipModule_t module = nullptr;     // loaded lazily, on first launch
   std::map<std::string, hipFunction_t> fns;
   KernelSource meta;                // argument plan (source text dropped after compilation)
@@ -58,7 +61,11 @@ class Context : public std::enable_shared_from_this<Context> {
   void fill0(void* dev, size_t bytes);
   void sync();
 
+  // Looks the kernel up (memory, then disk) or starts its compilation on a worker thread:
+  // the kernels of a program compile side by side.  wait() returns when the code object is
+  // there, and throws what the compiler reported.
   KernelP kernel(const KernelSource& ks);
+  void wait(const KernelP& k);
   void launch(const KernelP& k, const char* fn, unsigned grid, unsigned block, const std::vector<uint64_t>& args);
 
   // persistent device scratch for single-pass scans (tile descriptors + ticket counter)
