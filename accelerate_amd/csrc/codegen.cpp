@@ -201,6 +201,7 @@ std::string Codegen::toIndex(const ValP& sh, const ValP& ix, Emit& em) {
   shapeDims(ix, i);
   if (d.size() != i.size()) throw Error("toIndex: rank mismatch between shape and index");
   if (d.empty()) return "((i64)0)";
+  if (d.size() == 1) return i[0];
   std::string e = i[0];
   for (size_t k = 1; k < d.size(); ++k) e = "(" + e + " * " + d[k] + " + " + i[k] + ")";
   return bindLeaf(ST::I64, e, em)->ex;
@@ -229,7 +230,11 @@ ValP Codegen::readArray(const ArraySlot& s, const std::string& lin, Emit& em) {
     static ValP go(Codegen& cg, const TypeP& t, const ArraySlot& s, const std::string& lin, int& leaf, Emit& em) {
       if (t->k == Type::Unit) return vUnit();
       if (t->k == Type::Scalar)
-        return cg.bindLeaf(t->st, "env." + s.name + "_" + std::to_string(leaf++) + "[" + lin + "]", em);
+      {
+        const std::string at = "env." + s.name + "_" + std::to_string(leaf++) + "[" + lin + "]";
+        // read at the skeleton's own linear index: each element once, in order
+        return cg.bindLeaf(t->st, lin == "i" ? "acc_ld<kStream>(&" + at + ")" : at, em);
+      }
       ValP a = go(cg, t->a, s, lin, leaf, em);
       return vPair(a, go(cg, t->b, s, lin, leaf, em));
     }
@@ -795,8 +800,9 @@ KernelSource Codegen::finish(const std::string& specBody, const TypeP& elt, cons
     s += "  ACC_DEV Elt load(const Out& o, i64 i) {\n    Elt r_;\n";
     for (size_t k = 0; k < el.size(); ++k) s += "    r_.c" + std::to_string(k) + " = o.o" + std::to_string(k) + "[i];\n";
     s += "    return r_;\n  }\n";
-    s += "  ACC_DEV void store(const Out& o, i64 i, const Elt& v) {\n";
-    for (size_t k = 0; k < el.size(); ++k) s += "    o.o" + std::to_string(k) + "[i] = v.c" + std::to_string(k) + ";\n";
+    s += "  template <bool kStream = false>\n  ACC_DEV void store(const Out& o, i64 i, const Elt& v) {\n";
+    for (size_t k = 0; k < el.size(); ++k)
+      s += "    acc_st<kStream>(&o.o" + std::to_string(k) + "[i], v.c" + std::to_string(k) + ");\n";
     s += "  }\n";
   }
   s += "};\n\n";
@@ -815,6 +821,11 @@ KernelSource Codegen::finish(const std::string& specBody, const TypeP& elt, cons
 
 static std::string fnHead(const char* ret, const char* name, const char* params) {
   return std::string("  ACC_DEV ") + ret + " " + name + "(" + params + ") {\n";
+}
+
+// a function with a streaming variant: kStream selects non-temporal reads at index i
+static std::string streamHead(const char* ret, const char* name, const char* params) {
+  return "  template <bool kStream = false>\n" + fnHead(ret, name, params);
 }
 
 static void structLayout(const std::vector<ST>& leaves, int& size, int& align);
@@ -850,7 +861,7 @@ KernelSource Codegen::fold(const Sx& f, const Sx* seed, const Operand& src) {
     em.ind = 4;
     ValP v = operandLinear(src, "i", em);
     if (!typeEq(valType(v), elt)) throw Error("fold: fused producer does not return the element type");
-    body += fnHead("Elt", "in_linear", "const Env& env, i64 i") + returnElt(v, em) + "  }\n";
+    body += streamHead("Elt", "in_linear", "const Env& env, i64 i") + returnElt(v, em) + "  }\n";
   }
   // geometry of the kernel for many short rows (acc_fold_rows): 256 threads, about 64 bytes
   // of (value, flag) pairs per lane
@@ -874,6 +885,7 @@ KernelSource Codegen::fold(const Sx& f, const Sx* seed, const Operand& src) {
   ks.commutative = comm;
   ks.group = g;
   ks.block = 256;
+  ks.streaming = true;
   return ks;
 }
 
@@ -1076,8 +1088,10 @@ KernelSource Codegen::map(const TypeP& outElt, const Sx* f, const Operand& src) 
   ValP v = operandLinear(src, "i", em);
   ValP r = f ? applyFun(*f, {v}, {}, em) : v;
   if (!typeEq(valType(r), outElt)) throw Error("map: function result does not match the declared element type");
-  std::string body = fnHead("Elt", "produce", "const Env& env, i64 i") + returnElt(r, em) + "  }\n";
-  return finish(body, outElt, typeLeaves(outElt), "map.hpp", 0);
+  std::string body = streamHead("Elt", "produce", "const Env& env, i64 i") + returnElt(r, em) + "  }\n";
+  KernelSource ks = finish(body, outElt, typeLeaves(outElt), "map.hpp", 0);
+  ks.streaming = true;
+  return ks;
 }
 
 static void declareOut(std::map<std::string, ArraySlot>& used, int rank) {
@@ -1106,8 +1120,10 @@ KernelSource Codegen::zipWith(const TypeP& outElt, const Sx& f, const Operand& a
   }
   ValP r = applyFun(f, {x, y}, {}, em);
   if (!typeEq(valType(r), outElt)) throw Error("zipWith: function result does not match the declared element type");
-  std::string body = fnHead("Elt", "produce", "const Env& env, i64 i") + returnElt(r, em) + "  }\n";
-  return finish(body, outElt, typeLeaves(outElt), "map.hpp", 0);
+  std::string body = streamHead("Elt", "produce", "const Env& env, i64 i") + returnElt(r, em) + "  }\n";
+  KernelSource ks = finish(body, outElt, typeLeaves(outElt), "map.hpp", 0);
+  ks.streaming = true;
+  return ks;
 }
 
 KernelSource Codegen::generate(const ArrayR& out, const Sx& f) {
@@ -1118,8 +1134,10 @@ KernelSource Codegen::generate(const ArrayR& out, const Sx& f) {
   ValP ix = fromIndex(out.rank, shapeOf(o), "i", em);
   ValP r = applyFun(f, {ix}, {}, em);
   if (!typeEq(valType(r), out.elt)) throw Error("generate: function result does not match the declared element type");
-  std::string body = fnHead("Elt", "produce", "const Env& env, i64 i") + returnElt(r, em) + "  }\n";
-  return finish(body, out.elt, typeLeaves(out.elt), "map.hpp", 0);
+  std::string body = streamHead("Elt", "produce", "const Env& env, i64 i") + returnElt(r, em) + "  }\n";
+  KernelSource ks = finish(body, out.elt, typeLeaves(out.elt), "map.hpp", 0);
+  ks.streaming = true;
+  return ks;
 }
 
 KernelSource Codegen::backpermute(int outRank, const Sx& p, const Sx* f, const TypeP& outElt, const Operand& src) {
@@ -1132,8 +1150,10 @@ KernelSource Codegen::backpermute(int outRank, const Sx& p, const Sx* f, const T
   ValP v = operandIndex(src, sx, em);
   ValP r = f ? applyFun(*f, {v}, {}, em) : v;
   if (!typeEq(valType(r), outElt)) throw Error("backpermute: result does not match the declared element type");
-  std::string body = fnHead("Elt", "produce", "const Env& env, i64 i") + returnElt(r, em) + "  }\n";
-  return finish(body, outElt, typeLeaves(outElt), "map.hpp", 0);
+  std::string body = streamHead("Elt", "produce", "const Env& env, i64 i") + returnElt(r, em) + "  }\n";
+  KernelSource ks = finish(body, outElt, typeLeaves(outElt), "map.hpp", 0);
+  ks.streaming = true;
+  return ks;
 }
 
 // does the function's second argument (the old value) go unused?  `\x _ -> ..`
@@ -1742,7 +1762,7 @@ KernelSource Codegen::scalarKernel(const Sx& e) {
   em.ind = 4;
   ValP r = exp(e, {}, em);
   TypeP t = valType(r);
-  std::string body = fnHead("Elt", "produce", "const Env& env, i64 i") + returnElt(r, em) + "  }\n";
+  std::string body = streamHead("Elt", "produce", "const Env& env, i64 i") + returnElt(r, em) + "  }\n";
   return finish(body, t, typeLeaves(t), "map.hpp", 1);
 }
 

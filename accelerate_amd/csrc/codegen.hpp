@@ -54,6 +54,7 @@ struct KernelSource {
   int words = 1;                      // 32-bit words of Spec::Elt (scan descriptors)
   int block = 256;                    // threads per workgroup of the main kernel
   bool commutative = false;
+  bool streaming = false;             // has acc_*_stream entry points (non-temporal variant)
   std::string permuteMode;            // permute only: "atomic", "cas", "lock", "store"
 };
 

@@ -124,9 +124,9 @@ ACC_DEV bool acc_fold_block(const typename S::Env& env, const Src& src, i64 off,
   return have;
 }
 
-template <class S> struct AccFoldSrcIn {
+template <class S, bool NT = false> struct AccFoldSrcIn {
   const typename S::Env& env;
-  __device__ __forceinline__ typename S::Elt operator()(i64 i) const { return S::in_linear(env, i); }
+  __device__ __forceinline__ typename S::Elt operator()(i64 i) const { return S::template in_linear<NT>(env, i); }
 };
 template <class S> struct AccFoldSrcTmp {
   const typename S::Out& tmp;
@@ -145,15 +145,15 @@ ACC_DEV void acc_fold_finish(const typename S::Env& env, const typename S::Out& 
   }
 }
 
-extern "C" __global__ void __launch_bounds__(ACC_BLOCK)
-acc_fold_main(Spec::Env env, Spec::Out out, Spec::Out tmp, FoldParams p) {
+template <bool NT>
+ACC_DEV void acc_fold_main_body(const Spec::Env& env, const Spec::Out& out, const Spec::Out& tmp, const FoldParams& p) {
   typedef Spec S;
   i64 bid = (i64)blockIdx.x;
   i64 row = bid / p.bpr;
   i64 b = bid - row * p.bpr;
   i64 lo = b * p.chunk;
   i64 hi = lo + p.chunk < p.n ? lo + p.chunk : p.n;
-  AccFoldSrcIn<S> src{env};
+  AccFoldSrcIn<S, NT> src{env};
   S::Elt r;
   bool have = acc_fold_block<S>(env, src, row * p.n, lo, hi, r);
   if (p.bpr == 1) {
@@ -161,6 +161,18 @@ acc_fold_main(Spec::Env env, Spec::Out out, Spec::Out tmp, FoldParams p) {
   } else if (threadIdx.x == 0 && have) {
     S::store(tmp, bid, r);
   }
+}
+
+extern "C" __global__ void __launch_bounds__(ACC_BLOCK)
+acc_fold_main(Spec::Env env, Spec::Out out, Spec::Out tmp, FoldParams p) {
+  acc_fold_main_body<false>(env, out, tmp, p);
+}
+
+// the variant for sources far larger than the last-level cache: reads at the row's own
+// linear index are marked non-temporal
+extern "C" __global__ void __launch_bounds__(ACC_BLOCK)
+acc_fold_main_stream(Spec::Env env, Spec::Out out, Spec::Out tmp, FoldParams p) {
+  acc_fold_main_body<true>(env, out, tmp, p);
 }
 
 extern "C" __global__ void __launch_bounds__(ACC_BLOCK)

@@ -10,8 +10,8 @@ struct MapParams {
   i64 n;  // number of results
 };
 
-extern "C" __global__ void __launch_bounds__(ACC_BLOCK)
-acc_map(Spec::Env env, Spec::Out out, MapParams p) {
+template <bool NT>
+ACC_DEV void acc_map_body(const Spec::Env& env, const Spec::Out& out, const MapParams& p) {
   typedef Spec S;
   const int V = S::V;
 #ifdef ACC_MAP_XCD
@@ -48,15 +48,28 @@ acc_map(Spec::Env env, Spec::Out out, MapParams p) {
   if (i0 + V <= p.n) {
     S::Elt r[S::V];
 #pragma unroll
-    for (int k = 0; k < V; ++k) r[k] = S::produce(env, i0 + k);
+    for (int k = 0; k < V; ++k) r[k] = S::produce<NT>(env, i0 + k);
 #pragma unroll
-    for (int k = 0; k < V; ++k) S::store(out, i0 + k, r[k]);
+    for (int k = 0; k < V; ++k) S::store<NT>(out, i0 + k, r[k]);
   } else {
     for (int k = 0; k < V; ++k)
       if (i0 + k < p.n) S::store(out, i0 + k, S::produce(env, i0 + k));
   }
 #endif
 }
+
+extern "C" __global__ void __launch_bounds__(ACC_BLOCK)
+acc_map(Spec::Env env, Spec::Out out, MapParams p) {
+  acc_map_body<false>(env, out, p);
+}
+
+#ifndef ACC_MAP_INDEXED
+// the variant for launches that move far more than the last-level cache holds
+extern "C" __global__ void __launch_bounds__(ACC_BLOCK)
+acc_map_stream(Spec::Env env, Spec::Out out, MapParams p) {
+  acc_map_body<true>(env, out, p);
+}
+#endif
 
 // The same over two-dimensional tiles of the result: a workgroup produces 32 rows x 8*V
 // columns of the (outer dimensions flattened) x (innermost dimension) view, 8 lanes a row.

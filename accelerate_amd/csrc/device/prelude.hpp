@@ -39,6 +39,22 @@ ACC_DEV i64 acc_xcd_contiguous(i64 b, i64 nb) {
   return xcd * q + (xcd < r ? xcd : r) + k;
 }
 
+// Streaming accesses.  A launch that moves several times what the last-level cache holds
+// gains from telling the caches that an operand is touched once (the `nt` hint): map over
+// 2^28 Float32 348 -> 331 us, dotp 370 -> 340 us.  A launch whose operands fit the cache
+// loses (the next kernel finds less of them there), so the host picks the variant by size.
+// The generated functions that read at the skeleton's own linear index, and the plain
+// stores, are templates over kStream; everywhere else the name refers to this constant.
+static constexpr bool kStream = false;
+template <bool NT, class T> ACC_DEV T acc_ld(const T* p) {
+  if constexpr (NT) return __builtin_nontemporal_load(p);
+  else return *p;
+}
+template <bool NT, class T> ACC_DEV void acc_st(T* p, const T& v) {
+  if constexpr (NT) __builtin_nontemporal_store(v, p);
+  else *p = v;
+}
+
 ACC_DEV int acc_lane() { return (int)(threadIdx.x & (ACC_WAVE - 1)); }
 ACC_DEV int acc_wave() { return (int)(threadIdx.x / ACC_WAVE); }
 

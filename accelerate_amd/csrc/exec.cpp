@@ -681,6 +681,27 @@ std::vector<uint64_t> Program::packArgs(const KernelSource& ks, const AEnv& aenv
   return args;
 }
 
+static int64_t arrayBytes(const DArray& a) {
+  int64_t per = 0;
+  for (ST st : typeLeaves(a.r.elt)) per += stSize(st);
+  return a.size() * per;
+}
+
+bool Program::streams(const KernelSource& ks, const AEnv& aenv, const std::vector<DArrayP>& temps, int64_t more) {
+  if (!ks.streaming) return false;
+  // Measured on MI355X (256 MiB last-level cache): the non-temporal variants win once a launch
+  // moves more than about twice that, and lose below.
+  const char* e = std::getenv("ACCHIP_STREAM_BYTES");  // override, for tests and tuning
+  const int64_t threshold = e ? (int64_t)std::atoll(e) : (int64_t)512 << 20;
+  int64_t bytes = more;
+  for (const ArraySlot& s : ks.arrays) {
+    if (s.name == "out") continue;
+    const DArrayP& a = s.temp ? temps.at(s.index) : aenv.at(aenv.size() - 1 - s.index);
+    bytes += arrayBytes(*a);
+  }
+  return bytes >= threshold;
+}
+
 HValP Program::hostExp(const Sx& e, const AEnv& aenv, const Plan& plan) {
   auto it = plan.scalarKernels.find(&e);
   if (it == plan.scalarKernels.end()) return hostEval(e, {}, aenv);
@@ -768,7 +789,8 @@ void Program::launchMap(const KernelP& k, const AEnv& aenv, const std::vector<DA
   packOut(args, out);
   args.push_back((uint64_t)n);
   int64_t per = (int64_t)256 * k->meta.vec;
-  ctx_.launch(k, "acc_map", (unsigned)((n + per - 1) / per), 256, args);
+  const bool st = streams(k->meta, aenv, temps, arrayBytes(out));
+  ctx_.launch(k, st ? "acc_map_stream" : "acc_map", (unsigned)((n + per - 1) / per), 256, args);
 }
 
 AValP Program::evalFun(const Sx& f, AEnv& aenv, const std::vector<AValP>& args) {
@@ -1010,7 +1032,8 @@ AValP Program::eval(const Sx& n, AEnv& aenv) {
     args.push_back((uint64_t)len);
     args.push_back((uint64_t)bpr);
     args.push_back((uint64_t)chunk);
-    ctx_.launch(plan.k, "acc_fold_main", (unsigned)(rows * bpr), 256, args);
+    const bool st = streams(plan.k->meta, aenv, temps, 0);
+    ctx_.launch(plan.k, st ? "acc_fold_main_stream" : "acc_fold_main", (unsigned)(rows * bpr), 256, args);
     if (bpr > 1) ctx_.launch(plan.k, "acc_fold_final", (unsigned)rows, 256, args);
     return avArr(out);
   }

@@ -123,6 +123,9 @@ class Program {
   std::vector<uint64_t> packArgs(const KernelSource& ks, const AEnv& aenv, const std::vector<DArrayP>& temps,
                                  const std::vector<int64_t>& outShape);
   static void packOut(std::vector<uint64_t>& args, const DArray& a);
+  // does a launch of ks move so much more than the last-level cache holds that its
+  // streaming variant pays?  (the whole of every array it reads, plus `more` bytes)
+  static bool streams(const KernelSource& ks, const AEnv& aenv, const std::vector<DArrayP>& temps, int64_t more);
   void launchMap(const KernelP& k, const AEnv& aenv, const std::vector<DArrayP>& temps, DArray& out);
 };
 

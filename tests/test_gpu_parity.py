@@ -84,6 +84,28 @@ def test_folds_with_and_without_the_rows_kernel(gpu_ctx, monkeypatch, case, rows
         assert same(got, O.run_n(prog.text(), *args), exact=False, atol=last)
 
 
+ELEMENTWISE = [(c, g) for cs, g in ((GOLDEN, True), (PARITY, False)) for c in cs
+               if c[0].startswith(("map", "transpose", "gather", "identity", "issue185", "misc", "filter", "smvm",
+                                   "radix", "fold", "dotp", "mss", "issue228"))
+               and "foldseg" not in c[0]]
+
+
+@pytest.mark.parametrize("case", ELEMENTWISE, ids=[c[0][0] for c in ELEMENTWISE])
+def test_streaming_variants_of_map_and_fold(gpu_ctx, monkeypatch, case):
+    # launches that move far more than the last-level cache holds use kernels with
+    # non-temporal accesses; forced here at every size, the answers must not change
+    monkeypatch.setenv("ACCHIP_STREAM_BYTES", "0")
+    monkeypatch.setenv("ACCHIP_FOLD_ROWS", "0")
+    (_, prog, args, last), golden = case
+    got = gpu_ctx.compile(prog)(*args)
+    if golden:
+        assert same(got, last)
+    elif last is None:
+        assert same(got, O.run_n(prog.text(), *args))
+    else:
+        assert same(got, O.run_n(prog.text(), *args), exact=False, atol=last)
+
+
 # ---- the five benchmark configurations at the size the oracle's C loops handle in seconds ----
 
 def test_dotp_2pow24(gpu_ctx):
