@@ -50,6 +50,9 @@ def golden_cases():
         np.array(v["identity_permute"]["expected"], I64))
     add("transpose_backpermute", Q.transpose(), [np.array(v["transpose_backpermute"]["mat"], I64)],
         np.array(v["transpose_backpermute"]["expected"], I64))
+    for name, prog in (("scanlseg_doctest", Q.scanl_seg()), ("scanl1seg_doctest", Q.scan1_seg("l")),
+                       ("scanr1seg_doctest", Q.scan1_seg("r"))):
+        add(name, prog, [np.array(v[name]["mat"], I64), np.array(v[name]["seg"], I64)], np.array(v[name]["expected"], I64))
     t = v["issue228"]
     pair_in = [np.array(t["fst"], I64), np.array(t["snd"], I64)]
     pair_out = [np.array(t["expected"][0], I64), np.array(t["expected"][1], I64)]
@@ -195,6 +198,16 @@ def parity_cases():
     add("filter_none_pass", Q.filter_positive(), [-np.abs(_rand(rng, A.i64, (200,), -50, 50)) - 1], None)
     add("radix_4_passes", Q.radix_passes(4), [rng.integers(0, 16, 500).astype(np.int64)], None)
     add("radix_6_passes", Q.radix_passes(6), [rng.integers(0, 64, 3000).astype(np.int64)], None)
+    # ---- segmented scans (Prelude.hs:958-1322): scan', permute, a flagged scan over a fused zip
+    for shp, nseg in (((7, 900), 60), ((3, 6000), 25), ((2, 40), 0)):
+        lens = rng.integers(0, max(2, 2 * shp[1] // max(1, nseg)), nseg).astype(np.int64)
+        while lens.sum() > shp[1]:
+            lens[int(np.argmax(lens))] //= 2
+        m = _rand(rng, A.i64, shp, -20, 20)
+        if nseg:     # the inclusive scans need a non-empty segment descriptor (Prelude.hs:1107-1110)
+            add("scanl1seg_%s_%d" % (shp, nseg), Q.scan1_seg("l"), [m, lens], None)
+            add("scanr1seg_%s_%d" % (shp, nseg), Q.scan1_seg("r"), [m, lens], None)
+        add("scanlseg_%s_%d" % (shp, nseg), Q.scanl_seg(A.i64, 3), [m, lens], None)
     # ---- the benchmark programs at small size
     add("dotp_1000", P.dotp(), [_rand(rng, A.f32, (1000,)), _rand(rng, A.f32, (900,))], 1e-4 * 16 * 900)
     add("histogram_zipf", P.histogram(97), [rng.integers(0, 97, 3000).astype(np.int32)], None)

@@ -55,6 +55,17 @@ V["misc_scanl1"] = {"cite": "Test/NoFib/Misc/Scanl1.hs:32-39", "rows": 257, "col
 # Prelude.hs:689-708  foldSeg with an empty segment
 V["foldseg_doctest"] = {"cite": "Prelude.hs:689-708", "mat": iota5x10, "seg": [1, 4, 0, 3], "expected": [
     [0, 10, 0, 18], [10, 50, 0, 48], [20, 90, 0, 78], [30, 130, 0, 108], [40, 170, 0, 138]]}
+# Prelude.hs:958-991, 1117-1135, 1293-1312  segmented scans (same matrix and segments; one empty segment)
+V["scanlseg_doctest"] = {"cite": "Prelude.hs:958-978", "mat": iota5x10, "seg": [1, 4, 0, 3], "seed": 0, "expected": [
+    [0, 0, 0, 1, 3, 6, 10, 0, 0, 5, 11, 18], [0, 10, 0, 11, 23, 36, 50, 0, 0, 15, 31, 48],
+    [0, 20, 0, 21, 43, 66, 90, 0, 0, 25, 51, 78], [0, 30, 0, 31, 63, 96, 130, 0, 0, 35, 71, 108],
+    [0, 40, 0, 41, 83, 126, 170, 0, 0, 45, 91, 138]]}
+V["scanl1seg_doctest"] = {"cite": "Prelude.hs:1117-1135", "mat": iota5x10, "seg": [1, 4, 0, 3], "expected": [
+    [0, 1, 3, 6, 10, 5, 11, 18], [10, 11, 23, 36, 50, 15, 31, 48], [20, 21, 43, 66, 90, 25, 51, 78],
+    [30, 31, 63, 96, 130, 35, 71, 108], [40, 41, 83, 126, 170, 45, 91, 138]]}
+V["scanr1seg_doctest"] = {"cite": "Prelude.hs:1293-1312", "mat": iota5x10, "seg": [1, 4, 0, 3], "expected": [
+    [0, 10, 9, 7, 4, 18, 13, 7], [10, 50, 39, 27, 14, 48, 33, 17], [20, 90, 69, 47, 24, 78, 53, 27],
+    [30, 130, 99, 67, 34, 108, 73, 37], [40, 170, 129, 87, 44, 138, 93, 47]]}
 # Language.hs:716-728  histogram via permute (+)
 V["histogram_doctest"] = {"cite": "Language.hs:716-728",
                           "keys": [0, 0, 1, 2, 1, 1, 2, 4, 8, 3, 4, 9, 8, 3, 2, 5, 5, 3, 1, 2], "bins": 10,

@@ -321,3 +321,101 @@ def radix_passes(bits):
         return one_pass(keys, b, lambda moved: build(moved, b + 1))
 
     return A.alam([V1], lambda keys: build(keys, 0))
+
+
+# -- segmented scans as Prelude.hs builds them from scan', permute and a flagged scan
+#    (mkHeadFlags / mkTailFlags :1364-1389, segmentedL / segmentedR :1395-1407)
+def _seg_flags(seg_src, nseg_sh, direction, k):
+    """Head flags (left scans) or tail flags (right scans) of a segment descriptor given as an
+    operand: permute (+) zeros (\\ix -> Just (offset!ix)) ones.  k receives the array of
+    total+1 entries; `init` is left to the consumer (it reads all but the last entry)."""
+    sh1 = A.tshape(1)
+    V1, S0 = A.tarray(1, Int), A.tarray(0, Int)
+
+    def with_offsets(st):
+        offset, total = st
+        ln = lambda: A.index(total, A.nil)
+
+        def target(ix):
+            o = A.index(offset, A.vexp(ix))
+            return A.just(A.sh(o if direction == "l" else A.sub(Int, A.sub(Int, ln(), A.constI(1)), o)))
+
+        ones = A.delayed(V1, A.shape(offset), A.lam([sh1], lambda ix: A.constI(1)), A.lam([Int], lambda i: A.constI(1)))
+        zeros = A.generate(V1, A.sh(A.add(Int, ln(), A.constI(1))), A.lam([sh1], lambda ix: A.constI(0)))
+        return A.alet(V1, A.permute(binop(A.add, Int), zeros, A.lam([sh1], target), ones), k)
+
+    return A.alet(A.tpair(V1, S0), A.scan_(direction, binop(A.add, Int), A.constI(0), seg_src), with_offsets)
+
+
+def _scan1_seg(direction, ty, mat, seg_src, nseg_sh):
+    """scanl1Seg / scanr1Seg (Prelude.hs:1136-1145, 1313-1322) of a matrix operand variable:
+    map snd . scan1 (segmented f) $ zip (replicate flags) arr, the zip fused into the scan."""
+    sh2 = A.tshape(2)
+    t2 = A.ttup(Int, ty)
+
+    def seg_op(x, y):
+        # scanl1: x = running value, y = new element; scanr1: x = new element, y = running value
+        (af, av), (bf, bv) = (A.untup(x), A.untup(y)) if direction == "l" else (A.untup(y), A.untup(x))
+        f = A.add(ty, av, bv) if direction == "l" else A.add(ty, bv, av)
+        return A.tup(A.bor(Int, af, bf), A.cond(A.neq(Int, bf, A.constI(0)), bv, f))
+
+    def with_flags(fl):
+        def extent():
+            rows, cols = A.untup_shape(mat)
+            nfl = A.sub(Int, A.untup_shape(fl)[0], A.constI(1))
+            return A.sh(rows, A.min_(Int, nfl, cols))
+
+        def at(ix):
+            _, x = A.untup(ix)
+            return A.tup(A.index(fl, A.sh(x)), A.index(mat, A.vexp(ix)))
+
+        src = A.delayed(A.tarray(2, t2), extent(), A.lam([sh2], at),
+                        A.lam([Int], lambda i: A.let(sh2, A.fromindex(2, extent(), i), at)))
+        return A.map_(ty, A.lam([t2], lambda v: A.untup(v)[1]), A.scan(direction, A.lam([t2, t2], seg_op), None, src))
+
+    return _seg_flags(seg_src, nseg_sh, direction, with_flags)
+
+
+def scan1_seg(direction, ty=Int):
+    return A.alam([A.tarray(2, ty), A.tarray(1, Int)], lambda mat, seg: _scan1_seg(direction, ty, mat, seg, None))
+
+
+def scanl_seg(ty=Int, z=0):
+    """scanlSeg (Prelude.hs:979-1012): the seed is injected at the head of every segment by a
+    permute into an array of seeds, then an inclusive segmented scan over segments one longer."""
+    sh1, sh2 = A.tshape(1), A.tshape(2)
+    V1, M = A.tarray(1, Int), A.tarray(2, ty)
+
+    def body(mat, seg):
+        def with_flags(fl):
+            nflags = lambda: A.sub(Int, A.untup_shape(fl)[0], A.constI(1))
+            # (terms are built where they are used: binder levels are fixed at construction)
+            rows = lambda: A.untup_shape(mat)[0]
+            cols = lambda: A.untup_shape(mat)[1]
+            nseg = lambda: A.untup_shape(seg)[0]
+            taken_sh = lambda: A.sh(rows(), A.min_(Int, nflags(), cols()))
+            filled = lambda: A.generate(M, A.sh(rows(), A.add(Int, cols(), nseg())),
+                                        A.lam([sh2], lambda ix: A.const(ty, z)))
+            # inc = scanl1 (+) flags, with flags = init fl fused in
+            flags = A.delayed(V1, A.sh(nflags()), A.lam([sh1], lambda ix: A.index(fl, A.vexp(ix))),
+                              A.lam([Int], lambda i: A.linearindex(fl, i)))
+
+            def with_inc(inc):
+                def to(ix):
+                    y, x = A.untup(ix)
+                    return A.just(A.sh(y, A.add(Int, x, A.index(inc, A.sh(x)))))
+                # take (length flags) arr
+                taken = A.delayed(M, taken_sh(), A.lam([sh2], lambda ix: A.index(mat, A.vexp(ix))),
+                                  A.lam([Int], lambda i: A.let(sh2, A.fromindex(2, taken_sh(), i),
+                                                               lambda ix: A.index(mat, A.vexp(ix)))))
+                arr1 = A.permute(A.lam([ty, A.wild(ty)], lambda x, _: x), filled(), A.lam([sh2], to), taken)
+                seg1 = A.delayed(V1, A.shape(seg), A.lam([sh1], lambda ix: A.add(Int, A.index(seg, A.vexp(ix)), A.constI(1))),
+                                 A.lam([Int], lambda i: A.add(Int, A.linearindex(seg, i), A.constI(1))))
+                return A.alet(M, arr1, lambda a1: _scan1_seg("l", ty, a1, seg1, None))
+
+            empty = A.lor(A.eq(Int, A.mul(Int, rows(), cols()), A.constI(0)), A.eq(Int, nflags(), A.constI(0)))
+            return A.acond(empty, filled(),
+                           A.alet(V1, A.scan("l", binop(A.add, Int), None, flags), with_inc))
+        return _seg_flags(seg, None, "l", with_flags)
+
+    return A.alam([M, V1], body)

@@ -275,3 +275,24 @@ def test_oracle_on_whole_programs_against_numpy():
     assert np.array_equal(O.run_n(Q.filter_positive().text(), x), x[x > 0])
     k = rng.integers(0, 16, 500).astype(np.int64)
     assert np.array_equal(O.run_n(Q.radix_passes(4).text(), k), np.sort(k, kind="stable"))
+
+
+def test_oracle_on_segmented_scans_against_numpy():
+    # scanl1Seg / scanr1Seg / scanlSeg as Prelude.hs builds them, against per-segment cumulative
+    # sums: pins the oracle on scan', permute into generated defaults, and a scan over a fused zip
+    from . import progs as Q
+    rng = np.random.default_rng(12)
+    seg = np.array([3, 0, 5, 1, 0, 0, 7, 2], np.int64)
+    m = rng.integers(-9, 9, (4, 21)).astype(np.int64)     # 18 elements in segments, 3 beyond them
+    off = np.concatenate([[0], np.cumsum(seg)])
+    l1 = np.concatenate([np.cumsum(m[:, a:b], axis=1) for a, b in zip(off[:-1], off[1:])], axis=1)
+    r1 = np.concatenate([np.cumsum(m[:, a:b][:, ::-1], axis=1)[:, ::-1] for a, b in zip(off[:-1], off[1:])], axis=1)
+    assert np.array_equal(O.run_n(Q.scan1_seg("l").text(), m, seg), l1)
+    assert np.array_equal(O.run_n(Q.scan1_seg("r").text(), m, seg), r1)
+    z = 5
+    ex = np.concatenate([np.concatenate([np.full((4, 1), z), z + np.cumsum(m[:, a:b], axis=1)], axis=1)
+                         for a, b in zip(off[:-1], off[1:])], axis=1)
+    got = O.run_n(Q.scanl_seg(A.i64, z).text(), m, seg)
+    # the flagged scan zips with the flags of the lengthened segments: what lies beyond them is cut
+    assert got.shape == (4, int(seg.sum()) + len(seg))
+    assert np.array_equal(got, ex)
