@@ -315,6 +315,21 @@ int acchip_sha3_256(const void* data, size_t length, uint8_t digest[32]) {
   ACCHIP_END
 }
 
+int acchip_set_trace(acchip_ctx* ctx, acchip_trace_fn fn, void* user) {
+  ACCHIP_TRY
+  if (!fn) {
+    ctx->ctx->traceSink = nullptr;
+  } else {
+    ctx->ctx->traceSink = [fn, user](const std::string& msg, const std::shared_ptr<void>& arrays) {
+      acchip_array* h = wrapVal(std::static_pointer_cast<AVal>(arrays));
+      fn(user, msg.c_str(), h);
+      delete h;
+    };
+  }
+  return ACCHIP_OK;
+  ACCHIP_END
+}
+
 int acchip_execute(acchip_ctx* ctx, acchip_program* p, acchip_array* const* args, int n_args,
                    acchip_array* const* uses, int n_uses, acchip_array** result) {
   ACCHIP_TRY

@@ -432,6 +432,15 @@ ATyP Program::prepare(const Sx& n, TEnv& tenv) {
     prepare(n.at(2), tenv);
     return prepareFun(n.at(1), tenv, nullptr);
   }
+  if (h == "atrace") {  // (atrace hex-of-message as bs): Interpreter.hs:215
+    prepare(n.at(2), tenv);
+    return prepare(n.at(3), tenv);
+  }
+  if (h == "aforeign") {  // (aforeign hex-of-name afun acc): the pure fallback, closed (Interpreter.hs:217)
+    prepare(n.at(3), tenv);
+    TEnv empty;
+    return prepareFun(n.at(2), empty, nullptr);
+  }
   if (h == "acond") {
     Plan& plan = plans_[&n];
     prepareHostExp(n.at(1), tenv, plan);
@@ -681,6 +690,21 @@ std::vector<uint64_t> Program::packArgs(const KernelSource& ks, const AEnv& aenv
   return args;
 }
 
+// text carried as the hexadecimal digits of its bytes ("-" for the empty string)
+static std::string unhex(const std::string& h) {
+  std::string out;
+  if (h == "-") return out;
+  if (h.size() % 2) throw Error("malformed hexadecimal text '" + h + "'");
+  auto nib = [&](char c) -> int {
+    if (c >= '0' && c <= '9') return c - '0';
+    if (c >= 'a' && c <= 'f') return c - 'a' + 10;
+    if (c >= 'A' && c <= 'F') return c - 'A' + 10;
+    throw Error("malformed hexadecimal text '" + h + "'");
+  };
+  for (size_t i = 0; i < h.size(); i += 2) out.push_back((char)(nib(h[i]) * 16 + nib(h[i + 1])));
+  return out;
+}
+
 static int64_t arrayBytes(const DArray& a) {
   int64_t per = 0;
   for (ST st : typeLeaves(a.r.elt)) per += stSize(st);
@@ -840,6 +864,38 @@ AValP Program::eval(const Sx& n, AEnv& aenv) {
   if (h == "apply") {
     AValP a = eval(n.at(2), aenv);
     return evalFun(n.at(1), aenv, {a});
+  }
+  if (h == "atrace") {
+    // evaluate the traced arrays, hand them over complete, then go on with the body
+    AValP traced = eval(n.at(2), aenv);
+    materializeAll(traced);
+    ctx_.sync();
+    const std::string msg = unhex(n.at(1).str());
+    if (ctx_.traceSink) {
+      ctx_.traceSink(msg, traced);
+    } else {
+      std::string line = msg;
+      std::function<void(const AValP&)> show = [&](const AValP& v) {
+        if (v->k == AVal::Pair) {
+          show(v->a);
+          show(v->b);
+        } else if (v->k == AVal::Arr) {
+          line += line.size() > msg.size() ? ", " : ": ";
+          line += "Array (Z";
+          for (int64_t d : v->arr->shape) line += " :. " + std::to_string(d);
+          line += ") " + typeStr(v->arr->r.elt);
+        }
+      };
+      show(traced);
+      std::fprintf(stderr, "%s\n", line.c_str());
+      std::fflush(stderr);
+    }
+    return eval(n.at(3), aenv);
+  }
+  if (h == "aforeign") {
+    AValP a = eval(n.at(3), aenv);
+    AEnv closed;
+    return evalFun(n.at(2), closed, {a});
   }
   if (h == "acond") {
     const Plan& plan = plans_.at(&n);

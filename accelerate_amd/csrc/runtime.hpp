@@ -5,6 +5,7 @@
 
 #include <atomic>
 #include <condition_variable>
+#include <functional>
 #include <future>
 #include <map>
 #include <memory>
@@ -67,6 +68,10 @@ class Context : public std::enable_shared_from_this<Context> {
   KernelP kernel(const KernelSource& ks);
   void wait(const KernelP& k);
   void launch(const KernelP& k, const char* fn, unsigned grid, unsigned block, const std::vector<uint64_t>& args);
+
+  // Where Atrace nodes deliver their message and the arrays they were given (the C ABI
+  // installs the caller's callback here; the value is an AVal); empty: a line on stderr.
+  std::function<void(const std::string& msg, const std::shared_ptr<void>& arrays)> traceSink;
 
   // persistent device scratch for single-pass scans (tile descriptors + ticket counter)
   struct ScanState {

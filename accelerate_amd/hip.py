@@ -78,6 +78,7 @@ def lib():
         "acchip_program_arity": (C.c_int, [vp]),
         "acchip_program_num_kernels": (C.c_int, [vp]),
         "acchip_sha3_256": (C.c_int, [vp, C.c_size_t, C.c_char_p]),
+        "acchip_set_trace": (C.c_int, [vp, vp, vp]),
         "acchip_execute": (C.c_int, [vp, vp, C.POINTER(vp), C.c_int, C.POINTER(vp), C.c_int, C.POINTER(vp)]),
     }
     for name, (res, args) in sigs.items():
@@ -111,6 +112,9 @@ def _parse_type(text):
     return rd(0)[0]
 
 
+TRACE_FN = C.CFUNCTYPE(None, C.c_void_p, C.c_char_p, C.c_void_p)
+
+
 class Context:
     """One device, one stream, one memory pool, one kernel cache (acchip_init)."""
 
@@ -129,6 +133,24 @@ class Context:
             self.close()
         except Exception:
             pass
+
+    def set_trace(self, fn):
+        """fn(message, arrays) receives what Atrace nodes report (arrays already copied to the
+        host); None restores the default, a line on stderr."""
+        if fn is None:
+            self._trace_cb = None
+            _check(lib().acchip_set_trace(self._h, None, None))
+            return
+
+        def cb(_user, msg, handle):
+            view = DeviceArray(self, C.c_void_p(handle))
+            try:
+                fn(msg.decode(errors="replace"), view.to_host())
+            finally:
+                view._h = C.c_void_p()     # the library owns the handle
+
+        self._trace_cb = TRACE_FN(cb)      # keep the thunk alive while it is installed
+        _check(lib().acchip_set_trace(self._h, C.cast(self._trace_cb, C.c_void_p), None))
 
     # memory --------------------------------------------------------------------------
     def mem_info(self):

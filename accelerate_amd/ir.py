@@ -509,6 +509,31 @@ def apply(afun, acc):
     return Raw("apply", afun, acc)
 
 
+def _hex(text):
+    return text.encode().hex() or "-"
+
+
+def atrace(msg, traced, body):
+    """Atrace msg traced body (AST.hs Atrace; evaluated as Interpreter.hs:215)."""
+    return Raw("atrace", _hex(msg), traced, body)
+
+
+class _Closed(Node):
+    """A closed term (built outside every binder): rendered in an empty environment."""
+
+    def __init__(self, term):
+        self.term = term
+
+    def sx(self, d, ad):
+        return self.term.sx(0, 0)
+
+
+def aforeign(name, afun, acc):
+    """Aforeign with its pure fallback afun, a closed array function built outside every
+    binder (Interpreter.hs:217 evaluates it in the empty environment)."""
+    return Raw("aforeign", _hex(name), _Closed(afun), acc)
+
+
 def acond(e, a1, a2):
     return Raw("acond", e, a1, a2)
 

@@ -130,6 +130,15 @@ int acchip_program_num_kernels(const acchip_program* p);
  * Crypto.Hash.XKCP (src/Crypto/Hash/XKCP.hs:93-170, cbits/xkcp SHA3_256). */
 int acchip_sha3_256(const void* data, size_t length, uint8_t digest[32]);
 
+/* Atrace nodes (`atraceArray` and friends; Interpreter.hs:215, atraceOp :873-880): the
+ * traced arrays are evaluated, the stream is synchronised, and the callback receives the
+ * message and a handle to the arrays (a tuple handle for several), valid during the call
+ * only, so that the caller can print them with its own Show instances; then the body
+ * runs.  Without a callback (fn = NULL, the default) one line with the message and the
+ * arrays' shapes goes to stderr. */
+typedef void (*acchip_trace_fn)(void* user, const char* message, acchip_array* arrays);
+int acchip_set_trace(acchip_ctx* ctx, acchip_trace_fn fn, void* user);
+
 /* Apply a prepared function to device-resident arguments (the `go` closure returned by
  * runN, Interpreter.hs:118-126): args[i] is the i-th lambda's argument; uses[k] fills
  * `(use .. k)` nodes.  All work is queued on the context's stream; the result handle may

@@ -44,6 +44,9 @@ class OracleError(Exception):
 # --------------------------------------------------------------------------------------
 # reader
 
+TRACE = []   # (message, traced arrays) of every Atrace node evaluated, in order
+
+
 def parse(text):
     toks = text.replace("(", " ( ").replace(")", " ) ").split()
     pos = 0
@@ -577,6 +580,12 @@ def eval_acc(a, aenv, uses):
         return (x, man(a[2]))
     if k == "apply":
         return eval_afun(a[1], aenv, uses)(man(a[2]))
+    if k == "atrace":       # Interpreter.hs:215: evaluate the traced arrays, report, then the body
+        traced = man(a[2])
+        TRACE.append(("" if a[1] == "-" else bytes.fromhex(a[1]).decode(), traced))
+        return man(a[3])
+    if k == "aforeign":     # Interpreter.hs:217: the pure fallback in an empty environment
+        return eval_afun(a[2], (), uses)(man(a[3]))
     if k == "acond":
         return man(a[2]) if evE(a[1]) != 0 else man(a[3])
     if k == "awhile":

@@ -112,6 +112,18 @@ def runtime_cases():
             [A.tshape(2)], lambda ix: A.add(Int, A.mul(Int, A.untup(ix)[0], A.constI(100)), A.untup(ix)[1])))
     add("generate_dynamic_extent", A.alam([A.tarray(0, Int)], iota), [np.array(7, np.int64)], [])
 
+    # atrace: the traced arrays are evaluated and reported, the result is the body's
+    def traced(xs):
+        return A.atrace("partial sums", A.apair(A.scan("l", Q.binop(A.add, Int), None, xs), A.unit_(Int, A.constI(7))),
+                        A.map_(Int, A.lam([Int], lambda v: A.add(Int, v, A.constI(1))), xs))
+    add("atrace_reports_then_continues", A.alam([V(Int)], traced), [x], [])
+
+    # aforeign: no foreign implementation for this backend, so the pure fallback runs -- a closed
+    # function applied to the evaluated argument (a fold nested under it, an outer variable unused)
+    fallback = A.alam([V(Int)], lambda a: A.map_(Int, A.lam([Int], lambda v: A.mul(Int, v, A.constI(3))), a))
+    add("aforeign_runs_the_fallback", A.alam([V(Int), V(Int)], lambda xs, ys: A.aforeign(
+        "cublas_saxpy", fallback, A.zipwith(Int, Q.binop(A.add, Int), xs, ys))), [x, y], [])
+
     # permute whose defaults are a variable: the caller's array must not change
     sh1 = A.tshape(1)
     keep = A.alam([V(Int), V(Int)], lambda src, dfl: A.apair(

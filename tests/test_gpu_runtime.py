@@ -26,6 +26,25 @@ def test_control_flow_matches_oracle(gpu_ctx, case):
     assert same(got, exp)
 
 
+def test_atrace_hands_message_and_arrays_to_the_callback(gpu_ctx, capfd):
+    # Atrace (Interpreter.hs:215, atraceOp :873-880): the callback sees the message and the
+    # evaluated arrays before the body's result comes back; without one, a line on stderr
+    case = [c for c in CASES if c[0] == "atrace_reports_then_continues"][0]
+    _, prog, args, _ = case
+    run = gpu_ctx.compile(prog)
+    seen = []
+    gpu_ctx.set_trace(lambda msg, arrays: seen.append((msg, arrays)))
+    try:
+        got = run(*args)
+    finally:
+        gpu_ctx.set_trace(None)
+    assert same(got, args[0] + 1)
+    assert len(seen) == 1 and seen[0][0] == "partial sums"
+    assert same(seen[0][1], (np.cumsum(args[0]), np.array(7, np.int64)))
+    run(*args)
+    assert "partial sums: Array (Z :. 500) i64, Array (Z) i64" in capfd.readouterr().err
+
+
 def test_awhile_jacobi_counts_iterations(gpu_ctx):
     # 20 sweeps driven by awhile (Interpreter.hs:222-229).  The loop counter is a rank-0
     # array made by `unit` from index arithmetic, so the host follows its value and the
