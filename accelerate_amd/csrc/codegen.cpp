@@ -297,6 +297,8 @@ ValP Codegen::prim(const std::string& name, const std::vector<ST>& tys, const Va
   auto needFloat = [&](ST t) {
     if (!stIsFloat(t)) throw Error("primitive '" + name + "' needs a floating type");
   };
+  for (ST ty : tys)
+    if (stIsVec(ty)) throw Error("primitive '" + name + "' applied at a SIMD vector type");
   const ST t = tys.empty() ? ST::U8 : tys[0];
   const std::string bits = std::to_string(stBits(t));
   const std::string U = T(stUnsigned(t));
@@ -523,11 +525,43 @@ ValP Codegen::exp(const Sx& e, const Env& env, Emit& em) {
   }
   if (h == "const") {
     ST t = parseST(e.at(1));
+    if (stIsVec(t)) {  // (const v<n><t> (lit ..))
+      const Sx& ls = e.at(2);
+      if (ls.atom || (int)ls.size() != stWidth(t)) throw Error("vector constant needs one literal per component");
+      std::string x = std::string(stName(t)) + "{{";
+      for (int k = 0; k < stWidth(t); ++k) x += (k ? ", " : "") + literalText(stBase(t), ls.at(k).s);
+      return vLeaf(t, x + "}}");
+    }
     return vLeaf(t, literalText(t, e.at(2).s));
   }
   if (h == "undef") {
     ST t = parseST(e.at(1));
+    if (stIsVec(t)) return vLeaf(t, std::string(stName(t)) + "{}");
     return vLeaf(t, literalText(t, "0"));
+  }
+  if (h == "vecpack" || h == "vecunpack") {  // (vecpack N T e) / (vecunpack N T e): Interpreter.hs:942-943
+    const int w = (int)e.at(1).asInt();
+    const ST base = parseST(e.at(2));
+    if (!stVecWidthOk(w) || stIsVec(base)) throw Error("malformed vector type in " + h);
+    const ST vt = stVec(base, w);
+    ValP v = exp(e.at(3), env, em);
+    if (h == "vecpack") {
+      std::vector<ValP> parts;
+      valLeaves(v, parts);
+      if ((int)parts.size() != w) throw Error("vecpack: expected a tuple of " + std::to_string(w) + " components");
+      std::string x = std::string(stName(vt)) + "{{";
+      for (int k = 0; k < w; ++k) {
+        if (parts[k]->st != base) throw Error("vecpack: component type does not match the vector type");
+        x += (k ? ", " : "") + parts[k]->ex;
+      }
+      return bindLeaf(vt, x + "}}", em);
+    }
+    ValP l = leaf1(v, "vecunpack");
+    if (l->st != vt) throw Error("vecunpack: operand is not of the stated vector type");
+    ValP l2 = bindLeaf(vt, l->ex, em);  // a name, so that components can be selected
+    ValP out = vUnit();
+    for (int k = 0; k < w; ++k) out = vPair(out, bindLeaf(base, l2->ex + ".e[" + std::to_string(k) + "]", em));
+    return out;
   }
   if (h == "minbound" || h == "maxbound") {
     ST t = parseST(e.at(1));
@@ -894,8 +928,8 @@ static void structLayout(const std::vector<ST>& leaves, int& size, int& align) {
   int off = 0;
   align = 1;
   for (ST s : leaves) {
-    int a = stSize(s);
-    off = (off + a - 1) / a * a + a;
+    int a = stAlign(s);
+    off = (off + a - 1) / a * a + stSize(s);
     align = std::max(align, a);
   }
   if (off == 0) off = 1;
@@ -1211,7 +1245,7 @@ KernelSource Codegen::permute(const Sx& f, const ArrayR& dst, const Sx& p, const
   std::string mode = "lock", op;
   ST st = ST::I32;
   const bool single = leaves.size() == 1;
-  const bool wide = single && (stSize(leaves[0]) == 4 || stSize(leaves[0]) == 8);
+  const bool wide = single && !stIsVec(leaves[0]) && (stSize(leaves[0]) == 4 || stSize(leaves[0]) == 8);
   if (ignoresSecond(f)) mode = "store";
   else if (wide && isCommutative(f, &op, &st) && st == leaves[0] &&
            (op == "add" ? (st != ST::F16) : (op != "mul" && stIsInt(st))))
@@ -1256,11 +1290,21 @@ KernelSource Codegen::permute(const Sx& f, const ArrayR& dst, const Sx& p, const
     // lanes of one wave with the same destination then never finish.
     u += "    u32* lk_ = locks + j;\n    bool done_ = false;\n    while (__ballot(!done_) != 0ull) {\n";
     u += "      if (!done_ && __hip_atomic_exchange(lk_, 1u, __ATOMIC_ACQUIRE, __HIP_MEMORY_SCOPE_AGENT) == 0u) {\n        Elt y_;\n";
+    // leaf by leaf (component by component for SIMD vector leaves) through relaxed atomics
+    auto each = [&](size_t k, const std::function<void(const std::string& cell, const std::string& field)>& fn) {
+      const std::string cell = "out.o" + std::to_string(k) + "[j]", field = ".c" + std::to_string(k);
+      if (!stIsVec(leaves[k])) return fn(cell, field);
+      for (int m = 0; m < stWidth(leaves[k]); ++m) fn(cell + ".e[" + std::to_string(m) + "]", field + ".e[" + std::to_string(m) + "]");
+    };
     for (size_t k = 0; k < leaves.size(); ++k)
-      u += "        y_.c" + std::to_string(k) + " = __hip_atomic_load(&out.o" + std::to_string(k) + "[j], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);\n";
+      each(k, [&](const std::string& cell, const std::string& field) {
+        u += "        y_" + field + " = __hip_atomic_load(&" + cell + ", __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);\n";
+      });
     u += "        Elt r_ = combine(env, x, y_);\n";
     for (size_t k = 0; k < leaves.size(); ++k)
-      u += "        __hip_atomic_store(&out.o" + std::to_string(k) + "[j], r_.c" + std::to_string(k) + ", __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);\n";
+      each(k, [&](const std::string& cell, const std::string& field) {
+        u += "        __hip_atomic_store(&" + cell + ", r_" + field + ", __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);\n";
+      });
     u += "        __hip_atomic_store(lk_, 0u, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_AGENT);\n        done_ = true;\n      }\n    }\n";
   }
   u += "  }\n" + lds;

@@ -14,6 +14,15 @@ typedef _Float16 f16;
 typedef float f32;
 typedef double f64;
 
+// SIMD vector element types Vec n t: n components side by side, aligned like one of them
+template <class T, int N> struct acc_vec { T e[N]; };
+#define ACC_VEC_TYPES(T)                                                                          \
+  typedef acc_vec<T, 2> v2##T; typedef acc_vec<T, 3> v3##T; typedef acc_vec<T, 4> v4##T;           \
+  typedef acc_vec<T, 8> v8##T; typedef acc_vec<T, 16> v16##T;
+ACC_VEC_TYPES(i8) ACC_VEC_TYPES(i16) ACC_VEC_TYPES(i32) ACC_VEC_TYPES(i64)
+ACC_VEC_TYPES(u8) ACC_VEC_TYPES(u16) ACC_VEC_TYPES(u32) ACC_VEC_TYPES(u64)
+ACC_VEC_TYPES(f16) ACC_VEC_TYPES(f32) ACC_VEC_TYPES(f64)
+
 #define ACC_DEV static __device__ __forceinline__
 #define ACC_WAVE 64
 #define ACC_BLOCK 256
@@ -53,6 +62,17 @@ template <bool NT, class T> ACC_DEV T acc_ld(const T* p) {
 template <bool NT, class T> ACC_DEV void acc_st(T* p, const T& v) {
   if constexpr (NT) __builtin_nontemporal_store(v, p);
   else *p = v;
+}
+
+template <bool NT, class T, int N> ACC_DEV acc_vec<T, N> acc_ld(const acc_vec<T, N>* p) {
+  acc_vec<T, N> r;
+#pragma unroll
+  for (int k = 0; k < N; ++k) r.e[k] = acc_ld<NT>(&p->e[k]);
+  return r;
+}
+template <bool NT, class T, int N> ACC_DEV void acc_st(acc_vec<T, N>* p, const acc_vec<T, N>& v) {
+#pragma unroll
+  for (int k = 0; k < N; ++k) acc_st<NT>(&p->e[k], v.e[k]);
 }
 
 ACC_DEV int acc_lane() { return (int)(threadIdx.x & (ACC_WAVE - 1)); }

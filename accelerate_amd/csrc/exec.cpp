@@ -559,7 +559,13 @@ ATyP Program::prepare(const Sx& n, TEnv& tenv) {
       srcs.push_back(operandOf(n.at(8), cg, tenv, plan));
       if (srcs[0].r.rank != srcs[1].r.rank) throw Error("stencil2: operands of different rank");
     }
-    if (!two && srcs[0].r.rank == 2) {
+    // the LDS-tiled skeletons move 32-bit and 128-bit words; SIMD vector leaves go the generic way
+    bool simd = false;
+    for (ST st : typeLeaves(outElt)) simd = simd || stIsVec(st);
+    for (ST st : typeLeaves(srcs[0].r.elt)) simd = simd || stIsVec(st);
+    if (simd) {
+      plan.k = ctx_.kernel(cg.stencil(pats, outElt, *f, bnds, srcs));
+    } else if (!two && srcs[0].r.rank == 2) {
       plan.k = ctx_.kernel(cg.stencil2d(pats[0], outElt, *f, bnds[0], srcs[0]));
       plan.mode = "lds2d";
     } else if (!two && srcs[0].r.rank == 3 && !std::getenv("ACCHIP_STENCIL_NO3D")) {
@@ -752,6 +758,7 @@ HValP Program::hostExp(const Sx& e, const AEnv& aenv, const Plan& plan) {
   for (size_t i = 0; i < out->bufs.size(); ++i) {
     ST st = k->meta.outLeaves[i];
     unsigned char raw[8] = {0};
+    if (stIsVec(st)) throw Error("a SIMD vector value cannot be read back as a host scalar");
     ctx_.peek(raw, out->bufs[i]->p, stSize(st));
     auto v = std::make_shared<HVal>();
     v->k = HVal::Leaf;

@@ -11,34 +11,66 @@ namespace acchip {
 
 enum class ST : int { I8, I16, I32, I64, U8, U16, U32, U64, F16, F32, F64 };
 
+// SIMD vector types `Vec n t` (Type.hs VectorType; n in 2, 3, 4, 8, 16), written v<n><t>:
+// one leaf whose n components are stored next to each other, n*size(t) bytes per element
+// with the alignment of t (Array/Data.hs:119, 190: a buffer of w * size scalars).  Encoded
+// in ST as base | n << 8.
+inline int stWidth(ST t) { return ((int)t >> 8) ? ((int)t >> 8) : 1; }
+inline ST stBase(ST t) { return (ST)((int)t & 0xff); }
+inline bool stIsVec(ST t) { return ((int)t >> 8) != 0; }
+inline ST stVec(ST base, int n) { return (ST)((int)base | (n << 8)); }
+inline bool stVecWidthOk(int n) { return n == 2 || n == 3 || n == 4 || n == 8 || n == 16; }
+
 inline const char* stName(ST t) {
   static const char* n[] = {"i8", "i16", "i32", "i64", "u8", "u16", "u32", "u64", "f16", "f32", "f64"};
-  return n[(int)t];
+  if (!stIsVec(t)) return n[(int)t];
+  static const std::vector<std::string> names = [] {
+    std::vector<std::string> v(17 * 16);
+    for (int w = 2; w <= 16; ++w)
+      for (int b = 0; b < 11; ++b) v[w * 16 + b] = "v" + std::to_string(w) + n[b];
+    return v;
+  }();
+  return names[stWidth(t) * 16 + (int)stBase(t)].c_str();
 }
-inline int stSize(ST t) {
+inline int stAlign(ST t) {
   static const int n[] = {1, 2, 4, 8, 1, 2, 4, 8, 2, 4, 8};
-  return n[(int)t];
+  return n[(int)stBase(t)];
 }
+inline int stSize(ST t) { return stAlign(t) * stWidth(t); }
 inline int stBits(ST t) { return stSize(t) * 8; }
 inline bool stIsFloat(ST t) { return t == ST::F16 || t == ST::F32 || t == ST::F64; }
 inline bool stIsSigned(ST t) { return (int)t <= (int)ST::I64; }
-inline bool stIsInt(ST t) { return !stIsFloat(t); }
+inline bool stIsInt(ST t) { return !stIsVec(t) && !stIsFloat(t); }
 inline ST stUnsigned(ST t) { return stIsSigned(t) ? (ST)((int)t + 4) : t; }
 // type the wrap-around arithmetic of an integer type is carried out in
 inline const char* stWide(ST t) { return stSize(t) == 8 ? "u64" : "u32"; }
 
-inline ST parseST(const Sx& s) {
-  if (s.atom) {
-    for (int i = 0; i <= (int)ST::F64; ++i)
-      if (s.s == stName((ST)i)) return (ST)i;
+inline bool parseSTName(const std::string& s, ST& out) {
+  for (int i = 0; i <= (int)ST::F64; ++i)
+    if (s == stName((ST)i)) {
+      out = (ST)i;
+      return true;
+    }
+  if (s.size() >= 4 && s[0] == 'v' && s[1] >= '1' && s[1] <= '9') {
+    size_t p = 1;
+    int w = 0;
+    while (p < s.size() && s[p] >= '0' && s[p] <= '9' && w < 100) w = w * 10 + (s[p++] - '0');
+    ST base;
+    if (stVecWidthOk(w) && parseSTName(s.substr(p), base) && !stIsVec(base)) {
+      out = stVec(base, w);
+      return true;
+    }
   }
+  return false;
+}
+inline ST parseST(const Sx& s) {
+  ST t;
+  if (s.atom && parseSTName(s.s, t)) return t;
   throw Error("unknown scalar type '" + s.str() + "'");
 }
 inline bool isST(const Sx& s) {
-  if (!s.atom) return false;
-  for (int i = 0; i <= (int)ST::F64; ++i)
-    if (s.s == stName((ST)i)) return true;
-  return false;
+  ST t;
+  return s.atom && parseSTName(s.s, t);
 }
 
 struct Type;

@@ -184,8 +184,10 @@ class Context:
         parts = list(data) if isinstance(data, (list, tuple)) else [data]
         if len(parts) != len(lv):
             raise ValueError("one numpy array per scalar leaf of the element type")
-        parts = [np.asarray(p, dtype=NP[t], order="C") for p, t in zip(parts, lv)]  # keeps rank 0
-        shape = parts[0].shape if parts else ()
+        # a SIMD vector leaf carries its components in one more, innermost numpy dimension
+        vecs = [ir.vec_of(t) for t in lv]
+        parts = [np.asarray(p, dtype=NP[v[1] if v else t], order="C") for p, t, v in zip(parts, lv, vecs)]  # keeps rank 0
+        shape = (parts[0].shape[:-1] if vecs[0] else parts[0].shape) if parts else ()
         if len(shape) != rank:
             raise ValueError("array of rank %d passed where rank %d is declared" % (len(shape), rank))
         h = C.c_void_p()
@@ -265,7 +267,8 @@ class DeviceArray:
         shape = self.shape
         outs = []
         for i, t in enumerate(ir.tleaves(self.elt_type)):
-            out = np.empty(shape, NP[t])
+            v = ir.vec_of(t)
+            out = np.empty(tuple(shape) + (v[0],), NP[v[1]]) if v else np.empty(shape, NP[t])
             if out.nbytes:
                 _check(lib().acchip_peek(self.ctx._h, out.ctypes.data, lib().acchip_array_buffer(self._h, i), out.nbytes))
             outs.append(out)

@@ -13,7 +13,8 @@ reference's own tests do; it contains no evaluation logic.
 Grammar (atoms are bare words; every list starts with its constructor name):
 
   scalar type   i8 i16 i32 i64 u8 u16 u32 u64 f16 f32 f64   (Int = i64, Word = u64,
-                PrimBool / TAG = u8, ``Type.hs:112-152``)
+                PrimBool / TAG = u8, ``Type.hs:112-152``) | v<N><SCALAR> for the SIMD
+                vector `Vec N t`, N in 2 3 4 8 16 (one leaf, components side by side)
   tuple type    unit | SCALAR | (pair T T)
   array type    (array RANK T)          arrays type  unit | ARRAY | (pair AS AS)
   lhs           (single T) | (wild T) | (pair LHS LHS)        (``AST/LeftHandSide.hs``)
@@ -23,7 +24,7 @@ Grammar (atoms are bare words; every list starts with its constructor name):
        (fromindex RANK sh i) (indexslice SLICE slix sh) (indexfull SLICE slix sl)
        (case e ((TAG e)..) DEFAULT|none) (cond e e e) (while FUN FUN e)
        (index A ix) (linearindex A i) (shape A) (shapesize RANK sh)
-       (coerce T T e) (foreign FUN e)
+       (coerce T T e) (foreign FUN e) (vecpack N SCALAR e) (vecunpack N SCALAR e)
   fun  (lam LHS fun) | exp
   acc  (avar I) (alet ALHS acc acc) (apair acc acc) anil (apply AFUN acc)
        (acond exp acc acc) (awhile AFUN AFUN acc) (use ARRAY SLOT) (unit T exp)
@@ -54,6 +55,23 @@ unit = "unit"
 
 INTEGRAL = ("i8", "i16", "i32", "i64", "u8", "u16", "u32", "u64")
 FLOATING = ("f16", "f32", "f64")
+
+
+def tvec(n, t):
+    """SIMD vector type `Vec n t` (n in 2, 3, 4, 8, 16), one scalar leaf written v<n><t>."""
+    assert n in (2, 3, 4, 8, 16) and t in SCALARS
+    return "v%d%s" % (n, t)
+
+
+def vec_of(t):
+    """'v3i32' -> (3, 'i32'), anything else -> None."""
+    if isinstance(t, str) and t[0] == "v":
+        k = 1
+        while k < len(t) and t[k].isdigit():
+            k += 1
+        if 1 < k < len(t) and t[k:] in SCALARS:
+            return int(t[1:k]), t[k:]
+    return None
 
 
 def tpair(a, b):
@@ -442,6 +460,16 @@ def untup_shape(av):
 
 def shapesize(rank, sh_):
     return Raw("shapesize", rank, sh_)
+
+
+def vecpack(n, t, e):
+    """VecPack: a tuple of n components of type t -> Vec n t  (Interpreter.hs:942)."""
+    return Raw("vecpack", n, t, e)
+
+
+def vecunpack(n, t, e):
+    """VecUnpack: Vec n t -> the tuple of its components  (Interpreter.hs:943)."""
+    return Raw("vecunpack", n, t, e)
 
 
 def coerce(t1, t2, e):

@@ -37,6 +37,24 @@ NP = {"i8": np.int8, "i16": np.int16, "i32": np.int32, "i64": np.int64,
 FLOATS = ("f16", "f32", "f64")
 
 
+def vec_of(ty):
+    """'v3i32' -> (3, 'i32') for a SIMD vector type `Vec n t`, else None.  A vector value is a
+    Python tuple of its components; its buffer holds them side by side (Array/Data.hs:119,190)."""
+    if isinstance(ty, str) and ty[0] == "v":
+        k = 1
+        while k < len(ty) and ty[k].isdigit():
+            k += 1
+        if 1 < k < len(ty) and ty[k:] in NP and int(ty[1:k]) in (2, 3, 4, 8, 16):
+            return int(ty[1:k]), ty[k:]
+    return None
+
+
+def _scalar_out(ty, v):
+    if ty in INT_BITS:
+        return int(v)
+    return float(v) if ty == "f64" else v
+
+
 class OracleError(Exception):
     """A condition the reference reports through boundsCheck / internalError."""
 
@@ -344,7 +362,8 @@ class Arr:
     def __init__(self, sh, ty, bufs=None):
         self.sh, self.ty = sh, ty
         n = size(sh)
-        self.bufs = bufs if bufs is not None else [np.zeros(n, NP[t]) for t in leaves(ty)]
+        self.bufs = bufs if bufs is not None else [
+            np.zeros((n, vec_of(t)[0]), NP[vec_of(t)[1]]) if vec_of(t) else np.zeros(n, NP[t]) for t in leaves(ty)]
 
     def read(self, i):
         it = iter(self.bufs)
@@ -354,9 +373,9 @@ class Arr:
                 return ()
             if isinstance(ty, str):
                 v = next(it)[i]
-                if ty in INT_BITS:
-                    return int(v)
-                return float(v) if ty == "f64" else v
+                if vec_of(ty):
+                    return tuple(_scalar_out(vec_of(ty)[1], x) for x in v)
+                return _scalar_out(ty, v)
             a = go(ty[1])
             return (a, go(ty[2]))
         return go(self.ty)
@@ -469,9 +488,25 @@ def eval_exp(e, env, aenv):
         a = ev(e[1])
         return (a, ev(e[2]))
     if k == "const":
+        if vec_of(e[1]):
+            return tuple(literal(vec_of(e[1])[1], t) for t in e[2])
         return literal(e[1], e[2])
     if k == "undef":
+        if vec_of(e[1]):
+            return tuple(literal(vec_of(e[1])[1], "0") for _ in range(vec_of(e[1])[0]))
         return literal(e[1], "0")
+    if k == "vecpack":       # Interpreter.hs:942: the tuple (((), a), b) .. becomes one vector value
+        parts, v = [], ev(e[3])
+        while v != ():
+            v, x = v
+            parts.append(x)
+        assert len(parts) == int(e[1])
+        return tuple(parts[::-1])
+    if k == "vecunpack":     # Interpreter.hs:943
+        out = ()
+        for x in ev(e[3]):
+            out = (out, x)
+        return out
     if k == "minbound":
         b = INT_BITS[e[1]]
         return -(1 << (b - 1)) if e[1][0] == "i" else 0
@@ -801,13 +836,22 @@ def to_arr(a, aty):
     lv = leaves(ty)
     parts = [a] if not isinstance(a, (list, tuple)) else list(a)
     assert len(parts) == len(lv), "one buffer per scalar leaf"
-    shp = sh_of([int(x) for x in np.asarray(parts[0]).shape]) if lv else sh_of(a)
-    return Arr(shp, ty, [np.ascontiguousarray(p, NP[t]).reshape(-1).copy() for p, t in zip(parts, lv)])
+    if lv:      # a vector leaf carries its components in one more, innermost numpy dimension
+        dims = [int(x) for x in np.asarray(parts[0]).shape]
+        shp = sh_of(dims[:-1] if vec_of(lv[0]) else dims)
+    else:
+        shp = sh_of(a)
+    bufs = []
+    for p, t in zip(parts, lv):
+        v = vec_of(t)
+        bufs.append(np.ascontiguousarray(p, NP[v[1]]).reshape(-1, v[0]).copy() if v
+                    else np.ascontiguousarray(p, NP[t]).reshape(-1).copy())
+    return Arr(shp, ty, bufs)
 
 
 def from_arr(arr):
     dims = sh_list(arr.sh)
-    outs = [b.reshape(dims) for b in arr.bufs]
+    outs = [b.reshape(dims + [vec_of(t)[0]] if vec_of(t) else dims) for b, t in zip(arr.bufs, leaves(arr.ty))]
     return outs[0] if len(outs) == 1 else outs
 
 

@@ -208,6 +208,26 @@ def parity_cases():
             add("scanl1seg_%s_%d" % (shp, nseg), Q.scan1_seg("l"), [m, lens], None)
             add("scanr1seg_%s_%d" % (shp, nseg), Q.scan1_seg("r"), [m, lens], None)
         add("scanlseg_%s_%d" % (shp, nseg), Q.scanl_seg(A.i64, 3), [m, lens], None)
+    # ---- SIMD vector element types (Prelude/SIMD.hs:40-190): extract and inject for every base type
+    #      and width, then vectors as the elements of scans, folds, permute, backpermute, stencil
+    for k, ty in enumerate((A.i8, A.i16, A.i32, A.i64, A.u8, A.u16, A.u32, A.u64, A.f16, A.f32, A.f64)):
+        for n in (2, 3, 4):
+            xs = _rand(rng, ty, (157, n), -50, 50) if ty not in (A.f16, A.f32, A.f64) else _rand(rng, ty, (157, n))
+            add("simd_extract_v%d_%s" % (n, ty), Q.vec_extract(n, ty, (k + n) % n), [xs], None)
+            add("simd_inject_v%d_%s" % (n, ty), Q.vec_inject(n, ty), [xs[:150 - 7 * j, j].copy() for j in range(n)], None)
+    add("simd_extract_v8_f16_rank2", Q.vec_extract(8, A.f16, 5, 2), [_rand(rng, A.f16, (9, 13, 8))], None)
+    add("simd_extract_v16_i8", Q.vec_extract(16, A.i8, 11), [_rand(rng, A.i8, (300, 16), -100, 100)], None)
+    add("simd_extract_empty", Q.vec_extract(3, A.i32, 2), [np.zeros((0, 3), np.int32)], None)
+    for shp in ((1,), (300,), (5000,), (7, 900)):
+        add("scan1_simd_v3i32_%s" % (shp,), Q.vec_scan(3, A.i32, "l", len(shp)), [_rand(rng, A.i32, shp + (3,), -50, 50)], None)
+        add("scan1_simd_v2i64_r_%s" % (shp,), Q.vec_scan(2, A.i64, "r", len(shp)), [_rand(rng, A.i64, shp + (2,), -50, 50)], None)
+    add("scan1_simd_v16i8", Q.vec_scan(16, A.i8), [_rand(rng, A.i8, (3000, 16), -100, 100)], None)
+    add("fold_simd_v2i64", Q.vec_fold(2, A.i64), [_rand(rng, A.i64, (37, 1000, 2), -50, 50)], None)
+    add("fold_simd_v3i16_rows", Q.vec_fold(3, A.i16), [_rand(rng, A.i16, (900, 7, 3), -50, 50)], None)
+    add("permute_simd_v3i32", Q.vec_accumulate(3, A.i32, 17),
+        [_rand(rng, A.i32, (2000, 3), -50, 50), rng.integers(0, 17, 2000).astype(np.int64)], None)
+    add("simd_reverse_v3i16", Q.vec_reverse(3, A.i16), [_rand(rng, A.i16, (1001, 3), -50, 50)], None)
+    add("stencil_simd_v2f32", Q.vec_stencil_1d(), [_rand(rng, A.f32, (777, 2))], None)
     # ---- the benchmark programs at small size
     add("dotp_1000", P.dotp(), [_rand(rng, A.f32, (1000,)), _rand(rng, A.f32, (900,))], 1e-4 * 16 * 900)
     add("histogram_zipf", P.histogram(97), [rng.integers(0, 97, 3000).astype(np.int32)], None)

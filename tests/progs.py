@@ -419,3 +419,82 @@ def scanl_seg(ty=Int, z=0):
         return _seg_flags(seg, None, "l", with_flags)
 
     return A.alam([M, V1], body)
+
+
+# -- SIMD vector element types (Test/NoFib/Prelude/SIMD.hs): extract a component, inject components
+def _unpacked(n, ty, v, k):
+    """let (c0, .., c{n-1}) = unpack v in k [c0, ..]"""
+    return A.let(A.ttup(*[ty] * n), A.vecunpack(n, ty, v), lambda t: k(A.untup(t)))
+
+
+def _vec_add(n, ty):
+    def f(x, y):
+        return _unpacked(n, ty, x, lambda xs: _unpacked(n, ty, y, lambda ys: A.vecpack(
+            n, ty, A.tup(*[A.add(ty, a, b) for a, b in zip(xs, ys)]))))
+    vt = A.tvec(n, ty)
+    return A.lam([vt, vt], f)
+
+
+def vec_extract(n, ty, k, rank=1):
+    """map (view _k . unpackVec) xs"""
+    vt = A.tvec(n, ty)
+    return A.alam([A.tarray(rank, vt)], lambda xs: A.map_(
+        ty, A.lam([vt], lambda v: _unpacked(n, ty, v, lambda cs: cs[k])), xs))
+
+
+def vec_inject(n, ty):
+    """zipWith{n} V{n} xs ys ..: one Generate over the intersection after fusion"""
+    sh1 = A.tshape(1)
+    vt = A.tvec(n, ty)
+
+    def body(*arrs):
+        def ext():
+            e = A.untup_shape(arrs[0])[0]
+            for a in arrs[1:]:
+                e = A.min_(Int, e, A.untup_shape(a)[0])
+            return A.sh(e)
+        return A.generate(A.tarray(1, vt), ext(), A.lam([sh1], lambda ix: A.vecpack(
+            n, ty, A.tup(*[A.index(a, A.vexp(ix)) for a in arrs]))))
+
+    return A.alam([A.tarray(1, ty)] * n, body)
+
+
+def vec_scan(n, ty, direction="l", rank=1):
+    """scanl1 / scanr1 of the component-wise sum over Vec n t elements"""
+    return A.alam([A.tarray(rank, A.tvec(n, ty))], lambda xs: A.scan(direction, _vec_add(n, ty), None, xs))
+
+
+def vec_fold(n, ty, rank=2):
+    vt = A.tvec(n, ty)
+    zero = A.vecpack(n, ty, A.tup(*[A.const(ty, 0)] * n))
+    return A.alam([A.tarray(rank, vt)], lambda xs: A.fold(_vec_add(n, ty), zero, xs))
+
+
+def vec_accumulate(n, ty, nbins):
+    """permute (component-wise +) into zeros: no hardware atomic fits, cells are locked"""
+    sh1 = A.tshape(1)
+    vt = A.tvec(n, ty)
+    zero = lambda: A.vecpack(n, ty, A.tup(*[A.const(ty, 0)] * n))
+    return A.alam([A.tarray(1, vt), A.tarray(1, Int)], lambda xs, to: A.permute(
+        _vec_add(n, ty), A.generate(A.tarray(1, vt), A.sh(nbins), A.lam([sh1], lambda ix: zero())),
+        A.lam([sh1], lambda ix: A.just(A.sh(A.index(to, A.vexp(ix))))), xs))
+
+
+def vec_reverse(n, ty):
+    sh1 = A.tshape(1)
+    return A.alam([A.tarray(1, A.tvec(n, ty))], lambda xs: A.backpermute(
+        1, A.shape(xs), A.lam([sh1], lambda ix: A.sh(A.sub(Int, A.sub(Int, A.untup_shape(xs)[0], A.constI(1)),
+                                                            A.untup(ix)[0]))), xs))
+
+
+def vec_stencil_1d(ty=A.f32):
+    """3-point sum of V2 elements, clamp: component-wise left + centre + right"""
+    vt = A.tvec(2, ty)
+
+    def f(st):
+        l, c, r = A.untup(st)
+        return _unpacked(2, ty, l, lambda ls: _unpacked(2, ty, c, lambda cs: _unpacked(2, ty, r, lambda rs: A.vecpack(
+            2, ty, A.tup(*[A.add(ty, A.add(ty, ls[k], cs[k]), rs[k]) for k in range(2)])))))
+
+    sr = A.sunit(3, vt)
+    return A.alam([A.tarray(1, vt)], lambda xs: A.stencil(sr, vt, A.lam([A.stencil_type(sr)], f), "clamp", xs))
