@@ -93,7 +93,9 @@ int acchip_sync(acchip_ctx* ctx); /* wait for everything queued on the context's
  * acchip_malloc): rank, extents (outermost first, row-major: Representation/Shape.hs:98-106)
  * element type as text ("f32", "(pair (pair unit i32) f32)", ...), and one device pointer
  * per scalar leaf of the element type in left-to-right order -- the struct-of-arrays
- * payload of Array/Data.hs:95-119.  The handle does not take ownership of the buffers. */
+ * payload of Array/Data.hs:95-119.  A SIMD vector type `Vec n t` is one leaf, written
+ * "v<n><t>" ("v3f32"); its buffer holds the n components of each element side by side
+ * (Array/Data.hs:119,190).  The handle does not take ownership of the buffers. */
 int acchip_array_wrap(acchip_ctx* ctx, int rank, const int64_t* shape, const char* elt_type,
                       void* const* buffers, int n_buffers, acchip_array** out);
 /* Allocate an array from the pool (allocateArray + mallocRemote); owned by the handle. */
