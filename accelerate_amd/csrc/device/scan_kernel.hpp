@@ -25,7 +25,13 @@ acc_scan(Spec::Env env, Spec::Out out, Spec::Out tot, ScanParams p) {
       else S::store(out, outBase + (S::kRight ? m - 1 - u : u), y);
     }
   };
-  acc_scan_tile<S>(env, rowDesc, p.tpr, tile, n, p.epoch, load, store);
+  // scan' keeps the row's total apart: only the row's last tile can hold it, the others
+  // store without the test
+  auto inner = [&](i64 t, const Elt& y) {
+    if (S::kKind == 0) S::store(out, outBase + (S::kRight ? n - 1 - t : t), y);
+    else S::store(out, outBase + (S::kRight ? m - 2 - t : t + 1), y);
+  };
+  acc_scan_tile<S>(env, rowDesc, p.tpr, tile, n, p.epoch, load, store, inner, S::kKind != 2 || tile + 1 < p.tpr);
 
   if (S::kKind != 0 && tile == 0 && threadIdx.x == 0) {
     Elt z = S::seed(env);
