@@ -1510,6 +1510,32 @@ KernelSource Codegen::stencil(const std::vector<Sx>& patterns, const TypeP& outE
   if (!typeEq(valType(rb), outElt) || !typeEq(valType(ri), outElt))
     throw Error("stencil: function result does not match the declared element type");
 
+  // A thread whose V results and all their taps lie inside one row of the array evaluates
+  // them without any test (interior_run / produce_in): the taps of neighbouring results are
+  // then the same loads, and what is left becomes a few wide requests.
+  std::string runFns;
+  if (!interior.empty() && srcs.size() == 1) {
+    std::vector<int> halo;
+    stencilHalo(patterns[0], 0, halo);
+    std::string cond;
+    for (int d = 0; d < rank; ++d) {
+      const bool inner = d == rank - 1;
+      if (halo[d] == 0 && !inner) continue;
+      cond += (cond.empty() ? "" : " && ") + std::string("(") + fx[d] + " >= (i64)" + std::to_string(halo[d]) + ") && (" +
+              fx[d] + " + (i64)" + std::to_string(halo[d]) + (inner ? " + (i64)(V - 1)" : "") + " < " + dimsOf[0][d] + ")";
+    }
+    Emit er;
+    er.ind = 4;
+    er.code = em.code;  // extents and strides bound so far
+    er.line("return " + cond + ";");
+    runFns += fnHead("bool", "interior_run", "const Env& env, const i64* ix") + er.code + "  }\n";
+    Emit ep;
+    ep.ind = 4;
+    ep.code = em.code + ei.code;
+    runFns += fnHead("Elt", "produce_in", "const Env& env, i64 i") + returnElt(ri, ep) + "  }\n";
+    runFns += "#define ACC_MAP_INTERIOR_RUN 1\n";
+  }
+
   ValP r = rb;
   if (interior.empty()) {
     em.code += eb.code;  // no halo at all: nothing can leave the array (eb was emitted one level deeper)
@@ -1527,7 +1553,7 @@ KernelSource Codegen::stencil(const std::vector<Sx>& patterns, const TypeP& outE
     em.ind -= 2;
     em.line("}");
   }
-  std::string body = indexFns + fnHead("Elt", "produce_at", "const Env& env, i64 i, const i64* ix") + returnElt(r, em) + "  }\n";
+  std::string body = indexFns + runFns + fnHead("Elt", "produce_at", "const Env& env, i64 i, const i64* ix") + returnElt(r, em) + "  }\n";
   body += "  static constexpr int kRank = " + std::to_string(rank) + ";\n#define ACC_MAP_INDEXED 1\n";
   if (rank >= 2) body += "#define ACC_MAP_XCD 1\n";
   return finish(body, outElt, typeLeaves(outElt), "map.hpp", 0);

@@ -29,6 +29,17 @@ ACC_DEV void acc_map_body(const Spec::Env& env, const Spec::Out& out, const MapP
   if (i0 >= p.n) return;
   i64 ix[S::kRank];
   S::from_index(env, i0, ix);
+#ifdef ACC_MAP_INTERIOR_RUN
+  // all V results and their taps inside one row: no boundary tests, shared wide loads
+  if (S::interior_run(env, ix)) {
+    S::Elt r[S::V];
+#pragma unroll
+    for (int k = 0; k < V; ++k) r[k] = S::produce_in(env, i0 + k);
+#pragma unroll
+    for (int k = 0; k < V; ++k) S::store(out, i0 + k, r[k]);
+    return;
+  }
+#endif
   if (i0 + V <= p.n) {
     S::Elt r[S::V];
 #pragma unroll
