@@ -1418,28 +1418,33 @@ KernelSource Codegen::stencil(const std::vector<Sx>& patterns, const TypeP& outE
   Emit ei;
   ei.ind = em.ind + 2;
   ValP ri;
+  std::vector<std::string> focusLin, focusDefs;
   {
-    std::vector<std::string> stride(rank);
-    if (srcs.size() == 1) {
+    // every source is read at its own linear index of the focus (for one source that is the
+    // result's linear index; for two, whose extents may differ, it is computed from ix)
+    std::vector<std::vector<std::string>> stride(srcs.size(), std::vector<std::string>(rank));
+    for (size_t a = 0; a < srcs.size(); ++a) {
       std::string acc = "(i64)1";
       for (int d = rank - 1; d >= 0; --d) {
-        stride[d] = acc;
-        if (d > 0) acc = bindLeaf(ST::I64, acc + " * " + dimsOf[0][d], em)->ex;
+        stride[a][d] = acc;
+        if (d > 0) acc = bindLeaf(ST::I64, acc + " * " + dimsOf[a][d], em)->ex;
+      }
+      if (srcs.size() == 1) {
+        focusLin.push_back("i");
+      } else {
+        std::string e = fx[0];
+        for (int d = 1; d < rank; ++d) e = "(" + e + " * " + dimsOf[a][d] + " + " + fx[d] + ")";
+        focusLin.push_back("b" + std::to_string(a));
+        focusDefs.push_back("const i64 b" + std::to_string(a) + " = " + e);
       }
     }
     std::vector<ValP> args;
     for (size_t a = 0; a < srcs.size(); ++a) {
       auto access = [&](const std::vector<int>& off) -> ValP {
-        if (srcs.size() == 1) {
-          std::string lin = "i";
-          for (int d = 0; d < rank; ++d)
-            if (off[d] != 0) lin += " + (i64)" + std::to_string(off[d]) + " * " + stride[d];
-          return operandLinear(srcs[a], bindLeaf(ST::I64, lin, ei)->ex, ei);
-        }
-        std::vector<std::string> raw(rank);
+        std::string lin = focusLin[a];
         for (int d = 0; d < rank; ++d)
-          raw[d] = off[d] == 0 ? fx[d] : bindLeaf(ST::I64, fx[d] + " + (i64)" + std::to_string(off[d]), ei)->ex;
-        return operandIndex(srcs[a], mk(raw), ei);
+          if (off[d] != 0) lin += " + (i64)" + std::to_string(off[d]) + " * " + stride[a][d];
+        return operandLinear(srcs[a], bindLeaf(ST::I64, lin, ei)->ex, ei);
       };
       std::vector<int> off(rank, 0);
       args.push_back(Rec::go(patterns[a], 0, rank, off, access));
@@ -1514,25 +1519,30 @@ KernelSource Codegen::stencil(const std::vector<Sx>& patterns, const TypeP& outE
   // them without any test (interior_run / produce_in): the taps of neighbouring results are
   // then the same loads, and what is left becomes a few wide requests.
   std::string runFns;
-  if (!interior.empty() && srcs.size() == 1) {
-    std::vector<int> halo;
-    stencilHalo(patterns[0], 0, halo);
+  if (!interior.empty()) {
     std::string cond;
-    for (int d = 0; d < rank; ++d) {
-      const bool inner = d == rank - 1;
-      if (halo[d] == 0 && !inner) continue;
-      cond += (cond.empty() ? "" : " && ") + std::string("(") + fx[d] + " >= (i64)" + std::to_string(halo[d]) + ") && (" +
-              fx[d] + " + (i64)" + std::to_string(halo[d]) + (inner ? " + (i64)(V - 1)" : "") + " < " + dimsOf[0][d] + ")";
+    for (size_t a = 0; a < srcs.size(); ++a) {
+      std::vector<int> halo;
+      stencilHalo(patterns[a], 0, halo);
+      for (int d = 0; d < rank; ++d) {
+        const bool inner = d == rank - 1;
+        if (halo[d] == 0 && !inner) continue;
+        cond += (cond.empty() ? "" : " && ") + std::string("(") + fx[d] + " >= (i64)" + std::to_string(halo[d]) + ") && (" +
+                fx[d] + " + (i64)" + std::to_string(halo[d]) + (inner ? " + (i64)(V - 1)" : "") + " < " + dimsOf[a][d] + ")";
+      }
     }
     Emit er;
     er.ind = 4;
     er.code = em.code;  // extents and strides bound so far
     er.line("return " + cond + ";");
     runFns += fnHead("bool", "interior_run", "const Env& env, const i64* ix") + er.code + "  }\n";
+    // result k of the run that starts at ix (i: its linear index in the result)
     Emit ep;
     ep.ind = 4;
-    ep.code = em.code + ei.code;
-    runFns += fnHead("Elt", "produce_in", "const Env& env, i64 i") + returnElt(ri, ep) + "  }\n";
+    ep.code = em.code;
+    for (const std::string& d : focusDefs) ep.line(d + " + (i64)k;");
+    ep.code += ei.code;
+    runFns += fnHead("Elt", "produce_in", "const Env& env, i64 i, const i64* ix, int k") + returnElt(ri, ep) + "  }\n";
     runFns += "#define ACC_MAP_INTERIOR_RUN 1\n";
   }
 
@@ -1542,6 +1552,9 @@ KernelSource Codegen::stencil(const std::vector<Sx>& patterns, const TypeP& outE
   } else {
     r = declareVars(outElt, em);
     em.line("if (" + interior + ") {");
+    em.ind += 2;
+    for (const std::string& d : focusDefs) em.line(d + ";");
+    em.ind -= 2;
     em.code += ei.code;
     em.ind += 2;
     assign(r, ri, em);

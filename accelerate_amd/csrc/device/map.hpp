@@ -34,7 +34,7 @@ ACC_DEV void acc_map_body(const Spec::Env& env, const Spec::Out& out, const MapP
   if (S::interior_run(env, ix)) {
     S::Elt r[S::V];
 #pragma unroll
-    for (int k = 0; k < V; ++k) r[k] = S::produce_in(env, i0 + k);
+    for (int k = 0; k < V; ++k) r[k] = S::produce_in(env, i0 + k, ix, k);
 #pragma unroll
     for (int k = 0; k < V; ++k) S::store(out, i0 + k, r[k]);
     return;
