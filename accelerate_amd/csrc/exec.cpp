@@ -565,7 +565,7 @@ ATyP Program::prepare(const Sx& n, TEnv& tenv) {
     for (ST st : typeLeaves(srcs[0].r.elt)) simd = simd || stIsVec(st);
     if (simd) {
       plan.k = ctx_.kernel(cg.stencil(pats, outElt, *f, bnds, srcs));
-    } else if (!two && srcs[0].r.rank == 2) {
+    } else if (!two && srcs[0].r.rank == 2 && !std::getenv("ACCHIP_STENCIL_NO2D")) {
       plan.k = ctx_.kernel(cg.stencil2d(pats[0], outElt, *f, bnds[0], srcs[0]));
       plan.mode = "lds2d";
     } else if (!two && srcs[0].r.rank == 3 && !std::getenv("ACCHIP_STENCIL_NO3D")) {

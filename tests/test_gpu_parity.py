@@ -234,6 +234,21 @@ def test_stencil3d_plane_ring_matches_oracle(gpu_ctx, monkeypatch, bname, chain)
         assert same(gpu_ctx.compile(prog)(x), _ORACLE_3D[(bname, n)])
 
 
+def test_stencil2d_direct_evaluation_matches_oracle(monkeypatch):
+    # the same direct evaluation forced for rank 2: rows long enough for threads whose results
+    # and taps all lie inside a row (evaluated without tests) next to threads at the borders
+    monkeypatch.setenv("ACCHIP_STENCIL_NO2D", "1")
+    ctx = hip.Context(0)
+    rng = np.random.default_rng(32)
+    for bname in ("clamp", "mirror", "wrap", "constant", "function"):
+        for ty, widths in ((A.i64, [3, 5]), (A.i32, [5, 3])):
+            b = {"constant": A.constant(ty, -3), "function": Q.boundary_function(ty, 2)}.get(bname, bname)
+            prog = Q.stencil_weighted(ty, widths, b)
+            x = rng.integers(-9, 10, (9, 70)).astype(np.int64 if ty == A.i64 else np.int32)
+            assert same(ctx.compile(prog)(x), O.run_n(prog.text(), x))
+    ctx.close()
+
+
 def test_stencil3d_direct_evaluation_matches_oracle(monkeypatch):
     # the direct (one thread per result) evaluation that ranks other than 2 and 3 use, forced
     # here for rank 3
