@@ -70,7 +70,21 @@ ACC_DEV bool acc_fold_span(const typename S::Env& env, const Src& src, i64 off, 
     return nvalid > 0;
   } else {
     Elt carry;
-    for (i64 base = lo; base < hi; base += T) {
+    i64 base = lo;
+    // full tiles: V unconditional loads per lane (one wide request), all lanes take part
+    for (; base + T <= hi; base += T) {
+      const i64 q = off + base + (i64)lane * V;
+      Elt x[S::V];
+#pragma unroll
+      for (int k = 0; k < V; ++k) x[k] = src(q + k);
+      Elt t = x[0];
+#pragma unroll
+      for (int k = 1; k < V; ++k) t = S::combine(env, t, x[k]);
+      t = acc_wave_reduce<S>(env, t, lane, ACC_WAVE);
+      carry = have ? S::combine(env, carry, t) : t;
+      have = true;
+    }
+    for (; base < hi; base += T) {
       i64 cnt = hi - base < T ? hi - base : T;
       int nl = (int)((cnt + V - 1) / V);
       i64 p0 = base + (i64)lane * V;

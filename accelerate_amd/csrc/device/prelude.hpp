@@ -113,18 +113,6 @@ template <class T> ACC_DEV T acc_shfl(const T& v, int src) {
   return acc_from_words<T>(w);
 }
 
-// Ordered reduction of the values held by lanes [0, nvalid) of a wave: the result, in
-// lane 0, is v0 (+) v1 (+) .. with operands kept left to right, so the operator need
-// only be associative.
-template <class S> ACC_DEV typename S::Elt acc_wave_reduce(const typename S::Env& env, typename S::Elt v, int lane, int nvalid) {
-#pragma unroll
-  for (int d = 1; d < ACC_WAVE; d <<= 1) {
-    typename S::Elt o = acc_shfl_down(v, d);
-    if (lane + d < nvalid) v = S::combine(env, v, o);
-  }
-  return v;
-}
-
 // Data-parallel-primitive moves (VALU, no LDS traffic).  Controls of the gfx9 family:
 // row_shr:n = 0x110 + n (shift right by n inside each row of 16 lanes), wave_shr:1 = 0x138
 // (whole wave shifted by one lane), row_bcast:15 = 0x142 (lane 15 of each row to the next
@@ -148,6 +136,38 @@ template <class T> ACC_DEV T acc_readlane(const T& v, int src) {
   for (int k = 0; k < AccWords<T>::N; ++k) w[k] = (u32)__builtin_amdgcn_readlane((int)w[k], s);
   return acc_from_words<T>(w);
 }
+
+// Ordered reduction of the values held by lanes [0, nvalid) of a wave: the result, valid in
+// lane 0, is v0 (+) v1 (+) .. with operands kept left to right, so the operator need
+// only be associative.  Inside each row of 16 lanes the partner's value comes through
+// row_shl (a lane receives from the lane n places above it); the four row results are read
+// with readlane and combined in order.
+template <class S> ACC_DEV typename S::Elt acc_wave_reduce(const typename S::Env& env, typename S::Elt v, int lane, int nvalid) {
+  typedef typename S::Elt Elt;
+  const int col = lane & 15;
+  {
+    Elt o = acc_dpp<0x101, 0xf>(v);
+    if (col + 1 < 16 && lane + 1 < nvalid) v = S::combine(env, v, o);
+  }
+  {
+    Elt o = acc_dpp<0x102, 0xf>(v);
+    if (col + 2 < 16 && lane + 2 < nvalid) v = S::combine(env, v, o);
+  }
+  {
+    Elt o = acc_dpp<0x104, 0xf>(v);
+    if (col + 4 < 16 && lane + 4 < nvalid) v = S::combine(env, v, o);
+  }
+  {
+    Elt o = acc_dpp<0x108, 0xf>(v);
+    if (col + 8 < 16 && lane + 8 < nvalid) v = S::combine(env, v, o);
+  }
+  Elt r = acc_readlane(v, 0);
+  if (nvalid > 16) r = S::combine(env, r, acc_readlane(v, 16));
+  if (nvalid > 32) r = S::combine(env, r, acc_readlane(v, 32));
+  if (nvalid > 48) r = S::combine(env, r, acc_readlane(v, 48));
+  return r;
+}
+
 
 // Ordered inclusive scan across the lanes of a wave (valid lanes must form a prefix):
 // four shifts inside the rows of 16 lanes, then the row totals are handed to the next row
