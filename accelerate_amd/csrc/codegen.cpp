@@ -838,6 +838,15 @@ KernelSource Codegen::finish(const std::string& specBody, const TypeP& elt, cons
     for (size_t k = 0; k < el.size(); ++k)
       s += "    acc_st<kStream>(&o.o" + std::to_string(k) + "[i], v.c" + std::to_string(k) + ");\n";
     s += "  }\n";
+    // V consecutive results at once: one wide request per leaf whatever the compiler can
+    // prove about the alignment of position i
+    s += "  ACC_DEV void store_run(const Out& o, i64 i, const Elt* v) {\n";
+    for (size_t k = 0; k < el.size(); ++k) {
+      const std::string K = std::to_string(k), T = stName(el[k]);
+      s += "    {\n      acc_run<" + T + ", V> r_;\n#pragma unroll\n      for (int k_ = 0; k_ < V; ++k_) r_.e[k_] = v[k_].c" + K +
+           ";\n      *(acc_run<" + T + ", V>*)&o.o" + K + "[i] = r_;\n    }\n";
+    }
+    s += "  }\n";
   }
   s += "};\n\n";
   for (size_t b = 0; b <= skeleton.size();) {  // one or more headers joined by '+'

@@ -23,6 +23,10 @@ ACC_VEC_TYPES(i8) ACC_VEC_TYPES(i16) ACC_VEC_TYPES(i32) ACC_VEC_TYPES(i64)
 ACC_VEC_TYPES(u8) ACC_VEC_TYPES(u16) ACC_VEC_TYPES(u32) ACC_VEC_TYPES(u64)
 ACC_VEC_TYPES(f16) ACC_VEC_TYPES(f32) ACC_VEC_TYPES(f64)
 
+// N values that lie side by side in memory, aligned like one of them: assigning through a
+// pointer to it moves them with one request
+template <class T, int N> struct __attribute__((packed, aligned(alignof(T)))) acc_run { T e[N]; };
+
 #define ACC_DEV static __device__ __forceinline__
 #define ACC_WAVE 64
 #define ACC_BLOCK 256

@@ -263,12 +263,12 @@ ACC_DEV void acc_rake(const typename S::Env& env, typename S::Elt* mine, const t
 // receives val[t] (the inclusive combination up to t, seed included when S::kSeeded).
 // `desc` holds the descriptors of this sequence's tiles.  Called by all threads of the
 // workgroup (ACC_SCAN_BLOCK threads).  When `plain` holds, a tile that lies completely inside
-// the sequence stores through storePlain instead: a caller whose store tests for a special
-// position (the total of scan') passes a test-free version for the tiles that cannot hold
-// it, which keeps the V stores of a lane one wide request.
-template <class S, class Load, class Store, class StorePlain>
+// the sequence hands the V consecutive values of a lane to storeRun(t0, y) instead, which
+// can move them with one wide request: a caller whose store tests for a special position
+// (the total of scan') sets it for the tiles that cannot hold that position.
+template <class S, class Load, class Store, class StoreRun>
 ACC_DEV void acc_scan_tile(const typename S::Env& env, u64* desc, i64 tiles, i64 tile, i64 n, u64 epoch,
-                           const Load& load, const Store& store, const StorePlain& storePlain, bool plain) {
+                           const Load& load, const Store& store, const StoreRun& storeRun, bool plain) {
   typedef typename S::Elt Elt;
   typedef AccScanCfg<S> C;
   const int V = C::V, G = C::G, W = C::W;
@@ -419,8 +419,7 @@ ACC_DEV void acc_scan_tile(const typename S::Env& env, u64* desc, i64 tiles, i64
 #pragma unroll
       for (int k = 0; k < V; ++k) y[k] = hasBase ? S::combine(env, base, x[g][k]) : x[g][k];
       if (plain) {
-#pragma unroll
-        for (int k = 0; k < V; ++k) storePlain(t0 + k, y[k]);
+        storeRun(t0, y);
       } else {
 #pragma unroll
         for (int k = 0; k < V; ++k) store(t0 + k, y[k]);

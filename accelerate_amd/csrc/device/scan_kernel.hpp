@@ -25,13 +25,21 @@ acc_scan(Spec::Env env, Spec::Out out, Spec::Out tot, ScanParams p) {
       else S::store(out, outBase + (S::kRight ? m - 1 - u : u), y);
     }
   };
-  // scan' keeps the row's total apart: only the row's last tile can hold it, the others
-  // store without the test
-  auto inner = [&](i64 t, const Elt& y) {
-    if (S::kKind == 0) S::store(out, outBase + (S::kRight ? n - 1 - t : t), y);
-    else S::store(out, outBase + (S::kRight ? m - 2 - t : t + 1), y);
+  // the V consecutive values of a lane, moved with one wide request per leaf (a right scan
+  // writes them in reverse).  scan' keeps the row's total apart: only the row's last tile can
+  // hold it, the others need no test.
+  auto storeRun = [&](i64 t0, const Elt* y) {
+    const i64 shift = S::kKind == 0 ? 0 : 1;
+    if (!S::kRight) {
+      S::store_run(out, outBase + t0 + shift, y);
+    } else {
+      Elt z[S::V];
+#pragma unroll
+      for (int k = 0; k < S::V; ++k) z[k] = y[S::V - 1 - k];
+      S::store_run(out, outBase + (m - 1 - shift) - (t0 + S::V - 1), z);
+    }
   };
-  acc_scan_tile<S>(env, rowDesc, p.tpr, tile, n, p.epoch, load, store, inner, S::kKind != 2 || tile + 1 < p.tpr);
+  acc_scan_tile<S>(env, rowDesc, p.tpr, tile, n, p.epoch, load, store, storeRun, S::kKind != 2 || tile + 1 < p.tpr);
 
   if (S::kKind != 0 && tile == 0 && threadIdx.x == 0) {
     Elt z = S::seed(env);
