@@ -1134,7 +1134,12 @@ AValP Program::eval(const Sx& n, AEnv& aenv) {
     // Many sources into a destination of a few LDS-fuls with a hardware-atomic combination:
     // combine in workgroup-private LDS copies first (see permute.hpp).
     const int64_t partMax = 131072 / stSize(plan.k->meta.outLeaves.empty() ? ST::I32 : plan.k->meta.outLeaves[0]);
-    if (plan.mode == "atomic" && cnt >= (1 << 20) && out->size() <= 8 * partMax) {
+    // Up to 128 LDS-fuls: every share re-reads the sources (from its XCD's L2), so the cost grows
+    // with the destination -- 2^26 keys into 2^20 / 2^22 Int32 bins take 0.5 / 2.0 ms, which is
+    // where plain global atomics are for uniform keys (2.5 ms); for Zipf keys those take 110 ms.
+    const char* pe = std::getenv("ACCHIP_PERMUTE_PARTS");
+    const int64_t maxParts = pe ? std::atoll(pe) : 128;
+    if (plan.mode == "atomic" && cnt >= (1 << 20) && out->size() <= maxParts * partMax) {
       const int64_t nparts = (out->size() + partMax - 1) / partMax;
       const int64_t part = (out->size() + nparts - 1) / nparts;
       // one workgroup per CU in total (each holds 128 KiB of LDS): fewer, longer workgroups

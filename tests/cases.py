@@ -244,6 +244,8 @@ def gpu_only_programs():
             b = {"constant": A.constant(A.i64, -3), "function": Q.boundary_function(A.i64, rank)}.get(bname, bname)
             for widths in widths_list:
                 out.append(("stencil_%s_%s" % (widths, bname), Q.stencil_weighted(A.i64, widths, b)))
+    for nb in (1 << 20, (1 << 21) + 12345, 1 << 22):
+        out.append(("histogram_%d" % nb, P.histogram(nb)))
     out.append(("transpose_i32", Q.transpose(A.i32)))
     out.append(("transpose_i64", Q.transpose(A.i64)))
     return out

@@ -180,6 +180,18 @@ def test_histogram_2pow26_bit_exact(gpu_ctx):
     assert got.sum(dtype=np.int64) == n and np.array_equal(got, np.bincount(keys, minlength=nbins))
 
 
+@pytest.mark.parametrize("nbins", [1 << 20, (1 << 21) + 12345, 1 << 22])
+def test_histogram_over_many_lds_fuls(gpu_ctx, monkeypatch, nbins):
+    # destinations of up to 128 LDS-fuls are still combined in workgroup-private copies, one
+    # range of the destination per pass; against numpy and against the plain global atomics
+    keys = W.zipf_keys(1 << 22, nbins, 5)
+    ref = np.bincount(keys, minlength=nbins)
+    run = gpu_ctx.compile(P.histogram(nbins))
+    assert np.array_equal(run(keys), ref)
+    monkeypatch.setenv("ACCHIP_PERMUTE_PARTS", "0")
+    assert np.array_equal(run(keys), ref)
+
+
 def test_jacobi_8192_bit_equal(gpu_ctx):
     g = W.uniform_f32(8192 * 8192, 8, 0.0, 1.0).reshape(8192, 8192)
     step = gpu_ctx.compile(P.jacobi_step())
