@@ -53,6 +53,39 @@ def golden_cases():
     for name, prog in (("scanlseg_doctest", Q.scanl_seg()), ("scanl1seg_doctest", Q.scan1_seg("l")),
                        ("scanr1seg_doctest", Q.scan1_seg("r"))):
         add(name, prog, [np.array(v[name]["mat"], I64), np.array(v[name]["seg"], I64)], np.array(v[name]["expected"], I64))
+    # regression tests of the reference with literal answers (Test/NoFib/Issues)
+    add("issue93", Q.issue93(), [np.array(v["issue93"]["mat"], I64)], np.array(v["issue93"]["expected"], I64))
+    add("issue102", Q.issue102(), [], np.array(v["issue102"]["expected"], I64))
+    for n in "ABCD":
+        e = v["issue119_" + n]
+        dt = np.int32 if e["type"] == "i32" else I64
+        add("issue119_" + n, Q.issue119_foldall(e["type"]), [np.array(e["xs"], dt).reshape(e["shape"])],
+            np.array(e["expected"][0], dt))
+    e = v["issue119_E"]
+    add("issue119_E", Q.fold_op(A.add, A.i32, 2, 0), [np.array(e["xs"], np.int32).reshape(e["shape"])],
+        np.array(e["expected"], np.int32))
+    for n, prog in (("F", Q.scan1_seg("l", A.i64, 1, A.i32)), ("G", Q.scan1_seg("r", A.i64, 1, A.i32)),
+                    ("H", Q.scanl_seg(A.i64, 0, 1, A.i32)), ("I", Q.scanr_seg(A.i64, 0, 1, A.i32))):
+        e = v["issue119_" + n]
+        add("issue119_" + n, prog, [np.array(e["xs"], I64), np.array(e["seg"], np.int32)], np.array(e["expected"], I64))
+    add("issue123", Q.issue123(v["issue123"]["n"]), [], np.array(v["issue123"]["expected"], I64))
+    add("issue184_A", Q.issue184a(v["issue184_A"]["n"]), [np.array(v["issue184_A"]["v"], I64)],
+        np.array(v["issue184_A"]["expected"], I64))
+    add("issue287_A", Q.issue287a(), [[np.zeros(v["issue287_A"]["n"], I64)] * 6],
+        [np.array(c, I64) for c in zip(*v["issue287_A"]["expected"])])
+    pairs = [np.arange(1, v["issue288"]["n"] + 1, dtype=I64)] * 2
+    add("issue288", Q.issue288(), [pairs], pairs)
+    for n in v["issue364"]["sizes"]:
+        add("issue364_%d" % n, Q.issue364(), [[np.arange(n, dtype=I64)] * 2],
+            [np.concatenate([[-1], np.zeros(n, I64)]), np.concatenate([[-1], np.arange(n, dtype=I64)])])
+    for ty, dt in ((A.f32, np.float32), (A.f64, np.float64)):
+        xs = np.array([float(t) for t in v["issue407"]["xs"]], dt)
+        add("issue407_isnan_" + ty, Q.issue407("isnan", ty), [xs], np.array(v["issue407"]["isnan"], np.uint8))
+        add("issue407_isinf_" + ty, Q.issue407("isinf", ty), [xs], np.array(v["issue407"]["isinf"], np.uint8))
+    e = v["issue436_A"]
+    add("issue436_A", Q.filter_take(e["take"]), [np.array(e["xs"], np.uint8)],
+        (np.array(e["expected"], np.uint8), np.array(e["count"], I64)))
+    add("issue439", Q.issue439(), [], np.array(v["issue439"]["expected"], np.float32))
     t = v["issue228"]
     pair_in = [np.array(t["fst"], I64), np.array(t["snd"], I64)]
     pair_out = [np.array(t["expected"][0], I64), np.array(t["expected"][1], I64)]
@@ -228,6 +261,10 @@ def parity_cases():
         [_rand(rng, A.i32, (2000, 3), -50, 50), rng.integers(0, 17, 2000).astype(np.int64)], None)
     add("simd_reverse_v3i16", Q.vec_reverse(3, A.i16), [_rand(rng, A.i16, (1001, 3), -50, 50)], None)
     add("stencil_simd_v2f32", Q.vec_stencil_1d(), [_rand(rng, A.f32, (777, 2))], None)
+    # ---- Issue114: compensated summation over (value, error) pairs, a non-commutative fold1 / scanl1
+    ef = [np.full(100, 1.01, np.float32), np.zeros(100, np.float32)]
+    add("fold1_issue114", Q.issue114("fold1"), [ef], 1e-4 * 101)
+    add("scan1_issue114", Q.issue114("scanl1"), [ef], 1e-4 * 101)
     # ---- the benchmark programs at small size
     add("dotp_1000", P.dotp(), [_rand(rng, A.f32, (1000,)), _rand(rng, A.f32, (900,))], 1e-4 * 16 * 900)
     add("histogram_zipf", P.histogram(97), [rng.integers(0, 97, 3000).astype(np.int32)], None)

@@ -100,6 +100,60 @@ V["issue137"] = {"cite": "Test/NoFib/Issues/Issue137.hs:33-59", "size": 3000, "b
                  "values": "abs (8 - (a mod 17)) for a in 1..size", "targets": "a div 8 for a in 1..size",
                  "expected": pairs}
 
+# Test/NoFib/Issues/Issue119.hs: sums of and segmented scans over literal arrays ("fold and scan
+# with a number of elements not a multiple of the workgroup size").  The arrays are read from the
+# reference's file in the order they appear: A-E give (expected, input), F-I (expected, input,
+# segments); J and K (scan'Seg) are not taken.
+text = open(os.path.join(SRC, "Test", "NoFib", "Issues", "Issue119.hs")).read()
+lists = [(tuple(int(d) for d in re.findall(r"\d+", sh)), [int(x) for x in body.split(",")])
+         for sh, body in re.findall(r"fromList \((Z(?: *:\. *\d+)*)\)\s*\[([-0-9,\s]+)\]", text)]
+totals = [int(x) for x in re.findall(r"ref\d = fromList Z \[(-?\d+)\]", text)]
+assert len(totals) == 4
+it = iter(lists)
+for name, kind in (("A", "foldall"), ("B", "foldall"), ("C", "foldall"), ("D", "foldall"), ("E", "fold")):
+    expected = [totals["ABCD".index(name)]] if name != "E" else next(it)[1]
+    shape, xs = next(it)
+    V["issue119_" + name] = {"cite": "Test/NoFib/Issues/Issue119.hs test " + name, "kind": kind,
+                             "type": "i32" if name in "ABE" else "i64", "shape": list(shape), "xs": xs,
+                             "expected": expected}
+for name, kind in (("F", "scanl1Seg"), ("G", "scanr1Seg"), ("H", "scanlSeg"), ("I", "scanrSeg")):
+    (_, expected), (_, xs), (_, seg) = next(it), next(it), next(it)
+    V["issue119_" + name] = {"cite": "Test/NoFib/Issues/Issue119.hs test " + name, "kind": kind,
+                             "xs": xs, "seg": seg, "expected": expected}
+assert V["issue119_A"]["expected"] == [734889155] and len(V["issue119_F"]["expected"]) == 748
+assert sum(V["issue119_F"]["seg"]) == 748 and len(V["issue119_H"]["expected"]) == 645
+
+# Test/NoFib/Issues/Issue93.hs: permute (\c _ -> c) (fill (shape xs) 0) Just xs on a 1x1 matrix
+V["issue93"] = {"cite": "Test/NoFib/Issues/Issue93.hs:27-34", "mat": [[5]], "expected": [[5]]}
+# Test/NoFib/Issues/Issue102.hs: [4,4,4] of shape 1x3x1
+V["issue102"] = {"cite": "Test/NoFib/Issues/Issue102.hs:31-62", "expected": [[[4], [4], [4]]]}
+# Test/NoFib/Issues/Issue114.hs: compensated summation over pairs, fold1 and scanl1 (compared with ~=)
+V["issue114"] = {"cite": "Test/NoFib/Issues/Issue114.hs:33-71", "n": 100, "x": 1.01,
+                 "expected_sum": [101.0, 0.0], "expected_prefix": "(1.01 * i, 0) for i in 1..n"}
+# Test/NoFib/Issues/Issue123.hs: fold (+) 0 (fill n 1) = n
+V["issue123"] = {"cite": "Test/NoFib/Issues/Issue123.hs:27-38", "n": 100, "expected": 100}
+# Test/NoFib/Issues/Issue184.hs test A: generate 1000 (\x -> x < 5 ? (v!!x)^2 : 0), v = [1..5]
+V["issue184_A"] = {"cite": "Test/NoFib/Issues/Issue184.hs:33-41", "v": [1, 2, 3, 4, 5], "n": 1000,
+                   "expected": [1, 4, 9, 16, 25] + [0] * 995}
+# Test/NoFib/Issues/Issue287.hs test A: scanl1 of a six-component combination over zeros stays zero
+V["issue287_A"] = {"cite": "Test/NoFib/Issues/Issue287.hs:26-56", "n": 4, "expected": [[0] * 6] * 4}
+# Test/NoFib/Issues/Issue288.hs: map (while (const False) id) leaves pairs unchanged
+V["issue288"] = {"cite": "Test/NoFib/Issues/Issue288.hs:26-36", "n": 10}
+# Test/NoFib/Issues/Issue364.hs: scanl iappend one over the intervals (i, i) for i in 0..n-1 gives
+# one, then (0, i); n = 64 and n = 65 (the second failed for integral types)
+V["issue364"] = {"cite": "Test/NoFib/Issues/Issue364.hs:41-93", "sizes": [64, 65], "one": [-1, -1], "top": [-2, -2]}
+# Test/NoFib/Issues/Issue407.hs: isNaN / isInfinite
+V["issue407"] = {"cite": "Test/NoFib/Issues/Issue407.hs:38-46",
+                 "xs": ["nan", "-inf", "nan", "0.1", "inf", "0.5", "inf"],
+                 "isnan": [1, 0, 1, 0, 0, 0, 0], "isinf": [0, 1, 0, 0, 1, 0, 1]}
+# Test/NoFib/Issues/Issue409.hs: y + tanh ((-y) * y) with y = recip 1  ==  1 + tanh (-1)
+V["issue409"] = {"cite": "Test/NoFib/Issues/Issue409.hs:36-53", "x": 1.0, "expected": "1 + tanh(-1)"}
+# Test/NoFib/Issues/Issue436.hs test A: filter (const True) (take 3 bools)
+V["issue436_A"] = {"cite": "Test/NoFib/Issues/Issue436.hs:27-50", "xs": [1, 0, 1, 0, 1], "take": 3,
+                   "expected": [1, 0, 1], "count": 3}
+# Test/NoFib/Issues/Issue439.hs: map (* 2) over the rank-0 array fill Z 1
+V["issue439"] = {"cite": "Test/NoFib/Issues/Issue439.hs:26-34", "expected": 2.0}
+
 with open(OUT, "w") as f:
     json.dump(V, f, indent=1, sort_keys=True)
 print("wrote", OUT, len(V), "vectors")

@@ -324,13 +324,15 @@ def radix_passes(bits):
 
 
 # -- segmented scans as Prelude.hs builds them from scan', permute and a flagged scan
-#    (mkHeadFlags / mkTailFlags :1364-1389, segmentedL / segmentedR :1395-1407)
-def _seg_flags(seg_src, nseg_sh, direction, k):
+#    (mkHeadFlags / mkTailFlags :1364-1389, segmentedL / segmentedR :1395-1407); `ity` is the
+#    integral type of the segment descriptor, `rank` the rank of the scanned array
+def _seg_flags(seg_src, direction, ity, k):
     """Head flags (left scans) or tail flags (right scans) of a segment descriptor given as an
     operand: permute (+) zeros (\\ix -> Just (offset!ix)) ones.  k receives the array of
     total+1 entries; `init` is left to the consumer (it reads all but the last entry)."""
     sh1 = A.tshape(1)
-    V1, S0 = A.tarray(1, Int), A.tarray(0, Int)
+    V1, S0 = A.tarray(1, ity), A.tarray(0, ity)
+    toint = lambda e: e if ity == Int else A.fromintegral(ity, Int, e)
 
     def with_offsets(st):
         offset, total = st
@@ -338,85 +340,91 @@ def _seg_flags(seg_src, nseg_sh, direction, k):
 
         def target(ix):
             o = A.index(offset, A.vexp(ix))
-            return A.just(A.sh(o if direction == "l" else A.sub(Int, A.sub(Int, ln(), A.constI(1)), o)))
+            return A.just(A.sh(toint(o if direction == "l" else A.sub(ity, A.sub(ity, ln(), A.const(ity, 1)), o))))
 
-        ones = A.delayed(V1, A.shape(offset), A.lam([sh1], lambda ix: A.constI(1)), A.lam([Int], lambda i: A.constI(1)))
-        zeros = A.generate(V1, A.sh(A.add(Int, ln(), A.constI(1))), A.lam([sh1], lambda ix: A.constI(0)))
-        return A.alet(V1, A.permute(binop(A.add, Int), zeros, A.lam([sh1], target), ones), k)
+        ones = A.delayed(V1, A.shape(offset), A.lam([sh1], lambda ix: A.const(ity, 1)),
+                         A.lam([Int], lambda i: A.const(ity, 1)))
+        zeros = A.generate(V1, A.sh(A.add(Int, toint(ln()), A.constI(1))), A.lam([sh1], lambda ix: A.const(ity, 0)))
+        return A.alet(V1, A.permute(binop(A.add, ity), zeros, A.lam([sh1], target), ones), k)
 
-    return A.alet(A.tpair(V1, S0), A.scan_(direction, binop(A.add, Int), A.constI(0), seg_src), with_offsets)
+    return A.alet(A.tpair(V1, S0), A.scan_(direction, binop(A.add, ity), A.const(ity, 0), seg_src), with_offsets)
 
 
-def _scan1_seg(direction, ty, mat, seg_src, nseg_sh):
-    """scanl1Seg / scanr1Seg (Prelude.hs:1136-1145, 1313-1322) of a matrix operand variable:
+def _scan1_seg(direction, ty, arr, seg_src, rank=2, ity=Int):
+    """scanl1Seg / scanr1Seg (Prelude.hs:1136-1145, 1313-1322) of an array variable:
     map snd . scan1 (segmented f) $ zip (replicate flags) arr, the zip fused into the scan."""
-    sh2 = A.tshape(2)
-    t2 = A.ttup(Int, ty)
+    shr = A.tshape(rank)
+    t2 = A.ttup(ity, ty)
 
     def seg_op(x, y):
         # scanl1: x = running value, y = new element; scanr1: x = new element, y = running value
         (af, av), (bf, bv) = (A.untup(x), A.untup(y)) if direction == "l" else (A.untup(y), A.untup(x))
         f = A.add(ty, av, bv) if direction == "l" else A.add(ty, bv, av)
-        return A.tup(A.bor(Int, af, bf), A.cond(A.neq(Int, bf, A.constI(0)), bv, f))
+        return A.tup(A.bor(ity, af, bf), A.cond(A.neq(ity, bf, A.const(ity, 0)), bv, f))
 
     def with_flags(fl):
         def extent():
-            rows, cols = A.untup_shape(mat)
+            dims = A.untup_shape(arr)
             nfl = A.sub(Int, A.untup_shape(fl)[0], A.constI(1))
-            return A.sh(rows, A.min_(Int, nfl, cols))
+            return A.sh(*(dims[:-1] + [A.min_(Int, nfl, dims[-1])]))
 
         def at(ix):
-            _, x = A.untup(ix)
-            return A.tup(A.index(fl, A.sh(x)), A.index(mat, A.vexp(ix)))
+            x = A.untup(ix)[-1]
+            return A.tup(A.index(fl, A.sh(x)), A.index(arr, A.vexp(ix)))
 
-        src = A.delayed(A.tarray(2, t2), extent(), A.lam([sh2], at),
-                        A.lam([Int], lambda i: A.let(sh2, A.fromindex(2, extent(), i), at)))
+        src = A.delayed(A.tarray(rank, t2), extent(), A.lam([shr], at),
+                        A.lam([Int], lambda i: A.let(shr, A.fromindex(rank, extent(), i), at)))
         return A.map_(ty, A.lam([t2], lambda v: A.untup(v)[1]), A.scan(direction, A.lam([t2, t2], seg_op), None, src))
 
-    return _seg_flags(seg_src, nseg_sh, direction, with_flags)
+    return _seg_flags(seg_src, direction, ity, with_flags)
 
 
-def scan1_seg(direction, ty=Int):
-    return A.alam([A.tarray(2, ty), A.tarray(1, Int)], lambda mat, seg: _scan1_seg(direction, ty, mat, seg, None))
+def scan1_seg(direction, ty=Int, rank=2, ity=Int):
+    return A.alam([A.tarray(rank, ty), A.tarray(1, ity)],
+                  lambda arr, seg: _scan1_seg(direction, ty, arr, seg, rank, ity))
 
 
-def scanl_seg(ty=Int, z=0):
+def scanl_seg(ty=Int, z=0, rank=2, ity=Int):
     """scanlSeg (Prelude.hs:979-1012): the seed is injected at the head of every segment by a
     permute into an array of seeds, then an inclusive segmented scan over segments one longer."""
-    sh1, sh2 = A.tshape(1), A.tshape(2)
-    V1, M = A.tarray(1, Int), A.tarray(2, ty)
+    sh1, shr = A.tshape(1), A.tshape(rank)
+    V1, M = A.tarray(1, ity), A.tarray(rank, ty)
+    toint = lambda e: e if ity == Int else A.fromintegral(ity, Int, e)
 
     def body(mat, seg):
         def with_flags(fl):
-            nflags = lambda: A.sub(Int, A.untup_shape(fl)[0], A.constI(1))
             # (terms are built where they are used: binder levels are fixed at construction)
-            rows = lambda: A.untup_shape(mat)[0]
-            cols = lambda: A.untup_shape(mat)[1]
+            nflags = lambda: A.sub(Int, A.untup_shape(fl)[0], A.constI(1))
+            outer = lambda: A.untup_shape(mat)[:-1]
+            cols = lambda: A.untup_shape(mat)[-1]
             nseg = lambda: A.untup_shape(seg)[0]
-            taken_sh = lambda: A.sh(rows(), A.min_(Int, nflags(), cols()))
-            filled = lambda: A.generate(M, A.sh(rows(), A.add(Int, cols(), nseg())),
-                                        A.lam([sh2], lambda ix: A.const(ty, z)))
+            size = lambda: A.shapesize(rank, A.shape(mat))
+            taken_sh = lambda: A.sh(*(outer() + [A.min_(Int, nflags(), cols())]))
+            filled = lambda: A.generate(M, A.sh(*(outer() + [A.add(Int, cols(), nseg())])),
+                                        A.lam([shr], lambda ix: A.const(ty, z)))
             # inc = scanl1 (+) flags, with flags = init fl fused in
             flags = A.delayed(V1, A.sh(nflags()), A.lam([sh1], lambda ix: A.index(fl, A.vexp(ix))),
                               A.lam([Int], lambda i: A.linearindex(fl, i)))
 
             def with_inc(inc):
                 def to(ix):
-                    y, x = A.untup(ix)
-                    return A.just(A.sh(y, A.add(Int, x, A.index(inc, A.sh(x)))))
+                    parts = A.untup(ix)
+                    x = parts[-1]
+                    return A.just(A.sh(*(parts[:-1] + [A.add(Int, x, toint(A.index(inc, A.sh(x))))])))
                 # take (length flags) arr
-                taken = A.delayed(M, taken_sh(), A.lam([sh2], lambda ix: A.index(mat, A.vexp(ix))),
-                                  A.lam([Int], lambda i: A.let(sh2, A.fromindex(2, taken_sh(), i),
+                taken = A.delayed(M, taken_sh(), A.lam([shr], lambda ix: A.index(mat, A.vexp(ix))),
+                                  A.lam([Int], lambda i: A.let(shr, A.fromindex(rank, taken_sh(), i),
                                                                lambda ix: A.index(mat, A.vexp(ix)))))
-                arr1 = A.permute(A.lam([ty, A.wild(ty)], lambda x, _: x), filled(), A.lam([sh2], to), taken)
-                seg1 = A.delayed(V1, A.shape(seg), A.lam([sh1], lambda ix: A.add(Int, A.index(seg, A.vexp(ix)), A.constI(1))),
-                                 A.lam([Int], lambda i: A.add(Int, A.linearindex(seg, i), A.constI(1))))
-                return A.alet(M, arr1, lambda a1: _scan1_seg("l", ty, a1, seg1, None))
+                arr1 = A.permute(A.lam([ty, A.wild(ty)], lambda x, _: x), filled(), A.lam([shr], to), taken)
+                seg1 = A.delayed(V1, A.shape(seg),
+                                 A.lam([sh1], lambda ix: A.add(ity, A.index(seg, A.vexp(ix)), A.const(ity, 1))),
+                                 A.lam([Int], lambda i: A.add(ity, A.linearindex(seg, i), A.const(ity, 1))))
+                return A.alet(M, arr1, lambda a1: _scan1_seg("l", ty, a1, seg1, rank, ity))
 
-            empty = A.lor(A.eq(Int, A.mul(Int, rows(), cols()), A.constI(0)), A.eq(Int, nflags(), A.constI(0)))
+            empty = A.lor(A.eq(Int, size(), A.constI(0)), A.eq(Int, nflags(), A.constI(0)))
             return A.acond(empty, filled(),
-                           A.alet(V1, A.scan("l", binop(A.add, Int), None, flags), with_inc))
-        return _seg_flags(seg, None, "l", with_flags)
+                           A.alet(V1, A.scan("l", binop(A.add, ity), None, flags), with_inc))
+        return _seg_flags(seg, "l", ity, with_flags)
 
     return A.alam([M, V1], body)
 
@@ -498,3 +506,190 @@ def vec_stencil_1d(ty=A.f32):
 
     sr = A.sunit(3, vt)
     return A.alam([A.tarray(1, vt)], lambda xs: A.stencil(sr, vt, A.lam([A.stencil_type(sr)], f), "clamp", xs))
+
+
+def scanr_seg(ty=Int, z=0, rank=1, ity=Int):
+    """scanrSeg (Prelude.hs:1202-1228): as scanlSeg, the seeds injected by a permute whose targets
+    are one less than for the left scan, over `drop (sz - length flags) arr`, then scanr1Seg."""
+    sh1, shr = A.tshape(1), A.tshape(rank)
+    V1, M = A.tarray(1, ity), A.tarray(rank, ty)
+    toint = lambda e: e if ity == Int else A.fromintegral(ity, Int, e)
+
+    def body(mat, seg):
+        def with_flags(fl):
+            nflags = lambda: A.sub(Int, A.untup_shape(fl)[0], A.constI(1))
+            outer = lambda: A.untup_shape(mat)[:-1]
+            cols = lambda: A.untup_shape(mat)[-1]
+            nseg = lambda: A.untup_shape(seg)[0]
+            size = lambda: A.shapesize(rank, A.shape(mat))
+            dropped = lambda: A.min_(Int, A.sub(Int, cols(), nflags()), cols())     # drop n: n `min` sz
+            rest_sh = lambda: A.sh(*(outer() + [A.sub(Int, cols(), dropped())]))
+            filled = lambda: A.generate(M, A.sh(*(outer() + [A.add(Int, cols(), nseg())])),
+                                        A.lam([shr], lambda ix: A.const(ty, z)))
+            flags = A.delayed(V1, A.sh(nflags()), A.lam([sh1], lambda ix: A.index(fl, A.vexp(ix))),
+                              A.lam([Int], lambda i: A.linearindex(fl, i)))
+
+            def with_inc(inc):
+                def to(ix):
+                    parts = A.untup(ix)
+                    x = parts[-1]
+                    return A.just(A.sh(*(parts[:-1] + [A.sub(Int, A.add(Int, x, toint(A.linearindex(inc, x))), A.constI(1))])))
+
+                def from_rest(ix):
+                    parts = A.untup(ix)
+                    return A.index(mat, A.sh(*(parts[:-1] + [A.add(Int, parts[-1], dropped())])))
+                rest = A.delayed(M, rest_sh(), A.lam([shr], from_rest),
+                                 A.lam([Int], lambda i: A.let(shr, A.fromindex(rank, rest_sh(), i), from_rest)))
+                arr1 = A.permute(A.lam([ty, A.wild(ty)], lambda x, _: x), filled(), A.lam([shr], to), rest)
+                seg1 = A.delayed(V1, A.shape(seg),
+                                 A.lam([sh1], lambda ix: A.add(ity, A.index(seg, A.vexp(ix)), A.const(ity, 1))),
+                                 A.lam([Int], lambda i: A.add(ity, A.linearindex(seg, i), A.const(ity, 1))))
+                return A.alet(M, arr1, lambda a1: _scan1_seg("r", ty, a1, seg1, rank, ity))
+
+            empty = A.lor(A.eq(Int, size(), A.constI(0)), A.eq(Int, nflags(), A.constI(0)))
+            return A.acond(empty, filled(),
+                           A.alet(V1, A.scan("l", binop(A.add, ity), None, flags), with_inc))
+        return _seg_flags(seg, "l", ity, with_flags)
+
+    return A.alam([M, V1], body)
+
+
+# -- regression tests of the reference with known answers (Test/NoFib/Issues)
+def issue93():
+    sh2 = A.tshape(2)
+    M = A.tarray(2, Int)
+    return A.alam([M], lambda xs: A.permute(
+        A.lam([Int, A.wild(Int)], lambda c, _: c),
+        A.generate(M, A.shape(xs), A.lam([sh2], lambda ix: A.constI(0))),
+        A.lam([sh2], lambda ix: A.just(A.vexp(ix))), xs))
+
+
+def issue102():
+    """p = 3: y = generate (1,3,1) (i == 0 ? 0 : 2) [the reshaped fill 2 inlined], then the
+    DFT as fold (+) 0 over coefficients that are all 1 [fill 1 inlined through the replicate],
+    reshaped to the shape of y."""
+    sh3, sh4 = A.tshape(3), A.tshape(4)
+    Y = A.tarray(3, Int)
+
+    def with_y(y):
+        def at(ix):
+            l, _, r, col = A.untup(ix)
+            return A.mul(Int, A.constI(1), A.index(y, A.sh(l, col, r)))
+        ext = lambda: A.sh(1, 3, 1, 3)
+        src = A.delayed(A.tarray(4, Int), ext(), A.lam([sh4], at),
+                        A.lam([Int], lambda i: A.let(sh4, A.fromindex(4, ext(), i), at)))
+        return A.reshape(3, A.shape(y), A.reshape(1, A.sh(3), A.fold(binop(A.add, Int), A.constI(0), src)))
+
+    y = A.generate(Y, A.sh(1, 3, 1), A.lam([sh3], lambda ix: A.cond(
+        A.eq(Int, A.untup(ix)[1], A.constI(0)), A.constI(0), A.constI(2))))
+    return A.alet(Y, y, with_y)
+
+
+def issue114(kind):
+    """Compensated summation over (value, error) pairs: fold1 / scanl1 of a non-commutative add."""
+    t2 = A.ttup(A.f32, A.f32)
+    f = A.f32
+
+    def add(x, y):
+        aval, aerr = A.untup(x)
+        bval, berr = A.untup(y)
+        return A.let(f, A.add(f, aval, bval), lambda val: A.let(f, A.sub(f, val, aval), lambda det: A.tup(
+            val, A.add(f, A.add(f, A.add(f, A.sub(f, aval, A.sub(f, val, det)), A.sub(f, bval, det)), aerr), berr))))
+    fn = A.lam([t2, t2], add)
+    if kind == "fold1":
+        return A.alam([A.tarray(1, t2)], lambda xs: A.fold(fn, None, xs))
+    return A.alam([A.tarray(1, t2)], lambda xs: A.scan("l", fn, None, xs))
+
+
+def issue119_foldall(ty):
+    return A.alam([A.tarray(2, ty)], lambda xs: A.fold(
+        binop(A.add, ty), A.const(ty, 0), A.reshape(1, A.sh(A.shapesize(2, A.shape(xs))), xs)))
+
+
+def issue123(n=100):
+    sh1 = A.tshape(1)
+    ones = A.delayed(A.tarray(1, Int), A.sh(n), A.lam([sh1], lambda ix: A.constI(1)), A.lam([Int], lambda i: A.constI(1)))
+    return A.fold(binop(A.add, Int), A.constI(0), ones)
+
+
+def issue184a(n=1000):
+    sh1 = A.tshape(1)
+
+    def f(v):
+        def at(ix):
+            x = A.untup(ix)[0]
+            return A.cond(A.lt(Int, x, A.constI(5)), A.let(Int, A.linearindex(v, x), lambda y: A.mul(Int, y, y)), A.constI(0))
+        return A.generate(A.tarray(1, Int), A.sh(n), A.lam([sh1], at))
+    return A.alam([A.tarray(1, Int)], f)
+
+
+def issue287a():
+    t6 = A.ttup(*[Int] * 6)
+
+    def f(x, y):
+        mi1, l1, c1, r1, li1, ri1 = A.untup(x)
+        _, l2, _, r2, _, ri2 = A.untup(y)
+        return A.tup(A.max_(Int, mi1, A.add(Int, ri1, l2)), l1, c1, A.mul(Int, r2, r1), li1, ri2)
+    return A.alam([A.tarray(1, t6)], lambda xs: A.scan("l", A.lam([t6, t6], f), None, xs))
+
+
+def issue288():
+    t2 = A.ttup(Int, Int)
+    loop = lambda e: A.while_(t2, lambda v: A.const(A.u8, 0), lambda v: A.vexp(v), e)
+    return A.alam([A.tarray(1, t2)], lambda xs: A.map_(t2, A.lam([t2], lambda v: loop(A.vexp(v))), xs))
+
+
+def issue364(ty=Int):
+    """scanl iappend one: the interval-of-summations monoid with identity `one` and absorbing `top`"""
+    t2 = A.ttup(ty, ty)
+    c = lambda v: A.const(ty, v)
+    is_ = lambda p, v: A.land(A.eq(ty, A.untup(p)[0], c(v)), A.eq(ty, A.untup(p)[1], c(v)))
+
+    def iappend(x, y):
+        x1, x2 = A.untup(x)
+        y1, y2 = A.untup(y)
+        top = A.tup(c(-2), c(-2))
+        return A.cond(is_(x, -1), A.vexp(y), A.cond(is_(y, -1), A.vexp(x), A.cond(
+            A.lor(is_(x, -2), is_(y, -2)), top,
+            A.cond(A.eq(ty, A.add(ty, x2, c(1)), y1), A.tup(x1, y2), top))))
+    return A.alam([A.tarray(1, t2)], lambda xs: A.scan("l", A.lam([t2, t2], iappend), A.tup(c(-1), c(-1)), xs))
+
+
+def issue407(which, ty):
+    op = A.isnan if which == "isnan" else A.isinf
+    return A.alam([A.tarray(1, ty)], lambda xs: A.map_(A.u8, A.lam([ty], lambda x: op(ty, x)), xs))
+
+
+def issue409(ty):
+    def f(x):
+        return A.let(ty, A.recip(ty, x), lambda y: A.let(ty, A.mul(ty, A.neg(ty, y), y), lambda b: A.add(ty, y, A.tanh(ty, b))))
+    return A.alam([A.tarray(0, ty)], lambda xs: A.map_(ty, A.lam([ty], f), xs))
+
+
+def filter_take(n, ty=A.u8):
+    """filter (const True) (take n xs) (Issue436): the kept elements and their number"""
+    sh1 = A.tshape(1)
+    V1, S0 = A.tarray(1, Int), A.tarray(0, Int)
+
+    def body(xs):
+        ext = lambda: A.sh(A.min_(Int, A.constI(n), A.untup_shape(xs)[0]))
+        flags = A.delayed(V1, ext(), A.lam([sh1], lambda ix: A.constI(1)), A.lam([Int], lambda i: A.constI(1)))
+        taken = A.delayed(A.tarray(1, ty), ext(), A.lam([sh1], lambda ix: A.index(xs, A.vexp(ix))),
+                          A.lam([Int], lambda i: A.linearindex(xs, i)))
+
+        def with_scan(st):
+            targets, total = st
+            kept = A.permute(
+                A.lam([ty, A.wild(ty)], lambda x, _: x),
+                A.generate(A.tarray(1, ty), A.sh(A.index(total, A.nil)), A.lam([sh1], lambda ix: A.const(ty, 0))),
+                A.lam([sh1], lambda ix: A.just(A.sh(A.index(targets, A.vexp(ix))))), taken)
+            return A.apair(kept, total)
+        return A.alet(A.tpair(V1, S0), A.scan_("l", binop(A.add, Int), A.constI(0), flags), with_scan)
+
+    return A.alam([A.tarray(1, ty)], body)
+
+
+def issue439():
+    S0 = A.tarray(0, A.f32)
+    one = A.generate(S0, A.nil, A.lam([A.unit], lambda ix: A.const(A.f32, 1)))
+    return A.alet(S0, one, lambda a: A.map_(A.f32, A.lam([A.f32], lambda x: A.mul(A.f32, x, A.const(A.f32, 2))), a))

@@ -96,6 +96,9 @@ def scalar_cases():
         for name in ("truncate", "round", "floor", "ceiling"):
             for to in ("i32", "i64"):
                 add("%s_%s_%s" % (name, ty, to), _map1(ty, to, lambda a, n=name, t=to: A.prim(n, [ty, t], a)), [x], None)
+        # Issue409: y + tanh ((-y) * y) with y = recip x, at x = 1 (1 + tanh (-1))
+        add("issue409_%s" % ty, _map1(ty, ty, lambda a: A.let(ty, A.recip(ty, a), lambda y: A.let(
+            ty, A.mul(ty, A.neg(ty, y), y), lambda b: A.add(ty, y, A.tanh(ty, b))))), [np.array([1.0, 2.0, -0.5], NPT[ty])], 4)
         special = np.array([np.nan, np.inf, -np.inf, 0.0, 1.0], NPT[ty])
         add("isnan_%s" % ty, _map1(ty, A.u8, lambda a: A.isnan(ty, a)), [special], None)
         add("isinf_%s" % ty, _map1(ty, A.u8, lambda a: A.isinf(ty, a)), [special], None)

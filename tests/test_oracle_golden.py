@@ -296,3 +296,22 @@ def test_oracle_on_segmented_scans_against_numpy():
     # the flagged scan zips with the flags of the lengthened segments: what lies beyond them is cut
     assert got.shape == (4, int(seg.sum()) + len(seg))
     assert np.array_equal(got, ex)
+
+
+def test_oracle_on_issue114_and_issue409():
+    # Issue114 (compared with ~= in the reference: 5e-5 absolute or 0.5 % relative for Float) and
+    # Issue409, whose expected value is 1 + tanh (-1)
+    import json
+    import math
+    import os
+    from . import progs as Q
+    v = json.load(open(os.path.join(os.path.dirname(__file__), "golden", "vectors.json")))
+    n, x = v["issue114"]["n"], v["issue114"]["x"]
+    ef = [np.full(n, x, np.float32), np.zeros(n, np.float32)]
+    close = lambda a, b: np.all((np.abs(a - b) < 5e-5) | (np.abs(a - b) <= 0.005 * np.maximum(np.abs(a), np.abs(b))))
+    val, err = O.run_n(Q.issue114("fold1").text(), ef)
+    assert close(val, v["issue114"]["expected_sum"][0]) and close(err, v["issue114"]["expected_sum"][1])
+    vals, errs = O.run_n(Q.issue114("scanl1").text(), ef)
+    assert close(vals, np.float32(x) * np.arange(1, n + 1, dtype=np.float32)) and close(errs, 0.0)
+    assert O.run_n(Q.issue409(A.f64).text(), np.array(v["issue409"]["x"])) == 1 + math.tanh(-1)
+    assert abs(float(O.run_n(Q.issue409(A.f32).text(), np.array(1.0, np.float32))) - (1 + math.tanh(-1))) < 1e-6
