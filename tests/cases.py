@@ -68,6 +68,14 @@ def golden_cases():
                     ("H", Q.scanl_seg(A.i64, 0, 1, A.i32)), ("I", Q.scanr_seg(A.i64, 0, 1, A.i32))):
         e = v["issue119_" + n]
         add("issue119_" + n, prog, [np.array(e["xs"], I64), np.array(e["seg"], np.int32)], np.array(e["expected"], I64))
+    for n, d in (("J", "l"), ("K", "r")):
+        e = v["issue119_" + n]
+        add("issue119_" + n, Q.scan_prime_seg(d, A.i64, 0, 1, A.i32), [np.array(e["xs"], I64), np.array(e["seg"], np.int32)],
+            (np.array(e["expected"], I64), np.array(e["expected_sums"], I64)))
+    for name, d in (("scanlprimeseg_doctest", "l"), ("scanrprimeseg_doctest", "r")):
+        e = v[name]
+        add(name, Q.scan_prime_seg(d), [np.array(e["mat"], I64), np.array(e["seg"], I64)],
+            (np.array(e["expected"], I64), np.array(e["expected_sums"], I64)))
     add("issue123", Q.issue123(v["issue123"]["n"]), [], np.array(v["issue123"]["expected"], I64))
     add("issue184_A", Q.issue184a(v["issue184_A"]["n"]), [np.array(v["issue184_A"]["v"], I64)],
         np.array(v["issue184_A"]["expected"], I64))

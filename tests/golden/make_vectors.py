@@ -66,6 +66,15 @@ V["scanl1seg_doctest"] = {"cite": "Prelude.hs:1117-1135", "mat": iota5x10, "seg"
 V["scanr1seg_doctest"] = {"cite": "Prelude.hs:1293-1312", "mat": iota5x10, "seg": [1, 4, 0, 3], "expected": [
     [0, 10, 9, 7, 4, 18, 13, 7], [10, 50, 39, 27, 14, 48, 33, 17], [20, 90, 69, 47, 24, 78, 53, 27],
     [30, 130, 99, 67, 34, 108, 73, 37], [40, 170, 129, 87, 44, 138, 93, 47]]}
+# Prelude.hs:1014-1039, 1230-1257  scanl'Seg / scanr'Seg: scanned bodies and per-segment totals
+V["scanlprimeseg_doctest"] = {"cite": "Prelude.hs:1014-1039", "mat": iota5x10, "seg": [1, 4, 0, 3], "seed": 0,
+    "expected": [[0, 0, 1, 3, 6, 0, 5, 11], [0, 0, 11, 23, 36, 0, 15, 31], [0, 0, 21, 43, 66, 0, 25, 51],
+                 [0, 0, 31, 63, 96, 0, 35, 71], [0, 0, 41, 83, 126, 0, 45, 91]],
+    "expected_sums": [[0, 10, 0, 18], [10, 50, 0, 48], [20, 90, 0, 78], [30, 130, 0, 108], [40, 170, 0, 138]]}
+V["scanrprimeseg_doctest"] = {"cite": "Prelude.hs:1230-1257", "mat": iota5x10, "seg": [1, 4, 0, 3], "seed": 0,
+    "expected": [[0, 15, 11, 6, 0, 17, 9, 0], [0, 45, 31, 16, 0, 37, 19, 0], [0, 75, 51, 26, 0, 57, 29, 0],
+                 [0, 105, 71, 36, 0, 77, 39, 0], [0, 135, 91, 46, 0, 97, 49, 0]],
+    "expected_sums": [[2, 18, 0, 24], [12, 58, 0, 54], [22, 98, 0, 84], [32, 138, 0, 114], [42, 178, 0, 144]]}
 # Language.hs:716-728  histogram via permute (+)
 V["histogram_doctest"] = {"cite": "Language.hs:716-728",
                           "keys": [0, 0, 1, 2, 1, 1, 2, 4, 8, 3, 4, 9, 8, 3, 2, 5, 5, 3, 1, 2], "bins": 10,
@@ -103,7 +112,7 @@ V["issue137"] = {"cite": "Test/NoFib/Issues/Issue137.hs:33-59", "size": 3000, "b
 # Test/NoFib/Issues/Issue119.hs: sums of and segmented scans over literal arrays ("fold and scan
 # with a number of elements not a multiple of the workgroup size").  The arrays are read from the
 # reference's file in the order they appear: A-E give (expected, input), F-I (expected, input,
-# segments); J and K (scan'Seg) are not taken.
+# segments), J and K (expected bodies, expected sums, input, segments).
 text = open(os.path.join(SRC, "Test", "NoFib", "Issues", "Issue119.hs")).read()
 lists = [(tuple(int(d) for d in re.findall(r"\d+", sh)), [int(x) for x in body.split(",")])
          for sh, body in re.findall(r"fromList \((Z(?: *:\. *\d+)*)\)\s*\[([-0-9,\s]+)\]", text)]
@@ -120,6 +129,11 @@ for name, kind in (("F", "scanl1Seg"), ("G", "scanr1Seg"), ("H", "scanlSeg"), ("
     (_, expected), (_, xs), (_, seg) = next(it), next(it), next(it)
     V["issue119_" + name] = {"cite": "Test/NoFib/Issues/Issue119.hs test " + name, "kind": kind,
                              "xs": xs, "seg": seg, "expected": expected}
+for name, kind in (("J", "scanl'Seg"), ("K", "scanr'Seg")):
+    (_, ps), (_, rs), (_, xs), (_, seg) = next(it), next(it), next(it), next(it)
+    V["issue119_" + name] = {"cite": "Test/NoFib/Issues/Issue119.hs test " + name, "kind": kind,
+                             "xs": xs, "seg": seg, "expected": ps, "expected_sums": rs}
+assert len(V["issue119_J"]["expected_sums"]) == 30 and len(V["issue119_K"]["expected"]) == 750
 assert V["issue119_A"]["expected"] == [734889155] and len(V["issue119_F"]["expected"]) == 748
 assert sum(V["issue119_F"]["seg"]) == 748 and len(V["issue119_H"]["expected"]) == 645
 

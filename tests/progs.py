@@ -384,7 +384,7 @@ def scan1_seg(direction, ty=Int, rank=2, ity=Int):
                   lambda arr, seg: _scan1_seg(direction, ty, arr, seg, rank, ity))
 
 
-def scanl_seg(ty=Int, z=0, rank=2, ity=Int):
+def scanl_seg(ty=Int, z=0, rank=2, ity=Int, as_body=False):
     """scanlSeg (Prelude.hs:979-1012): the seed is injected at the head of every segment by a
     permute into an array of seeds, then an inclusive segmented scan over segments one longer."""
     sh1, shr = A.tshape(1), A.tshape(rank)
@@ -426,7 +426,7 @@ def scanl_seg(ty=Int, z=0, rank=2, ity=Int):
                            A.alet(V1, A.scan("l", binop(A.add, ity), None, flags), with_inc))
         return _seg_flags(seg, "l", ity, with_flags)
 
-    return A.alam([M, V1], body)
+    return body if as_body else A.alam([M, V1], body)
 
 
 # -- SIMD vector element types (Test/NoFib/Prelude/SIMD.hs): extract a component, inject components
@@ -508,7 +508,7 @@ def vec_stencil_1d(ty=A.f32):
     return A.alam([A.tarray(1, vt)], lambda xs: A.stencil(sr, vt, A.lam([A.stencil_type(sr)], f), "clamp", xs))
 
 
-def scanr_seg(ty=Int, z=0, rank=1, ity=Int):
+def scanr_seg(ty=Int, z=0, rank=1, ity=Int, as_body=False):
     """scanrSeg (Prelude.hs:1202-1228): as scanlSeg, the seeds injected by a permute whose targets
     are one less than for the left scan, over `drop (sz - length flags) arr`, then scanr1Seg."""
     sh1, shr = A.tshape(1), A.tshape(rank)
@@ -550,6 +550,69 @@ def scanr_seg(ty=Int, z=0, rank=1, ity=Int):
             return A.acond(empty, filled(),
                            A.alet(V1, A.scan("l", binop(A.add, ity), None, flags), with_inc))
         return _seg_flags(seg, "l", ity, with_flags)
+
+    return body if as_body else A.alam([M, V1], body)
+
+
+def scan_prime_seg(direction, ty=Int, z=0, rank=2, ity=Int):
+    """scanl'Seg / scanr'Seg (Prelude.hs:1041-1094, 1262-1288): the exclusive segmented scan taken
+    apart by two backpermutes into the scanned bodies and the per-segment totals."""
+    sh1, shr = A.tshape(1), A.tshape(rank)
+    V1, S0, M = A.tarray(1, ity), A.tarray(0, ity), A.tarray(rank, ty)
+    toint = lambda e: e if ity == Int else A.fromintegral(ity, Int, e)
+    inner = scanl_seg(ty, z, rank, ity, True) if direction == "l" else scanr_seg(ty, z, rank, ity, True)
+    addi = binop(A.add, ity)
+
+    def body(mat, seg):
+        outer = lambda: A.untup_shape(mat)[:-1]
+        nseg = lambda: A.untup_shape(seg)[0]
+        seg1 = lambda: A.delayed(V1, A.shape(seg),
+                                 A.lam([sh1], lambda ix: A.add(ity, A.index(seg, A.vexp(ix)), A.const(ity, 1))),
+                                 A.lam([Int], lambda i: A.add(ity, A.linearindex(seg, i), A.const(ity, 1))))
+
+        def with_scanned(arr1):
+            def with_starts(st):
+                starts, _ = st      # prescanl (+) 0 seg'
+
+                def total_at(ix):
+                    parts = A.untup(ix)
+                    i = parts[-1]
+                    at = A.index(starts, A.sh(i))
+                    if direction == "l":    # tails = zipWith (+) seg starts
+                        at = A.add(ity, A.index(seg, A.sh(i)), at)
+                    return A.sh(*(parts[:-1] + [toint(at)]))
+                sums = A.backpermute(rank, A.sh(*(outer() + [nseg()])), A.lam([shr], total_at), arr1)
+
+                def bodies(inc, length):
+                    def at(ix):
+                        parts = A.untup(ix)
+                        i = parts[-1]
+                        return A.sh(*(parts[:-1] + [A.add(Int, i, toint(A.index(inc, A.sh(i))))]))
+                    return A.apair(A.backpermute(rank, A.sh(*(outer() + [length()])), A.lam([shr], at), arr1), sums)
+
+                if direction == "l":
+                    def with_offset(offset):
+                        ones = A.delayed(V1, A.shape(seg), A.lam([sh1], lambda ix: A.const(ity, 1)),
+                                         A.lam([Int], lambda i: A.const(ity, 1)))
+                        marks = A.permute(addi, A.generate(V1, A.sh(A.add(Int, A.shapesize(rank, A.shape(mat)), A.constI(1))),
+                                                           A.lam([sh1], lambda ix: A.const(ity, 0))),
+                                          A.lam([sh1], lambda ix: A.just(A.sh(toint(A.index(offset, A.vexp(ix)))))), ones)
+                        length = lambda: toint(A.index(offset, A.sh(A.sub(Int, A.untup_shape(offset)[0], A.constI(1)))))
+                        return A.alet(V1, marks, lambda mk: A.alet(V1, A.scan("l", addi, None, mk),
+                                                                   lambda inc: bodies(inc, length)))
+                    return A.alet(V1, A.scan("l", addi, None, seg), with_offset)
+
+                def with_flags(fl):
+                    nflags = lambda: A.sub(Int, A.untup_shape(fl)[0], A.constI(1))
+                    flags = A.delayed(V1, A.sh(nflags()), A.lam([sh1], lambda ix: A.index(fl, A.vexp(ix))),
+                                      A.lam([Int], lambda i: A.linearindex(fl, i)))
+                    return A.alet(V1, A.scan("l", addi, None, flags), lambda inc: bodies(inc, nflags))
+                return _seg_flags(seg, "l", ity, with_flags)
+            return A.alet(A.tpair(V1, S0), A.scan_("l", addi, A.const(ity, 0), seg1()), with_starts)
+
+        empty = A.eq(Int, A.shapesize(rank, A.shape(mat)), A.constI(0))
+        return A.acond(empty, A.apair(mat, A.generate(M, A.sh(*(outer() + [nseg()])), A.lam([shr], lambda ix: A.const(ty, z)))),
+                       A.alet(M, inner(mat, seg), with_scanned))
 
     return A.alam([M, V1], body)
 
