@@ -76,6 +76,62 @@ def golden_cases():
         e = v[name]
         add(name, Q.scan_prime_seg(d), [np.array(e["mat"], I64), np.array(e["seg"], I64)],
             (np.array(e["expected"], I64), np.array(e["expected_sums"], I64)))
+    # doctests of Prelude.hs beyond the skeletons' own
+    e = v["scanrseg_doctest"]
+    add("scanrseg_doctest", Q.scanr_seg(A.Int, 0, 2), [np.array(e["mat"], I64), np.array(e["seg"], I64)], np.array(e["expected"], I64))
+    e = v["foldall_doctest"]
+    add("foldall_vec_doctest", Q.fold_all(A.f32, 1, e["seed"]), [np.array(e["vec"], np.float32)], np.array(e["expected_vec"], np.float32))
+    add("foldall_mat_doctest", Q.fold_all(A.f32, 2, 0), [np.array(e["mat"], np.float32)], np.array(e["expected_mat"], np.float32))
+    e = v["all_any_doctest"]
+    add("fold_all_even_doctest", Q.all_any("all"), [np.array(e["mat"], I64)], np.array(e["all"], np.uint8))
+    add("fold_any_even_doctest", Q.all_any("any"), [np.array(e["mat"], I64)], np.array(e["any"], np.uint8))
+    e = v["reductions_doctest"]
+    add("fold_sum_doctest", Q.fold_op(A.add, A.Int, 2, 0), [np.array(e["mat2x5"], I64)], np.array(e["sum"], I64))
+    add("fold_product_doctest", Q.fold_op(A.mul, A.Int, 2, 1), [np.array(e["mat2x5"], I64)], np.array(e["product"], I64))
+    add("fold1_minimum_doctest", Q.fold_op(A.min_, A.Int, 2), [np.array(e["mat3x4"], I64)], np.array(e["minimum"], I64))
+    add("fold1_maximum_doctest", Q.fold_op(A.max_, A.Int, 2), [np.array(e["mat3x4"], I64)], np.array(e["maximum"], I64))
+    e = v["prepostscanl_doctest"]
+    add("scan_prescanl_doctest", Q.prescanl_sum(), [np.array(e["vec"], I64)], np.array(e["prescanl"], I64))
+    add("scan_postscanl_doctest", Q.postscanl_sum(e["postscanl_seed"]), [np.array(e["vec"], I64)], np.array(e["postscanl"], I64))
+    e = v["filter_doctest"]
+    add("filter_even_doctest", Q.filter_even(), [np.array(e["vec"], I64)], (np.array(e["expected"], I64), np.array(e["count"], I64)))
+    e = v["gather_scatter_doctest"]
+    g = e["gather"]
+    add("gather_doctest", Q.gather(A.Int), [np.array(g["from"], I64), np.array(g["input"], I64)], np.array(g["expected"], I64))
+    g = e["gatherIf"]
+    add("gatherif_doctest", Q.gather_if(), [np.array(g["from"], I64), np.array(g["mask"], I64), np.array(g["defaults"], np.float32),
+                                            np.array(g["input"], np.float32)], np.array(g["expected"], np.float32))
+    g = e["scatter"]
+    add("scatter_doctest", Q.scatter(A.Int), [np.array(g["to"], I64), np.zeros(g["size"], I64), np.array(g["input"], I64)],
+        np.array(g["expected"], I64))
+    g = e["scatterIf"]
+    add("scatterif_doctest", Q.scatter_if(), [np.array(g["to"], I64), np.array(g["mask"], I64), np.zeros(g["size"], I64),
+                                              np.array(g["input"], I64)], np.array(g["expected"], I64))
+    e = v["reindex_doctest"]
+    mat, box = np.array(e["mat"], I64), np.arange(30, dtype=I64).reshape(e["box_shape"])
+    last = lambda d: A.sub(A.Int, d, A.constI(1))
+    add("reverseon_1_doctest", Q.reindex(2, lambda d: d(), lambda ix, d: [ix[0], A.sub(A.Int, last(d()[1]), ix[1])]),
+        [mat], np.array(e["reverseOn_1"], I64))
+    add("reverseon_2_doctest", Q.reindex(2, lambda d: d(), lambda ix, d: [A.sub(A.Int, last(d()[0]), ix[0]), ix[1]]),
+        [mat], np.array(e["reverseOn_2"], I64))
+    add("transposeon_1_2_box_doctest", Q.reindex(3, lambda d: [d()[0], d()[2], d()[1]], lambda ix, d: [ix[0], ix[2], ix[1]]),
+        [box], np.array(e["transposeOn_1_2_box"], I64).reshape(2, 5, 3))
+    add("transposeon_2_3_box_doctest", Q.reindex(3, lambda d: [d()[1], d()[0], d()[2]], lambda ix, d: [ix[1], ix[0], ix[2]]),
+        [box], np.array(e["transposeOn_2_3_box"], I64).reshape(3, 2, 5))
+    add("transposeon_1_3_box_doctest", Q.reindex(3, lambda d: [d()[2], d()[1], d()[0]], lambda ix, d: [ix[2], ix[1], ix[0]]),
+        [box], np.array(e["transposeOn_1_3_box"], I64).reshape(5, 3, 2))
+    add("take_5_doctest", Q.reindex(2, lambda d: [d()[0], A.min_(A.Int, A.constI(5), d()[1])], lambda ix, d: ix),
+        [mat], np.array(e["take_5"], I64))
+    add("drop_7_doctest", Q.reindex(2, lambda d: [d()[0], A.sub(A.Int, d()[1], A.min_(A.Int, A.constI(7), d()[1]))],
+                                    lambda ix, d: [ix[0], A.add(A.Int, ix[1], A.min_(A.Int, A.constI(7), d()[1]))]),
+        [mat], np.array(e["drop_7"], I64))
+    add("init_doctest", Q.reindex(2, lambda d: [d()[0], last(d()[1])], lambda ix, d: ix), [mat], np.array(e["init"], I64))
+    add("tail_doctest", Q.reindex(2, lambda d: [d()[0], last(d()[1])], lambda ix, d: [ix[0], A.add(A.Int, ix[1], A.constI(1))]),
+        [mat], np.array(e["tail"], I64))
+    e = v["concat_doctest"]
+    add("append_doctest", Q.concat_on(1), [np.array(e["m1"], I64), np.array(e["m2_10x3"], I64)], np.array(e["append"], I64))
+    add("concaton_1_doctest", Q.concat_on(1), [np.array(e["m1"], I64), np.array(e["m2_10x5"], I64)], np.array(e["concatOn_1"], I64))
+    add("concaton_2_doctest", Q.concat_on(2), [np.array(e["m1"], I64), np.array(e["m2_10x5"], I64)], np.array(e["concatOn_2"], I64))
     add("issue123", Q.issue123(v["issue123"]["n"]), [], np.array(v["issue123"]["expected"], I64))
     add("issue184_A", Q.issue184a(v["issue184_A"]["n"]), [np.array(v["issue184_A"]["v"], I64)],
         np.array(v["issue184_A"]["expected"], I64))

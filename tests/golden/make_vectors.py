@@ -75,6 +75,56 @@ V["scanrprimeseg_doctest"] = {"cite": "Prelude.hs:1230-1257", "mat": iota5x10, "
     "expected": [[0, 15, 11, 6, 0, 17, 9, 0], [0, 45, 31, 16, 0, 37, 19, 0], [0, 75, 51, 26, 0, 57, 29, 0],
                  [0, 105, 71, 36, 0, 77, 39, 0], [0, 135, 91, 46, 0, 97, 49, 0]],
     "expected_sums": [[2, 18, 0, 24], [12, 58, 0, 54], [22, 98, 0, 84], [32, 138, 0, 114], [42, 178, 0, 144]]}
+# Prelude.hs:1175-1200  scanrSeg
+V["scanrseg_doctest"] = {"cite": "Prelude.hs:1175-1200", "mat": iota5x10, "seg": [1, 4, 0, 3], "seed": 0, "expected": [
+    [2, 0, 18, 15, 11, 6, 0, 0, 24, 17, 9, 0], [12, 0, 58, 45, 31, 16, 0, 0, 54, 37, 19, 0],
+    [22, 0, 98, 75, 51, 26, 0, 0, 84, 57, 29, 0], [32, 0, 138, 105, 71, 36, 0, 0, 114, 77, 39, 0],
+    [42, 0, 178, 135, 91, 46, 0, 0, 144, 97, 49, 0]]}
+# Prelude.hs:656-662  foldAll
+V["foldall_doctest"] = {"cite": "Prelude.hs:656-662", "vec": list(range(10)), "seed": 42, "expected_vec": 87.0,
+                        "mat": iota5x10, "expected_mat": 1225.0}
+# Prelude.hs:770-797  all even / any even along rows
+evens_mat = [[1, 2, 3, 4, 5, 6, 7, 8, 9, 10], [1, 1, 1, 1, 1, 2, 2, 2, 2, 2], [2, 4, 6, 8, 10, 12, 14, 16, 18, 20],
+             [1, 3, 5, 7, 9, 11, 13, 15, 17, 19]]
+V["all_any_doctest"] = {"cite": "Prelude.hs:770-797", "mat": evens_mat, "all": [0, 0, 1, 0], "any": [1, 1, 1, 0]}
+# Prelude.hs:822-878  sum, product, minimum, maximum along rows
+V["reductions_doctest"] = {"cite": "Prelude.hs:822-878", "mat2x5": [list(range(5)), list(range(5, 10))], "sum": [10, 35],
+                           "product": [0, 15120], "mat3x4": [[1, 4, 3, 8], [0, 2, 8, 4], [7, 9, 8, 8]],
+                           "minimum": [1, 0, 7], "maximum": [8, 8, 9]}
+# Prelude.hs:895-914  prescanl, postscanl
+V["prepostscanl_doctest"] = {"cite": "Prelude.hs:895-914", "vec": list(range(1, 11)), "prescanl_seed": 0,
+                             "prescanl": [0, 1, 3, 6, 10, 15, 21, 28, 36, 45], "postscanl_seed": 42,
+                             "postscanl": [43, 45, 48, 52, 57, 63, 70, 78, 87, 97]}
+# Prelude.hs:1620-1625  filter even
+V["filter_doctest"] = {"cite": "Prelude.hs:1620-1625", "vec": list(range(1, 11)), "expected": [2, 4, 6, 8, 10], "count": 5}
+# Prelude.hs:1696-1724, 1748-1778  gather, gatherIf, scatter, scatterIf
+V["gather_scatter_doctest"] = {
+    "cite": "Prelude.hs:1696-1724, 1748-1778",
+    "gather": {"from": [1, 3, 7, 2, 5, 3], "input": [1, 9, 6, 4, 4, 2, 0, 1, 2], "expected": [9, 4, 1, 6, 2, 4]},
+    "gatherIf": {"from": [1, 3, 7, 2, 5, 3], "mask": [3, 4, 9, 2, 7, 5], "defaults": [6.0] * 6,
+                 "input": [1, 9, 6, 4, 4, 2, 0, 1, 2], "expected": [6.0, 6.0, 1.0, 6.0, 2.0, 4.0]},
+    "scatter": {"to": [1, 3, 7, 2, 5, 8], "input": [1, 9, 6, 4, 4, 2, 5], "size": 10, "expected": [0, 1, 4, 9, 0, 4, 0, 6, 2, 0]},
+    "scatterIf": {"to": [1, 3, 7, 2, 5, 8], "mask": [3, 4, 9, 2, 7, 5], "input": [1, 9, 6, 4, 4, 2, 5], "size": 10,
+                  "expected": [0, 0, 0, 0, 0, 4, 0, 6, 2, 0]}}
+# Prelude.hs:1812-1892  reverseOn, transposeOn; 1915-2010 take, drop, init, tail (the 5x10 iota matrix, the 2x3x5 iota box)
+V["reindex_doctest"] = {
+    "cite": "Prelude.hs:1812-1892, 1915-2010", "mat": iota5x10, "box_shape": [2, 3, 5],
+    "reverseOn_1": [[r * 10 + 9 - c for c in range(10)] for r in range(5)],
+    "reverseOn_2": [[(4 - r) * 10 + c for c in range(10)] for r in range(5)],
+    "transposeOn_1_2_box": [0, 5, 10, 1, 6, 11, 2, 7, 12, 3, 8, 13, 4, 9, 14, 15, 20, 25, 16, 21, 26, 17, 22, 27, 18, 23, 28, 19, 24, 29],
+    "transposeOn_2_3_box": [0, 1, 2, 3, 4, 15, 16, 17, 18, 19, 5, 6, 7, 8, 9, 20, 21, 22, 23, 24, 10, 11, 12, 13, 14, 25, 26, 27, 28, 29],
+    "transposeOn_1_3_box": [0, 15, 5, 20, 10, 25, 1, 16, 6, 21, 11, 26, 2, 17, 7, 22, 12, 27, 3, 18, 8, 23, 13, 28, 4, 19, 9, 24, 14, 29],
+    "take_5": [[r * 10 + c for c in range(5)] for r in range(5)],
+    "drop_7": [[r * 10 + c for c in range(7, 10)] for r in range(5)],
+    "init": [[r * 10 + c for c in range(9)] for r in range(5)],
+    "tail": [[r * 10 + c for c in range(1, 10)] for r in range(5)]}
+# Prelude.hs:1490-1575  (++) and concatOn
+V["concat_doctest"] = {
+    "cite": "Prelude.hs:1490-1575", "m1": iota5x10, "m2_10x3": [[r * 3 + c for c in range(3)] for r in range(10)],
+    "append": [[r * 10 + c for c in range(10)] + [r * 3 + c for c in range(3)] for r in range(5)],
+    "m2_10x5": [[r * 5 + c for c in range(5)] for r in range(10)],
+    "concatOn_1": [[r * 10 + c for c in range(10)] + [r * 5 + c for c in range(5)] for r in range(5)],
+    "concatOn_2": [[r * 10 + c for c in range(5)] for r in range(5)] + [[r * 5 + c for c in range(5)] for r in range(10)]}
 # Language.hs:716-728  histogram via permute (+)
 V["histogram_doctest"] = {"cite": "Language.hs:716-728",
                           "keys": [0, 0, 1, 2, 1, 1, 2, 4, 8, 3, 4, 9, 8, 3, 2, 5, 5, 3, 1, 2], "bins": 10,

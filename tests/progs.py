@@ -756,3 +756,116 @@ def issue439():
     S0 = A.tarray(0, A.f32)
     one = A.generate(S0, A.nil, A.lam([A.unit], lambda ix: A.const(A.f32, 1)))
     return A.alet(S0, one, lambda a: A.map_(A.f32, A.lam([A.f32], lambda x: A.mul(A.f32, x, A.const(A.f32, 2))), a))
+
+
+# -- doctests of Language.hs / Prelude.hs, as the terms fusion would hand over
+def fold_all(ty, rank, z):
+    """foldAll f z = fold f z . flatten (Prelude.hs:665-672)"""
+    return A.alam([A.tarray(rank, ty)], lambda xs: A.fold(
+        binop(A.add, ty), A.const(ty, z), xs if rank == 1 else A.reshape(1, A.sh(A.shapesize(rank, A.shape(xs))), xs)))
+
+
+def all_any(which):
+    """all even / any even (Prelude.hs:777-806): and / or over a fused map"""
+    sh2 = A.tshape(2)
+    B = A.u8
+    even = lambda x: A.eq(Int, A.rem(Int, x, A.constI(2)), A.constI(0))
+    op, z = (A.land, 1) if which == "all" else (A.lor, 0)
+
+    def body(xs):
+        src = A.delayed(A.tarray(2, B), A.shape(xs), A.lam([sh2], lambda ix: even(A.index(xs, A.vexp(ix)))),
+                        A.lam([Int], lambda i: even(A.linearindex(xs, i))))
+        return A.fold(A.lam([B, B], lambda x, y: op(x, y)), A.const(B, z), src)
+    return A.alam([A.tarray(2, Int)], body)
+
+
+def prescanl_sum():
+    """prescanl f e = afst . scanl' f e (Prelude.hs:896-903)"""
+    V1, S0 = A.tarray(1, Int), A.tarray(0, Int)
+    return A.alam([V1], lambda xs: A.alet(A.tpair(V1, S0), A.scan_("l", binop(A.add, Int), A.constI(0), xs),
+                                           lambda st: st[0]))
+
+
+def postscanl_sum(e):
+    """postscanl f e = map (e `f`) . scanl1 f (Prelude.hs:913-921)"""
+    return A.alam([A.tarray(1, Int)], lambda xs: A.map_(
+        Int, A.lam([Int], lambda x: A.add(Int, A.constI(e), x)), A.scan("l", binop(A.add, Int), None, xs)))
+
+
+def filter_even():
+    """filter even over a vector (Prelude.hs:1623-1662): the kept elements and their number"""
+    sh1 = A.tshape(1)
+    V1, S0 = A.tarray(1, Int), A.tarray(0, Int)
+    even = lambda x: A.eq(Int, A.rem(Int, x, A.constI(2)), A.constI(0))
+
+    def body(xs):
+        flags = A.map_(Int, A.lam([Int], lambda x: A.cond(even(x), A.constI(1), A.constI(0))), xs)
+
+        def with_flags(fl):
+            def with_scan(st):
+                targets, total = st
+                kept = A.permute(
+                    A.lam([Int, A.wild(Int)], lambda x, _: x),
+                    A.generate(V1, A.sh(A.index(total, A.nil)), A.lam([sh1], lambda ix: A.constI(0))),
+                    A.lam([sh1], lambda ix: A.cond(A.eq(Int, A.index(fl, A.vexp(ix)), A.constI(0)), A.nothing(sh1),
+                                                   A.just(A.sh(A.index(targets, A.vexp(ix)))))), xs)
+                return A.apair(kept, total)
+            return A.alet(A.tpair(V1, S0), A.scan_("l", binop(A.add, Int), A.constI(0), fl), with_scan)
+        return A.alet(V1, flags, with_flags)
+    return A.alam([V1], body)
+
+
+def gather_if(ty=A.f32):
+    """gatherIf from mask (> 4) defaults input = zipWith (\\p g -> p ? g) (map pred mask) (zip (gather ..) defaults)"""
+    sh1 = A.tshape(1)
+
+    def body(frm, mask, defaults, xs):
+        ext = lambda: A.sh(A.min_(Int, A.untup_shape(mask)[0], A.min_(Int, A.untup_shape(frm)[0], A.untup_shape(defaults)[0])))
+
+        def at(ix):
+            return A.cond(A.gt(Int, A.index(mask, A.vexp(ix)), A.constI(4)),
+                          A.index(xs, A.sh(A.index(frm, A.vexp(ix)))), A.index(defaults, A.vexp(ix)))
+        return A.generate(A.tarray(1, ty), ext(), A.lam([sh1], at))
+    return A.alam([A.tarray(1, Int), A.tarray(1, Int), A.tarray(1, ty), A.tarray(1, ty)], body)
+
+
+def scatter_if(ty=Int):
+    """scatterIf to mask (> 4) defaults input (Prelude.hs:1788-1793)"""
+    sh1 = A.tshape(1)
+
+    def body(to, mask, over, xs):
+        ext = A.sh(A.min_(Int, A.untup_shape(to)[0], A.untup_shape(xs)[0]))
+        src = A.delayed(A.tarray(1, ty), ext, A.lam([sh1], lambda ix: A.index(xs, A.vexp(ix))),
+                        A.lam([Int], lambda i: A.linearindex(xs, i)))
+        return A.permute(A.lam([ty, A.wild(ty)], lambda x, _: x), over, A.lam([sh1], lambda ix: A.cond(
+            A.gt(Int, A.index(mask, A.vexp(ix)), A.constI(4)), A.just(A.sh(A.index(to, A.vexp(ix)))), A.nothing(sh1))), src)
+    return A.alam([A.tarray(1, Int), A.tarray(1, Int), A.tarray(1, ty), A.tarray(1, ty)], body)
+
+
+def reindex(rank, extent_of, source_of, ty=Int):
+    """backpermute with the result's extent and the source index given as functions of lists of
+    expressions (outermost first): reverseOn, transposeOn, take, drop, init, tail"""
+    shr = A.tshape(rank)
+    return A.alam([A.tarray(rank, ty)], lambda xs: A.backpermute(
+        rank, A.sh(*extent_of(lambda: A.untup_shape(xs))),
+        A.lam([shr], lambda ix: A.sh(*source_of(A.untup(ix), lambda: A.untup_shape(xs)))), xs))
+
+
+def concat_on(dim):
+    """concatOn _1 (the (++) of Prelude.hs:1518-1545) or _2 over matrices: one Generate"""
+    sh2 = A.tshape(2)
+
+    def body(m1, m2):
+        d1, d2 = (lambda: A.untup_shape(m1)), (lambda: A.untup_shape(m2))
+        if dim == 1:    # along the innermost dimension: rows = min, columns = sum
+            ext = lambda: A.sh(A.min_(Int, d1()[0], d2()[0]), A.add(Int, d1()[1], d2()[1]))
+        else:
+            ext = lambda: A.sh(A.add(Int, d1()[0], d2()[0]), A.min_(Int, d1()[1], d2()[1]))
+
+        def at(ix):
+            y, x = A.untup(ix)
+            if dim == 1:
+                return A.cond(A.lt(Int, x, d1()[1]), A.index(m1, A.sh(y, x)), A.index(m2, A.sh(y, A.sub(Int, x, d1()[1]))))
+            return A.cond(A.lt(Int, y, d1()[0]), A.index(m1, A.sh(y, x)), A.index(m2, A.sh(A.sub(Int, y, d1()[0]), x)))
+        return A.generate(A.tarray(2, Int), ext(), A.lam([sh2], at))
+    return A.alam([A.tarray(2, Int), A.tarray(2, Int)], body)
