@@ -329,6 +329,14 @@ def parity_cases():
     ef = [np.full(100, 1.01, np.float32), np.zeros(100, np.float32)]
     add("fold1_issue114", Q.issue114("fold1"), [ef], 1e-4 * 101)
     add("scan1_issue114", Q.issue114("scanl1"), [ef], 1e-4 * 101)
+    # ---- Spectral/BlackScholes, Imaginary/SAXPY and SASUM (transcendental functions come from
+    #      different libraries on the two sides: a few units in the last place)
+    for ty, tol in ((A.f32, 2e-4), (A.f64, 1e-11)):
+        psy = [rng.uniform(5, 30, 3000).astype(NPT[ty]), rng.uniform(1, 100, 3000).astype(NPT[ty]),
+               rng.uniform(0.25, 10, 3000).astype(NPT[ty])]
+        add("map_blackscholes_%s" % ty, Q.blackscholes(ty), [psy], tol)
+        add("map_saxpy_%s" % ty, Q.saxpy(ty), [np.array(1.75, NPT[ty]), _rand(rng, ty, (2000,)), _rand(rng, ty, (1900,))], None)
+        add("fold_sasum_%s" % ty, Q.sasum(ty), [_rand(rng, ty, (5000,))], 1e-4 * 4 * 5000 if ty == A.f32 else 1e-9)
     # ---- the benchmark programs at small size
     add("dotp_1000", P.dotp(), [_rand(rng, A.f32, (1000,)), _rand(rng, A.f32, (900,))], 1e-4 * 16 * 900)
     add("histogram_zipf", P.histogram(97), [rng.integers(0, 97, 3000).astype(np.int32)], None)

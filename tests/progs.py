@@ -869,3 +869,53 @@ def concat_on(dim):
             return A.cond(A.lt(Int, y, d1()[0]), A.index(m1, A.sh(y, x)), A.index(m2, A.sh(A.sub(Int, y, d1()[0]), x)))
         return A.generate(A.tarray(2, Int), ext(), A.lam([sh2], at))
     return A.alam([A.tarray(2, Int), A.tarray(2, Int)], body)
+
+
+# -- Test/NoFib/Spectral/BlackScholes.hs and Imaginary/{SAXPY,SASUM}.hs
+def blackscholes(ty=A.f32):
+    t3, t2 = A.ttup(ty, ty, ty), A.ttup(ty, ty)
+    c = lambda x: A.const(ty, x)
+    mul, add, sub, div = (lambda a, b: A.mul(ty, a, b)), (lambda a, b: A.add(ty, a, b)), \
+        (lambda a, b: A.sub(ty, a, b)), (lambda a, b: A.fdiv(ty, a, b))
+    let = lambda e, k: A.let(ty, e, k)
+    coeff = [0.31938153, -0.356563782, 1.781477937, -1.821255978, 1.330274429]
+
+    def cnd(d, k):
+        def tail(kk):
+            # horner coeff x = x * foldr1 (\a b -> a + x*b) coeff
+            acc = c(coeff[-1])
+            for a in coeff[-2::-1]:
+                acc = add(c(a), mul(kk, acc))
+            poly = mul(kk, acc)
+            cn = mul(mul(c(0.39894228040143267793994605993438), A.exp(ty, mul(mul(c(-0.5), d), d))), poly)
+            return let(cn, lambda cv: k(A.cond(A.gt(ty, d, c(0)), sub(c(1.0), cv), cv)))
+        return let(div(c(1.0), add(c(1.0), mul(c(0.2316419), A.abs_(ty, d)))), tail)
+
+    def go(v):
+        price, strike, years = A.untup(v)
+        r, vol = c(0.02), c(0.30)
+        return let(mul(vol, A.sqrt(ty, years)), lambda vsq: let(
+            div(add(A.log(ty, div(price, strike)), mul(add(r, mul(mul(c(0.5), vol), vol)), years)), vsq), lambda d1: let(
+                sub(d1, vsq), lambda d2: cnd(d1, lambda c1: let(c1, lambda cd1: cnd(d2, lambda c2: let(c2, lambda cd2: let(
+                    mul(strike, A.exp(ty, mul(A.neg(ty, r), years))), lambda xe: A.tup(
+                        sub(mul(price, cd1), mul(xe, cd2)),
+                        sub(mul(xe, sub(c(1.0), cd2)), mul(price, sub(c(1.0), cd1))))))))))))
+
+    return A.alam([A.tarray(1, t3)], lambda xs: A.map_(t2, A.lam([t3], go), xs))
+
+
+def saxpy(ty=A.f32):
+    """zipWith (\\x y -> alpha * x + y) with alpha a rank-0 argument"""
+    return A.alam([A.tarray(0, ty), A.tarray(1, ty), A.tarray(1, ty)], lambda alpha, xs, ys: A.zipwith(
+        ty, A.lam([ty, ty], lambda x, y: A.add(ty, A.mul(ty, A.index(alpha, A.nil), x), y)), xs, ys))
+
+
+def sasum(ty=A.f32):
+    """fold (+) 0 . map abs: the map fused into the fold"""
+    sh1 = A.tshape(1)
+
+    def body(xs):
+        src = A.delayed(A.tarray(1, ty), A.shape(xs), A.lam([sh1], lambda ix: A.abs_(ty, A.index(xs, A.vexp(ix)))),
+                        A.lam([Int], lambda i: A.abs_(ty, A.linearindex(xs, i))))
+        return A.fold(binop(A.add, ty), A.const(ty, 0), src)
+    return A.alam([A.tarray(1, ty)], body)

@@ -315,3 +315,24 @@ def test_oracle_on_issue114_and_issue409():
     assert close(vals, np.float32(x) * np.arange(1, n + 1, dtype=np.float32)) and close(errs, 0.0)
     assert O.run_n(Q.issue409(A.f64).text(), np.array(v["issue409"]["x"])) == 1 + math.tanh(-1)
     assert abs(float(O.run_n(Q.issue409(A.f32).text(), np.array(1.0, np.float32))) - (1 + math.tanh(-1))) < 1e-6
+
+
+def test_oracle_on_blackscholes_against_numpy():
+    # Spectral/BlackScholes.hs restated with numpy in Float64 (blackscholesRef, :96-118)
+    from . import progs as Q
+    rng = np.random.default_rng(13)
+    p, s, y = rng.uniform(5, 30, 500), rng.uniform(1, 100, 500), rng.uniform(0.25, 10, 500)
+    r, v = 0.02, 0.30
+
+    def cnd(d):
+        k = 1.0 / (1.0 + 0.2316419 * np.abs(d))
+        poly = k * (0.31938153 + k * (-0.356563782 + k * (1.781477937 + k * (-1.821255978 + k * 1.330274429))))
+        c = 0.39894228040143267793994605993438 * np.exp(-0.5 * d * d) * poly
+        return np.where(d > 0, 1.0 - c, c)
+    vs = v * np.sqrt(y)
+    d1 = (np.log(p / s) + (r + 0.5 * v * v) * y) / vs
+    d2 = d1 - vs
+    xe = s * np.exp(-r * y)
+    call, put = O.run_n(Q.blackscholes(A.f64).text(), [p, s, y])
+    assert np.allclose(call, p * cnd(d1) - xe * cnd(d2), rtol=1e-12, atol=1e-12)
+    assert np.allclose(put, xe * (1.0 - cnd(d2)) - p * (1.0 - cnd(d1)), rtol=1e-12, atol=1e-12)
