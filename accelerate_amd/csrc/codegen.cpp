@@ -804,6 +804,54 @@ bool Codegen::isCommutative(const Sx& f, std::string* op, ST* st) {
   return true;
 }
 
+// Is f a component-wise combination of tuples, \(x0, .., xn) (y0, .., yn) -> (x0 (+)0 y0, ..),
+// with every (+)k one of the commutative primitives that exist as hardware atomics?  Then the
+// components can be combined independently of each other, one atomic each.  Accepts the form
+// the front end produces: both arguments bound by fully destructuring left-hand sides, the body
+// a tuple of primitive applications to the matching pair of variables (in either order).
+static bool componentwiseAtomic(const Sx& f, const std::vector<ST>& leaves, std::vector<std::string>& ops) {
+  struct Lhs {
+    static bool singles(const Sx& l, int& n) {  // counts variables; false on wildcards
+      if (l.is("single")) { ++n; return true; }
+      if (l.is("pair") && l.size() == 3) return singles(l.at(1), n) && singles(l.at(2), n);
+      if (l.is("wild")) return l.at(1).isAtom("unit");
+      return false;
+    }
+    static bool flat(const Sx& e, std::vector<const Sx*>& out) {  // leaves of a tuple expression
+      if (e.isAtom("nil")) return true;
+      if (e.is("pair") && e.size() == 3) return flat(e.at(1), out) && flat(e.at(2), out);
+      out.push_back(&e);
+      return true;
+    }
+  };
+  const int n = (int)leaves.size();
+  if (n < 2 || !f.is("lam")) return false;
+  const Sx& g = f.at(2);
+  if (!g.is("lam")) return false;
+  int nx = 0, ny = 0;
+  if (!Lhs::singles(f.at(1), nx) || !Lhs::singles(g.at(1), ny) || nx != n || ny != n) return false;
+  std::vector<const Sx*> parts;
+  if (!Lhs::flat(g.at(2), parts) || (int)parts.size() != n) return false;
+  ops.clear();
+  for (int k = 0; k < n; ++k) {
+    const Sx& b = *parts[k];
+    if (!b.is("prim") || b.size() != 4 || !isST(b.at(2)) || parseST(b.at(2)) != leaves[k]) return false;
+    const ST t = leaves[k];
+    if (stIsVec(t) || (stSize(t) != 4 && stSize(t) != 8)) return false;
+    const std::string& o = b.at(1).s;
+    const bool okOp = o == "add" || (stIsInt(t) && (o == "min" || o == "max" || o == "band" || o == "bor" || o == "bxor"));
+    if (!okOp) return false;
+    const Sx& arg = b.at(3);
+    if (!arg.is("pair") || !arg.at(1).is("var") || !arg.at(2).is("var")) return false;
+    // variable levels: x_k = k, y_k = n + k; de Bruijn index = 2n - 1 - level
+    const long long ix = 2 * n - 1 - k, iy = n - 1 - k;
+    const long long a = arg.at(1).at(1).asInt(), c = arg.at(2).at(1).asInt();
+    if (!((a == ix && c == iy) || (a == iy && c == ix))) return false;
+    ops.push_back(o);
+  }
+  return true;
+}
+
 static int vecFor(const std::vector<ST>& leaves, const std::vector<ArraySlot>& arrays) {
   int maxLeaf = 1, eltBytes = 0;
   for (ST s : leaves) {
@@ -1260,6 +1308,8 @@ KernelSource Codegen::permute(const Sx& f, const ArrayR& dst, const Sx& p, const
            (op == "add" ? (st != ST::F16) : (op != "mul" && stIsInt(st))))
     mode = "atomic";
   else if (wide) mode = "cas";
+  std::vector<std::string> leafOps;
+  if (mode == "lock" && componentwiseAtomic(f, leaves, leafOps)) mode = "atomics";
   std::string lds;
   std::string u = "  ACC_DEV void update(const Env& env, const Out& out, i64 j, const Elt& x, u32* locks) {\n";
   if (mode == "store") {
@@ -1285,6 +1335,16 @@ KernelSource Codegen::permute(const Sx& f, const ArrayR& dst, const Sx& p, const
     lds += "  ACC_DEV Prim identity() { return " + idv + "; }\n";
     lds += "  ACC_DEV void lds_update(Prim* p, const Elt& x) { (void)" + fn + "(p, x.c0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP); }\n";
     lds += "  ACC_DEV void global_update(const Out& out, i64 j, Prim v) { (void)" + fn + "(&out.o0[j], v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); }\n";
+  } else if (mode == "atomics") {
+    // component-wise combination: the components do not see each other, one atomic each
+    for (size_t k = 0; k < leaves.size(); ++k) {
+      const std::string& o = leafOps[k];
+      std::string fn = o == "add" ? "__hip_atomic_fetch_add" : o == "min" ? "__hip_atomic_fetch_min"
+                     : o == "max" ? "__hip_atomic_fetch_max" : o == "band" ? "__hip_atomic_fetch_and"
+                     : o == "bor" ? "__hip_atomic_fetch_or" : "__hip_atomic_fetch_xor";
+      const std::string K = std::to_string(k);
+      u += "    (void)" + fn + "(&out.o" + K + "[j], x.c" + K + ", __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);\n";
+    }
   } else if (mode == "cas") {
     std::string B = stSize(leaves[0]) == 4 ? "u32" : "u64", T = stName(leaves[0]);
     u += "    " + B + "* a_ = (" + B + "*)&out.o0[j];\n";

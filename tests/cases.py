@@ -262,6 +262,15 @@ def parity_cases():
                 xs = np.round(xs * 4) / 4     # sums of quarters are exact in any order
             add("permute_add_%s_%d_%d" % (ty, sr, dr), Q.accumulate(ty, sr, dr), [xs, to, _rand(rng, ty, dshape, -5, 5)
                 if ty != A.f32 else np.zeros(dshape, np.float32)], None)
+    # ---- permute with a component-wise combination over pairs (one atomic per component)
+    to = rng.integers(0, 29, 3000).astype(np.int64)
+    quarters = lambda n: (np.round(rng.uniform(-20, 20, n) * 4) / 4).astype(np.float32)
+    add("permute_pairs_f32_add_add", Q.accumulate_pairs(), [[quarters(3000), quarters(3000)], to,
+                                                            [np.zeros(29, np.float32), quarters(29)]], None)
+    add("permute_pairs_i64_add_i32_max", Q.accumulate_pairs(A.i64, A.i32, A.max_),
+        [[_rand(rng, A.i64, (3000,)), _rand(rng, A.i32, (3000,))], to, [_rand(rng, A.i64, (29,)), _rand(rng, A.i32, (29,))]], None)
+    add("permute_pairs_u32_add_u64_bxor", Q.accumulate_pairs(A.u32, A.u64, A.bxor),
+        [[_rand(rng, A.u32, (3000,)), _rand(rng, A.u64, (3000,))], to, [_rand(rng, A.u32, (29,)), _rand(rng, A.u64, (29,))]], None)
     # ---- backpermute (Prelude/Backpermute.hs)
     add("transpose_33x17", Q.transpose(A.i32), [_rand(rng, A.i32, (33, 17))], None)
     add("gather", Q.gather(A.f32), [rng.integers(0, 100, 257).astype(np.int64), _rand(rng, A.f32, (100,))], None)

@@ -919,3 +919,17 @@ def sasum(ty=A.f32):
                         A.lam([Int], lambda i: A.abs_(ty, A.linearindex(xs, i))))
         return A.fold(binop(A.add, ty), A.const(ty, 0), src)
     return A.alam([A.tarray(1, ty)], body)
+
+
+def accumulate_pairs(t0=A.f32, t1=A.f32, op1=A.add):
+    """permute of a component-wise combination over pairs: (a, b) (c, d) -> (a + c, b `op1` d)
+    (complex numbers, sum-and-maximum): no cell sees the other component, one atomic each"""
+    sh1 = A.tshape(1)
+    t2 = A.ttup(t0, t1)
+
+    def f(x, y):
+        a, b = A.untup(x)
+        c, d = A.untup(y)
+        return A.tup(A.add(t0, a, c), op1(t1, d, b))
+    return A.alam([A.tarray(1, t2), A.tarray(1, Int), A.tarray(1, t2)], lambda xs, to, dfl: A.permute(
+        A.lam([t2, t2], f), dfl, A.lam([sh1], lambda ix: A.just(A.sh(A.index(to, A.vexp(ix))))), xs))
