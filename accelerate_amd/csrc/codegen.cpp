@@ -809,7 +809,8 @@ bool Codegen::isCommutative(const Sx& f, std::string* op, ST* st) {
 // components can be combined independently of each other, one atomic each.  Accepts the form
 // the front end produces: both arguments bound by fully destructuring left-hand sides, the body
 // a tuple of primitive applications to the matching pair of variables (in either order).
-static bool componentwiseAtomic(const Sx& f, const std::vector<ST>& leaves, std::vector<std::string>& ops) {
+static bool componentwiseAtomic(const Sx& f, const std::vector<ST>& leaves, std::vector<std::string>& ops,
+                                bool anyCommutative = false) {
   struct Lhs {
     static bool singles(const Sx& l, int& n) {  // counts variables; false on wildcards
       if (l.is("single")) { ++n; return true; }
@@ -837,10 +838,15 @@ static bool componentwiseAtomic(const Sx& f, const std::vector<ST>& leaves, std:
     const Sx& b = *parts[k];
     if (!b.is("prim") || b.size() != 4 || !isST(b.at(2)) || parseST(b.at(2)) != leaves[k]) return false;
     const ST t = leaves[k];
-    if (stIsVec(t) || (stSize(t) != 4 && stSize(t) != 8)) return false;
     const std::string& o = b.at(1).s;
-    const bool okOp = o == "add" || (stIsInt(t) && (o == "min" || o == "max" || o == "band" || o == "bor" || o == "bxor"));
-    if (!okOp) return false;
+    if (anyCommutative) {  // for reductions: any commutative primitive at any scalar type
+      if (stIsVec(t) || !(o == "add" || o == "mul" || o == "min" || o == "max" || o == "band" || o == "bor" || o == "bxor"))
+        return false;
+    } else {
+      if (stIsVec(t) || (stSize(t) != 4 && stSize(t) != 8)) return false;
+      const bool okOp = o == "add" || (stIsInt(t) && (o == "min" || o == "max" || o == "band" || o == "bor" || o == "bxor"));
+      if (!okOp) return false;
+    }
     const Sx& arg = b.at(3);
     if (!arg.is("pair") || !arg.at(1).is("var") || !arg.at(2).is("var")) return false;
     // variable levels: x_k = k, y_k = n + k; de Bruijn index = 2n - 1 - level
@@ -925,6 +931,11 @@ KernelSource Codegen::fold(const Sx& f, const Sx* seed, const Operand& src) {
   const TypeP elt = src.r.elt;
   std::string body;
   bool comm = isCommutative(f);
+  {
+    // component-wise combinations of tuples of commutative primitives commute as a whole
+    std::vector<std::string> ops;
+    if (!comm && componentwiseAtomic(f, typeLeaves(elt), ops, true)) comm = true;
+  }
   body += std::string("  static constexpr bool kCommutative = ") + (comm ? "true" : "false") + ";\n";
   body += std::string("  static constexpr bool kSeeded = ") + (seed ? "true" : "false") + ";\n";
   {
