@@ -28,6 +28,7 @@ struct FoldSegParams {
   void* carry;    // [tiles] (head seen, value since the last head) of each tile
   void* pend;     // [tiles] value of the tile's one segment end that precedes all its heads
   i64* pend_at;   // [tiles] boundary number of that end, or -1
+  u32* err;       // host-visible word: 1 = "empty segment" (what the reference's boundsCheck reports)
 };
 
 // part[t] = number of boundaries that lie before position t * TILE of the stream.  One
@@ -66,6 +67,10 @@ acc_foldseg_partition(Spec::Env env, Spec::Out out, FoldSegParams p) {
       lo = prev < 0 ? 0 : prev / (i64)C::TILE + 1;
       // an empty segment yields z; it is written here, where every boundary has a thread of its own
       if (Spec::kSeeded && s > 0 && prev == pos) Spec::store(out, row * p.nseg + s - 1, Spec::seed(env));
+      // foldSeg: offsets must not decrease; fold1Seg: every segment needs an element
+      // (Interpreter.hs:407, 424)
+      if (s > 0 && (prev > pos || (!Spec::kSeeded && prev == pos)))
+        __hip_atomic_store(p.err, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
     }
     hi = pos < 0 ? -1 : pos / (i64)C::TILE;
     if (hi > p.tiles - 1) hi = p.tiles - 1;

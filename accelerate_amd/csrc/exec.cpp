@@ -1255,6 +1255,7 @@ AValP Program::eval(const Sx& n, AEnv& aenv) {
     args.push_back((uint64_t)(uintptr_t)carry->bufs[0]->p);
     args.push_back((uint64_t)(uintptr_t)pend->bufs[0]->p);
     args.push_back((uint64_t)(uintptr_t)pendAt->bufs[0]->p);
+    args.push_back((uint64_t)(uintptr_t)ctx_.errorWord());
     const int64_t boundaries = rows * (nseg + 1);
     if ((boundaries + 255) / 256 > 0x7fffffffLL) throw Error("foldSeg: too many segments for one launch");
     ctx_.launch(plan.k, "acc_foldseg_partition", (unsigned)((boundaries + 255) / 256), 256, args);

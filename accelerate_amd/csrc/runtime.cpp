@@ -65,6 +65,7 @@ Context::~Context() {
   purge();
   for (auto& kv : live_) (void)hipFree(kv.first);
   if (staging_) (void)hipHostFree(staging_);
+  if (errHost_) (void)hipHostFree(errHost_);
   if (scan_.desc) (void)hipFree(scan_.desc);
   if (scan_.ticket) (void)hipFree(scan_.ticket);
   (void)hipStreamDestroy(stream_);
@@ -194,6 +195,7 @@ void Context::peek(void* host, const void* dev, size_t bytes) {
     std::memcpy(dst + off, st, n);
   }
   stats.bytesCopiedFromRemote += (long long)bytes;
+  raiseDeviceError();
 }
 
 void Context::copy(void* dst, const void* src, size_t bytes) {
@@ -208,6 +210,24 @@ void Context::fill0(void* dev, size_t bytes) {
 
 void Context::sync() {
   if (device_ >= 0) hipCheck(hipStreamSynchronize(stream_), "hipStreamSynchronize");
+  raiseDeviceError();
+}
+
+unsigned* Context::errorWord() {
+  if (!errDev_) {
+    hipCheck(hipHostMalloc((void**)&errHost_, 64, hipHostMallocMapped), "hipHostMalloc(error word)");
+    *errHost_ = 0;
+    hipCheck(hipHostGetDevicePointer((void**)&errDev_, errHost_, 0), "hipHostGetDevicePointer");
+  }
+  return errDev_;
+}
+
+// call after the stream has been waited for
+void Context::raiseDeviceError() {
+  if (!errHost_) return;
+  const unsigned code = __atomic_exchange_n(errHost_, 0u, __ATOMIC_ACQ_REL);
+  if (code == 1) throw Error("empty segment");  // foldSegOp / fold1SegOp, Interpreter.hs:407, 424
+  if (code != 0) throw Error("a kernel reported error " + std::to_string(code));
 }
 
 Context::ScanState& Context::scanState(size_t descBytes) {

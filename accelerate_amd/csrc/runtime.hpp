@@ -61,6 +61,11 @@ class Context : public std::enable_shared_from_this<Context> {
   void copy(void* dst, const void* src, size_t bytes);    // D->D
   void fill0(void* dev, size_t bytes);
   void sync();
+  // A word of pinned host memory that kernels write when they meet what the reference reports
+  // through boundsCheck (Error.hs:33-62; e.g. an empty segment under fold1Seg).  Kernels get
+  // errorWord(); every call that waits for the stream (sync, peek) then raises the error.
+  unsigned* errorWord();
+  void raiseDeviceError();
 
   // Looks the kernel up (memory, then disk) or starts its compilation on a worker thread:
   // the kernels of a program compile side by side.  wait() returns when the code object is
@@ -95,6 +100,8 @@ class Context : public std::enable_shared_from_this<Context> {
   std::map<size_t, std::vector<void*>> nursery_;            // rounded size -> free blocks
   std::unordered_map<std::string, KernelP> kernels_;
   void* staging_ = nullptr;
+  unsigned* errHost_ = nullptr;  // pinned, mapped: written by kernels, read here
+  unsigned* errDev_ = nullptr;
   size_t stagingBytes_ = 0;
   ScanState scan_;
   void ensureLoaded(const KernelP& k);

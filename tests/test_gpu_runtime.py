@@ -45,6 +45,27 @@ def test_atrace_hands_message_and_arrays_to_the_callback(gpu_ctx, capfd):
     assert "partial sums: Array (Z :. 500) i64, Array (Z) i64" in capfd.readouterr().err
 
 
+def test_fold1seg_reports_an_empty_segment(gpu_ctx):
+    # fold1SegOp checks every segment for an element (boundsCheck "empty segment",
+    # Interpreter.hs:424); the kernel that walks the boundaries reports it, and the next call
+    # that waits for the stream raises it.  The context stays usable.
+    from . import progs as Q
+    V1 = A.tarray(1, A.i64)
+    prog = A.alam([V1, V1], lambda vals, seg: A.alet(
+        V1, A.scan("l", Q.binop(A.add, A.i64), A.const(A.i64, 0), seg),
+        lambda offs: A.foldseg(A.i64, Q.binop(A.add, A.i64), None, vals, offs)))
+    run = gpu_ctx.compile(prog)
+    vals = np.arange(10, dtype=np.int64)
+    assert same(run(vals, np.array([3, 2, 5], np.int64)), np.array([3, 7, 35], np.int64))
+    res = run.execute(gpu_ctx.to_device(vals, V1), gpu_ctx.to_device(np.array([3, 0, 7], np.int64), V1))
+    with pytest.raises(hip.AccError, match="empty segment"):
+        res.to_host()
+    assert same(run(vals, np.array([4, 6], np.int64)), np.array([6, 39], np.int64))
+    # with a seed the empty segment is legal and yields the seed (Interpreter.hs:407)
+    assert same(gpu_ctx.compile(P.foldseg_sum(A.i64, A.i64, 1, 5))(vals, np.array([3, 0, 7], np.int64)),
+                np.array([8, 5, 47], np.int64))
+
+
 def test_awhile_jacobi_counts_iterations(gpu_ctx):
     # 20 sweeps driven by awhile (Interpreter.hs:222-229).  The loop counter is a rank-0
     # array made by `unit` from index arithmetic, so the host follows its value and the
