@@ -1304,10 +1304,23 @@ KernelSource Codegen::permute(const Sx& f, const ArrayR& dst, const Sx& p, const
     if (m->k != Val::Pair || m->a->k != Val::Leaf || m->b->k != Val::Pair)
       throw Error("permute: index function must return a Maybe index (tag, ((), ix))");
     std::string tag = m->a->ex;
-    em.line("if (" + tag + " == 0) return false;");
-    em.line("j = " + toIndex(shapeOf(o), m->b->b, em) + ";");
-    em.line("return true;");
-    body += fnHead("bool", "target", "const Env& env, i64 i, i64& j") + em.code + "  }\n";
+    {
+      // a target outside the destination is an error in the reference (toIndex's bounds check,
+      // Shape.hs:98-106); here it is dropped instead of written, and the skeleton reports it.  The
+      // function stays free of stores and branches, so that the loads of many sources can be in
+      // flight.  0: Nothing, 1: j is the target, 2: the target lies outside the destination.
+      std::vector<std::string> dd, ii;
+      shapeDims(shapeOf(o), dd);
+      shapeDims(m->b->b, ii);
+      if (dd.size() != ii.size()) throw Error("permute: index function returns an index of the wrong rank");
+      std::string bad;
+      for (size_t d = 0; d < dd.size(); ++d)
+        bad += (bad.empty() ? "" : " | ") + std::string("((u64)") + ii[d] + " >= (u64)" + dd[d] + ")";
+      if (bad.empty()) bad = "false";
+      em.line("j = " + toIndex(shapeOf(o), m->b->b, em) + ";");
+      em.line("return " + tag + " == 0 ? 0 : ((" + bad + ") ? 2 : 1);");
+    }
+    body += fnHead("int", "target", "const Env& env, i64 i, i64& j") + em.code + "  }\n";
   }
   // how to combine into the destination
   std::string mode = "lock", op;

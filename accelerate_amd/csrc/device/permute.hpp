@@ -3,8 +3,8 @@
 // out[dst] with f new old.  Sources are visited in parallel, so the result is defined for
 // associative and commutative f only (AST.hs:420-423).
 //
-// S::target turns the linear source index into the linear destination index (false for
-// Nothing); S::update applies the combination with the cheapest mechanism the generated
+// S::target turns the linear source index into the linear destination index (0 for Nothing,
+// 2 for an index outside the destination, which the skeleton drops and reports); S::update applies the combination with the cheapest mechanism the generated
 // code could prove correct for f and the element type:
 //   store   f ignores the old value: plain store
 //   atomic  f is +, min, max, and, or, xor on a 32/64-bit scalar: one hardware atomic
@@ -16,19 +16,24 @@
 struct PermuteParams {
   i64 n;       // number of source elements
   u32* locks;  // one word per destination element, zero when free (lock mode only)
+  u32* err;    // host-visible word: 2 = a target outside the destination
 };
 
 extern "C" __global__ void __launch_bounds__(ACC_BLOCK)
 acc_permute(Spec::Env env, Spec::Out out, PermuteParams p) {
   typedef Spec S;
   const i64 stride = (i64)gridDim.x * ACC_BLOCK;
+  bool bad = false;
   for (i64 i = (i64)blockIdx.x * ACC_BLOCK + threadIdx.x; i < p.n; i += stride) {
     i64 j;
-    if (S::target(env, i, j)) {
+    const int t = S::target(env, i, j);
+    if (t == 1) {
       S::Elt x = S::in_linear(env, i);
       S::update(env, out, j, x, p.locks);
     }
+    bad = bad || t == 2;
   }
+  if (bad) __hip_atomic_store(p.err, 2u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
 }
 
 #ifdef ACC_PERMUTE_LDS
@@ -67,6 +72,7 @@ struct PermuteLdsParams {
   i64 nparts;  // destination ranges
   i64 part;    // elements per range
   i64 dst_n;   // destination elements
+  u32* err;    // host-visible word: 2 = a target outside the destination
 };
 
 extern "C" __global__ void __launch_bounds__(ACC_PERMUTE_LDS_BLOCK)
@@ -88,6 +94,7 @@ acc_permute_lds(Spec::Env env, Spec::Out out, PermuteLdsParams p) {
   // a step are computed (their loads issued) before the first update, which keeps enough
   // loads in flight for a single resident workgroup per CU to stream at HBM speed
   const i64 step = (i64)ACC_PERMUTE_LDS_BLOCK * 4 * ACC_PERMUTE_UNROLL;
+  bool bad = false;  // a target outside the destination was met (reported once, at the end)
   for (i64 base = begin; base < end; base += step) {
     if (base + step <= end) {
       i64 j[ACC_PERMUTE_UNROLL][4];
@@ -96,7 +103,11 @@ acc_permute_lds(Spec::Env env, Spec::Out out, PermuteLdsParams p) {
       for (int g = 0; g < ACC_PERMUTE_UNROLL; ++g) {
         const i64 i0 = base + ((i64)g * ACC_PERMUTE_LDS_BLOCK + threadIdx.x) * 4;
 #pragma unroll
-        for (int k = 0; k < 4; ++k) ok[g][k] = S::target(env, i0 + k, j[g][k]);
+        for (int k = 0; k < 4; ++k) {
+          const int t = S::target(env, i0 + k, j[g][k]);
+          ok[g][k] = t == 1;
+          bad = bad || t == 2;
+        }
       }
 #pragma unroll
       for (int g = 0; g < ACC_PERMUTE_UNROLL; ++g) {
@@ -108,7 +119,9 @@ acc_permute_lds(Spec::Env env, Spec::Out out, PermuteLdsParams p) {
     } else {
       for (i64 i = base + threadIdx.x; i < end; i += ACC_PERMUTE_LDS_BLOCK) {
         i64 j;
-        if (S::target(env, i, j) && j >= lo && j < hi) S::lds_update(&priv[j - lo], S::in_linear(env, i));
+        const int t = S::target(env, i, j);
+        if (t == 1 && j >= lo && j < hi) S::lds_update(&priv[j - lo], S::in_linear(env, i));
+        bad = bad || t == 2;
       }
     }
   }
@@ -117,5 +130,6 @@ acc_permute_lds(Spec::Env env, Spec::Out out, PermuteLdsParams p) {
     const Prim v = priv[i];
     if (v != id) S::global_update(out, lo + i, v);
   }
+  if (bad) __hip_atomic_store(p.err, 2u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
 }
 #endif

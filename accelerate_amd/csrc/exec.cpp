@@ -1153,11 +1153,13 @@ AValP Program::eval(const Sx& n, AEnv& aenv) {
       args.push_back((uint64_t)nparts);
       args.push_back((uint64_t)part);
       args.push_back((uint64_t)out->size());
+      args.push_back((uint64_t)(uintptr_t)ctx_.errorWord());
       ctx_.launch(plan.k, "acc_permute_lds", (unsigned)(groups * nparts), 1024, args);
       return avArr(out);
     }
     args.push_back((uint64_t)cnt);
     args.push_back(locks ? (uint64_t)(uintptr_t)locks->bufs[0]->p : 0);
+    args.push_back((uint64_t)(uintptr_t)ctx_.errorWord());
     int64_t grid = std::min<int64_t>((cnt + 255) / 256, 256 * 32);
     ctx_.launch(plan.k, "acc_permute", (unsigned)grid, 256, args);
     return avArr(out);

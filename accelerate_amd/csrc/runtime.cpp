@@ -227,6 +227,7 @@ void Context::raiseDeviceError() {
   if (!errHost_) return;
   const unsigned code = __atomic_exchange_n(errHost_, 0u, __ATOMIC_ACQ_REL);
   if (code == 1) throw Error("empty segment");  // foldSegOp / fold1SegOp, Interpreter.hs:407, 424
+  if (code == 2) throw Error("index out of bounds");  // permute target, Shape.hs:98-106
   if (code != 0) throw Error("a kernel reported error " + std::to_string(code));
 }
 

@@ -87,7 +87,8 @@ int acchip_event_elapsed_ms(acchip_event* start, acchip_event* stop, float* ms);
 void acchip_event_destroy(acchip_event* ev);
 /* Wait for everything queued on the context's stream.  Conditions that only a kernel can see and
  * that the reference reports through boundsCheck (Error.hs:33-62; "empty segment" of fold1Seg,
- * Interpreter.hs:424) are raised here and by acchip_peek, i.e. by the first call after the
+ * Interpreter.hs:424; "index out of bounds" for a permute target outside the destination, which
+ * is not written) are raised here and by acchip_peek, i.e. by the first call after the
  * offending launch that waits for the stream: it fails with that message. */
 int acchip_sync(acchip_ctx* ctx);
 

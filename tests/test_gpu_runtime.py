@@ -66,6 +66,23 @@ def test_fold1seg_reports_an_empty_segment(gpu_ctx):
                 np.array([8, 5, 47], np.int64))
 
 
+@pytest.mark.parametrize("n", [1000, 1 << 21])
+def test_permute_reports_a_target_outside_the_destination(gpu_ctx, n):
+    # the reference's toIndex checks the target (Shape.hs:98-106); here such a source is dropped
+    # instead of written, reported, and raised by the next call that waits for the stream --
+    # through both permute kernels (global atomics; workgroup-private copies from 2^20 sources on)
+    keys = (np.arange(n) % 10).astype(np.int32)
+    run = gpu_ctx.compile(P.histogram(10))
+    assert same(run(keys), np.bincount(keys, minlength=10).astype(np.int32))
+    bad = keys.copy()
+    bad[n // 2] = 10
+    bad[7] = -3
+    res = run.execute(gpu_ctx.to_device(bad, A.tarray(1, A.i32)))
+    with pytest.raises(hip.AccError, match="index out of bounds"):
+        res.to_host()
+    assert same(run(keys), np.bincount(keys, minlength=10).astype(np.int32))    # the context goes on
+
+
 def test_awhile_jacobi_counts_iterations(gpu_ctx):
     # 20 sweeps driven by awhile (Interpreter.hs:222-229).  The loop counter is a rank-0
     # array made by `unit` from index arithmetic, so the host follows its value and the
