@@ -1139,13 +1139,19 @@ AValP Program::eval(const Sx& n, AEnv& aenv) {
     // where plain global atomics are for uniform keys (2.5 ms); for Zipf keys those take 110 ms.
     const char* pe = std::getenv("ACCHIP_PERMUTE_PARTS");
     const int64_t maxParts = pe ? std::atoll(pe) : 128;
-    if (plan.mode == "atomic" && cnt >= (1 << 20) && out->size() <= maxParts * partMax) {
+    // From 2^20 sources on, and from 2^12 on when every destination element receives several of
+    // them (few destinations under many sources contend in the memory-side atomic units: 2^16
+    // keys into 256 bins take 33 us through global atomics, 2^14 keys into 16 bins 47 us,
+    // against 9 us this way).
+    const bool many = cnt >= (1 << 20) || (cnt >= (1 << 12) && cnt >= 4 * out->size());
+    if (plan.mode == "atomic" && many && out->size() <= maxParts * partMax) {
       const int64_t nparts = (out->size() + partMax - 1) / partMax;
       const int64_t part = (out->size() + nparts - 1) / nparts;
       // one workgroup per CU in total (each holds 128 KiB of LDS): fewer, longer workgroups
-      // mean fewer private copies to add into the destination at the end
+      // mean fewer private copies to add into the destination at the end; at least 16 Ki
+      // sources per workgroup
       const char* ge = std::getenv("ACCHIP_PERMUTE_GROUPS");
-      int64_t groups = ge ? std::atoll(ge) : 256 / nparts;
+      int64_t groups = ge ? std::atoll(ge) : std::min<int64_t>(256 / nparts, cnt / 16384);
       groups = std::max<int64_t>(8, groups / 8 * 8);
       int64_t chunk = ((cnt + groups - 1) / groups + 3) / 4 * 4;
       args.push_back((uint64_t)cnt);
