@@ -1343,22 +1343,7 @@ KernelSource Codegen::permute(const Sx& f, const ArrayR& dst, const Sx& p, const
                    : op == "max" ? "__hip_atomic_fetch_max" : op == "band" ? "__hip_atomic_fetch_and"
                    : op == "bor" ? "__hip_atomic_fetch_or" : "__hip_atomic_fetch_xor";
     u += "    (void)" + fn + "(&out.o0[j], x.c0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);\n";
-    // pieces of the LDS-privatised variant (permute.hpp): identity, LDS and global updates
-    std::string T = stName(st), idv;
-    if (op == "add" || op == "bor" || op == "bxor") idv = "(" + T + ")0";
-    else if (op == "band") idv = "(" + T + ")~(" + T + ")0";
-    else {
-      int bits = stBits(st);
-      unsigned long long mx = stIsSigned(st) ? ((1ULL << (bits - 1)) - 1) : (bits == 64 ? ~0ULL : ((1ULL << bits) - 1));
-      unsigned long long mn = stIsSigned(st) ? (1ULL << (bits - 1)) : 0ULL;
-      char buf[64];
-      snprintf(buf, sizeof buf, "(%s)0x%llxULL", T.c_str(), op == "min" ? mx : mn);
-      idv = buf;
-    }
-    lds = "#define ACC_PERMUTE_LDS 1\n  typedef " + T + " Prim;\n";
-    lds += "  ACC_DEV Prim identity() { return " + idv + "; }\n";
-    lds += "  ACC_DEV void lds_update(Prim* p, const Elt& x) { (void)" + fn + "(p, x.c0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP); }\n";
-    lds += "  ACC_DEV void global_update(const Out& out, i64 j, Prim v) { (void)" + fn + "(&out.o0[j], v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); }\n";
+    leafOps = {op};
   } else if (mode == "atomics") {
     // component-wise combination: the components do not see each other, one atomic each
     for (size_t k = 0; k < leaves.size(); ++k) {
@@ -1399,6 +1384,42 @@ KernelSource Codegen::permute(const Sx& f, const ArrayR& dst, const Sx& p, const
         u += "        __hip_atomic_store(&" + cell + ", r_" + field + ", __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);\n";
       });
     u += "        __hip_atomic_store(lk_, 0u, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_AGENT);\n        done_ = true;\n      }\n    }\n";
+  }
+  if (mode == "atomic" || mode == "atomics") {
+    // pieces of the LDS-privatised variant (permute.hpp): one private array per component, its
+    // identity, the LDS update and the addition of a private value to the destination
+    int bytes = 0;
+    for (ST t : leaves) bytes += stSize(t);
+    lds = "#define ACC_PERMUTE_LDS 1\n  static constexpr int kPart = 131072 / " + std::to_string(bytes) + ";\n  struct Priv {\n";
+    std::string init, upd, flush;
+    for (size_t k = 0; k < leaves.size(); ++k) {
+      const ST t = leaves[k];
+      const std::string& o = leafOps[k];
+      const std::string T = stName(t), K = std::to_string(k);
+      std::string fn = o == "add" ? "__hip_atomic_fetch_add" : o == "min" ? "__hip_atomic_fetch_min"
+                     : o == "max" ? "__hip_atomic_fetch_max" : o == "band" ? "__hip_atomic_fetch_and"
+                     : o == "bor" ? "__hip_atomic_fetch_or" : "__hip_atomic_fetch_xor";
+      std::string idv;
+      if (o == "add" || o == "bor" || o == "bxor") idv = "(" + T + ")0";
+      else if (o == "band") idv = "(" + T + ")~(" + T + ")0";
+      else {
+        int bits = stBits(t);
+        unsigned long long mx = stIsSigned(t) ? ((1ULL << (bits - 1)) - 1) : (bits == 64 ? ~0ULL : ((1ULL << bits) - 1));
+        unsigned long long mn = stIsSigned(t) ? (1ULL << (bits - 1)) : 0ULL;
+        char buf[64];
+        snprintf(buf, sizeof buf, "(%s)0x%llxULL", T.c_str(), o == "min" ? mx : mn);
+        idv = buf;
+      }
+      lds += "    " + T + " c" + K + "[kPart];\n";
+      init += "    p.c" + K + "[i] = " + idv + ";\n";
+      upd += "    (void)" + fn + "(&p.c" + K + "[i], x.c" + K + ", __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);\n";
+      flush += "    {\n      const " + T + " v_ = p.c" + K + "[i];\n      if (v_ != " + idv + ") (void)" + fn + "(&out.o" + K +
+               "[j], v_, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);\n    }\n";
+    }
+    lds += "  };\n";
+    lds += "  ACC_DEV void lds_init(Priv& p, int i) {\n" + init + "  }\n";
+    lds += "  ACC_DEV void lds_update(Priv& p, int i, const Elt& x) {\n" + upd + "  }\n";
+    lds += "  ACC_DEV void lds_flush(const Priv& p, int i, const Out& out, i64 j) {\n" + flush + "  }\n";
   }
   u += "  }\n" + lds;
   // update() uses store()/combine(): it must come after them, and finish() appends load/store

@@ -55,8 +55,8 @@ acc_permute(Spec::Env env, Spec::Out out, PermuteParams p) {
 // one range) changed nothing for Zipf keys and cost the uniform ones a third through the
 // extra index arithmetic: the update loop is bound by its instructions.
 //
-// The destination is cut into `nparts` ranges of `part` elements (part <= ACC_PERMUTE_PART,
-// 128 KiB of LDS).  The sources are cut into `groups` chunks; workgroup b serves chunk
+// The destination is cut into `nparts` ranges of `part` elements (part <= S::kPart, the
+// elements that fit 128 KiB of LDS; a tuple element has one private array per component).  The sources are cut into `groups` chunks; workgroup b serves chunk
 // (b / (8 * nparts)) * 8 + b % 8 and range (b / 8) % nparts: workgroups are dealt to the 8
 // XCDs round-robin, so the nparts workgroups that read the same chunk run on the same XCD
 // and share its L2 -- the sources come from HBM once.
@@ -64,7 +64,6 @@ acc_permute(Spec::Env env, Spec::Out out, PermuteParams p) {
 #ifndef ACC_PERMUTE_UNROLL
 #define ACC_PERMUTE_UNROLL 4
 #endif
-#define ACC_PERMUTE_PART (131072 / (int)sizeof(Spec::Prim))
 
 struct PermuteLdsParams {
   i64 n;       // number of source elements
@@ -78,15 +77,13 @@ struct PermuteLdsParams {
 extern "C" __global__ void __launch_bounds__(ACC_PERMUTE_LDS_BLOCK)
 acc_permute_lds(Spec::Env env, Spec::Out out, PermuteLdsParams p) {
   typedef Spec S;
-  typedef S::Prim Prim;
-  __shared__ Prim priv[ACC_PERMUTE_PART];
+  __shared__ S::Priv priv;
   const i64 b = (i64)blockIdx.x;
   const i64 range = (b / 8) % p.nparts;
   const i64 chunkId = (b / (8 * p.nparts)) * 8 + (b % 8);
   const i64 lo = range * p.part;
   const i64 hi = lo + p.part < p.dst_n ? lo + p.part : p.dst_n;
-  const Prim id = S::identity();
-  for (int i = threadIdx.x; i < (int)(hi - lo); i += ACC_PERMUTE_LDS_BLOCK) priv[i] = id;
+  for (int i = threadIdx.x; i < (int)(hi - lo); i += ACC_PERMUTE_LDS_BLOCK) S::lds_init(priv, i);
   __syncthreads();
   const i64 begin = chunkId * p.chunk;
   const i64 end = begin + p.chunk < p.n ? begin + p.chunk : p.n;
@@ -114,21 +111,20 @@ acc_permute_lds(Spec::Env env, Spec::Out out, PermuteLdsParams p) {
         const i64 i0 = base + ((i64)g * ACC_PERMUTE_LDS_BLOCK + threadIdx.x) * 4;
 #pragma unroll
         for (int k = 0; k < 4; ++k)
-          if (ok[g][k] && j[g][k] >= lo && j[g][k] < hi) S::lds_update(&priv[j[g][k] - lo], S::in_linear(env, i0 + k));
+          if (ok[g][k] && j[g][k] >= lo && j[g][k] < hi) S::lds_update(priv, (int)(j[g][k] - lo), S::in_linear(env, i0 + k));
       }
     } else {
       for (i64 i = base + threadIdx.x; i < end; i += ACC_PERMUTE_LDS_BLOCK) {
         i64 j;
         const int t = S::target(env, i, j);
-        if (t == 1 && j >= lo && j < hi) S::lds_update(&priv[j - lo], S::in_linear(env, i));
+        if (t == 1 && j >= lo && j < hi) S::lds_update(priv, (int)(j - lo), S::in_linear(env, i));
         bad = bad || t == 2;
       }
     }
   }
   __syncthreads();
   for (int i = threadIdx.x; i < (int)(hi - lo); i += ACC_PERMUTE_LDS_BLOCK) {
-    const Prim v = priv[i];
-    if (v != id) S::global_update(out, lo + i, v);
+    S::lds_flush(priv, i, out, lo + i);  // components that still hold the identity are skipped
   }
   if (bad) __hip_atomic_store(p.err, 2u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
 }

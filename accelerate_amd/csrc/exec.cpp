@@ -1133,7 +1133,9 @@ AValP Program::eval(const Sx& n, AEnv& aenv) {
     packOut(args, *out);
     // Many sources into a destination of a few LDS-fuls with a hardware-atomic combination:
     // combine in workgroup-private LDS copies first (see permute.hpp).
-    const int64_t partMax = 131072 / stSize(plan.k->meta.outLeaves.empty() ? ST::I32 : plan.k->meta.outLeaves[0]);
+    int64_t eltBytes = 0;
+    for (ST st : plan.k->meta.outLeaves) eltBytes += stSize(st);
+    const int64_t partMax = 131072 / std::max<int64_t>(1, eltBytes);  // Spec::kPart
     // Up to 128 LDS-fuls: every share re-reads the sources (from its XCD's L2), so the cost grows
     // with the destination -- 2^26 keys into 2^20 / 2^22 Int32 bins take 0.5 / 2.0 ms, which is
     // where plain global atomics are for uniform keys (2.5 ms); for Zipf keys those take 110 ms.
@@ -1144,7 +1146,7 @@ AValP Program::eval(const Sx& n, AEnv& aenv) {
     // keys into 256 bins take 33 us through global atomics, 2^14 keys into 16 bins 47 us,
     // against 9 us this way).
     const bool many = cnt >= (1 << 20) || (cnt >= (1 << 12) && cnt >= 4 * out->size());
-    if (plan.mode == "atomic" && many && out->size() <= maxParts * partMax) {
+    if ((plan.mode == "atomic" || plan.mode == "atomics") && many && out->size() <= maxParts * partMax) {
       const int64_t nparts = (out->size() + partMax - 1) / partMax;
       const int64_t part = (out->size() + nparts - 1) / nparts;
       // one workgroup per CU in total (each holds 128 KiB of LDS): fewer, longer workgroups

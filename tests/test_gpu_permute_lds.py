@@ -53,3 +53,26 @@ def test_privatised_permute_matches_sequential_updates(gpu_ctx, case):
     keep = to >= 0
     uf.at(ref, to[keep], xs[keep])
     assert np.array_equal(got, ref)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dst", [7, 300, 20000, 50000])
+def test_privatised_permute_of_pairs(gpu_ctx, dst):
+    # component-wise combinations of tuples keep one private array per component: sums of
+    # (Int64, Int32 maximum) pairs and of Float32 pairs (quarters: exact in any order) into
+    # 1 .. 5 ranges of the destination
+    rng = np.random.default_rng(dst)
+    to = np.minimum((rng.pareto(1.1, N) * 3).astype(np.int64), dst - 1)
+    a, b = rng.integers(-1000, 1000, N).astype(np.int64), rng.integers(-1000, 1000, N).astype(np.int32)
+    da, db = rng.integers(-1000, 1000, dst).astype(np.int64), rng.integers(-1000, 1000, dst).astype(np.int32)
+    got = gpu_ctx.compile(Q.accumulate_pairs(A.i64, A.i32, A.max_))([a, b], to, [da, db])
+    ra, rb = da.copy(), db.copy()
+    np.add.at(ra, to, a)
+    np.maximum.at(rb, to, b)
+    assert np.array_equal(got[0], ra) and np.array_equal(got[1], rb)
+    x, y = (rng.integers(-8, 9, N) / 4).astype(np.float32), (rng.integers(-8, 9, N) / 4).astype(np.float32)
+    got = gpu_ctx.compile(Q.accumulate_pairs())([x, y], to, [np.zeros(dst, np.float32)] * 2)
+    rx, ry = np.zeros(dst, np.float64), np.zeros(dst, np.float64)
+    np.add.at(rx, to, x)
+    np.add.at(ry, to, y)
+    assert np.array_equal(got[0], rx.astype(np.float32)) and np.array_equal(got[1], ry.astype(np.float32))
