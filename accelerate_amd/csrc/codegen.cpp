@@ -215,8 +215,10 @@ ValP Codegen::fromIndex(int rank, const ValP& sh, const std::string& lin, Emit& 
   std::vector<std::string> ix(rank);
   std::string cur = lin;
   for (int k = rank - 1; k >= 1; --k) {
-    ix[k] = bindLeaf(ST::I64, "acc_rem(" + cur + ", " + d[k] + ")", em)->ex;
-    cur = bindLeaf(ST::I64, "acc_quot(" + cur + ", " + d[k] + ")", em)->ex;
+    // one division per dimension: the remainder follows from the quotient
+    const std::string q = bindLeaf(ST::I64, "acc_quot(" + cur + ", " + d[k] + ")", em)->ex;
+    ix[k] = bindLeaf(ST::I64, cur + " - " + q + " * " + d[k], em)->ex;
+    cur = q;
   }
   ix[0] = cur;  // the outermost component needs no remainder (Shape.hs:110-120)
   ValP v = vUnit();
@@ -1184,6 +1186,41 @@ KernelSource Codegen::scan(const Sx& f, const Sx* seed, const Operand& src, bool
   return ks;
 }
 
+// Producers of rank >= 2 that need the multi-dimensional index of a result: the skeleton splits
+// the linear index of a thread's first result once (the divisions) and steps from result to
+// result, instead of dividing for every result.
+std::string Codegen::indexedFns(int rank, const ArraySlot& o) {
+  std::string fns;
+  Emit ef;
+  ef.ind = 4;
+  ValP ix0 = fromIndex(rank, shapeOf(o), "i", ef);
+  std::vector<std::string> c;
+  shapeDims(ix0, c);
+  for (int d = 0; d < rank; ++d) ef.line("ix[" + std::to_string(d) + "] = " + c[d] + ";");
+  fns += fnHead("void", "from_index", "const Env& env, i64 i, i64* ix") + ef.code + "  }\n";
+  std::vector<std::string> od;
+  shapeDims(shapeOf(o), od);
+  Emit en;
+  en.ind = 4;
+  for (int d = rank - 1; d >= 1; --d) {
+    en.line("if (++ix[" + std::to_string(d) + "] < " + od[d] + ") return;");
+    en.line("ix[" + std::to_string(d) + "] = 0;");
+  }
+  en.line("++ix[0];");
+  fns += fnHead("void", "next_index", "const Env& env, i64* ix") + en.code + "  }\n";
+  return fns;
+}
+
+ValP Codegen::indexedIx(int rank) {
+  ValP v = vUnit();
+  for (int d = 0; d < rank; ++d) v = vPair(v, vLeaf(ST::I64, "ix[" + std::to_string(d) + "]"));
+  return v;
+}
+
+std::string Codegen::indexedTail(int rank) {
+  return "  static constexpr int kRank = " + std::to_string(rank) + ";\n#define ACC_MAP_INDEXED 1\n";
+}
+
 KernelSource Codegen::map(const TypeP& outElt, const Sx* f, const Operand& src) {
   Emit em;
   em.ind = 4;
@@ -1216,9 +1253,14 @@ KernelSource Codegen::zipWith(const TypeP& outElt, const Sx& f, const Operand& a
   } else {
     declareOut(used_, rank);
     ArraySlot o = used_.at("out");
-    ValP ix = fromIndex(rank, shapeOf(o), "i", em);
+    ValP ix = indexedIx(rank);
     x = operandIndex(a, ix, em);
     y = operandIndex(b, ix, em);
+    ValP r = applyFun(f, {x, y}, {}, em);
+    if (!typeEq(valType(r), outElt)) throw Error("zipWith: function result does not match the declared element type");
+    std::string body = indexedFns(rank, o) + fnHead("Elt", "produce_at", "const Env& env, i64 i, const i64* ix") +
+                       returnElt(r, em) + "  }\n" + indexedTail(rank);
+    return finish(body, outElt, typeLeaves(outElt), "map.hpp", 0);
   }
   ValP r = applyFun(f, {x, y}, {}, em);
   if (!typeEq(valType(r), outElt)) throw Error("zipWith: function result does not match the declared element type");
@@ -1233,6 +1275,13 @@ KernelSource Codegen::generate(const ArrayR& out, const Sx& f) {
   em.ind = 4;
   declareOut(used_, out.rank);
   ArraySlot o = used_.at("out");
+  if (out.rank >= 2) {
+    ValP r = applyFun(f, {indexedIx(out.rank)}, {}, em);
+    if (!typeEq(valType(r), out.elt)) throw Error("generate: function result does not match the declared element type");
+    std::string body = indexedFns(out.rank, o) + fnHead("Elt", "produce_at", "const Env& env, i64 i, const i64* ix") +
+                       returnElt(r, em) + "  }\n" + indexedTail(out.rank);
+    return finish(body, out.elt, typeLeaves(out.elt), "map.hpp", 0);
+  }
   ValP ix = fromIndex(out.rank, shapeOf(o), "i", em);
   ValP r = applyFun(f, {ix}, {}, em);
   if (!typeEq(valType(r), out.elt)) throw Error("generate: function result does not match the declared element type");
@@ -1247,11 +1296,16 @@ KernelSource Codegen::backpermute(int outRank, const Sx& p, const Sx* f, const T
   em.ind = 4;
   declareOut(used_, outRank);
   ArraySlot o = used_.at("out");
-  ValP ix = fromIndex(outRank, shapeOf(o), "i", em);
+  ValP ix = outRank >= 2 ? indexedIx(outRank) : fromIndex(outRank, shapeOf(o), "i", em);
   ValP sx = applyFun(p, {ix}, {}, em);
   ValP v = operandIndex(src, sx, em);
   ValP r = f ? applyFun(*f, {v}, {}, em) : v;
   if (!typeEq(valType(r), outElt)) throw Error("backpermute: result does not match the declared element type");
+  if (outRank >= 2) {
+    std::string body = indexedFns(outRank, o) + fnHead("Elt", "produce_at", "const Env& env, i64 i, const i64* ix") +
+                       returnElt(r, em) + "  }\n" + indexedTail(outRank);
+    return finish(body, outElt, typeLeaves(outElt), "map.hpp", 0);
+  }
   std::string body = streamHead("Elt", "produce", "const Env& env, i64 i") + returnElt(r, em) + "  }\n";
   KernelSource ks = finish(body, outElt, typeLeaves(outElt), "map.hpp", 0);
   ks.streaming = true;
@@ -1462,26 +1516,7 @@ KernelSource Codegen::stencil(const std::vector<Sx>& patterns, const TypeP& outE
   // of a thread's first result once and steps to the following results by increments
   std::vector<std::string> fx(rank);
   for (int d = 0; d < rank; ++d) fx[d] = "ix[" + std::to_string(d) + "]";
-  std::string indexFns;
-  {
-    Emit ef;
-    ef.ind = 4;
-    ValP ix0 = fromIndex(rank, shapeOf(o), "i", ef);
-    std::vector<std::string> c;
-    shapeDims(ix0, c);
-    for (int d = 0; d < rank; ++d) ef.line("ix[" + std::to_string(d) + "] = " + c[d] + ";");
-    indexFns += fnHead("void", "from_index", "const Env& env, i64 i, i64* ix") + ef.code + "  }\n";
-    std::vector<std::string> od;
-    shapeDims(shapeOf(o), od);
-    Emit en;
-    en.ind = 4;
-    for (int d = rank - 1; d >= 1; --d) {
-      en.line("if (++ix[" + std::to_string(d) + "] < " + od[d] + ") return;");
-      en.line("ix[" + std::to_string(d) + "] = 0;");
-    }
-    en.line("++ix[0];");
-    indexFns += fnHead("void", "next_index", "const Env& env, i64* ix") + en.code + "  }\n";
-  }
+  std::string indexFns = indexedFns(rank, o);
 
   // stencilAccess (Interpreter.hs:670-794): the outermost tuple walks the left-most
   // dimension, offsets -k..+k left to right

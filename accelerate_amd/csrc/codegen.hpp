@@ -111,6 +111,11 @@ class Codegen {
   ValP shapeOf(const ArraySlot& s);
   std::string toIndex(const ValP& sh, const ValP& ix, Emit& em);
   ValP fromIndex(int rank, const ValP& sh, const std::string& lin, Emit& em);
+  // from_index / next_index over the result's extents, the index value (ix[0], ix[1], ..) and
+  // the tail that marks a producer as taking the multi-dimensional index (map.hpp)
+  std::string indexedFns(int rank, const ArraySlot& o);
+  ValP indexedIx(int rank);
+  std::string indexedTail(int rank);
   ValP operandLinear(const Operand& o, const std::string& lin, Emit& em);
   ValP operandIndex(const Operand& o, const ValP& ix, Emit& em);
   ValP operandShape(const Operand& o, Emit& em);
