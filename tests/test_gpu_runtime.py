@@ -83,6 +83,32 @@ def test_permute_reports_a_target_outside_the_destination(gpu_ctx, n):
     assert same(run(keys), np.bincount(keys, minlength=10).astype(np.int32))    # the context goes on
 
 
+def test_issue255_endurance_blocks_are_recycled():
+    # Test/NoFib/Issues/Issue255.hs: a 160 MiB array stepped a hundred times by `zipWith (+) a b`,
+    # the function prepared anew for every step, old results dropped as the loop goes.  The kernel
+    # cache answers every preparation after the first, and the memory table hands the dropped
+    # blocks out again: device memory does not grow with the number of steps.
+    ctx = hip.Context(0)
+    n = 20 * 1024 * 1024
+    V, S0 = A.tarray(1, A.f64), A.tarray(0, A.Int)
+    step = A.alam([V, V, S0], lambda a, b, _i: A.zipwith(A.f64, A.lam([A.f64, A.f64], lambda x, y: A.add(A.f64, x, y)), a, b))
+    total = A.alam([V], lambda a: A.fold(A.lam([A.f64, A.f64], lambda x, y: A.add(A.f64, x, y)), A.const(A.f64, 0), a))
+    a = ctx.to_device(np.zeros(n), V)
+    b = ctx.to_device(np.ones(n), V)
+    after_two = None
+    for i in range(101):
+        go = ctx.compile(step)
+        a = go.execute(a, b, ctx.to_device(np.array(i, np.int64), S0))     # the old `a` is released here
+        if i == 1:
+            ctx.sync()
+            after_two = ctx.stat("bytes_allocated_remote")
+    assert float(ctx.compile(total)(a)) == 101.0 * n
+    assert ctx.stat("bytes_allocated_remote") - after_two < 8 * n       # less than one more array
+    assert ctx.stat("pool_hits") >= 98
+    del a, b, go
+    ctx.close()
+
+
 def test_awhile_jacobi_counts_iterations(gpu_ctx):
     # 20 sweeps driven by awhile (Interpreter.hs:222-229).  The loop counter is a rank-0
     # array made by `unit` from index arithmetic, so the host follows its value and the
