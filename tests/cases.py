@@ -17,6 +17,14 @@ VEC = json.load(open(os.path.join(HERE, "golden", "vectors.json")))
 I64 = np.int64
 
 
+def _nest(parts):
+    """Value (((), p0), p1) .. of the given components, outermost first."""
+    v = A.nil
+    for p in parts:
+        v = A.pair(v, p)
+    return v
+
+
 def golden_cases():
     """(id, program, args, expected): expected is what the reference's own doctests /
     regression tests state (tests/golden/vectors.json)."""
@@ -132,6 +140,20 @@ def golden_cases():
     add("append_doctest", Q.concat_on(1), [np.array(e["m1"], I64), np.array(e["m2_10x3"], I64)], np.array(e["append"], I64))
     add("concaton_1_doctest", Q.concat_on(1), [np.array(e["m1"], I64), np.array(e["m2_10x5"], I64)], np.array(e["concatOn_1"], I64))
     add("concaton_2_doctest", Q.concat_on(2), [np.array(e["m1"], I64), np.array(e["m2_10x5"], I64)], np.array(e["concatOn_2"], I64))
+    e = v["replicate_slice_doctest"]
+    vec, mat, cube = np.array(e["vec"], I64), np.array(e["mat"], I64), np.arange(60, dtype=I64).reshape(e["cube_shape"])
+    fx, un = (lambda n: A.constI(n)), A.nil
+    sl = lambda *parts: (lambda: _nest(parts))      # slice index, outermost component first
+    add("replicate_4_all_doctest", Q.replicate_(("all", "fixed"), sl(fx(4), un), 1, 2), [vec], np.array(e["replicate_4_All"], I64))
+    add("replicate_all_4_doctest", Q.replicate_(("fixed", "all"), sl(un, fx(4)), 1, 2), [vec], np.array(e["replicate_All_4"], I64))
+    add("replicate_2_all_3_doctest", Q.replicate_(("fixed", "all", "fixed"), sl(fx(2), un, fx(3)), 1, 3), [vec],
+        np.array(e["replicate_2_All_3"], I64))
+    add("slice_2_all_doctest", Q.slice_of(("all", "fixed"), sl(fx(2), un), 2, 1), [mat], np.array(e["slice_2_All"], I64))
+    add("slice_4_2_doctest", Q.slice_of(("fixed", "fixed"), sl(fx(4), fx(2)), 2, 0), [mat], np.array(e["slice_4_2"], I64))
+    add("slice_sl0_vec_doctest", Q.slice_of(("fixed",), sl(fx(4)), 1, 0), [vec], np.array(e["sl0_vec_4"], I64))
+    add("slice_sl0_mat_doctest", Q.slice_of(("fixed", "all"), sl(un, fx(4)), 2, 1), [mat], np.array(e["sl0_mat_4"], I64))
+    add("slice_sl1_mat_doctest", Q.slice_of(("all", "fixed"), sl(fx(4), un), 2, 1), [mat], np.array(e["sl1_mat_4"], I64))
+    add("slice_sl1_cube_doctest", Q.slice_of(("all", "fixed", "all"), sl(un, fx(2), un), 3, 2), [cube], np.array(e["sl1_cube_2"], I64))
     add("issue123", Q.issue123(v["issue123"]["n"]), [], np.array(v["issue123"]["expected"], I64))
     add("issue184_A", Q.issue184a(v["issue184_A"]["n"]), [np.array(v["issue184_A"]["v"], I64)],
         np.array(v["issue184_A"]["expected"], I64))

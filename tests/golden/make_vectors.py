@@ -125,6 +125,15 @@ V["concat_doctest"] = {
     "m2_10x5": [[r * 5 + c for c in range(5)] for r in range(10)],
     "concatOn_1": [[r * 10 + c for c in range(10)] + [r * 5 + c for c in range(5)] for r in range(5)],
     "concatOn_2": [[r * 10 + c for c in range(5)] for r in range(5)] + [[r * 5 + c for c in range(5)] for r in range(10)]}
+# Language.hs:186-260  replicate; 340-400 slice (vec = [0..9], mat = the 5x10 iota matrix, cube = 3x4x5 iota)
+V["replicate_slice_doctest"] = {
+    "cite": "Language.hs:186-260, 340-400", "vec": list(range(10)), "mat": iota5x10, "cube_shape": [3, 4, 5],
+    "replicate_4_All": [list(range(10))] * 4,
+    "replicate_All_4": [[i] * 4 for i in range(10)],
+    "replicate_2_All_3": [[[i] * 3 for i in range(10)]] * 2,
+    "slice_2_All": list(range(20, 30)), "slice_4_2": 42,
+    "sl0_vec_4": 4, "sl0_mat_4": [4, 14, 24, 34, 44], "sl1_mat_4": list(range(40, 50)),
+    "sl1_cube_2": [[10, 11, 12, 13, 14], [30, 31, 32, 33, 34], [50, 51, 52, 53, 54]]}
 # Language.hs:716-728  histogram via permute (+)
 V["histogram_doctest"] = {"cite": "Language.hs:716-728",
                           "keys": [0, 0, 1, 2, 1, 1, 2, 4, 8, 3, 4, 9, 8, 3, 2, 5, 5, 3, 1, 2], "bins": 10,

@@ -933,3 +933,21 @@ def accumulate_pairs(t0=A.f32, t1=A.f32, op1=A.add):
         return A.tup(A.add(t0, a, c), op1(t1, d, b))
     return A.alam([A.tarray(1, t2), A.tarray(1, Int), A.tarray(1, t2)], lambda xs, to, dfl: A.permute(
         A.lam([t2, t2], f), dfl, A.lam([sh1], lambda ix: A.just(A.sh(A.index(to, A.vexp(ix))))), xs))
+
+
+def replicate_(spec, slix, src_rank, out_rank, ty=Int):
+    """Replicate as fusion leaves it (Trafo/Fusion.hs replicateD): a Backpermute whose extent is
+    IndexFull of the source's shape and whose index map is IndexSlice.  spec lists all / fixed
+    from the innermost dimension outwards, slix is the matching slice index."""
+    sho = A.tshape(out_rank)
+    return A.alam([A.tarray(src_rank, ty)], lambda xs: A.backpermute(
+        out_rank, A.indexfull(spec, slix(), A.shape(xs)),
+        A.lam([sho], lambda ix: A.indexslice(spec, slix(), A.vexp(ix))), xs))
+
+
+def slice_of(spec, slix, src_rank, out_rank, ty=Int):
+    """Slice as fusion leaves it (sliceD): extent IndexSlice of the source's shape, index map IndexFull"""
+    sho = A.tshape(out_rank)
+    return A.alam([A.tarray(src_rank, ty)], lambda xs: A.backpermute(
+        out_rank, A.indexslice(spec, slix(), A.shape(xs)),
+        A.lam([sho], lambda ix: A.indexfull(spec, slix(), A.vexp(ix))), xs))
