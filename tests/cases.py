@@ -154,6 +154,22 @@ def golden_cases():
     add("slice_sl0_mat_doctest", Q.slice_of(("fixed", "all"), sl(un, fx(4)), 2, 1), [mat], np.array(e["sl0_mat_4"], I64))
     add("slice_sl1_mat_doctest", Q.slice_of(("all", "fixed"), sl(fx(4), un), 2, 1), [mat], np.array(e["sl1_mat_4"], I64))
     add("slice_sl1_cube_doctest", Q.slice_of(("all", "fixed", "all"), sl(un, fx(2), un), 3, 2), [cube], np.array(e["sl1_cube_2"], I64))
+    e = v["map_zipwith_doctest"]
+    add("map_plus1_doctest", A.alam([A.tarray(1, A.Int)], lambda xs: A.map_(A.Int, A.lam([A.Int], lambda x: A.add(A.Int, x, A.constI(1))), xs)),
+        [np.array(e["xs"], I64)], np.array(e["map_plus1"], I64))
+    add("zipwith_plus_doctest", A.alam([A.tarray(2, A.Int)] * 2, lambda a, b: A.zipwith(A.Int, Q.binop(A.add, A.Int), a, b)),
+        [np.array(e["m3x5"], I64), np.array(e["m5x10"], I64)], np.array(e["zipwith_plus"], I64))
+    e = v["producers_doctest"]
+    xs5 = np.array(e["indexed_vec"], np.float32)
+    add("indexed_vec_doctest", Q.indexed(1), [xs5], [np.arange(5, dtype=I64), xs5])
+    m34 = np.arange(12, dtype=np.float32).reshape(e["indexed_mat_shape"])
+    add("indexed_mat_doctest", Q.indexed(2), [m34], [np.repeat(np.arange(3, dtype=I64), 4).reshape(3, 4),
+                                                     np.tile(np.arange(4, dtype=I64), 3).reshape(3, 4), m34])
+    add("enumfromn_doctest", Q.enum_from_step_n(2, (5, 10), A.Int, 0, 1), [], np.array(e["enumFromN_5x10"], I64))
+    add("enumfromstepn_doctest", Q.enum_from_step_n(2, (5, 10), A.f32, 0.0, 0.5), [], np.array(e["enumFromStepN_5x10"], np.float32))
+    odd = lambda x: A.neq(A.Int, A.rem(A.Int, x, A.constI(2)), A.constI(0))
+    add("filter_odd_mat_doctest", Q.filter_rows(odd), [np.array(e["filter_odd_mat"], I64)],
+        (np.array(e["filter_odd"], I64), np.array(e["filter_odd_counts"], I64)))
     add("issue123", Q.issue123(v["issue123"]["n"]), [], np.array(v["issue123"]["expected"], I64))
     add("issue184_A", Q.issue184a(v["issue184_A"]["n"]), [np.array(v["issue184_A"]["v"], I64)],
         np.array(v["issue184_A"]["expected"], I64))

@@ -134,6 +134,18 @@ V["replicate_slice_doctest"] = {
     "slice_2_All": list(range(20, 30)), "slice_4_2": 42,
     "sl0_vec_4": 4, "sl0_mat_4": [4, 14, 24, 34, 44], "sl1_mat_4": list(range(40, 50)),
     "sl1_cube_2": [[10, 11, 12, 13, 14], [30, 31, 32, 33, 34], [50, 51, 52, 53, 54]]}
+# Language.hs:405-455  map (+1), zipWith (+) over matrices of different extents
+V["map_zipwith_doctest"] = {"cite": "Language.hs:405-455", "xs": list(range(10)), "map_plus1": list(range(1, 11)),
+                            "m3x5": [[r * 5 + c for c in range(5)] for r in range(3)],
+                            "m5x10": [[r * 10 + c + 1 for c in range(10)] for r in range(5)],
+                            "zipwith_plus": [[1, 3, 5, 7, 9], [16, 18, 20, 22, 24], [31, 33, 35, 37, 39]]}
+# Prelude.hs:157-172 indexed; 1436-1478 fill, enumFromN, enumFromStepN; 1627-1635 filter odd over a matrix
+V["producers_doctest"] = {"cite": "Prelude.hs:157-172, 1436-1478, 1627-1635",
+                          "indexed_vec": [0.0, 1.0, 2.0, 3.0, 4.0], "indexed_mat_shape": [3, 4],
+                          "enumFromN_5x10": iota5x10,
+                          "enumFromStepN_5x10": [[(r * 10 + c) * 0.5 for c in range(10)] for r in range(5)],
+                          "filter_odd_mat": evens_mat, "filter_odd": [1, 3, 5, 7, 9, 1, 1, 1, 1, 1, 1, 3, 5, 7, 9, 11, 13, 15, 17, 19],
+                          "filter_odd_counts": [5, 5, 0, 10]}
 # Language.hs:716-728  histogram via permute (+)
 V["histogram_doctest"] = {"cite": "Language.hs:716-728",
                           "keys": [0, 0, 1, 2, 1, 1, 2, 4, 8, 3, 4, 9, 8, 3, 2, 5, 5, 3, 1, 2], "bins": 10,

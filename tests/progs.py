@@ -951,3 +951,56 @@ def slice_of(spec, slix, src_rank, out_rank, ty=Int):
     return A.alam([A.tarray(src_rank, ty)], lambda xs: A.backpermute(
         out_rank, A.indexslice(spec, slix(), A.shape(xs)),
         A.lam([sho], lambda ix: A.indexfull(spec, slix(), A.vexp(ix))), xs))
+
+
+def filter_rows(pred, ty=Int):
+    """filter over a matrix (compact, Prelude.hs:1670-1686): per-row exclusive scans of the keep
+    flags give the targets inside a row and the row's count, an exclusive scan of the counts
+    the rows' offsets, a permute gathers the kept elements; returns (elements, counts per row)."""
+    sh1, sh2 = A.tshape(1), A.tshape(2)
+    V1, S0, M = A.tarray(1, Int), A.tarray(0, Int), A.tarray(2, Int)
+
+    def body(xs):
+        flags = A.delayed(M, A.shape(xs),
+                          A.lam([sh2], lambda ix: A.cond(pred(A.index(xs, A.vexp(ix))), A.constI(1), A.constI(0))),
+                          A.lam([Int], lambda i: A.cond(pred(A.linearindex(xs, i)), A.constI(1), A.constI(0))))
+
+        def with_rows(st):
+            target, length = st
+
+            def with_offsets(so):
+                offset, valid = so
+
+                def prj(ix):
+                    y, _ = A.untup(ix)
+                    return A.cond(pred(A.index(xs, A.vexp(ix))),
+                                  A.just(A.sh(A.add(Int, A.linearindex(offset, y), A.index(target, A.vexp(ix))))),
+                                  A.nothing(sh1))
+                result = A.permute(A.lam([ty, A.wild(ty)], lambda x, _: x),
+                                   A.generate(A.tarray(1, ty), A.sh(A.index(valid, A.nil)), A.lam([sh1], lambda ix: A.undef(ty))),
+                                   A.lam([sh2], prj), xs)
+                return A.apair(result, length)
+            return A.alet(A.tpair(V1, S0), A.scan_("l", binop(A.add, Int), A.constI(0), length), with_offsets)
+        return A.alet(A.tpair(M, V1), A.scan_("l", binop(A.add, Int), A.constI(0), flags), with_rows)
+
+    return A.alam([A.tarray(2, ty)], body)
+
+
+def indexed(rank, ty=A.f32):
+    """indexed = imap (\\ix x -> (ix, x)) (Prelude.hs:157-177): a Transform over the source"""
+    shr = A.tshape(rank)
+    out = A.ttup(shr, ty)
+    return A.alam([A.tarray(rank, ty)], lambda xs: A.generate(
+        A.tarray(rank, out), A.shape(xs), A.lam([shr], lambda ix: A.tup(A.vexp(ix), A.index(xs, A.vexp(ix))))))
+
+
+def enum_from_step_n(rank, dims, ty, x0, dx):
+    """enumFromStepN sh x y = reshape sh (generate (size sh) (\\i -> x + fromIntegral i * y))  (Prelude.hs:1475-1488)"""
+    sh1 = A.tshape(1)
+    n = 1
+    for d in dims:
+        n *= d
+    conv = (lambda i: A.fromintegral(Int, ty, i)) if ty in A.INTEGRAL else (lambda i: A.tofloating(Int, ty, i))
+    gen = A.generate(A.tarray(1, ty), A.sh(n), A.lam([sh1], lambda ix: A.add(
+        ty, A.const(ty, x0), A.mul(ty, conv(A.untup(ix)[0]), A.const(ty, dx)))))
+    return A.reshape(rank, A.sh(*dims), gen)
