@@ -170,6 +170,10 @@ def golden_cases():
     odd = lambda x: A.neq(A.Int, A.rem(A.Int, x, A.constI(2)), A.constI(0))
     add("filter_odd_mat_doctest", Q.filter_rows(odd), [np.array(e["filter_odd_mat"], I64)],
         (np.array(e["filter_odd"], I64), np.array(e["filter_odd_counts"], I64)))
+    e = v["misc_cache"]
+    for which in ("generate", "backpermute"):
+        add("misc_cache_" + which, Q.misc_cache(which), [np.array(e["a"], np.float32), np.array(e["b"], np.float32)],
+            np.array(e[which], np.float32))
     add("issue123", Q.issue123(v["issue123"]["n"]), [], np.array(v["issue123"]["expected"], I64))
     add("issue184_A", Q.issue184a(v["issue184_A"]["n"]), [np.array(v["issue184_A"]["v"], I64)],
         np.array(v["issue184_A"]["expected"], I64))

@@ -146,6 +146,9 @@ V["producers_doctest"] = {"cite": "Prelude.hs:157-172, 1436-1478, 1627-1635",
                           "enumFromStepN_5x10": [[(r * 10 + c) * 0.5 for c in range(10)] for r in range(5)],
                           "filter_odd_mat": evens_mat, "filter_odd": [1, 3, 5, 7, 9, 1, 1, 1, 1, 1, 1, 3, 5, 7, 9, 11, 13, 15, 17, 19],
                           "filter_odd_counts": [5, 5, 0, 10]}
+# Test/NoFib/Misc/Cache.hs:44-73: a = [0..9], b = [10..19]
+V["misc_cache"] = {"cite": "Test/NoFib/Misc/Cache.hs:44-73", "a": [float(i) for i in range(10)],
+                   "b": [float(i) for i in range(10, 20)], "generate": 5 * 45.0, "backpermute": 2 * 45.0}
 # Language.hs:716-728  histogram via permute (+)
 V["histogram_doctest"] = {"cite": "Language.hs:716-728",
                           "keys": [0, 0, 1, 2, 1, 1, 2, 4, 8, 3, 4, 9, 8, 3, 2, 5, 5, 3, 1, 2], "bins": 10,

@@ -1004,3 +1004,25 @@ def enum_from_step_n(rank, dims, ty, x0, dx):
     gen = A.generate(A.tarray(1, ty), A.sh(n), A.lam([sh1], lambda ix: A.add(
         ty, A.const(ty, x0), A.mul(ty, conv(A.untup(ix)[0]), A.const(ty, dx)))))
     return A.reshape(rank, A.sh(*dims), gen)
+
+
+def misc_cache(which):
+    """Test/NoFib/Misc/Cache.hs: two nodes with the same scalar code but different extent
+    expressions; a kernel cache whose key leaves the extents out must still give each its own."""
+    sh1 = A.tshape(1)
+    V, S0 = A.tarray(1, A.f32), A.tarray(0, A.f32)
+    plus = binop(A.add, A.f32)
+
+    def body(a, b):
+        n, m = (lambda: A.untup_shape(a)[0]), (lambda: A.untup_shape(b)[0])
+        if which == "generate":
+            f = lambda: A.lam([sh1], lambda ix: A.index(a, A.sh(A.rem(Int, A.untup(ix)[0], A.constI(10)))))
+            c = A.generate(V, A.sh(A.add(Int, n(), m())), f())
+            d = lambda: A.generate(V, A.sh(A.mul(Int, A.constI(3), n())), f())
+        else:
+            ident = lambda: A.lam([sh1], lambda ix: A.vexp(ix))
+            c = A.backpermute(1, A.sh(A.min_(Int, n(), m())), ident(), a)
+            d = lambda: A.backpermute(1, A.sh(n()), ident(), a)
+        return A.alet(V, c, lambda cv: A.alet(V, d(), lambda dv: A.zipwith(
+            A.f32, plus, A.fold(plus, A.const(A.f32, 0), cv), A.fold(plus, A.const(A.f32, 0), dv))))
+    return A.alam([V, V], body)
