@@ -1298,7 +1298,7 @@ AValP Program::eval(const Sx& n, AEnv& aenv) {
     if (plan.k2) {
       const KernelSource& sm = plan.k2->meta;
       const int64_t smallTile = (int64_t)sm.block * sm.group * sm.vec;
-      small = rows * ((len + bigTile - 1) / bigTile) < 128 || len <= 2 * smallTile;
+      small = rows * ((len + bigTile - 1) / bigTile) < 80 || len <= 2 * smallTile;
     }
     if (const char* v = std::getenv("ACCHIP_SCAN_TILES")) {  // "large" / "small": override, for tests
       if (std::string(v) == "large") small = false;
