@@ -343,11 +343,7 @@ ACC_DEV void acc_scan_tile(const typename S::Env& env, u64* desc, i64 tiles, i64
   for (int g = 0; g < G; ++g) {
     i64 cnt = n - (wlo + (i64)g * C::GROUP);
     cnt = cnt < 0 ? 0 : (cnt > C::GROUP ? C::GROUP : cnt);
-#ifdef ACC_X_NOWAVESCAN
-    Elt ts = x[g][V - 1];
-#else
     Elt ts = acc_wave_scan<S>(env, x[g][V - 1], lane);
-#endif
     Elt lanePre = acc_prev_lane(ts);  // exclusive prefix of the lane inside its group (lane > 0)
     const int last = cnt > 0 ? (int)((cnt - 1) / V) : 0;
     Elt gt = acc_readlane(ts, last);
@@ -383,11 +379,7 @@ ACC_DEV void acc_scan_tile(const typename S::Env& env, u64* desc, i64 tiles, i64
 
   Elt excl;
   bool hasExcl = false;
-#ifdef ACC_X_NOLOOKBACK
-  if (true) {
-#else
   if (tile == 0) {
-#endif
     if (S::kSeeded) {
       excl = S::seed(env);
       hasExcl = true;
@@ -612,9 +604,6 @@ ACC_DEV void acc_rows_tile(const typename S::Env& env, int cnt, int n, const Loa
 }
 
 ACC_DEV i64 acc_take_ticket(u64* ticket, u64 base) {
-#ifdef ACC_X_NOTICKET
-  return (i64)blockIdx.x;
-#endif
   __shared__ i64 sh_tile;
   if (threadIdx.x == 0)
     sh_tile = (i64)(__hip_atomic_fetch_add(ticket, 1ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) - base);
