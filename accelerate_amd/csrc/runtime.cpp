@@ -370,7 +370,8 @@ KernelP Context::kernel(const KernelSource& ks0) {
   k->meta.source.clear();
   std::string path = cacheDir + "/" + hash + ".hsaco";
   if (dumpCC) fprintf(stderr, "[acchip] kernel %s\n%s\n", hash.c_str(), ks.source.c_str());
-  if (!forceRecomp && readFile(path, k->code) && !k->code.empty()) {
+  // a cached code object must at least look like one (an ELF image); anything else is compiled anew
+  if (!forceRecomp && readFile(path, k->code) && k->code.size() > 64 && k->code.compare(0, 4, "\177ELF") == 0) {
     stats.kernelsFromDisk++;
   } else {
     // compile on a worker thread, at most as many at once as there are cores

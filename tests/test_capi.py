@@ -74,6 +74,29 @@ def test_kernel_cache_is_shared_between_equal_terms(cc_ctx):
     assert cc_ctx.stat("kernels_from_memory") == before + 1
 
 
+def test_disk_cache_round_trip_and_damaged_entries(tmp_path, monkeypatch):
+    # a second context finds the code object on disk; an entry that is not a code object (here:
+    # overwritten with text) is compiled anew instead of being handed to the loader
+    monkeypatch.setenv("ACCHIP_CACHE_DIR", str(tmp_path))
+    prog = P.fold_sum(A.i64, 1, 7)
+    c1 = hip.Context(-1)
+    c1.compile(prog)
+    assert c1.stat("kernels_compiled") >= 1
+    c1.close()
+    files = sorted(tmp_path.glob("*.hsaco"))
+    assert files and all(f.read_bytes()[:4] == b"\x7fELF" for f in files)
+    c2 = hip.Context(-1)
+    c2.compile(prog)
+    assert c2.stat("kernels_from_disk") == len(files) and c2.stat("kernels_compiled") == 0
+    c2.close()
+    files[0].write_bytes(b"not a code object" * 10)
+    c3 = hip.Context(-1)
+    c3.compile(prog)
+    assert c3.stat("kernels_compiled") == 1 and c3.stat("kernels_from_disk") == len(files) - 1
+    c3.close()
+    assert files[0].read_bytes()[:4] == b"\x7fELF"
+
+
 def test_errors_are_reported_not_thrown(cc_ctx):
     with pytest.raises(hip.AccError) as e:
         cc_ctx.compile("(alam (single (array 1 f32)) (fold (lam (single f32) 3) nothing (avar 0)")
