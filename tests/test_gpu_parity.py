@@ -180,6 +180,30 @@ def test_histogram_2pow26_bit_exact(gpu_ctx):
     assert got.sum(dtype=np.int64) == n and np.array_equal(got, np.bincount(keys, minlength=nbins))
 
 
+TILE_EDGES = sorted({t * k + d for t in (4096, 8192, 12288, 24576, 49152) for k in (1, 2, 5) for d in (-1, 0, 1)})
+
+
+@pytest.mark.parametrize("tiles", ["large", "small"])
+@pytest.mark.parametrize("ty", [A.i32, A.i64])
+def test_scans_and_folds_at_tile_borders(gpu_ctx, monkeypatch, ty, tiles):
+    # lengths one short of, equal to and one beyond multiples of every tile size the scans use,
+    # through both tile variants: left, right and exclusive scans and the fold, against numpy
+    monkeypatch.setenv("ACCHIP_SCAN_TILES", tiles)
+    dt = np.int32 if ty == A.i32 else np.int64
+    rng = np.random.default_rng(77)
+    progs = {"scanl1": gpu_ctx.compile(P.scanl1_sum(ty)), "scanl'": gpu_ctx.compile(P.scan_prime_sum("l", ty, 1, 3)),
+             "scanr": gpu_ctx.compile(P.scan_sum("r", ty, 1, 3)), "fold": gpu_ctx.compile(P.fold_sum(ty, 1, 3))}
+    for n in TILE_EDGES:
+        x = rng.integers(-1000, 1000, n).astype(dt)
+        inc = np.cumsum(x, dtype=dt)
+        assert np.array_equal(progs["scanl1"](x), inc), n
+        body, total = progs["scanl'"](x)
+        assert np.array_equal(body, np.concatenate([[3], 3 + inc[:-1]]).astype(dt)) and total == dt(3) + inc[-1], n
+        rinc = np.cumsum(x[::-1], dtype=dt)[::-1]
+        assert np.array_equal(progs["scanr"](x), np.concatenate([rinc + dt(3), [3]]).astype(dt)), n
+        assert progs["fold"](x) == dt(3) + inc[-1], n
+
+
 @pytest.mark.parametrize("nbins", [1 << 20, (1 << 21) + 12345, 1 << 22])
 def test_histogram_over_many_lds_fuls(gpu_ctx, monkeypatch, nbins):
     # destinations of up to 128 LDS-fuls are still combined in workgroup-private copies, one
