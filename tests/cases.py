@@ -192,6 +192,36 @@ def golden_cases():
     add("issue436_A", Q.filter_take(e["take"]), [np.array(e["xs"], np.uint8)],
         (np.array(e["expected"], np.uint8), np.array(e["count"], I64)))
     add("issue439", Q.issue439(), [], np.array(v["issue439"]["expected"], np.float32))
+    F32 = np.float32
+    for which in "ABC":
+        add("issue168_" + which, Q.issue168(which), [], [np.array([x], F32) for x in v["issue168"][which]])
+    rng = np.random.default_rng(264)
+    for ty, dt in ((A.i8, np.int8), (A.i16, np.int16), (A.i32, np.int32), (A.i64, np.int64), (A.u8, np.uint8),
+                   (A.u16, np.uint16), (A.u32, np.uint32), (A.u64, np.uint64)):
+        info = np.iinfo(dt)
+        xs = np.concatenate([np.array([info.min, info.max, 0], dt), rng.integers(info.min, info.max, 61, dtype=dt, endpoint=True)])
+        add("issue264_negneg_" + ty, Q.issue264_neg(ty), [xs], xs)
+    for ty, dt in ((A.f32, np.float32), (A.f64, np.float64)):
+        xs = np.concatenate([[0.0, -0.0, np.inf, -np.inf], rng.standard_normal(60)]).astype(dt)
+        add("issue264_negneg_" + ty, Q.issue264_neg(ty), [xs], xs)
+    table = {"not.not": lambda u: u, "not(&&)": lambda u, w: 1 - (u & w), "not(||)": lambda u, w: 1 - (u | w),
+             "not(not(&&))": lambda u, w: u & w, "not(not(||))": lambda u, w: u | w}
+    assert set(table) == set(v["issue264"]["bool"])
+    for which, f in table.items():
+        for bits in ((0,), (1,)) if which == "not.not" else ((0, 0), (0, 1), (1, 0), (1, 1)):
+            add("issue264_%s_%s" % (which, "".join(map(str, bits))), Q.issue264_bool(which),
+                [np.array(b, np.uint8) for b in bits], np.array(f(*bits), np.uint8))
+    t = v["issue286"]
+    add("issue286", Q.issue286(), [np.full(t["shape"], t["fill"], np.uint8)], np.array(t["expected"], F32))
+    for shp in v["issue427"]["shapes"]:
+        cells = (np.random.default_rng(427).random(shp) < 0.4).astype(np.uint8)
+        add("issue427_%dx%d" % tuple(shp), Q.indices_of_truth(), [cells], [c.astype(I64) for c in np.nonzero(cells)])
+    t = v["issue517"]
+    add("issue517", Q.issue517(), [], [np.array(x, dt) for tag, val in zip(t["tags"], t["values"])
+                                        for x, dt in ((tag, np.uint8), (0.0 if val is None else val, F32))])
+    n = v["issue551"]["n"]
+    add("issue551_eq", Q.issue551("eq"), [], np.eye(n, dtype=np.uint8))
+    add("issue551_digits", Q.issue551("digits"), [], np.arange(n, dtype=np.uint16))
     t = v["issue228"]
     pair_in = [np.array(t["fst"], I64), np.array(t["snd"], I64)]
     pair_out = [np.array(t["expected"][0], I64), np.array(t["expected"][1], I64)]

@@ -242,6 +242,29 @@ V["issue436_A"] = {"cite": "Test/NoFib/Issues/Issue436.hs:27-50", "xs": [1, 0, 1
 # Test/NoFib/Issues/Issue439.hs: map (* 2) over the rank-0 array fill Z 1
 V["issue439"] = {"cite": "Test/NoFib/Issues/Issue439.hs:26-34", "expected": 2.0}
 
+# Test/NoFib/Issues/Issue168.hs: fill (Z:.1) of an iterated tuple function
+V["issue168"] = {"cite": "Test/NoFib/Issues/Issue168.hs:31-66", "A": [3.0, 2.0], "B": [3.0, 2.0],
+                 "C": [1.0, 2.0, 3.0, 4.0, 5.0, 6.0]}
+# Test/NoFib/Issues/Issue264.hs: negate . negate = id for every number type; not . not = id and
+# De Morgan's pairs over Bool (the reference checks them as properties against the host functions)
+V["issue264"] = {"cite": "Test/NoFib/Issues/Issue264.hs:36-130",
+                 "bool": {"not.not": "x", "not(&&)": "not (u and v)", "not(||)": "not (u or v)",
+                          "not(not(&&))": "u and v", "not(not(||))": "u or v"}}
+# Test/NoFib/Issues/Issue286.hs: sum . flatten . map fromIntegral over a 120x659 matrix of ones
+V["issue286"] = {"cite": "Test/NoFib/Issues/Issue286.hs:47-48,107", "shape": [120, 659], "fill": 1,
+                 "expected": 120.0 * 659.0}
+# Test/NoFib/Issues/Issue427.hs: indices of the True cells of a matrix, row-major (property against
+# a list filter; shapes n-by-64, n-by-8, n-by-m)
+V["issue427"] = {"cite": "Test/NoFib/Issues/Issue427.hs:34-84", "shapes": [[33, 64], [129, 8], [0, 8], [17, 31], [1, 1]]}
+# Test/NoFib/Issues/Issue437.hs: runN id returns its arguments; nothing is allocated, 4 bytes at most
+# go to the device and nothing comes back
+V["issue437"] = {"cite": "Test/NoFib/Issues/Issue437.hs:45-83", "unit": 42.0, "shape": [10000, 10000], "fill": 1.0}
+# Test/NoFib/Issues/Issue517.hs: (Nothing, Just 2, Just 3, Just 5, Just 7) from (<>) on Maybe (Max Float)
+V["issue517"] = {"cite": "Test/NoFib/Issues/Issue517.hs:31-43", "tags": [0, 1, 1, 1, 1], "values": [None, 2.0, 3.0, 5.0, 7.0]}
+# Test/NoFib/Issues/Issue551.hs: equality of a nine-constructor enumeration is the 9x9 identity, the
+# digits map back to 0..8
+V["issue551"] = {"cite": "Test/NoFib/Issues/Issue551.hs:80-83", "n": 9}
+
 with open(OUT, "w") as f:
     json.dump(V, f, indent=1, sort_keys=True)
 print("wrote", OUT, len(V), "vectors")

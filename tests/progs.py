@@ -752,6 +752,146 @@ def filter_take(n, ty=A.u8):
     return A.alam([A.tarray(1, ty)], body)
 
 
+def issue168(which):
+    """fill (Z:.1) of a tuple made by iterating a tuple-to-tuple function (Issue168): A applies
+    it in the host language, B and C through `iterate` (Prelude.hs: a `while` over (count, value))"""
+    F = A.f32
+    c = lambda v: A.const(F, v)
+    sh1 = A.tshape(1)
+    if which == "C":
+        ty, seed = A.ttup(*[F] * 6), lambda: A.tup(*[c(v) for v in (6, 5, 4, 3, 2, 1)])
+        step = lambda t: A.tup(*reversed(A.untup(t)))
+    else:
+        ty, seed = A.ttup(F, F), lambda: A.tup(c(2), c(1))
+        step = lambda t: A.tup(c(3), A.untup(t)[0])
+
+    def value():
+        if which == "A":
+            return A.let(ty, seed(), lambda t: step(t))
+        st = A.ttup(Int, ty)
+        loop = A.while_(st, lambda v: A.lt(Int, A.untup(v)[0], A.constI(1)),
+                        lambda v: A.tup(A.add(Int, A.untup(v)[0], A.constI(1)), step(A.untup(v)[1])),
+                        A.tup(A.constI(0), seed()))
+        return A.let(st, loop, lambda r: A.vexp(A.untup(r)[1]))
+    return A.generate(A.tarray(1, ty), A.sh(A.constI(1)), A.lam([sh1], lambda ix: value()))
+
+
+def issue264_neg(ty):
+    """map negate . map negate, fused (Issue264)"""
+    return A.alam([A.tarray(1, ty)], lambda xs: A.map_(ty, A.lam([ty], lambda x: A.neg(ty, A.neg(ty, x))), xs))
+
+
+def issue264_bool(which):
+    """not.not over a scalar array of Bool; not (u && v), not (u || v) and their negations
+    through zipWith (Issue264)"""
+    B = A.u8
+    S0 = A.tarray(0, B)
+    if which == "not.not":
+        return A.alam([S0], lambda xs: A.map_(B, A.lam([B], lambda x: A.lnot(A.lnot(x))), xs))
+    op = A.land if "&&" in which else A.lor
+    f = (lambda u, v: A.lnot(A.lnot(op(u, v)))) if which.startswith("not(not") else (lambda u, v: A.lnot(op(u, v)))
+    return A.alam([S0, S0], lambda xs, ys: A.zipwith(B, A.lam([B, B], f), xs, ys))
+
+
+def issue286():
+    """sum . flatten . map fromIntegral over a matrix of Word8 (Issue286): one fold over a
+    delayed, flattened source"""
+    sh1 = A.tshape(1)
+    get = lambda xs, i: A.fromintegral(A.u8, A.f32, A.linearindex(xs, i))
+    return A.alam([A.tarray(2, A.u8)], lambda xs: A.fold(
+        binop(A.add, A.f32), A.const(A.f32, 0),
+        A.delayed(A.tarray(1, A.f32), A.sh(A.shapesize(2, A.shape(xs))),
+                  A.lam([sh1], lambda ix: get(xs, A.untup(ix)[0])), A.lam([Int], lambda i: get(xs, i)))))
+
+
+def indices_of_truth():
+    """map dropBool (afst (filter accept (imap addInds xs))) over a matrix of Bool (Issue427):
+    the indexed source is fused into the filter's scans and its permute"""
+    B = A.u8
+    sh1, sh2 = A.tshape(1), A.tshape(2)
+    t3, t2 = A.ttup(Int, Int, B), A.ttup(Int, Int)
+    V1, S0, M = A.tarray(1, Int), A.tarray(0, Int), A.tarray(2, Int)
+
+    def body(xs):
+        keep = lambda b: A.cond(b, A.constI(1), A.constI(0))
+        flags = A.delayed(M, A.shape(xs), A.lam([sh2], lambda ix: keep(A.index(xs, A.vexp(ix)))),
+                          A.lam([Int], lambda i: keep(A.linearindex(xs, i))))
+
+        def with_inds_at(ix):
+            y, x = A.untup(ix)
+            return A.tup(y, x, A.index(xs, A.vexp(ix)))
+        with_inds = A.delayed(A.tarray(2, t3), A.shape(xs), A.lam([sh2], with_inds_at),
+                              A.lam([Int], lambda i: A.let(sh2, A.fromindex(2, A.shape(xs), i), with_inds_at)))
+
+        def with_rows(st):
+            target, length = st
+
+            def with_offsets(so):
+                offset, valid = so
+
+                def prj(ix):
+                    y, _ = A.untup(ix)
+                    return A.cond(A.index(xs, A.vexp(ix)),
+                                  A.just(A.sh(A.add(Int, A.linearindex(offset, y), A.index(target, A.vexp(ix))))),
+                                  A.nothing(sh1))
+                kept = A.permute(A.lam([t3, A.wild(t3)], lambda x, _: A.vexp(x)),
+                                 A.generate(A.tarray(1, t3), A.sh(A.index(valid, A.nil)), A.lam([sh1], lambda ix: A.tup(A.undef(Int), A.undef(Int), A.undef(B)))),
+                                 A.lam([sh2], prj), with_inds)
+                return A.map_(t2, A.lam([t3], lambda v: A.tup(*A.untup(v)[:2])), kept)
+            return A.alet(A.tpair(V1, S0), A.scan_("l", binop(A.add, Int), A.constI(0), length), with_offsets)
+        return A.alet(A.tpair(M, V1), A.scan_("l", binop(A.add, Int), A.constI(0), flags), with_rows)
+
+    return A.alam([A.tarray(2, B)], body)
+
+
+def issue437():
+    """runN id over (Scalar Float, Matrix Float) (Issue437)"""
+    aty = A.tpair(A.tarray(0, A.f32), A.tarray(2, A.f32))
+    return A.alam([aty], lambda xs: A.apair(*xs))
+
+
+def issue517():
+    """unit of five `Maybe (Max Float)` combined with (<>) (Issue517): Maybe a is (tag, ((), a)),
+    Nothing's payload is undef, and (<>) matches on both tags"""
+    F = A.f32
+    mb = A.ttup(A.u8, A.ttup(F))
+    nothing = lambda: A.tup(A.const(A.u8, 0), A.tup(A.undef(F)))
+    just = lambda v: (lambda: A.tup(A.const(A.u8, 1), A.tup(A.const(F, v))))
+
+    def append(a, b):
+        def both(x, y):
+            both_just = lambda: A.tup(A.const(A.u8, 1), A.tup(A.max_(F, A.untup(A.untup(x)[1])[0], A.untup(A.untup(y)[1])[0])))
+            return A.case(A.untup(x)[0], [(0, A.vexp(y)), (1, A.case(A.untup(y)[0], [(0, A.vexp(x)), (1, both_just())]))])
+        return A.let(mb, a(), lambda x: A.let(mb, b(), lambda y: both(x, y)))
+    t5 = A.ttup(*[mb] * 5)
+    return A.unit_(t5, A.tup(append(nothing, nothing), append(nothing, just(2)), append(just(3), nothing),
+                             append(just(4), just(5)), append(just(7), just(6))))
+
+
+def issue551(which):
+    """A nine-constructor enumeration (Issue551): word16ToDigit is a chain of conds ending in undef,
+    (==) a match on the pair of tags, digitToWord16 a match on the tag"""
+    T, W = A.u8, A.u16
+    sh1, sh2 = A.tshape(1), A.tshape(2)
+
+    def to_digit(i):
+        e = A.undef(T)
+        for k in range(8, -1, -1):
+            e = A.cond(A.eq(W, i, A.const(W, k)), A.const(T, k), e)
+        return e
+    to_word = lambda d: A.case(d, [(k, A.const(W, k)) for k in range(9)])
+    same = lambda a, b: A.case(a, [(k, A.case(b, [(k, A.const(A.u8, 1))], A.const(A.u8, 0))) for k in range(9)])
+    nine = lambda: A.constI(9)
+    if which == "eq":
+        def at(ix):
+            i, j = A.untup(ix)
+            return A.let(W, A.fromintegral(Int, W, i), lambda a: A.let(W, A.fromintegral(Int, W, j), lambda b: same(to_digit(a), to_digit(b))))
+        return A.generate(A.tarray(2, A.u8), A.sh(nine(), nine()), A.lam([sh2], at))
+    digits = A.generate(A.tarray(1, T), A.sh(nine()),
+                        A.lam([sh1], lambda ix: A.let(W, A.fromintegral(Int, W, A.untup(ix)[0]), to_digit)))
+    return A.alet(A.tarray(1, T), digits, lambda ds: A.map_(W, A.lam([T], to_word), ds))
+
+
 def issue439():
     S0 = A.tarray(0, A.f32)
     one = A.generate(S0, A.nil, A.lam([A.unit], lambda ix: A.const(A.f32, 1)))

@@ -9,6 +9,7 @@ from accelerate_amd import programs as P
 from oracle import c as OC
 from oracle import interp as O
 
+from . import progs as Q
 from .cases import same
 from .runtime_cases import runtime_cases
 
@@ -107,6 +108,42 @@ def test_issue255_endurance_blocks_are_recycled():
     assert ctx.stat("pool_hits") >= 98
     del a, b, go
     ctx.close()
+
+
+def test_issue437_identity_allocates_and_copies_nothing(gpu_ctx):
+    # Test/NoFib/Issues/Issue437.hs: `runN id` applied to (unit 42, fill (Z:.10000:.10000) 1), itself
+    # the result of a run: no remote allocation, nothing copied to the device beyond the unit's 4
+    # bytes (here not even those: the pair was made on the device), nothing copied back until the
+    # first component is read, and then its 4 bytes only.
+    F = A.f32
+    sh2 = A.tshape(2)
+    make = A.apair(A.unit_(F, A.const(F, 42)),
+                   A.generate(A.tarray(2, F), A.sh(A.constI(10000), A.constI(10000)), A.lam([sh2], lambda ix: A.const(F, 1))))
+    xs = gpu_ctx.compile(make).execute()
+    go = gpu_ctx.compile(Q.issue437())
+    gpu_ctx.sync()
+    names = ("bytes_allocated_remote", "bytes_copied_to_remote", "bytes_copied_from_remote")
+    before = [gpu_ctx.stat(n) for n in names]
+    res = go.execute(xs)
+    gpu_ctx.sync()
+    assert [gpu_ctx.stat(n) for n in names] == before
+    a, b = res.parts()
+    assert a.to_host() == np.float32(42) and b.shape == (10000, 10000)
+    assert gpu_ctx.stat("bytes_copied_from_remote") - before[2] == 4
+
+
+def test_issue286_repeated_runs_hold_memory_steady(gpu_ctx):
+    # Test/NoFib/Issues/Issue286.hs ("check heap profile"): the same prepared function applied to a
+    # fresh 120x659 matrix of Word8 over and over; every run's blocks come back from the pool
+    go = gpu_ctx.compile(Q.issue286())
+    ones = np.ones((120, 659), np.uint8)
+    total, steady = 0.0, None
+    for n in range(300):
+        total += float(go(ones))
+        if n == 4:
+            steady = gpu_ctx.stat("bytes_allocated_remote")
+    assert total == 300 * 79080.0
+    assert gpu_ctx.stat("bytes_allocated_remote") == steady
 
 
 def test_awhile_jacobi_counts_iterations(gpu_ctx):
