@@ -73,6 +73,12 @@ template <class S> struct AccScanCfg {
 #ifndef ACC_SCAN_SLEEP
 #define ACC_SCAN_SLEEP 16    // s_sleep argument between two polls of the same window
 #endif
+#ifndef ACC_SCAN_SETTLE
+#define ACC_SCAN_SETTLE 32   // s_sleep argument before the first poll of a tile in a long launch
+#endif
+#ifndef ACC_SCAN_SETTLE_TILES
+#define ACC_SCAN_SETTLE_TILES 4096  // a launch of at least this many tiles is a long one
+#endif
 
 template <class E> ACC_DEV void acc_publish(u64* slot, const E& v, u64 epoch, u64 state) {
   u32 w[AccWords<E>::N];
@@ -165,7 +171,8 @@ ACC_DEV void acc_window(const typename S::Env& env, const u64* rowDesc, i64 look
 // Exclusive prefix of tile `tile` (> 0) of a row whose descriptors start at `rowDesc`.
 // Called by all threads of the workgroup; the result is valid in thread 0.
 template <class S>
-ACC_DEV bool acc_lookback(const typename S::Env& env, const u64* rowDesc, i64 tile, u64 epoch, typename S::Elt& excl) {
+ACC_DEV bool acc_lookback(const typename S::Env& env, const u64* rowDesc, i64 tile, u64 epoch, bool settle,
+                          typename S::Elt& excl) {
   typedef typename S::Elt Elt;
   enum { LB = ACC_SCAN_LBWAVES < ACC_SCAN_WAVES ? ACC_SCAN_LBWAVES : ACC_SCAN_WAVES };
   __shared__ Elt sh_win[LB];
@@ -176,6 +183,13 @@ ACC_DEV bool acc_lookback(const typename S::Env& env, const u64* rowDesc, i64 ti
   bool have = false;
   Elt running;
   i64 look = tile - 1;
+  // In a long launch the nearest predecessors have published a little less than one trip to
+  // their descriptors ago, so a poll sent at once finds them a moment too early and costs a
+  // whole further round trip; one sent 2048 cycles later mostly succeeds (2^28 Int64: 0.770 ->
+  // 0.757 ms).  Short launches, where every tile's wait is on the critical path, poll at once.
+  // (the condition goes through a scalar register: under a mere lane mask the scalar s_sleep
+  // would run whether or not any lane is enabled)
+  if (__builtin_amdgcn_readfirstlane((int)(settle && w < LB))) __builtin_amdgcn_s_sleep(ACC_SCAN_SETTLE);
   for (;;) {
     if (w < LB) {
       Elt r;
@@ -265,10 +279,11 @@ ACC_DEV void acc_rake(const typename S::Env& env, typename S::Elt* mine, const t
 // workgroup (ACC_SCAN_BLOCK threads).  When `plain` holds, a tile that lies completely inside
 // the sequence hands the V consecutive values of a lane to storeRun(t0, y) instead, which
 // can move them with one wide request: a caller whose store tests for a special position
-// (the total of scan') sets it for the tiles that cannot hold that position.
+// (the total of scan') sets it for the tiles that cannot hold that position.  `settle` delays
+// the first look at the predecessors (see acc_lookback).
 template <class S, class Load, class Store, class StoreRun>
 ACC_DEV void acc_scan_tile(const typename S::Env& env, u64* desc, i64 tiles, i64 tile, i64 n, u64 epoch,
-                           const Load& load, const Store& store, const StoreRun& storeRun, bool plain) {
+                           const Load& load, const Store& store, const StoreRun& storeRun, bool plain, bool settle) {
   typedef typename S::Elt Elt;
   typedef AccScanCfg<S> C;
   const int V = C::V, G = C::G, W = C::W;
@@ -385,7 +400,7 @@ ACC_DEV void acc_scan_tile(const typename S::Env& env, u64* desc, i64 tiles, i64
       hasExcl = true;
     }
   } else {
-    hasExcl = acc_lookback<S>(env, desc, tile, epoch, excl);  // valid in thread 0
+    hasExcl = acc_lookback<S>(env, desc, tile, epoch, settle, excl);  // valid in thread 0
   }
   if (threadIdx.x == 0) {
     if (successors && wavesWithData > 0) {

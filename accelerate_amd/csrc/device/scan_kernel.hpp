@@ -39,7 +39,8 @@ acc_scan(Spec::Env env, Spec::Out out, Spec::Out tot, ScanParams p) {
       S::store_run(out, outBase + (m - 1 - shift) - (t0 + S::V - 1), z);
     }
   };
-  acc_scan_tile<S>(env, rowDesc, p.tpr, tile, n, p.epoch, load, store, storeRun, S::kKind != 2 || tile + 1 < p.tpr);
+  acc_scan_tile<S>(env, rowDesc, p.tpr, tile, n, p.epoch, load, store, storeRun, S::kKind != 2 || tile + 1 < p.tpr,
+                   p.rows * p.tpr >= ACC_SCAN_SETTLE_TILES);
 
   if (S::kKind != 0 && tile == 0 && threadIdx.x == 0) {
     Elt z = S::seed(env);
