@@ -7,7 +7,9 @@
 // ACC_MAP_INDEXED (stencils) takes the multi-dimensional index as well.
 
 struct MapParams {
-  i64 n;  // number of results
+  i64 n;     // number of results
+  i64 base;  // workgroups of the launches that came before: index spaces of 2^32 threads
+             // and more are covered by several launches
 };
 
 template <bool NT>
@@ -18,9 +20,9 @@ ACC_DEV void acc_map_body(const Spec::Env& env, const Spec::Out& out, const MapP
   // producers that read neighbouring rows / planes (stencils): every XCD works on one
   // contiguous stretch of the result, so that what neighbouring workgroups share is found
   // in that XCD's L2
-  const i64 b = acc_xcd_contiguous((i64)blockIdx.x, (i64)gridDim.x);
+  const i64 b = p.base + acc_xcd_contiguous((i64)blockIdx.x, (i64)gridDim.x);
 #else
-  const i64 b = (i64)blockIdx.x;
+  const i64 b = p.base + (i64)blockIdx.x;
 #endif
   i64 i0 = (b * ACC_BLOCK + threadIdx.x) * V;
 #ifdef ACC_MAP_INDEXED

@@ -753,6 +753,7 @@ HValP Program::hostExp(const Sx& e, const AEnv& aenv, const Plan& plan) {
   std::vector<uint64_t> args = packArgs(k->meta, aenv, {}, {});
   packOut(args, *out);
   args.push_back(1);
+  args.push_back(0);
   ctx_.launch(k, "acc_map", 1, 256, args);
   std::vector<HValP> leaves;
   for (size_t i = 0; i < out->bufs.size(); ++i) {
@@ -819,9 +820,16 @@ void Program::launchMap(const KernelP& k, const AEnv& aenv, const std::vector<DA
   std::vector<uint64_t> args = packArgs(k->meta, aenv, temps, out.shape);
   packOut(args, out);
   args.push_back((uint64_t)n);
+  args.push_back(0);
   int64_t per = (int64_t)256 * k->meta.vec;
   const bool st = streams(k->meta, aenv, temps, arrayBytes(out));
-  ctx_.launch(k, st ? "acc_map_stream" : "acc_map", (unsigned)((n + per - 1) / per), 256, args);
+  // a launch holds fewer than 2^32 threads: larger index spaces take several
+  const char* me = std::getenv("ACCHIP_MAP_MAX_BLOCKS");  // for tests: several launches over a small index space
+  const int64_t blocks = (n + per - 1) / per, most = me && std::atoll(me) > 0 ? std::atoll(me) : (int64_t)1 << 23;
+  for (int64_t base = 0; base < blocks; base += most) {
+    args.back() = (uint64_t)base;
+    ctx_.launch(k, st ? "acc_map_stream" : "acc_map", (uint64_t)std::min(most, blocks - base), 256, args);
+  }
 }
 
 AValP Program::evalFun(const Sx& f, AEnv& aenv, const std::vector<AValP>& args) {
@@ -1015,7 +1023,7 @@ AValP Program::eval(const Sx& n, AEnv& aenv) {
       args.push_back((uint64_t)rows);
       args.push_back((uint64_t)w);
       args.push_back((uint64_t)tilesX);
-      ctx_.launch(plan.k, "acc_map_tiled", (unsigned)(tilesX * tilesY), 256, args);
+      ctx_.launch(plan.k, "acc_map_tiled", (uint64_t)(tilesX * tilesY), 256, args);
       return avArr(out);
     }
     launchMap(plan.k, aenv, temps, *out);
@@ -1067,7 +1075,7 @@ AValP Program::eval(const Sx& n, AEnv& aenv) {
         args.push_back((uint64_t)rows);
         args.push_back((uint64_t)len);
         args.push_back((uint64_t)rpt);
-        ctx_.launch(plan.k, "acc_fold_rows", (unsigned)groups, (unsigned)m.block, args);
+        ctx_.launch(plan.k, "acc_fold_rows", (uint64_t)groups, (unsigned)m.block, args);
         return avArr(out);
       }
     }
@@ -1096,8 +1104,8 @@ AValP Program::eval(const Sx& n, AEnv& aenv) {
     args.push_back((uint64_t)bpr);
     args.push_back((uint64_t)chunk);
     const bool st = streams(plan.k->meta, aenv, temps, 0);
-    ctx_.launch(plan.k, st ? "acc_fold_main_stream" : "acc_fold_main", (unsigned)(rows * bpr), 256, args);
-    if (bpr > 1) ctx_.launch(plan.k, "acc_fold_final", (unsigned)rows, 256, args);
+    ctx_.launch(plan.k, st ? "acc_fold_main_stream" : "acc_fold_main", (uint64_t)(rows * bpr), 256, args);
+    if (bpr > 1) ctx_.launch(plan.k, "acc_fold_final", (uint64_t)rows, 256, args);
     return avArr(out);
   }
   if (h == "permute") {
@@ -1162,14 +1170,14 @@ AValP Program::eval(const Sx& n, AEnv& aenv) {
       args.push_back((uint64_t)part);
       args.push_back((uint64_t)out->size());
       args.push_back((uint64_t)(uintptr_t)ctx_.errorWord());
-      ctx_.launch(plan.k, "acc_permute_lds", (unsigned)(groups * nparts), 1024, args);
+      ctx_.launch(plan.k, "acc_permute_lds", (uint64_t)(groups * nparts), 1024, args);
       return avArr(out);
     }
     args.push_back((uint64_t)cnt);
     args.push_back(locks ? (uint64_t)(uintptr_t)locks->bufs[0]->p : 0);
     args.push_back((uint64_t)(uintptr_t)ctx_.errorWord());
     int64_t grid = std::min<int64_t>((cnt + 255) / 256, 256 * 32);
-    ctx_.launch(plan.k, "acc_permute", (unsigned)grid, 256, args);
+    ctx_.launch(plan.k, "acc_permute", (uint64_t)grid, 256, args);
     return avArr(out);
   }
   if (h == "stencil" || h == "stencil2") {
@@ -1202,7 +1210,7 @@ AValP Program::eval(const Sx& n, AEnv& aenv) {
       chain = std::max<int64_t>(1, std::min(chain, tilesY));
       args.push_back((uint64_t)chain);
       const int64_t chunksY = (tilesY + chain - 1) / chain;
-      ctx_.launch(plan.k, "acc_stencil2d", (unsigned)(tilesX * chunksY), 256, args);
+      ctx_.launch(plan.k, "acc_stencil2d", (uint64_t)(tilesX * chunksY), 256, args);
       return avArr(out);
     }
     if (plan.mode == "lds3d") {
@@ -1223,7 +1231,7 @@ AValP Program::eval(const Sx& n, AEnv& aenv) {
       args.push_back((uint64_t)tilesX);
       args.push_back((uint64_t)tilesY);
       args.push_back((uint64_t)chain);
-      ctx_.launch(plan.k, "acc_stencil3d", (unsigned)(tilesX * tilesY * chunksZ), 256, args);
+      ctx_.launch(plan.k, "acc_stencil3d", (uint64_t)(tilesX * tilesY * chunksZ), 256, args);
       return avArr(out);
     }
     launchMap(plan.k, aenv, temps, *out);
@@ -1268,9 +1276,9 @@ AValP Program::eval(const Sx& n, AEnv& aenv) {
     args.push_back((uint64_t)(uintptr_t)ctx_.errorWord());
     const int64_t boundaries = rows * (nseg + 1);
     if ((boundaries + 255) / 256 > 0x7fffffffLL) throw Error("foldSeg: too many segments for one launch");
-    ctx_.launch(plan.k, "acc_foldseg_partition", (unsigned)((boundaries + 255) / 256), 256, args);
-    ctx_.launch(plan.k, "acc_foldseg", (unsigned)tiles, (unsigned)m.block, args);
-    ctx_.launch(plan.k, "acc_foldseg_fixup", (unsigned)((tiles + 3) / 4), 256, args);
+    ctx_.launch(plan.k, "acc_foldseg_partition", (uint64_t)((boundaries + 255) / 256), 256, args);
+    ctx_.launch(plan.k, "acc_foldseg", (uint64_t)tiles, (unsigned)m.block, args);
+    ctx_.launch(plan.k, "acc_foldseg_fixup", (uint64_t)((tiles + 3) / 4), 256, args);
     return avArr(out);
   }
   if (h == "scan" || h == "scan'") {
@@ -1320,7 +1328,7 @@ AValP Program::eval(const Sx& n, AEnv& aenv) {
         args.push_back((uint64_t)rows);
         args.push_back((uint64_t)len);
         args.push_back((uint64_t)rpt);
-        ctx_.launch(plan.k2, "acc_scan_rows", (unsigned)groups, (unsigned)sm.block, args);
+        ctx_.launch(plan.k2, "acc_scan_rows", (uint64_t)groups, (unsigned)sm.block, args);
         return result;
       }
     }
@@ -1341,7 +1349,7 @@ AValP Program::eval(const Sx& n, AEnv& aenv) {
     args.push_back((uint64_t)(uintptr_t)st.ticket);
     args.push_back((uint64_t)st.ticketBase);
     args.push_back((uint64_t)st.epoch);
-    ctx_.launch(kern, "acc_scan", (unsigned)tiles, (unsigned)m.block, args);
+    ctx_.launch(kern, "acc_scan", (uint64_t)tiles, (unsigned)m.block, args);
     st.ticketBase += (uint64_t)tiles;
     return result;
   }

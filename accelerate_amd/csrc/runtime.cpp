@@ -404,8 +404,12 @@ void Context::ensureLoaded(const KernelP& k) {
   hipCheck(hipModuleLoadData(&k->module, k->code.data()), "hipModuleLoadData");
 }
 
-void Context::launch(const KernelP& k, const char* fn, unsigned grid, unsigned block, const std::vector<uint64_t>& args) {
+void Context::launch(const KernelP& k, const char* fn, uint64_t grid, unsigned block, const std::vector<uint64_t>& args) {
   if (grid == 0) return;
+  // a launch holds fewer than 2^32 threads; a count cut to 32 bits would leave part of the work undone
+  if (grid > 0x7fffffffull || grid * block > 0xffffffffull)
+    throw Error(std::string(fn) + ": " + std::to_string(grid) + " workgroups of " + std::to_string(block) +
+                " threads exceed what one launch can hold");
   hipFunction_t f;
   {
     std::lock_guard<std::mutex> g(mu_);
@@ -421,8 +425,8 @@ void Context::launch(const KernelP& k, const char* fn, unsigned grid, unsigned b
   size_t size = args.size() * sizeof(uint64_t);
   void* config[] = {HIP_LAUNCH_PARAM_BUFFER_POINTER, (void*)args.data(), HIP_LAUNCH_PARAM_BUFFER_SIZE, &size,
                     HIP_LAUNCH_PARAM_END};
-  if (dumpExec) fprintf(stderr, "[acchip] launch %s<<<%u,%u>>> %s (%zu arg bytes)\n", fn, grid, block, k->hash.substr(0, 12).c_str(), size);
-  hipCheck(hipModuleLaunchKernel(f, grid, 1, 1, block, 1, 1, 0, stream_, nullptr, config), "hipModuleLaunchKernel");
+  if (dumpExec) fprintf(stderr, "[acchip] launch %s<<<%llu,%u>>> %s (%zu arg bytes)\n", fn, (unsigned long long)grid, block, k->hash.substr(0, 12).c_str(), size);
+  hipCheck(hipModuleLaunchKernel(f, (unsigned)grid, 1, 1, block, 1, 1, 0, stream_, nullptr, config), "hipModuleLaunchKernel");
   stats.launches++;
 }
 

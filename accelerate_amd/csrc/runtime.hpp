@@ -72,7 +72,7 @@ class Context : public std::enable_shared_from_this<Context> {
   // there, and throws what the compiler reported.
   KernelP kernel(const KernelSource& ks);
   void wait(const KernelP& k);
-  void launch(const KernelP& k, const char* fn, unsigned grid, unsigned block, const std::vector<uint64_t>& args);
+  void launch(const KernelP& k, const char* fn, uint64_t grid, unsigned block, const std::vector<uint64_t>& args);
 
   // Where Atrace nodes deliver their message and the arrays they were given (the C ABI
   // installs the caller's callback here; the value is an AVal); empty: a line on stderr.

@@ -1166,3 +1166,27 @@ def misc_cache(which):
         return A.alet(V, c, lambda cv: A.alet(V, d(), lambda dv: A.zipwith(
             A.f32, plus, A.fold(plus, A.const(A.f32, 0), cv), A.fold(plus, A.const(A.f32, 0), dv))))
     return A.alam([V, V], body)
+
+
+def long_array_programs(big, n):
+    """Three closed programs over arrays made on the device: fold (+) 7 over the delayed source
+    i -> i .&. 255 of `big` elements; the last 8 elements of map (+1) over `big` manifest bytes
+    i .&. 255; the last 6 elements of scanl1 (+) over n Int32 ones."""
+    sh1 = A.tshape(1)
+    low = lambda i: A.band(Int, i, A.constI(255))
+    src = A.delayed(A.tarray(1, Int), A.sh(A.constI(big)), A.lam([sh1], lambda ix: low(A.untup(ix)[0])), A.lam([Int], low))
+    fold = A.fold(binop(A.add, Int), A.constI(7), src)
+    B, I32 = A.u8, A.i32
+    tail = lambda ys, m, k: A.backpermute(1, A.sh(A.constI(k)), A.lam(
+        [sh1], lambda ix: A.sh(A.add(Int, A.untup(ix)[0], A.constI(m - k)))), ys)
+    bytes_ = A.generate(A.tarray(1, B), A.sh(A.constI(big)), A.lam([sh1], lambda ix: A.fromintegral(Int, B, low(A.untup(ix)[0]))))
+    far_end = A.alet(A.tarray(1, B), bytes_, lambda xs: A.alet(
+        A.tarray(1, B), A.map_(B, A.lam([B], lambda x: A.add(B, x, A.const(B, 1))), xs), lambda ys: tail(ys, big, 8)))
+    ones = A.generate(A.tarray(1, I32), A.sh(A.constI(n)), A.lam([sh1], lambda ix: A.const(I32, 1)))
+    scan_end = A.alet(A.tarray(1, I32), ones, lambda xs: A.alet(
+        A.tarray(1, I32), A.scan("l", binop(A.add, I32), None, xs), lambda ys: tail(ys, n, 6)))
+    return fold, far_end, scan_end
+
+
+def long_fold_expected(big):
+    return 7 + (big // 256) * (255 * 128) + sum(range(big % 256))

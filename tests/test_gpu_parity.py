@@ -180,6 +180,34 @@ def test_histogram_2pow26_bit_exact(gpu_ctx):
     assert got.sum(dtype=np.int64) == n and np.array_equal(got, np.bincount(keys, minlength=nbins))
 
 
+def test_map_over_several_launches(gpu_ctx, monkeypatch):
+    # index spaces of 2^32 threads and more are covered by several launches of the map skeleton;
+    # here the limit is lowered to 3 workgroups so that small arrays take that path: a plain map,
+    # an indexed generate of rank 3 and a directly evaluated stencil (XCD-contiguous numbering)
+    monkeypatch.setenv("ACCHIP_MAP_MAX_BLOCKS", "3")
+    monkeypatch.setenv("ACCHIP_STENCIL_NO2D", "1")
+    rng = np.random.default_rng(5)
+    x = rng.standard_normal(50001).astype(np.float32)
+    assert np.array_equal(gpu_ctx.compile(P.map_affine())(x), x * np.float32(2) + np.float32(1))
+    cube = rng.standard_normal((7, 33, 65)).astype(np.float32)
+    prog = Q.indexed(3)
+    assert same(gpu_ctx.compile(prog)(cube), O.run_n(prog.text(), cube))
+    g = rng.uniform(0, 1, (67, 131)).astype(np.float32)
+    assert same(gpu_ctx.compile(P.jacobi_step())(g), OC.jacobi_f32(g, 1))
+
+
+def test_arrays_of_more_than_2p32_elements(gpu_ctx):
+    # linear indices, grids and tile counts beyond 32 bits: a fold over a delayed source of
+    # 2^32 + 5 elements (closed form), a manifest map over as many bytes read back at its far
+    # end, and scanl1 over 2^31 + 3 Int32 ones, whose last prefixes wrap around
+    big, n = (1 << 32) + 5, (1 << 31) + 3
+    fold, far_end, scan_end = Q.long_array_programs(big, n)
+    assert int(gpu_ctx.compile(fold)()) == Q.long_fold_expected(big)
+    assert np.array_equal(gpu_ctx.compile(far_end)(), ((np.arange(big - 8, big) & 255) + 1).astype(np.uint8))
+    assert np.array_equal(gpu_ctx.compile(scan_end)(), np.arange(n - 5, n + 1, dtype=np.int64).astype(np.int32))
+    gpu_ctx.purge()
+
+
 TILE_EDGES = sorted({t * k + d for t in (4096, 8192, 12288, 24576, 49152) for k in (1, 2, 5) for d in (-1, 0, 1)})
 
 

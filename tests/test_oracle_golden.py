@@ -336,3 +336,13 @@ def test_oracle_on_blackscholes_against_numpy():
     call, put = O.run_n(Q.blackscholes(A.f64).text(), [p, s, y])
     assert np.allclose(call, p * cnd(d1) - xe * cnd(d2), rtol=1e-12, atol=1e-12)
     assert np.allclose(put, xe * (1.0 - cnd(d2)) - p * (1.0 - cnd(d1)), rtol=1e-12, atol=1e-12)
+
+
+def test_long_array_programs_at_a_small_size():
+    # the programs of the GPU test over more than 2^32 elements, at a size the oracle walks:
+    # their closed-form expectations are checked here
+    big, n = 1000 + 5, 50
+    fold, far_end, scan_end = Q.long_array_programs(big, n)
+    assert int(O.run_n(fold.text())) == Q.long_fold_expected(big) == 7 + sum(i & 255 for i in range(big))
+    assert same(O.run_n(far_end.text()), ((np.arange(big - 8, big) & 255) + 1).astype(np.uint8))
+    assert same(O.run_n(scan_end.text()), np.arange(n - 5, n + 1).astype(np.int32))
