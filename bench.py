@@ -142,7 +142,7 @@ def main():
         del dv, dl
         nk, nb = 1 << 26, 1 << 16
         dk = ctx.to_device(W.zipf_keys(nk, nb, 15), A.tarray(1, A.i32))
-        _, ev = time_program(ctx, ctx.compile(P.histogram(nb)), [dk], 3, 1)
+        _, ev = time_program(ctx, ctx.compile(P.histogram(nb)), [dk], 20, 5)
         sk.append(entry("histogram: permute (+) of 2^26 Zipf(1.1) keys into 2^16 Int32 bins", nk, 4 * nk + 8 * nb, ev))
         del dk
         side = 8192
