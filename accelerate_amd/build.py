@@ -44,10 +44,19 @@ def build(verbose=True):
     # so the host compiler builds it against the HIP runtime and hipRTC.
     rocm = os.environ.get("ROCM_PATH", "/opt/rocm")
     cxx = os.environ.get("CXX", "g++")
+    # ... except scratch.hip, which holds a static device array and is compiled by hipcc
+    hipcc = os.path.join(rocm, "bin", "hipcc")
+    obj = os.path.join(HERE, "build", "scratch.o")
+    hcmd = [hipcc, "--offload-arch=gfx950", "-O2", "-std=c++17", "-fPIC", "-c",
+            "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+            "-o", obj, os.path.join(CSRC, "scratch.hip")]
+    if verbose:
+        print(" ".join(hcmd), flush=True)
+    subprocess.run(hcmd, check=True, stderr=None if verbose else subprocess.DEVNULL)
     cmd = [cxx, "-O2", "-std=c++17", "-fPIC", "-shared", "-Wall", "-Wno-unused-function",
            "-D__HIP_PLATFORM_AMD__", "-I" + os.path.join(rocm, "include"),
            "-o", LIB] + [os.path.join(CSRC, s) for s in HOST_SOURCES] + [
-               gen, "-L" + os.path.join(rocm, "lib"), "-Wl,-rpath," + os.path.join(rocm, "lib"),
+               gen, obj, "-L" + os.path.join(rocm, "lib"), "-Wl,-rpath," + os.path.join(rocm, "lib"),
                "-lamdhip64", "-lhiprtc", "-pthread", "-ldl"]
     if verbose:
         print(" ".join(cmd), flush=True)

@@ -347,4 +347,22 @@ int acchip_execute(acchip_ctx* ctx, acchip_program* p, acchip_array* const* args
   ACCHIP_END
 }
 
+int acchip_execute_into(acchip_ctx* ctx, acchip_program* p, acchip_array* const* args, int n_args,
+                        acchip_array* const* uses, int n_uses, acchip_array* result) {
+  ACCHIP_TRY
+  if (!ctx->ctx->hasDevice()) throw Error("no device");
+  if (p->keep != ctx->ctx) throw Error("program was compiled in a different context");
+  if (!result) throw Error("acchip_execute_into: null result array");
+  std::vector<AValP> av;
+  for (int i = 0; i < n_args; ++i) av.push_back(args[i]->v);
+  std::vector<DArrayP> uv;
+  for (int i = 0; i < n_uses; ++i) {
+    if (uses[i]->v->k != AVal::Arr) throw Error("use slots take single arrays");
+    uv.push_back(uses[i]->v->arr);
+  }
+  p->prog.runInto(av, uv, result->v);
+  return ACCHIP_OK;
+  ACCHIP_END
+}
+
 }  // extern "C"

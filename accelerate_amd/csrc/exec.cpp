@@ -350,6 +350,13 @@ Program::Program(Context& ctx, const char* text, size_t len) : ctx_(ctx) {
     ctx_.wait(kv.second.k2);
     for (auto& sk : kv.second.scalarKernels) ctx_.wait(sk.second);
   }
+  // a program that is one scan can be run without allocating (runInto): its code objects are
+  // loaded now, so that no launch of it has set-up work left
+  if (ctx_.hasDevice() && (body_->is("scan") || body_->is("scan'"))) {
+    const Plan& plan = plans_.at(body_);
+    ctx_.preload(plan.k, {"acc_scan", "acc_scan_rows"});
+    ctx_.preload(plan.k2, {"acc_scan", "acc_scan_rows"});
+  }
 }
 
 std::vector<ArrayR> Program::aenvOf(const TEnv& tenv) {
@@ -619,6 +626,20 @@ ATyP Program::prepare(const Sx& n, TEnv& tenv) {
 // execution
 
 DArrayP Program::alloc(const ArrayR& r, const std::vector<int64_t>& shape) {
+  if (noAlloc_) {
+    if (destNext_ >= dest_.size())
+      throw Error("this program needs device memory beyond its results, which acchip_execute_into does not provide");
+    const DArrayP& d = dest_[destNext_++];
+    if (d->r.rank != r.rank || !typeEq(d->r.elt, r.elt))
+      throw Error("result array has the wrong type: the program yields rank " + std::to_string(r.rank) + ", " +
+                  typeStr(r.elt));
+    if (d->shape != shape) {
+      std::string want;
+      for (int64_t x : shape) want += (want.empty() ? "" : " x ") + std::to_string(x);
+      throw Error("result array has the wrong extents: the program yields " + (want.empty() ? std::string("a scalar") : want));
+    }
+    return d;
+  }
   auto a = std::make_shared<DArray>();
   a->r = r;
   a->shape = shape;
@@ -644,6 +665,7 @@ void Program::packOut(std::vector<uint64_t>& args, const DArray& a) {
 // something there reads it: a kernel that takes the array, a copy, or the caller.
 void Program::materialize(DArray& a) {
   if (!a.hostKnown || a.onDevice) return;
+  if (noAlloc_) throw Error("an argument of acchip_execute_into has not been written to the device yet");
   auto leaves = typeLeaves(a.r.elt);
   void* p = a.bufs.at(0)->p;
   const uint64_t v = (uint64_t)a.hostValue;
@@ -855,6 +877,43 @@ AValP Program::run(const std::vector<AValP>& args, const std::vector<DArrayP>& u
   AValP r = eval(*body_, aenv);
   materializeAll(r);  // what the caller gets is on the device
   return r;
+}
+
+void Program::runInto(const std::vector<AValP>& args, const std::vector<DArrayP>& uses, const AValP& dest) {
+  if (args.size() != lams_.size())
+    throw Error("program expects " + std::to_string(lams_.size()) + " arguments, got " + std::to_string(args.size()));
+  const bool prime = body_->is("scan'");
+  if (!prime && !body_->is("scan"))
+    throw Error("acchip_execute_into runs programs whose body is a single scan; this one is not");
+  const Plan& plan = plans_.at(body_);
+  if (!plan.temps.empty() || !plan.scalarKernels.empty())
+    throw Error("acchip_execute_into: the scan's operand must be an array variable or a fused producer whose extent "
+                "the host can compute");
+  std::vector<DArrayP> d;
+  if (prime) {
+    if (dest->k != AVal::Pair || dest->a->k != AVal::Arr || dest->b->k != AVal::Arr)
+      throw Error("acchip_execute_into: the result of scanl' / scanr' is a pair (array, totals)");
+    d = {dest->a->arr, dest->b->arr};
+  } else {
+    if (dest->k != AVal::Arr) throw Error("acchip_execute_into: the result is a single array");
+    d = {dest->arr};
+  }
+  struct Mode {  // left again however the call ends
+    Program& p;
+    ~Mode() {
+      p.noAlloc_ = false;
+      p.dest_.clear();
+      p.destNext_ = 0;
+    }
+  } mode{*this};
+  noAlloc_ = true;
+  dest_ = std::move(d);
+  destNext_ = 0;
+  uses_ = &uses;
+  AEnv aenv;
+  for (size_t i = 0; i < args.size(); ++i) pushVals(lams_[i]->at(1), args[i], aenv);
+  eval(*body_, aenv);
+  if (destNext_ != dest_.size()) throw Error("internal: acchip_execute_into left a result unwritten");
 }
 
 AValP Program::eval(const Sx& n, AEnv& aenv) {
@@ -1338,7 +1397,8 @@ AValP Program::eval(const Sx& n, AEnv& aenv) {
     const int64_t tpr = std::max<int64_t>(1, (len + tile - 1) / tile);
     const int64_t tiles = rows * tpr;
     if (tiles > 0x7fffffffLL) throw Error("scan: too many tiles for one launch");
-    Context::ScanState& st = ctx_.scanState((size_t)tiles * m.words * sizeof(uint64_t));
+    const size_t descBytes = (size_t)tiles * m.words * sizeof(uint64_t);
+    ScanState& st = noAlloc_ ? staticScanState(ctx_.device(), ctx_.stream(), descBytes) : ctx_.scanState(descBytes);
     std::vector<uint64_t> args = packArgs(m, aenv, temps, {});
     packOut(args, *out);
     packOut(args, *tot);

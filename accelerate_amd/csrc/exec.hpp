@@ -85,6 +85,11 @@ class Program {
   Program(Context& ctx, const char* text, size_t len);
   // args: one AVal per lambda of the program, in order; uses: arrays for (use ..) slots
   AValP run(const std::vector<AValP>& args, const std::vector<DArrayP>& uses);
+  // The same for a program whose body is one scan over array variables or fused producers,
+  // written into arrays the caller made (`dest`: the result array, or the pair (array, totals)
+  // of scanl' / scanr'); tile descriptors and ticket live in the device's static scratch, so the
+  // call allocates no device memory.  Throws when the program or its size does not qualify.
+  void runInto(const std::vector<AValP>& args, const std::vector<DArrayP>& uses, const AValP& dest);
 
   std::vector<ATyP> argTypes;
   ATyP resultType;
@@ -97,6 +102,11 @@ class Program {
   std::vector<const Sx*> lams_;
   std::map<const Sx*, Plan> plans_;
   const std::vector<DArrayP>* uses_ = nullptr;
+  // runInto: alloc() hands out the caller's arrays, in the order the node asks for its results,
+  // and fails once they are used up
+  bool noAlloc_ = false;
+  std::vector<DArrayP> dest_;
+  size_t destNext_ = 0;
 
   using TEnv = std::vector<ArrayR>;     // back() has de Bruijn index 0
   using AEnv = std::vector<DArrayP>;

@@ -47,6 +47,7 @@ Context::Context(int device) : device_(device) {
   if (device_ >= 0) {
     hipCheck(hipSetDevice(device_), "hipSetDevice");
     hipCheck(hipStreamCreateWithFlags(&stream_, hipStreamNonBlocking), "hipStreamCreate");
+    staticScratchSetup(device_);  // address of the static scan scratch on this device
   }
 }
 
@@ -231,7 +232,7 @@ void Context::raiseDeviceError() {
   if (code != 0) throw Error("a kernel reported error " + std::to_string(code));
 }
 
-Context::ScanState& Context::scanState(size_t descBytes) {
+ScanState& Context::scanState(size_t descBytes) {
   if (!scan_.ticket) {
     hipCheck(hipMalloc((void**)&scan_.ticket, 256), "hipMalloc(scan ticket)");
     hipCheck(hipMemsetAsync(scan_.ticket, 0, 256, stream_), "hipMemsetAsync");
@@ -402,6 +403,18 @@ void Context::ensureLoaded(const KernelP& k) {
   wait(k);
   if (device_ < 0) throw Error("this context has no device: programs can be compiled but not executed");
   hipCheck(hipModuleLoadData(&k->module, k->code.data()), "hipModuleLoadData");
+}
+
+void Context::preload(const KernelP& k, std::initializer_list<const char*> fns) {
+  if (!k || device_ < 0) return;
+  std::lock_guard<std::mutex> g(mu_);
+  ensureLoaded(k);
+  for (const char* fn : fns) {
+    if (k->fns.count(fn)) continue;
+    hipFunction_t f;
+    hipCheck(hipModuleGetFunction(&f, k->module, fn), fn);
+    k->fns[fn] = f;
+  }
 }
 
 void Context::launch(const KernelP& k, const char* fn, uint64_t grid, unsigned block, const std::vector<uint64_t>& args) {

@@ -15,6 +15,7 @@
 #include <vector>
 
 #include "codegen.hpp"
+#include "scratch.hpp"
 
 namespace acchip {
 
@@ -78,15 +79,12 @@ class Context : public std::enable_shared_from_this<Context> {
   // installs the caller's callback here; the value is an AVal); empty: a line on stderr.
   std::function<void(const std::string& msg, const std::shared_ptr<void>& arrays)> traceSink;
 
-  // persistent device scratch for single-pass scans (tile descriptors + ticket counter)
-  struct ScanState {
-    void* desc = nullptr;
-    size_t descBytes = 0;
-    unsigned long long* ticket = nullptr;
-    unsigned long long ticketBase = 0;
-    unsigned epoch = 0;
-  };
+  // persistent device scratch for single-pass scans (tile descriptors + ticket counter),
+  // allocated and grown on demand
   ScanState& scanState(size_t descBytes);
+  // Load the kernel's code object and look its entry points up now instead of at the first
+  // launch, so that a later launch does no set-up work on the device.
+  void preload(const KernelP& k, std::initializer_list<const char*> fns);
 
   Stats stats;
   std::string cacheDir;

@@ -80,6 +80,7 @@ def lib():
         "acchip_sha3_256": (C.c_int, [vp, C.c_size_t, C.c_char_p]),
         "acchip_set_trace": (C.c_int, [vp, vp, vp]),
         "acchip_execute": (C.c_int, [vp, vp, C.POINTER(vp), C.c_int, C.POINTER(vp), C.c_int, C.POINTER(vp)]),
+        "acchip_execute_into": (C.c_int, [vp, vp, C.POINTER(vp), C.c_int, C.POINTER(vp), C.c_int, vp]),
     }
     for name, (res, args) in sigs.items():
         fn = getattr(L, name)
@@ -198,6 +199,21 @@ class Context:
             if p.nbytes:
                 _check(lib().acchip_poke(self._h, lib().acchip_array_buffer(h, k), p.ctypes.data, p.nbytes))
         return arr
+
+    def empty(self, shape, aty):
+        """An uninitialised device array of the given extents (acchip_array_new)."""
+        rank, ety = int(aty[1]), aty[2]
+        if len(shape) != rank:
+            raise ValueError("array of rank %d asked for where rank %d is declared" % (len(shape), rank))
+        h = C.c_void_p()
+        shp = (C.c_int64 * max(1, rank))(*shape)
+        _check(lib().acchip_array_new(self._h, rank, shp, ir.render(ety).encode(), C.byref(h)))
+        return DeviceArray(self, h)
+
+    def pair(self, a, b):
+        h = C.c_void_p()
+        _check(lib().acchip_array_pair(a._h, b._h, C.byref(h)))
+        return DeviceArray(self, h)
 
     def compile(self, program):
         return Program(self, program)
@@ -340,6 +356,18 @@ class Program:
         res = C.c_void_p()
         _check(lib().acchip_execute(self.ctx._h, self._h, av, len(hs), uv, len(uses), C.byref(res)))
         return DeviceArray(self.ctx, res)
+
+    def execute_into(self, result, *args, uses=()):
+        """acchip_execute_into: a single-scan program written into `result`, a DeviceArray the
+        caller made; allocates no device memory."""
+        if len(args) != len(self.arg_types):
+            raise TypeError("program takes %d arguments" % len(self.arg_types))
+        if not all(isinstance(a, DeviceArray) for a in args):
+            raise TypeError("execute_into takes device arrays")
+        av = (C.c_void_p * max(1, len(args)))(*[a._h for a in args])
+        uv = (C.c_void_p * max(1, len(uses)))(*[u._h for u in uses])
+        _check(lib().acchip_execute_into(self.ctx._h, self._h, av, len(args), uv, len(uses), result._h))
+        return result
 
     def __call__(self, *args, uses=()):
         """numpy in, numpy out (the `go` closure of runN)."""

@@ -154,6 +154,22 @@ int acchip_set_trace(acchip_ctx* ctx, acchip_trace_fn fn, void* user);
 int acchip_execute(acchip_ctx* ctx, acchip_program* p, acchip_array* const* args, int n_args,
                    acchip_array* const* uses, int n_uses, acchip_array** result);
 
+/* No counterpart in the reference: a variant of acchip_execute for callers that cannot allocate
+ * device memory (code under HIP graph capture, tight serving loops, harnesses that forbid
+ * hipMalloc).  The program's body must be a single scan (any of the six) whose operand is an
+ * array variable or a fused producer with a host-computable extent; `result` is an array the
+ * caller made (acchip_array_wrap / acchip_array_new) with the type and extents of the
+ * program's result -- for scanl' / scanr' the pair (array, totals) built with
+ * acchip_array_pair.  The tile descriptors and the ticket counter that acchip_execute keeps in
+ * pool memory live in a static device array of 1 MiB + 256 B per GPU instead (131072 descriptor
+ * words: a scan may have at most 131072 / ceil(element bytes / 4) tiles, e.g. 2^28 Int64 or
+ * Float32 elements in one row take 10923 or 5462 tiles); larger scans fail with an error and
+ * nothing is launched.  The call performs no hipMalloc / hipFree and clears nothing with memset
+ * nodes; code objects were loaded by acchip_compile.  All contexts on one GPU share the array:
+ * calls of this entry point that overlap on one GPU (two streams, two threads) race. */
+int acchip_execute_into(acchip_ctx* ctx, acchip_program* p, acchip_array* const* args, int n_args,
+                        acchip_array* const* uses, int n_uses, acchip_array* result);
+
 #ifdef __cplusplus
 }
 #endif
