@@ -35,7 +35,8 @@ static int fail(const std::exception& e) {
   const std::string& m = g_lastError;
   if (m.find("Remote memory exhausted") != std::string::npos) return ACCHIP_OUT_OF_MEMORY;
   if (m.find("no device") != std::string::npos) return ACCHIP_NO_DEVICE;
-  if (m == "empty array" || m == "shape mismatch" || m == "empty segment descriptor" || m == "empty segment")
+  if (m == "empty array" || m == "shape mismatch" || m == "empty segment descriptor" || m == "empty segment" ||
+      m.compare(0, 19, "index out of bounds") == 0)
     return ACCHIP_BOUNDS;
   return ACCHIP_ERROR;
 }

@@ -1389,7 +1389,7 @@ KernelSource Codegen::permute(const Sx& f, const ArrayR& dst, const Sx& p, const
   std::vector<std::string> leafOps;
   if (mode == "lock" && componentwiseAtomic(f, leaves, leafOps)) mode = "atomics";
   std::string lds;
-  std::string u = "  ACC_DEV void update(const Env& env, const Out& out, i64 j, const Elt& x, u32* locks) {\n";
+  std::string u = "  ACC_DEV void update(const Env& env, const Out& out, i64 j, const Elt& x, u32* locks, u32* err) {\n";
   if (mode == "store") {
     u += "    Elt y_{};\n    store(out, j, combine(env, x, y_));\n";
   } else if (mode == "atomic") {
@@ -1420,7 +1420,10 @@ KernelSource Codegen::permute(const Sx& f, const ArrayR& dst, const Sx& p, const
     // ballot).  With a per-lane exit the compiler may move the critical section behind the
     // loop, where a lane that won the lock waits for the lanes still spinning on it: two
     // lanes of one wave with the same destination then never finish.
-    u += "    u32* lk_ = locks + j;\n    bool done_ = false;\n    while (__ballot(!done_) != 0ull) {\n";
+    // The wait for a lock is bounded (ACC_LOCK_SPIN_LIMIT rounds, seconds): a lane that never
+    // gets its lock reports through err and drops its update, so that the kernel always ends.
+    u += "    u32* lk_ = locks + j;\n    bool done_ = false;\n    u32 rounds_ = 0;\n    while (__ballot(!done_) != 0ull) {\n";
+    u += "      if (++rounds_ > ACC_LOCK_SPIN_LIMIT) {\n        if (!done_) __hip_atomic_store(err, 4u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);\n        break;\n      }\n";
     u += "      if (!done_ && __hip_atomic_exchange(lk_, 1u, __ATOMIC_ACQUIRE, __HIP_MEMORY_SCOPE_AGENT) == 0u) {\n        Elt y_;\n";
     // leaf by leaf (component by component for SIMD vector leaves) through relaxed atomics
     auto each = [&](size_t k, const std::function<void(const std::string& cell, const std::string& field)>& fn) {
@@ -1502,6 +1505,12 @@ static void stencilHalo(const Sx& sr, int dim, std::vector<int>& halo) {
   halo[dim] = std::max(halo[dim], w / 2);
   if (sr.head().compare(0, 4, "unit") != 0)
     for (size_t r = 1; r < sr.size(); ++r) stencilHalo(sr.at(r), dim + 1, halo);
+}
+
+std::vector<int> stencilHaloOf(const Sx& pattern) {
+  std::vector<int> halo;
+  stencilHalo(pattern, 0, halo);
+  return halo;
 }
 
 KernelSource Codegen::stencil(const std::vector<Sx>& patterns, const TypeP& outElt, const Sx& f,

@@ -133,6 +133,8 @@ class Codegen {
                       const std::string& skeleton, int vec);
 };
 
+// taps a stencil pattern reaches on either side of the focus, per dimension (outermost first)
+std::vector<int> stencilHaloOf(const Sx& pattern);
 std::string literalText(ST st, const std::string& tok);
 const std::string& deviceHeader(const std::string& name);  // embedded device/*.hpp text
 

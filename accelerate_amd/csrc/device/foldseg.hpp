@@ -229,6 +229,10 @@ ACC_DEV void acc_foldseg_tile(const Spec::Env& env, const Spec::Out& out, const 
     c = c < 0 ? 0 : (c > V ? V : c);
     const S::Elt* e = x[g];
     P a{};
+    // a run past the end of the stream stands for a real element without a head: the raking
+    // below applies the combination function to every run, and that function may only ever
+    // see values of the array
+    if (!FULL && c == 0 && n > 0) a.v = S::in_linear(env, tlo);
     bool has = false;
     pendIdx[g] = NOPEND;
 #pragma unroll

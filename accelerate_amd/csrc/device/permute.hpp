@@ -16,7 +16,7 @@
 struct PermuteParams {
   i64 n;       // number of source elements
   u32* locks;  // one word per destination element, zero when free (lock mode only)
-  u32* err;    // host-visible word: 2 = a target outside the destination
+  u32* err;    // host-visible word: 2 = a target outside the destination, 4 = a lock never came free
 };
 
 extern "C" __global__ void __launch_bounds__(ACC_BLOCK)
@@ -29,7 +29,7 @@ acc_permute(Spec::Env env, Spec::Out out, PermuteParams p) {
     const int t = S::target(env, i, j);
     if (t == 1) {
       S::Elt x = S::in_linear(env, i);
-      S::update(env, out, j, x, p.locks);
+      S::update(env, out, j, x, p.locks, p.err);
     }
     bad = bad || t == 2;
   }
@@ -71,7 +71,7 @@ struct PermuteLdsParams {
   i64 nparts;  // destination ranges
   i64 part;    // elements per range
   i64 dst_n;   // destination elements
-  u32* err;    // host-visible word: 2 = a target outside the destination
+  u32* err;    // host-visible word: 2 = a target outside the destination, 4 = a lock never came free
 };
 
 extern "C" __global__ void __launch_bounds__(ACC_PERMUTE_LDS_BLOCK)

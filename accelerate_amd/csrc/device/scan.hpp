@@ -43,6 +43,8 @@ struct ScanParams {
   u64* ticket;      // monotonically increasing counter shared by all launches of a context
   u64 ticket_base;  // value of the counter when this launch starts
   u64 epoch;        // tag of this launch, 1 .. 2^30 - 1
+  u64 spin_limit;   // polls of one window after which a tile stops waiting for its predecessors
+  u32* err;         // host-visible word: 3 = a tile gave up waiting, or took a ticket outside the launch
 };
 
 #ifndef ACC_SCAN_BLOCK
@@ -124,9 +126,16 @@ ACC_DEV bool acc_join(const typename S::Env& env, bool ha, const typename S::Elt
 // inclusive prefix, or the start of the row), or 64 aggregates.  On return lane 0 holds in
 // `r` the ordered combination of the `nv` values found (nv may be 0) and `terminal` says
 // whether the walk ends inside this window.
+//
+// The wait is bounded: every tile takes its number from the ticket, so all tiles it waits for
+// have started and the wait is short; should the host's idea of the ticket counter ever be
+// wrong (tiles then carry numbers their predecessors never get), the wave gives up after
+// `limit` polls, reports through `err` and returns as if the walk had ended with nothing
+// found, so that every workgroup still finishes and the next wait on the stream raises the
+// error instead of the launch never ending.
 template <class S>
-ACC_DEV void acc_window(const typename S::Env& env, const u64* rowDesc, i64 look, u64 epoch, typename S::Elt& r,
-                        int& nv, bool& terminal) {
+ACC_DEV void acc_window(const typename S::Env& env, const u64* rowDesc, i64 look, u64 epoch, u64 limit, u32* err,
+                        typename S::Elt& r, int& nv, bool& terminal) {
   typedef typename S::Elt Elt;
   const int W = AccScanCfg<S>::W;
   const int lane = acc_lane();
@@ -134,6 +143,7 @@ ACC_DEV void acc_window(const typename S::Env& env, const u64* rowDesc, i64 look
   int st;  // 0 not yet, 1 aggregate, 2 inclusive prefix, 3 before the row
   Elt val;
   int first;
+  u64 polls = 0;
   for (;;) {
     st = idx < 0 ? 3 : acc_try_read<Elt>(rowDesc + idx * W, val, epoch);
     if (st == 1 && S::stops(val)) st = 2;  // nothing before this aggregate can matter
@@ -142,6 +152,12 @@ ACC_DEV void acc_window(const typename S::Env& env, const u64* rowDesc, i64 look
     first = mEnd ? __builtin_ctzll(mEnd) : ACC_WAVE;
     const u64 need = first >= 63 ? ~0ull : ((2ull << first) - 1);
     if ((mInv & need) == 0) break;
+    if (++polls >= limit) {
+      if (lane == 0) __hip_atomic_store(err, 3u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+      nv = 0;
+      terminal = true;
+      return;
+    }
     __builtin_amdgcn_s_sleep(ACC_SCAN_SLEEP);
   }
   nv = ACC_WAVE;
@@ -171,8 +187,8 @@ ACC_DEV void acc_window(const typename S::Env& env, const u64* rowDesc, i64 look
 // Exclusive prefix of tile `tile` (> 0) of a row whose descriptors start at `rowDesc`.
 // Called by all threads of the workgroup; the result is valid in thread 0.
 template <class S>
-ACC_DEV bool acc_lookback(const typename S::Env& env, const u64* rowDesc, i64 tile, u64 epoch, bool settle,
-                          typename S::Elt& excl) {
+ACC_DEV bool acc_lookback(const typename S::Env& env, const u64* rowDesc, i64 tile, u64 epoch, bool settle, u64 limit,
+                          u32* err, typename S::Elt& excl) {
   typedef typename S::Elt Elt;
   enum { LB = ACC_SCAN_LBWAVES < ACC_SCAN_WAVES ? ACC_SCAN_LBWAVES : ACC_SCAN_WAVES };
   __shared__ Elt sh_win[LB];
@@ -195,7 +211,7 @@ ACC_DEV bool acc_lookback(const typename S::Env& env, const u64* rowDesc, i64 ti
       Elt r;
       int nv;
       bool term;
-      acc_window<S>(env, rowDesc, look - (i64)w * ACC_WAVE, epoch, r, nv, term);
+      acc_window<S>(env, rowDesc, look - (i64)w * ACC_WAVE, epoch, limit, err, r, nv, term);
       if (acc_lane() == 0) {
         sh_win[w] = r;
         sh_nv[w] = nv;
@@ -282,8 +298,9 @@ ACC_DEV void acc_rake(const typename S::Env& env, typename S::Elt* mine, const t
 // (the total of scan') sets it for the tiles that cannot hold that position.  `settle` delays
 // the first look at the predecessors (see acc_lookback).
 template <class S, class Load, class Store, class StoreRun>
-ACC_DEV void acc_scan_tile(const typename S::Env& env, u64* desc, i64 tiles, i64 tile, i64 n, u64 epoch,
-                           const Load& load, const Store& store, const StoreRun& storeRun, bool plain, bool settle) {
+ACC_DEV void acc_scan_tile(const typename S::Env& env, u64* desc, i64 tiles, i64 tile, i64 n, u64 epoch, u64 limit,
+                           u32* err, const Load& load, const Store& store, const StoreRun& storeRun, bool plain,
+                           bool settle) {
   typedef typename S::Elt Elt;
   typedef AccScanCfg<S> C;
   const int V = C::V, G = C::G, W = C::W;
@@ -299,6 +316,7 @@ ACC_DEV void acc_scan_tile(const typename S::Env& env, u64* desc, i64 tiles, i64
   // takes the branch without bounds tests, which lets the V consecutive accesses of a lane
   // become one wide request.
   Elt x[C::G][C::V];
+  Elt filler;
   const bool full = tlo + (i64)C::TILE <= n;
   if (full) {
 #pragma unroll
@@ -311,7 +329,13 @@ ACC_DEV void acc_scan_tile(const typename S::Env& env, u64* desc, i64 tiles, i64
 #pragma unroll
       for (int k = 1; k < V; ++k) x[g][k] = S::combine(env, x[g][k - 1], e[k]);
     }
+    filler = x[0][0];
   } else {
+    // Slots past the end repeat a real element (the tile's first one), and so do the totals
+    // of waves without data: the wave scans and the raking below apply the combination
+    // function to every lane, and that function may only ever see values of the array (it
+    // may index a table by its operands, or loop on them).  Nothing of this is stored.
+    filler = tlo < n ? load(tlo) : S::seed(env);
 #pragma unroll
     for (int g = 0; g < G; ++g) {
       const i64 t0 = wlo + ((i64)g * ACC_WAVE + lane) * V;
@@ -321,14 +345,14 @@ ACC_DEV void acc_scan_tile(const typename S::Env& env, u64* desc, i64 tiles, i64
         if (t < n) {
           Elt e = load(t);
           x[g][k] = k == 0 ? e : S::combine(env, x[g][k - 1], e);
-        } else if (k > 0) {
-          x[g][k] = x[g][k - 1];
+        } else {
+          x[g][k] = k > 0 ? x[g][k - 1] : filler;
         }
       }
     }
   }
 
-  Elt waveTot;
+  Elt waveTot = filler;
   bool hasWaveTot = false;
 #ifdef ACC_SCAN_RAKE
   // prefixes of the lane totals by raking (acc_rake), applied to the elements at once, so
@@ -400,7 +424,7 @@ ACC_DEV void acc_scan_tile(const typename S::Env& env, u64* desc, i64 tiles, i64
       hasExcl = true;
     }
   } else {
-    hasExcl = acc_lookback<S>(env, desc, tile, epoch, settle, excl);  // valid in thread 0
+    hasExcl = acc_lookback<S>(env, desc, tile, epoch, settle, limit, err, excl);  // valid in thread 0
   }
   if (threadIdx.x == 0) {
     if (successors && wavesWithData > 0) {
@@ -488,6 +512,8 @@ ACC_DEV void acc_rows_tile(const typename S::Env& env, int cnt, int n, const Loa
   const int lane = acc_lane(), w = acc_wave();
   const int wlo = w * G * C::GROUP;
   P x[C::G][C::V];
+  P filler;
+  bool haveFiller = false;
   int r0[C::G], t0[C::G];
 #pragma unroll
   for (int g = 0; g < G; ++g) {
@@ -512,6 +538,12 @@ ACC_DEV void acc_rows_tile(const typename S::Env& env, int cnt, int n, const Loa
 #pragma unroll
       for (int k = 1; k < V; ++k) x[g][k] = SS::combine(env, x[g][k - 1], e[k]);
     } else {
+      // slots past the end repeat the first element of the stretch (see acc_scan_tile)
+      if (!haveFiller) {
+        filler.v = load(0, 0, 0);
+        filler.f = 1u;
+        haveFiller = true;
+      }
 #pragma unroll
       for (int k = 0; k < V; ++k) {
         if (idx0 + k < cnt) {
@@ -519,8 +551,8 @@ ACC_DEV void acc_rows_tile(const typename S::Env& env, int cnt, int n, const Loa
           e.v = load(idx0 + k, r, t);
           e.f = t == 0 ? 1u : 0u;
           x[g][k] = k == 0 ? e : SS::combine(env, x[g][k - 1], e);
-        } else if (k > 0) {
-          x[g][k] = x[g][k - 1];
+        } else {
+          x[g][k] = k > 0 ? x[g][k - 1] : filler;
         }
         if (++t == n) {
           t = 0;
@@ -529,7 +561,7 @@ ACC_DEV void acc_rows_tile(const typename S::Env& env, int cnt, int n, const Loa
       }
     }
   }
-  P waveTot;
+  P waveTot = haveFiller ? filler : x[0][0];
   bool hasWaveTot = false;
 #ifdef ACC_ROWS_RAKE
   {

@@ -7,6 +7,11 @@ acc_scan(Spec::Env env, Spec::Out out, Spec::Out tot, ScanParams p) {
   typedef S::Elt Elt;
   const int W = AccScanCfg<S>::W;
   const i64 gtile = acc_take_ticket(p.ticket, p.ticket_base);
+  // a ticket outside the launch means that the host's count of tickets is off: touch nothing
+  if (gtile < 0 || gtile >= p.rows * p.tpr) {
+    if (threadIdx.x == 0) __hip_atomic_store(p.err, 3u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+    return;
+  }
   const i64 row = gtile / p.tpr;
   const i64 tile = gtile - row * p.tpr;
   const i64 n = p.n;
@@ -39,7 +44,7 @@ acc_scan(Spec::Env env, Spec::Out out, Spec::Out tot, ScanParams p) {
       S::store_run(out, outBase + (m - 1 - shift) - (t0 + S::V - 1), z);
     }
   };
-  acc_scan_tile<S>(env, rowDesc, p.tpr, tile, n, p.epoch, load, store, storeRun, S::kKind != 2 || tile + 1 < p.tpr,
+  acc_scan_tile<S>(env, rowDesc, p.tpr, tile, n, p.epoch, p.spin_limit, p.err, load, store, storeRun, S::kKind != 2 || tile + 1 < p.tpr,
                    p.rows * p.tpr >= ACC_SCAN_SETTLE_TILES);
 
   if (S::kKind != 0 && tile == 0 && threadIdx.x == 0) {

@@ -1,6 +1,8 @@
 #include "exec.hpp"
 
 #include <algorithm>
+#include <cmath>
+#include <cstdint>
 #include <cstring>
 
 namespace acchip {
@@ -317,6 +319,13 @@ static HValP hostEval(const Sx& e, std::vector<HValP> env, const std::vector<DAr
     if (uns) {
       if (n == "quot" || n == "idiv") return hvInt(st, (int64_t)(ua / ub));
       return hvInt(st, (int64_t)(ua % ub));
+    }
+    // minBound `quot` (-1) overflows: the reference raises (GHC.Real overflowError), C would trap
+    if (b == -1) {
+      if (n == "rem" || n == "mod") return hvInt(st, 0);
+      const int64_t lowest = stSize(st) == 8 ? INT64_MIN : -((int64_t)1 << (8 * stSize(st) - 1));
+      if (a == lowest) throw Error("arithmetic overflow");
+      return hvInt(st, wrapTo(st, (int64_t)(0 - (uint64_t)a)));
     }
     int64_t q = a / b, r = a % b;
     if (n == "quot") return hvInt(st, wrapTo(st, q));
@@ -797,7 +806,14 @@ HValP Program::hostExp(const Sx& e, const AEnv& aenv, const Plan& plan) {
       case ST::U64: v->i = (int64_t) * (uint64_t*)raw; break;
       case ST::F32: v->f = *(float*)raw; break;
       case ST::F64: v->f = *(double*)raw; break;
-      case ST::F16: v->f = 0; break;
+      case ST::F16: {  // binary16 -> double
+        const unsigned h16 = *(uint16_t*)raw, ex = (h16 >> 10) & 31, fr = h16 & 1023;
+        double mag = ex == 0 ? std::ldexp((double)fr, -24)
+                   : ex == 31 ? (fr ? std::nan("") : HUGE_VAL)
+                              : std::ldexp((double)(fr | 1024), (int)ex - 25);
+        v->f = (h16 & 0x8000) ? -mag : mag;
+        break;
+      }
     }
     leaves.push_back(v);
   }
@@ -1248,6 +1264,27 @@ AValP Program::eval(const Sx& n, AEnv& aenv) {
       std::vector<int64_t> e2 = operandExtent(n.at(8), aenv, plan, temps, cur);
       for (size_t k = 0; k < ext.size(); ++k) ext[k] = std::min(ext[k], e2[k]);
     }
+    // Mirror and Wrap remap an outside index once (Interpreter.hs:824-839); on an extent shorter
+    // than the taps reach (Mirror: extent <= halo, Wrap: extent < halo) the remapped index is
+    // still outside, which the reference reports when it indexes the source (indexCheck in
+    // toIndex, Shape.hs:98-106).  The kernels do not test their reads, so this is decided here.
+    {
+      bool nonEmpty = true;
+      for (int64_t d : ext) nonEmpty = nonEmpty && d > 0;
+      size_t cur2 = 0;
+      for (int a = 0; nonEmpty && a < (two ? 2 : 1); ++a) {
+        const Sx& bnd = n.at(two ? (a == 0 ? 5 : 7) : 4);
+        const std::vector<int64_t> sext = operandExtent(n.at(two ? (a == 0 ? 6 : 8) : 5), aenv, plan, temps, cur2);
+        const bool mirror = bnd.isAtom("mirror"), wrap = bnd.isAtom("wrap");
+        if (!mirror && !wrap) continue;
+        const std::vector<int> halo = stencilHaloOf(n.at(two ? 1 + a : 1));
+        for (size_t d = 0; d < halo.size() && d < sext.size(); ++d)
+          if (halo[d] > 0 && sext[d] < halo[d] + (mirror ? 1 : 0))
+            throw Error("index out of bounds: a " + std::string(mirror ? "mirror" : "wrap") + " boundary on an extent of " +
+                        std::to_string(sext[d]) + " under a stencil that reaches " + std::to_string(halo[d]) +
+                        " beyond the focus");
+      }
+    }
     DArrayP out = alloc(plan.ty->r, ext);
     if (plan.mode == "lds2d") {
       if (out->size() == 0) return avArr(out);
@@ -1407,8 +1444,18 @@ AValP Program::eval(const Sx& n, AEnv& aenv) {
     args.push_back((uint64_t)tpr);
     args.push_back((uint64_t)(uintptr_t)st.desc);
     args.push_back((uint64_t)(uintptr_t)st.ticket);
-    args.push_back((uint64_t)st.ticketBase);
+    // fault injection for the test of the bounded look-back wait: a ticket base that lags the
+    // counter by `skew` gives every tile a number `skew` too high, so the first tiles wait for
+    // predecessors that never run, give up after `spin` polls and report
+    const char* sk = std::getenv("ACCHIP_SCAN_TEST_SKEW");
+    const char* sp = std::getenv("ACCHIP_SCAN_SPIN_LIMIT");
+    const uint64_t skew = sk ? (uint64_t)std::atoll(sk) : 0;
+    // a legitimate wait lasts microseconds; 2^22 polls are several seconds
+    const uint64_t spin = sp && std::atoll(sp) > 0 ? (uint64_t)std::atoll(sp) : (uint64_t)1 << 22;
+    args.push_back((uint64_t)(st.ticketBase - skew));
     args.push_back((uint64_t)st.epoch);
+    args.push_back(spin);
+    args.push_back((uint64_t)(uintptr_t)ctx_.errorWord());
     ctx_.launch(kern, "acc_scan", (uint64_t)tiles, (unsigned)m.block, args);
     st.ticketBase += (uint64_t)tiles;
     return result;

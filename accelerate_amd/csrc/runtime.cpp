@@ -48,6 +48,7 @@ Context::Context(int device) : device_(device) {
     hipCheck(hipSetDevice(device_), "hipSetDevice");
     hipCheck(hipStreamCreateWithFlags(&stream_, hipStreamNonBlocking), "hipStreamCreate");
     staticScratchSetup(device_);  // address of the static scan scratch on this device
+    (void)errorWord();            // pinned now: launches allocate nothing for it later
   }
 }
 
@@ -229,6 +230,8 @@ void Context::raiseDeviceError() {
   const unsigned code = __atomic_exchange_n(errHost_, 0u, __ATOMIC_ACQ_REL);
   if (code == 1) throw Error("empty segment");  // foldSegOp / fold1SegOp, Interpreter.hs:407, 424
   if (code == 2) throw Error("index out of bounds");  // permute target, Shape.hs:98-106
+  if (code == 3) throw Error("internal error: a scan tile gave up waiting for its predecessors (ticket count out of step)");
+  if (code == 4) throw Error("internal error: a permute update gave up waiting for its destination's lock");
   if (code != 0) throw Error("a kernel reported error " + std::to_string(code));
 }
 
@@ -267,7 +270,8 @@ static bool readFile(const std::string& path, std::string& out) {
 }
 
 static void writeFile(const std::string& path, const std::string& data) {
-  std::string tmp = path + ".tmp" + std::to_string((long long)getpid());
+  static std::atomic<unsigned long> serial{0};  // several writers in one process get a file each
+  std::string tmp = path + ".tmp" + std::to_string((long long)getpid()) + "." + std::to_string(serial++);
   {
     std::ofstream f(tmp, std::ios::binary);
     if (!f) return;
@@ -372,13 +376,25 @@ KernelP Context::kernel(const KernelSource& ks0) {
   std::string path = cacheDir + "/" + hash + ".hsaco";
   if (dumpCC) fprintf(stderr, "[acchip] kernel %s\n%s\n", hash.c_str(), ks.source.c_str());
   // a cached code object must at least look like one (an ELF image); anything else is compiled anew
-  if (!forceRecomp && readFile(path, k->code) && k->code.size() > 64 && k->code.compare(0, 4, "\177ELF") == 0) {
+  const bool fromDisk =
+      !forceRecomp && readFile(path, k->code) && k->code.size() > 64 && k->code.compare(0, 4, "\177ELF") == 0;
+  // Two threads may miss on the same key: the one that enters the table first owns the
+  // compilation, the other takes its kernel.  The worker is started under the lock, after the
+  // entry is in the table, so no kernel with a worker attached is ever dropped.
+  std::lock_guard<std::mutex> g(mu_);
+  auto ins = kernels_.emplace(hash, k);
+  if (!ins.second) {
+    stats.kernelsFromMemory++;
+    return ins.first->second;
+  }
+  if (fromDisk) {
     stats.kernelsFromDisk++;
   } else {
     // compile on a worker thread, at most as many at once as there are cores
     stats.kernelsCompiled++;
     const bool dump = dumpCC;
     const std::string dir = cacheDir;
+    k->code.clear();
     Kernel* raw = k.get();  // kept alive by kernels_ until the context goes, which waits
     k->ready = std::async(std::launch::async, [raw, src = ks.source, path, dir, dump]() {
                  CompileSlot slot;
@@ -389,9 +405,7 @@ KernelP Context::kernel(const KernelSource& ks0) {
                  writeFile(path, raw->code);
                }).share();
   }
-  std::lock_guard<std::mutex> g(mu_);
-  auto ins = kernels_.emplace(hash, k);
-  return ins.first->second;
+  return k;
 }
 
 void Context::wait(const KernelP& k) {

@@ -21,11 +21,14 @@ namespace acchip {
 
 struct Kernel {
   std::string hash;
-  std::shared_future<void> ready;   // compilation in flight (valid only when hipRTC had to run)
   std::string code;                 // code object (hsaco), complete once `ready` is
   hipModule_t module = nullptr;     // loaded lazily, on first launch
   std::map<std::string, hipFunction_t> fns;
   KernelSource meta;                // argument plan (source text dropped after compilation)
+  // compilation in flight (valid only when hipRTC had to run).  Declared last: it is destroyed
+  // first, and destroying the last reference to an async task waits for the worker, which
+  // writes into `code`.
+  std::shared_future<void> ready;
 };
 using KernelP = std::shared_ptr<Kernel>;
 

@@ -322,6 +322,19 @@ def parity_cases():
                 lens[-1] = max(0, int(lens[-1]) - 3)     # leave a few trailing elements in no segment
             v = _rand(rng, A.i32, shp)
             add("foldseg_%s_%s_%d" % (ity, shp, nseg), P.foldseg_sum(A.i32, ity, len(shp), 5), [v, lens], None)
+    # ---- fold1Seg (Prelude/Fold.hs:102-121): DIM1-3, a sum and the non-commutative interval monoid,
+    #      both descriptor types; no empty segment (that is an error, tested apart)
+    for ity in (A.i32, A.i64):
+        for shp, nseg in [((200,), 1), ((5000,), 64), ((3, 700), 9), ((2, 5, 300), 4), ((9000,), 2500), ((40000,), 3)]:
+            n = shp[-1]
+            cuts = np.sort(rng.choice(np.arange(1, n), nseg - 1, replace=False)) if nseg > 1 else np.array([], np.int64)
+            lens = np.diff(np.concatenate([[0], cuts, [n]])).astype(NPT[ity])
+            if nseg > 2 and lens[-1] > 3:
+                lens[-1] -= 3                             # leave a few trailing elements in no segment
+            add("fold1seg_sum_%s_%s_%d" % (ity, shp, nseg), Q.fold1seg_sum(A.i64, len(shp), ity),
+                [_rand(rng, A.i64, shp), lens], None)
+            add("fold1seg_interval_%s_%s_%d" % (ity, shp, nseg), Q.fold1seg_interval(len(shp), A.Int, ity),
+                [[_rand(rng, A.i64, shp), _rand(rng, A.i64, shp)], lens], None)
     # ---- permute (Prelude/Permute.hs:46-146): (+) with collisions and drops, every rank pair
     for sr, dr in [(1, 1), (2, 1), (1, 2), (3, 2), (2, 3)]:
         sshape = {1: (400,), 2: (13, 31), 3: (4, 5, 21)}[sr]
@@ -362,6 +375,19 @@ def parity_cases():
     add("jacobi_37x53", P.jacobi_step(), [g], None)
     add("stencil2_clamp_const", Q.stencil2_sum(A.f32, "clamp", A.constant(A.f32, 0.5)),
         [g, rng.uniform(0, 1, (40, 50)).astype(np.float32)], None)
+    # stencil2 (Prelude/Stencil.hs): every boundary kind on either source, sources of different
+    # extents (the result has their intersection), Int64 so that the comparison is exact
+    s2 = lambda k: {"constant": A.constant(A.i64, 4), "function": Q.boundary_function(A.i64, 2)}.get(k, k)
+    for b1, b2 in (("clamp", "wrap"), ("mirror", "clamp"), ("wrap", "mirror"), ("constant", "function"),
+                   ("function", "constant"), ("wrap", "wrap"), ("mirror", "mirror")):
+        for sh1, sh2 in (((5, 8), (7, 6)), ((70, 300), (64, 310)), ((2, 2), (2, 2))):
+            add("stencil2_%s_%s_%s" % (b1, b2, sh1), Q.stencil2_sum(A.i64, s2(b1), s2(b2)),
+                [_rand(rng, A.i64, sh1, -9, 9), _rand(rng, A.i64, sh2, -9, 9)], None)
+    # ---- Transform (AST.hs:289-296): an index function and a value function in one node
+    for shp in ((5, 7), (64, 300), (1, 1), (0, 4)):
+        add("transform_transpose_affine_%s" % (shp,), Q.transform_transpose_affine(), [_rand(rng, A.i64, shp)], None)
+    add("transform_gather_scale", Q.transform_gather_scale(),
+        [rng.integers(0, 100, 257).astype(np.int64), _rand(rng, A.f32, (100,))], None)
     # ---- whole programs (Test/NoFib/Spectral: SMVM, RadixSort; Prelude/Filter.hs)
     for nrows, ncols in ((40, 30), (700, 500)):
         segd = rng.integers(0, 7, nrows).astype(np.int64)

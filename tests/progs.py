@@ -1190,3 +1190,62 @@ def long_array_programs(big, n):
 
 def long_fold_expected(big):
     return 7 + (big // 256) * (255 * 128) + sum(range(big % 256))
+
+
+# -- fold1Seg (Test/NoFib/Prelude/Fold.hs:102-121): the surface function scans the lengths into
+#    offsets first (Prelude.hs:730-737), the node consumes offsets and has no seed
+def fold1seg_sum(ty=Int, rank=1, ity=Int):
+    return A.alam([A.tarray(rank, ty), A.tarray(1, ity)], lambda vals, seg: A.alet(
+        A.tarray(1, ity), A.scan("l", binop(A.add, ity), A.const(ity, 0), seg),
+        lambda offs: A.foldseg(ity, binop(A.add, ty), None, vals, offs)))
+
+
+def fold1seg_interval(rank=1, ty=Int, ity=Int):
+    """fold1Seg of the interval monoid over pairs: (a, _) <> (_, d) = (a, d); neither commutative
+    nor indifferent to where a segment starts and ends"""
+    t2 = A.ttup(ty, ty)
+
+    def f(x, y):
+        a, _ = A.untup(x)
+        _, d = A.untup(y)
+        return A.tup(a, d)
+
+    return A.alam([A.tarray(rank, t2), A.tarray(1, ity)], lambda vals, seg: A.alet(
+        A.tarray(1, ity), A.scan("l", binop(A.add, ity), A.const(ity, 0), seg),
+        lambda offs: A.foldseg(ity, A.lam([t2, t2], f), None, vals, offs)))
+
+
+# -- Transform (AST.hs:289-296): out[ix] = f (a ! p ix); here the transpose of 3 * x + 1
+def transform_transpose_affine(ty=Int):
+    sh2 = A.tshape(2)
+
+    def swap(v):
+        y, x = A.untup(v)
+        return A.sh(x, y)
+
+    return A.alam([A.tarray(2, ty)], lambda m: A.transform(
+        A.tarray(2, ty), A.let(sh2, A.shape(m), swap), A.lam([sh2], swap),
+        A.lam([ty], lambda x: A.add(ty, A.mul(ty, A.const(ty, 3), x), A.const(ty, 1))), m))
+
+
+def transform_gather_scale(ty=A.f32):
+    """Transform with a data-dependent index function: out[i] = 0.5 * xs[from[i]]"""
+    sh1 = A.tshape(1)
+    return A.alam([A.tarray(1, Int), A.tarray(1, ty)], lambda frm, xs: A.transform(
+        A.tarray(1, ty), A.shape(frm), A.lam([sh1], lambda ix: A.sh(A.index(frm, A.vexp(ix)))),
+        A.lam([ty], lambda x: A.mul(ty, A.const(ty, 0.5), x)), xs))
+
+
+# -- a scan whose combination function looks its result up in a table indexed by both operands
+#    (composition of finite-state transitions): the function must only ever be applied to values
+#    of the array, or the lookup leaves the table
+def table_scan(k, direction="l", kind="scan1"):
+    sh1 = A.tshape(1)
+
+    def body(tbl, xs):
+        f = A.lam([Int, Int], lambda a, b: A.index(tbl, A.sh(A.add(Int, A.mul(Int, a, A.constI(k)), b))))
+        if kind == "scan1":
+            return A.scan(direction, f, None, xs)
+        return A.scan(direction, f, A.constI(0), xs)
+
+    return A.alam([A.tarray(1, Int), A.tarray(1, Int)], body)

@@ -232,6 +232,45 @@ def test_scans_and_folds_at_tile_borders(gpu_ctx, monkeypatch, ty, tiles):
         assert progs["fold"](x) == dt(3) + inc[-1], n
 
 
+@pytest.mark.parametrize("tiles", ["large", "small", "rows"])
+def test_scan_whose_function_indexes_a_table_at_tile_borders(gpu_ctx, monkeypatch, tiles):
+    # composition of finite-state transitions: the combination function reads tbl[a * k + b].  The
+    # kernels apply it to every lane of a tile, also to lanes past the end of a row, so those lanes
+    # must hold values of the array: anything else indexes outside the table.  Lengths around
+    # the multiples of every tile size, against a sequential fold of the same table.
+    monkeypatch.setenv("ACCHIP_SCAN_TILES", tiles)
+    k = 7
+    rng = np.random.default_rng(123)
+    tbl = rng.integers(0, k, k * k).astype(np.int64)
+    # make the table's operation associative: composition of functions on k states, elements
+    # are function numbers in a closed set; the simplest closed set is a cyclic group
+    tbl = np.array([(a + b) % k for a in range(k) for b in range(k)], np.int64)
+    runs = {(d, kind): gpu_ctx.compile(Q.table_scan(k, d, kind)) for d in "lr" for kind in ("scan1", "scan")}
+    edges = TILE_EDGES if tiles != "rows" else [1, 2, 63, 64, 65, 1000, 2047, 2048, 4095, 4096]
+    for n in edges:
+        x = rng.integers(0, k, n).astype(np.int64)
+        inc = np.cumsum(x) % k
+        rinc = (np.cumsum(x[::-1]) % k)[::-1]
+        assert np.array_equal(runs[("l", "scan1")](tbl, x), inc), n
+        assert np.array_equal(runs[("r", "scan1")](tbl, x), rinc), n
+        assert np.array_equal(runs[("l", "scan")](tbl, x), np.concatenate([[0], inc])), n
+        assert np.array_equal(runs[("r", "scan")](tbl, x), np.concatenate([rinc, [0]])), n
+
+
+def test_many_short_rows_of_a_table_scan(gpu_ctx):
+    # the rows kernel: several whole rows per workgroup, the last workgroup ragged
+    k = 5
+    tbl = np.array([(a + b) % k for a in range(k) for b in range(k)], np.int64)
+    rng = np.random.default_rng(5)
+    V1, V2 = A.tarray(1, A.Int), A.tarray(2, A.Int)
+    prog = A.alam([V1, V2], lambda t, xs: A.scan("l", A.lam([A.Int, A.Int], lambda a, b: A.index(
+        t, A.sh(A.add(A.Int, A.mul(A.Int, a, A.constI(k)), b)))), None, xs))
+    run = gpu_ctx.compile(prog)
+    for shape in ((1001, 7), (333, 100), (50, 1500), (3, 4097)):
+        x = rng.integers(0, k, shape).astype(np.int64)
+        assert np.array_equal(run(tbl, x), np.cumsum(x, axis=1) % k), shape
+
+
 @pytest.mark.parametrize("nbins", [1 << 20, (1 << 21) + 12345, 1 << 22])
 def test_histogram_over_many_lds_fuls(gpu_ctx, monkeypatch, nbins):
     # destinations of up to 128 LDS-fuls are still combined in workgroup-private copies, one
@@ -253,6 +292,17 @@ def test_jacobi_8192_bit_equal(gpu_ctx):
     got = d.to_host()
     assert np.array_equal(got, OC.jacobi_f32(g, 3))             # no reduction, no contraction: bit-equal
     assert got.min() >= g.min() and got.max() <= g.max()        # averaging never leaves the input's range
+
+
+def test_jacobi_8192_100_iterations_bit_equal(gpu_ctx):
+    # the stencil configuration at its full size: 100 sweeps over 8192 x 8192, every cell compared
+    g = W.uniform_f32(8192 * 8192, 8, 0.0, 1.0).reshape(8192, 8192)
+    step = gpu_ctx.compile(P.jacobi_step())
+    d = gpu_ctx.to_device(g, A.tarray(2, A.f32))
+    for _ in range(100):
+        d = step.execute(d)
+    got = d.to_host()
+    assert np.array_equal(got, OC.jacobi_f32(g, 100))
 
 
 def test_jacobi_100_iterations_small_grid_bit_equal(gpu_ctx):
@@ -360,6 +410,47 @@ def test_more_than_2_pow_31_elements(gpu_ctx):
     run = gpu_ctx.compile(P.scanl1_sum(A.u8)).execute(dx).to_host()
     assert run[-1] == total and np.array_equal(run[:4096], np.cumsum(x[:4096], dtype=np.uint8))
     assert np.array_equal(np.diff(run[-5000:]).astype(np.uint8), x[-4999:])
+
+
+@pytest.mark.parametrize("kind,widths,shape", [("mirror", [3, 3], (1, 5)), ("mirror", [3, 3], (5, 1)), ("wrap", [9], (3,)),
+                                               ("mirror", [9], (4,)), ("mirror", [3, 3, 3], (2, 1, 9)),
+                                               ("wrap", [5, 5], (1, 11))])
+def test_stencil_extent_too_short_for_its_boundary_is_a_bounds_error(gpu_ctx, kind, widths, shape):
+    # Mirror on an extent <= halo and Wrap on an extent < halo leave the remapped index outside the
+    # array; the reference reports it when it indexes the source (Shape.hs:98-106), so does the
+    # oracle, and here the host refuses the launch
+    prog = Q.stencil_weighted(A.i64, widths, kind)
+    x = np.ones(shape, np.int64)
+    with pytest.raises(O.OracleError, match="index out of bounds"):
+        O.run_n(prog.text(), x)
+    launches = gpu_ctx.stat("launches")
+    with pytest.raises(hip.AccError, match="index out of bounds") as e:
+        gpu_ctx.compile(prog)(x)
+    assert e.value.code == 4 and gpu_ctx.stat("launches") == launches
+    # one element more (Mirror) is enough
+    ok = tuple(max(s, w // 2 + (1 if kind == "mirror" else 0)) for s, w in zip(shape, widths))
+    y = np.arange(int(np.prod(ok)), dtype=np.int64).reshape(ok)
+    assert same(gpu_ctx.compile(prog)(y), O.run_n(prog.text(), y))
+
+
+def test_lookback_wait_is_bounded_and_reported(gpu_ctx, monkeypatch):
+    # Fault injection from the host: the launch is told a ticket count that lags the device's by
+    # 3, so its tiles take numbers 3 too high -- the first ones wait for predecessors that never
+    # run, the last ones fall outside the launch.  With a poll limit of 50 every workgroup still
+    # finishes within microseconds; the condition is raised by the next wait on the stream and
+    # the context stays usable.
+    x = W.uniform_int(400_000, 3)
+    run = gpu_ctx.compile(P.scanl1_sum(A.i64))
+    assert np.array_equal(run(x), np.cumsum(x))
+    monkeypatch.setenv("ACCHIP_SCAN_TEST_SKEW", "3")
+    monkeypatch.setenv("ACCHIP_SCAN_SPIN_LIMIT", "50")
+    res = run.execute(gpu_ctx.to_device(x, A.tarray(1, A.i64)))
+    with pytest.raises(hip.AccError, match="gave up waiting"):
+        gpu_ctx.sync()
+    res.release()
+    monkeypatch.delenv("ACCHIP_SCAN_TEST_SKEW")
+    monkeypatch.delenv("ACCHIP_SCAN_SPIN_LIMIT")
+    assert np.array_equal(run(x), np.cumsum(x))
 
 
 def test_fold1_of_empty_is_a_bounds_error(gpu_ctx):
