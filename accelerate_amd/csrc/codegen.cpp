@@ -1478,6 +1478,19 @@ KernelSource Codegen::permute(const Sx& f, const ArrayR& dst, const Sx& p, const
     lds += "  ACC_DEV void lds_update(Priv& p, int i, const Elt& x) {\n" + upd + "  }\n";
     lds += "  ACC_DEV void lds_flush(const Priv& p, int i, const Out& out, i64 j) {\n" + flush + "  }\n";
   }
+  // A sum of one and the same constant per source (a histogram: `permute (+) zeros p ones`, the ones
+  // fused into a constant producer): the skeleton only counts, in 16-bit LDS counters, and adds
+  // count * constant (acc_permute_count).
+  bool countable = false;
+  if (mode == "atomic" && op == "add" && stIsInt(st) && src.delayed && src.linearD.is("lam") &&
+      src.linearD.at(2).is("const") && isST(src.linearD.at(2).at(1)) && parseST(src.linearD.at(2).at(1)) == st) {
+    countable = true;
+    const std::string T = stName(st), U = stName(stUnsigned(st));
+    lds += "#define ACC_PERMUTE_COUNT 1\n";
+    lds += "  ACC_DEV void count_flush(const Out& out, i64 j, u32 n) {\n    (void)__hip_atomic_fetch_add(&out.o0[j], (" + T +
+           ")((" + U + ")n * (" + U + ")(" + literalText(st, src.linearD.at(2).at(2).s) +
+           ")), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);\n  }\n";
+  }
   u += "  }\n" + lds;
   // update() uses store()/combine(): it must come after them, and finish() appends load/store
   // last, so emit our own forward-safe copies by placing update in a trailing block
@@ -1488,6 +1501,7 @@ KernelSource Codegen::permute(const Sx& f, const ArrayR& dst, const Sx& p, const
   endSpec -= std::strlen("//@UPDATE@\n");
   ks.source.insert(endSpec, u);
   ks.permuteMode = mode;
+  ks.permuteCount = countable;
   return ks;
 }
 

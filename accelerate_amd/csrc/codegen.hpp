@@ -56,6 +56,7 @@ struct KernelSource {
   bool commutative = false;
   bool streaming = false;             // has acc_*_stream entry points (non-temporal variant)
   std::string permuteMode;            // permute only: "atomic", "cas", "lock", "store"
+  bool permuteCount = false;          // permute only: has acc_permute_count (sum of a constant per source)
 };
 
 class Codegen {

@@ -1229,6 +1229,42 @@ AValP Program::eval(const Sx& n, AEnv& aenv) {
     // keys into 256 bins take 33 us through global atomics, 2^14 keys into 16 bins 47 us,
     // against 9 us this way).
     const bool many = cnt >= (1 << 20) || (cnt >= (1 << 12) && cnt >= 4 * out->size());
+    const char* ce = std::getenv("ACCHIP_PERMUTE_COUNT");  // "0": never take the counting kernel (tests, tuning)
+    if (plan.k->meta.permuteCount && many && out->size() <= maxParts * 65536 && !(ce && ce[0] == '0')) {
+      // a sum of one constant per source: 16-bit counters, 65536 destination elements per LDS-ful
+      const int64_t nparts = (out->size() + 65535) / 65536;
+      const int64_t part = nparts == 1 ? out->size() : 65536;
+      const char* ge = std::getenv("ACCHIP_PERMUTE_GROUPS");
+      int64_t groups = ge ? std::atoll(ge) : std::min<int64_t>(256 / nparts, cnt / 16384);
+      groups = std::max<int64_t>(8, groups / 8 * 8);
+      int64_t chunk = ((cnt + groups - 1) / groups + 3) / 4 * 4;
+      args.push_back((uint64_t)cnt);
+      args.push_back((uint64_t)chunk);
+      args.push_back((uint64_t)nparts);
+      args.push_back((uint64_t)part);
+      args.push_back((uint64_t)out->size());
+      args.push_back((uint64_t)(uintptr_t)ctx_.errorWord());
+      // The workgroups leave their counters in memory and a second launch sums them, unless there
+      // are so few workgroups that adding them to the destination directly is as cheap.
+      const char* pe2 = std::getenv("ACCHIP_PERMUTE_PARTIALS");  // "0" / "1": override, for tests
+      bool viaPartials = groups >= 32;
+      if (pe2) viaPartials = pe2[0] != '0';
+      DArrayP partials;
+      int64_t slices = 1;
+      if (viaPartials) {
+        ArrayR pr;
+        pr.rank = 1;
+        pr.elt = tScalar(ST::U32);
+        partials = alloc(pr, {nparts * groups * 32768});
+        slices = std::max<int64_t>(1, std::min<int64_t>(16, groups / 16));
+      }
+      args.push_back(partials ? (uint64_t)(uintptr_t)partials->bufs[0]->p : 0);
+      args.push_back((uint64_t)groups);
+      args.push_back((uint64_t)slices);
+      ctx_.launch(plan.k, "acc_permute_count", (uint64_t)(groups * nparts), 1024, args);
+      if (partials) ctx_.launch(plan.k, "acc_permute_count_reduce", (uint64_t)(nparts * (32768 / 128)), 256, args);
+      return avArr(out);
+    }
     if ((plan.mode == "atomic" || plan.mode == "atomics") && many && out->size() <= maxParts * partMax) {
       const int64_t nparts = (out->size() + partMax - 1) / partMax;
       const int64_t part = (out->size() + nparts - 1) / nparts;
@@ -1245,6 +1281,9 @@ AValP Program::eval(const Sx& n, AEnv& aenv) {
       args.push_back((uint64_t)part);
       args.push_back((uint64_t)out->size());
       args.push_back((uint64_t)(uintptr_t)ctx_.errorWord());
+      args.push_back(0);  // (fields of the counting variant)
+      args.push_back((uint64_t)groups);
+      args.push_back(1);
       ctx_.launch(plan.k, "acc_permute_lds", (uint64_t)(groups * nparts), 1024, args);
       return avArr(out);
     }

@@ -76,3 +76,62 @@ def test_privatised_permute_of_pairs(gpu_ctx, dst):
     np.add.at(rx, to, x)
     np.add.at(ry, to, y)
     assert np.array_equal(got[0], rx.astype(np.float32)) and np.array_equal(got[1], ry.astype(np.float32))
+
+
+def _histogram_with_drops(nbins, ty=A.i32, value=1):
+    """permute (+) zeros (\\ix -> if k < 0 then Nothing else Just k) (fill value): a constant per source"""
+    sh1 = A.tshape(1)
+    return A.alam([A.tarray(1, A.Int)], lambda keys: A.permute(
+        Q.binop(A.add, ty),
+        A.generate(A.tarray(1, ty), A.sh(nbins), A.lam([sh1], lambda ix: A.const(ty, 0))),
+        A.lam([sh1], lambda ix: A.let(A.Int, A.index(keys, A.vexp(ix)), lambda t: A.cond(
+            A.lt(A.Int, t, A.constI(0)), A.nothing(sh1), A.just(A.sh(t))))),
+        A.delayed(A.tarray(1, ty), A.shape(keys), A.lam([sh1], lambda ix: A.const(ty, value)),
+                  A.lam([A.Int], lambda i: A.const(ty, value)))))
+
+
+COUNT_KEYS = ["one_key", "two_keys_one_word", "last_bin", "sorted", "zipf", "uniform", "drops"]
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("keys_kind", COUNT_KEYS)
+@pytest.mark.parametrize("nbins,ty,value", [(1 << 16, A.i32, 1), (40000, A.i64, -3), (65537, A.i32, 7), (300000, A.u32, 1),
+                                            (1 << 16, A.i32, 0x7fffffff)])
+def test_counting_permute_matches_bincount(gpu_ctx, keys_kind, nbins, ty, value):
+    # a sum of one constant per source is counted in 16-bit LDS counters that are relieved of 32768
+    # whenever they reach it: inputs that drive single counters through many such crossings (one key;
+    # two keys whose counters share a word), the range's last element, and ordinary distributions,
+    # over one and several ranges of the destination; sums wrap like the reference's fixed-width types
+    n = (1 << 22) + 4321
+    rng = np.random.default_rng(nbins)
+    if keys_kind == "one_key":
+        keys = np.full(n, min(12345, nbins - 1), np.int64)
+    elif keys_kind == "two_keys_one_word":
+        keys = np.where(rng.random(n) < 0.5, 77, 77 + 32768).astype(np.int64) % nbins
+    elif keys_kind == "last_bin":
+        keys = np.where(rng.random(n) < 0.7, nbins - 1, 65535 % nbins).astype(np.int64)
+    elif keys_kind == "sorted":
+        keys = np.sort(rng.integers(0, nbins, n)).astype(np.int64)
+    elif keys_kind == "zipf":
+        keys = np.minimum(rng.zipf(1.1, n) - 1, nbins - 1).astype(np.int64)
+    elif keys_kind == "uniform":
+        keys = rng.integers(0, nbins, n).astype(np.int64)
+    else:
+        keys = rng.integers(0, nbins, n).astype(np.int64)
+        keys[rng.random(n) < 0.3] = -1
+    got = gpu_ctx.compile(_histogram_with_drops(nbins, ty, value))(keys)
+    dt = {"i32": np.int32, "i64": np.int64, "u32": np.uint32}[ty]
+    counts = np.bincount(keys[keys >= 0], minlength=nbins).astype(np.int64)
+    want = (counts * value).astype(np.int64).astype(dt)      # wraps to the element type
+    assert got.dtype == dt and np.array_equal(got, want)
+
+
+@pytest.mark.gpu
+def test_counting_permute_agrees_with_the_atomic_paths(gpu_ctx, monkeypatch):
+    rng = np.random.default_rng(3)
+    keys = np.minimum(rng.zipf(1.1, 1 << 22) - 1, 65535).astype(np.int64)
+    prog = _histogram_with_drops(1 << 16)
+    a = gpu_ctx.compile(prog)(keys)
+    monkeypatch.setenv("ACCHIP_PERMUTE_COUNT", "0")
+    b = gpu_ctx.compile(prog)(keys)
+    assert np.array_equal(a, b) and np.array_equal(a, np.bincount(keys, minlength=1 << 16))
