@@ -18,6 +18,10 @@
 // in LDS: sh_first[p] = first boundary at position p of the tile.  Empty segments (two equal
 // consecutive offsets) get z from the partition kernel.
 
+#ifndef ACC_FOLDSEG_STAGE
+#define ACC_FOLDSEG_STAGE 1024  // segment results a tile collects in LDS before it writes them (a multiple of 32)
+#endif
+
 struct FoldSegParams {
   i64 rows;
   i64 n;       // elements per row
@@ -96,7 +100,8 @@ acc_foldseg_partition(Spec::Env env, Spec::Out out, FoldSegParams p) {
 // no division is needed.  FULL: the tile lies completely inside the stream.
 template <bool ONE_ROW, bool FULL>
 ACC_DEV void acc_foldseg_tile(const Spec::Env& env, const Spec::Out& out, const FoldSegParams& p, unsigned short* sh_first,
-                              AccSegSpec<Spec>::Elt* sh_wave, AccSegSpec<Spec>::Elt* sh_rake, Spec::Elt& sh_pend, int& sh_pend_at) {
+                              AccSegSpec<Spec>::Elt* sh_wave, AccSegSpec<Spec>::Elt* sh_rake, Spec::Elt& sh_pend, int& sh_pend_at,
+                              Spec::Elt* sh_stage, u32* sh_staged) {
   typedef Spec S;
   typedef AccSegSpec<Spec> SS;
   typedef AccScanCfg<SS> C;
@@ -167,6 +172,7 @@ ACC_DEV void acc_foldseg_tile(const Spec::Env& env, const Spec::Out& out, const 
   if (!crowded) loadBatch(j0);
   for (int i = threadIdx.x; i < C::TILE / 8 + 1; i += ACC_SCAN_BLOCK)
     reinterpret_cast<int4*>(sh_first)[i] = make_int4(-1, -1, -1, -1);
+  for (int i = threadIdx.x; i < ACC_FOLDSEG_STAGE / 32; i += ACC_SCAN_BLOCK) sh_staged[i] = 0u;
   __syncthreads();
   if (crowded) {
     // far more boundaries than positions (long runs of empty segments): every position
@@ -205,12 +211,24 @@ ACC_DEV void acc_foldseg_tile(const Spec::Env& env, const Spec::Out& out, const 
     }
     return (int)(a - j0);
   };
-  // the segment that ends where boundary j0 + idx sits
-  auto emit = [&](int idx, const S::Elt& v) {
+  // the segment that ends where boundary j0 + idx sits: written to the result
+  auto write = [&](int idx, const S::Elt& v) {
     const i64 j = j0 + idx;
     const i64 row = ONE_ROW ? 0 : acc_quot(j, sp1), s = j - row * sp1;
     if (s == 0) return;  // what precedes a row's first boundary belongs to no segment
     S::store(out, row * p.nseg + s - 1, S::kSeeded ? S::combine(env, S::seed(env), v) : v);
+  };
+  // A finished segment waits in LDS under its boundary's number: neighbouring boundaries are
+  // neighbouring segments, so the workgroup writes them to the result side by side at the end,
+  // instead of one scattered store (and one index division) where each segment happens to
+  // end.  Boundaries beyond the staging area (a tile crowded with short segments) are written at once.
+  auto emit = [&](int idx, const S::Elt& v) {
+    if (idx < ACC_FOLDSEG_STAGE) {
+      sh_stage[idx] = v;
+      (void)__hip_atomic_fetch_or(&sh_staged[idx >> 5], 1u << (idx & 31), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+    } else {
+      write(idx, v);
+    }
   };
 
   P waveTot;
@@ -317,6 +335,226 @@ ACC_DEV void acc_foldseg_tile(const Spec::Env& env, const Spec::Out& out, const 
     p.pend_at[tile] = sh_pend_at == NOPEND ? (i64)-1 : j0 + sh_pend_at;
     if (sh_pend_at != NOPEND) reinterpret_cast<P*>(p.pend)[tile].v = sh_pend;
   }
+  // the staged segments, in the order of their boundaries
+  {
+    const i64 inTile = jend - j0 + 1;  // boundary numbers the tile can have met, relative to j0
+    const int top = inTile < ACC_FOLDSEG_STAGE ? (int)inTile : ACC_FOLDSEG_STAGE;
+    for (int idx = threadIdx.x; idx < top; idx += ACC_SCAN_BLOCK)
+      if ((sh_staged[idx >> 5] >> (idx & 31)) & 1u) write(idx, sh_stage[idx]);
+  }
+}
+
+// The same tile for the ordinary case (at most 4 boundaries per position on average, so that
+// every boundary of the tile has a 16-bit number), arranged so that the pass over the elements
+// has no branches: next to the marks a bitmap says which positions hold a boundary, a run reads
+// its 9 bits at once and computes, with selects only, the running value after each of its
+// elements.  Segment ends are dealt with once, after the prefix of every run inside the tile is
+// known (raking inside the wave, wave totals through LDS): a lane that has none skips them
+// together, an end reads its boundary's number from the marks then, and its value is the
+// running value, preceded by the prefix unless the run itself holds the segment's head.
+// the tile's elements: lane l of wave w holds, per group g, the V consecutive elements from
+// position tile * TILE + ((w * G + g) * 64 + l) * V on
+template <bool FULL>
+ACC_DEV void acc_foldseg_load(const Spec::Env& env, i64 tile, i64 n,
+                              Spec::Elt (&x)[AccScanCfg<AccSegSpec<Spec>>::G][AccScanCfg<AccSegSpec<Spec>>::V]) {
+  typedef AccScanCfg<AccSegSpec<Spec>> C;
+  const i64 wlo = tile * (i64)C::TILE + (i64)acc_wave() * C::G * C::GROUP;
+#pragma unroll
+  for (int g = 0; g < C::G; ++g) {
+    const i64 t0 = wlo + ((i64)g * ACC_WAVE + acc_lane()) * C::V;
+    if (FULL) {
+#pragma unroll
+      for (int k = 0; k < C::V; ++k) x[g][k] = Spec::in_linear(env, t0 + k);
+    } else {
+#pragma unroll
+      for (int k = 0; k < C::V; ++k)
+        if (t0 + k < n) x[g][k] = Spec::in_linear(env, t0 + k);
+    }
+  }
+}
+
+template <bool ONE_ROW, bool FULL>
+ACC_DEV void acc_foldseg_tile_fast(const Spec::Env& env, const Spec::Out& out, const FoldSegParams& p, i64 j0, i64 j1,
+                                   unsigned short* sh_first, u32* sh_head, AccSegSpec<Spec>::Elt* sh_wave,
+                                   AccSegSpec<Spec>::Elt* sh_rake, Spec::Elt& sh_pend, int& sh_pend_at, Spec::Elt* sh_stage,
+                                   u32* sh_staged) {
+  typedef Spec S;
+  typedef AccSegSpec<Spec> SS;
+  typedef AccScanCfg<SS> C;
+  typedef SS::Elt P;
+  const int V = C::V, G = C::G;
+  static_assert(C::V <= 24, "a run's boundary bits are taken from two words of the bitmap");
+  const int NOPEND = 0x7fffffff;
+  const i64 tile = blockIdx.x;
+  const i64 tlo = tile * (i64)C::TILE;
+  const i64 sp1 = p.nseg + 1;
+  const i64 nb = p.rows * sp1;
+  const int lane = acc_lane(), w = acc_wave();
+  const i64 n = p.total;
+  const i64 wlo = tlo + (i64)w * G * C::GROUP;
+  // marks and bitmap: four boundaries per thread and step, their offsets loaded together; a
+  // boundary at the position of its predecessor is not the first there and is skipped, so every
+  // mark has one writer.  The next tile's first boundary is looked at too: it may sit on this
+  // tile's upper border, where it ends a segment of this tile.
+  const i64 jend = tile + 1 < p.tiles && j1 < nb ? j1 + 1 : j1;
+  i64 row[4], sg[4], o[4], before[4];
+  auto loadBatch = [&](i64 jb) {
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      const i64 j = jb + (i64)u * ACC_SCAN_BLOCK + threadIdx.x;
+      if (j < jend) {
+        row[u] = ONE_ROW ? 0 : acc_quot(j, sp1);
+        sg[u] = j - row[u] * sp1;
+        o[u] = S::seg_at(env, sg[u]);
+        before[u] = sg[u] > 0 ? S::seg_at(env, sg[u] - 1) : (row[u] > 0 ? S::seg_at(env, p.nseg) - p.n : -1);
+      }
+    }
+  };
+  auto markBatch = [&](i64 jb) {
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      const i64 j = jb + (i64)u * ACC_SCAN_BLOCK + threadIdx.x;
+      if (j < jend && o[u] != before[u]) {
+        const i64 rel = row[u] * p.n + o[u] - tlo;
+        if (rel >= 0 && rel <= C::TILE) {
+          sh_first[rel] = (unsigned short)(j - j0);
+          (void)__hip_atomic_fetch_or(&sh_head[rel >> 5], 1u << (rel & 31), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+        }
+      }
+    }
+  };
+  // The offsets of the first boundaries are asked for before the elements: a wave's loads
+  // come back in the order they were issued, and the marks, which everything else waits for,
+  // would otherwise queue behind the tile's 32 KiB of elements.
+  loadBatch(j0);
+  S::Elt x[C::G][C::V];
+  acc_foldseg_load<FULL>(env, tile, n, x);
+  for (int i = threadIdx.x; i < C::TILE / 32 + 2; i += ACC_SCAN_BLOCK) sh_head[i] = 0u;
+  for (int i = threadIdx.x; i < ACC_FOLDSEG_STAGE / 32; i += ACC_SCAN_BLOCK) sh_staged[i] = 0u;
+  if (threadIdx.x == 0) sh_pend_at = NOPEND;
+  __syncthreads();
+  markBatch(j0);
+  for (i64 jb = j0 + (i64)ACC_SCAN_BLOCK * 4; jb < jend; jb += (i64)ACC_SCAN_BLOCK * 4) {
+    loadBatch(jb);
+    markBatch(jb);
+  }
+  __syncthreads();
+
+  // the pass over the elements: s[g][k] = value of the segment piece that ends with element k of
+  // the run (starting afresh at every head), bits[g] = boundaries at the run's V + 1 positions
+  u32 bits[C::G];
+  P agg[C::G];
+#pragma unroll
+  for (int g = 0; g < G; ++g) {
+    const i64 t0 = wlo + ((i64)g * ACC_WAVE + lane) * V;
+    const int rel0 = (int)(t0 - tlo);
+    const u32 w0 = sh_head[rel0 >> 5], w1 = sh_head[(rel0 >> 5) + 1];
+    const u32 b = (u32)((((u64)w1 << 32) | (u64)w0) >> (rel0 & 31)) & ((2u << V) - 1u);
+    bits[g] = b;
+    i64 c = n - t0;
+    c = c < 0 ? 0 : (c > V ? V : c);
+    S::Elt* e = x[g];
+    if (!FULL && c == 0) {  // a run past the end stands for a real element (none exists in an empty stream)
+      S::Elt none{};
+      e[0] = n > 0 ? S::in_linear(env, tlo) : none;
+    }
+    // Most of a stream of long segments has no boundary for hundreds of elements: when none of
+    // the wave's runs of this group has one, a run is a plain fold (wave-uniform test, so the
+    // branch costs no divergence) and its running values are never looked at.
+    if (FULL && __ballot(b != 0u) == 0ull) {
+      S::Elt v = e[0];
+#pragma unroll
+      for (int k = 1; k < V; ++k) v = S::combine(env, v, e[k]);
+      agg[g].v = v;
+      agg[g].f = 0u;
+    } else {
+#pragma unroll
+      for (int k = 1; k < V; ++k) {
+        if (FULL || k < c) {
+          const S::Elt joined = S::combine(env, e[k - 1], e[k]);
+          if (!((b >> k) & 1u)) e[k] = joined;
+        } else {
+          e[k] = e[k - 1];
+        }
+      }
+      agg[g].v = e[V - 1];
+      agg[g].f = (b & ((1u << V) - 1u)) != 0u ? 1u : 0u;
+    }
+  }
+  // prefixes of the runs inside the wave by raking, wave totals through LDS
+  P pre[C::G], waveTot;
+  {
+    i64 wcnt = n - wlo;
+    wcnt = wcnt < 0 ? 0 : (wcnt > (i64)G * C::GROUP ? (i64)G * C::GROUP : wcnt);
+    const int entries = (int)((wcnt + V - 1) / V);
+    waveTot = agg[0];
+    acc_rake<SS, C::G>(env, sh_rake + w * (ACC_WAVE * (C::G + 1) + 1), agg, lane, entries, pre, waveTot);
+  }
+  if (lane == 0) sh_wave[w] = waveTot;
+  __syncthreads();
+  const i64 tcnt = n - tlo;
+  const i64 perWave = (i64)G * C::GROUP;
+  i64 wd = tcnt <= 0 ? 0 : (tcnt + perWave - 1) / perWave;
+  const int wavesWithData = wd > ACC_SCAN_WAVES ? ACC_SCAN_WAVES : (int)wd;
+  if (w == 0) {
+    P t = sh_wave[lane < ACC_SCAN_WAVES ? lane : 0];
+    t = acc_wave_scan<SS>(env, t, lane);
+    if (lane < ACC_SCAN_WAVES) sh_wave[lane] = t;
+    if (lane == wavesWithData - 1) reinterpret_cast<P*>(p.carry)[tile] = t;
+  }
+  __syncthreads();
+  const bool hasWavePre = w > 0 && w <= wavesWithData;
+  const P wavePre = sh_wave[w > 0 ? w - 1 : 0];
+
+  auto write = [&](int idx, const S::Elt& v) {
+    const i64 j = j0 + idx;
+    const i64 row = ONE_ROW ? 0 : acc_quot(j, sp1), s = j - row * sp1;
+    if (s == 0) return;  // what precedes a row's first boundary belongs to no segment
+    S::store(out, row * p.nseg + s - 1, S::kSeeded ? S::combine(env, S::seed(env), v) : v);
+  };
+  // the segment ends
+#pragma unroll
+  for (int g = 0; g < G; ++g) {
+    const u32 b = bits[g];
+    if ((b >> 1) != 0u) {  // a boundary behind one of the run's elements
+      const int rel0 = (int)(wlo - tlo) + (g * ACC_WAVE + lane) * V;
+      // everything of the tile in front of the run
+      P fore;
+      const bool hasFore = acc_join<SS>(env, hasWavePre, wavePre, g * ACC_WAVE + lane > 0, pre[g], fore);
+#pragma unroll
+      for (int k = 0; k < V; ++k) {
+        if ((b >> (k + 1)) & 1u) {
+          const int idx = sh_first[rel0 + k + 1];
+          const bool local = (b & ((2u << k) - 1u)) != 0u;  // the segment's head lies in this run
+          const S::Elt v = !local && hasFore ? S::combine(env, fore.v, x[g][k]) : x[g][k];
+          if (local || (hasFore && fore.f)) {
+            // finished: it waits in LDS under its boundary's number and is written with its
+            // neighbours; boundaries beyond the staging area are written at once
+            if (idx < ACC_FOLDSEG_STAGE) {
+              sh_stage[idx] = v;
+              (void)__hip_atomic_fetch_or(&sh_staged[idx >> 5], 1u << (idx & 31), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+            } else {
+              write(idx, v);
+            }
+          } else {
+            sh_pend_at = idx;  // no head of the tile precedes it: at most one such end per tile
+            sh_pend = v;
+          }
+        }
+      }
+    }
+  }
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    p.pend_at[tile] = sh_pend_at == NOPEND ? (i64)-1 : j0 + sh_pend_at;
+    if (sh_pend_at != NOPEND) reinterpret_cast<P*>(p.pend)[tile].v = sh_pend;
+  }
+  {
+    const i64 inTile = jend - j0 + 1;
+    const int top = inTile < ACC_FOLDSEG_STAGE ? (int)inTile : ACC_FOLDSEG_STAGE;
+    for (int idx = threadIdx.x; idx < top; idx += ACC_SCAN_BLOCK)
+      if ((sh_staged[idx >> 5] >> (idx & 31)) & 1u) write(idx, sh_stage[idx]);
+  }
 }
 
 extern "C" __global__ void __launch_bounds__(ACC_SCAN_BLOCK)
@@ -324,17 +562,31 @@ acc_foldseg(Spec::Env env, Spec::Out out, FoldSegParams p) {
   typedef AccScanCfg<AccSegSpec<Spec>> C;
   // sh_first[q]: first boundary (relative to the tile's first) at position q of the tile
   __shared__ __attribute__((aligned(16))) unsigned short sh_first[C::TILE + 8];
+  __shared__ u32 sh_head[C::TILE / 32 + 2];
   __shared__ AccSegSpec<Spec>::Elt sh_wave[ACC_SCAN_WAVES];
   __shared__ AccSegSpec<Spec>::Elt sh_rake[ACC_SCAN_WAVES * (ACC_WAVE * (C::G + 1) + 1)];
   __shared__ Spec::Elt sh_pend;
   __shared__ int sh_pend_at;
+  __shared__ Spec::Elt sh_stage[ACC_FOLDSEG_STAGE];
+  __shared__ u32 sh_staged[ACC_FOLDSEG_STAGE / 32];
   const bool full = ((i64)blockIdx.x + 1) * (i64)C::TILE <= p.total;
-  if (p.rows == 1) {
-    if (full) acc_foldseg_tile<true, true>(env, out, p, sh_first, sh_wave, sh_rake, sh_pend, sh_pend_at);
-    else acc_foldseg_tile<true, false>(env, out, p, sh_first, sh_wave, sh_rake, sh_pend, sh_pend_at);
+  // (clamped: offsets that do not ascend leave entries of part unwritten)
+  const i64 nb = p.rows * (p.nseg + 1);
+  i64 j0 = p.part[blockIdx.x], j1 = p.part[blockIdx.x + 1];
+  j0 = j0 < 0 ? 0 : (j0 > nb ? nb : j0);
+  j1 = j1 < j0 ? j0 : (j1 > nb ? nb : j1);
+  // far more boundaries than positions (long runs of empty segments): the tile that numbers
+  // its boundaries by searching
+  const bool crowded = j1 - j0 > (4 * (i64)C::TILE < 65000 ? 4 * (i64)C::TILE : 65000);
+  if (crowded) {
+    if (p.rows == 1) acc_foldseg_tile<true, false>(env, out, p, sh_first, sh_wave, sh_rake, sh_pend, sh_pend_at, sh_stage, sh_staged);
+    else acc_foldseg_tile<false, false>(env, out, p, sh_first, sh_wave, sh_rake, sh_pend, sh_pend_at, sh_stage, sh_staged);
+  } else if (p.rows == 1) {
+    if (full) acc_foldseg_tile_fast<true, true>(env, out, p, j0, j1, sh_first, sh_head, sh_wave, sh_rake, sh_pend, sh_pend_at, sh_stage, sh_staged);
+    else acc_foldseg_tile_fast<true, false>(env, out, p, j0, j1, sh_first, sh_head, sh_wave, sh_rake, sh_pend, sh_pend_at, sh_stage, sh_staged);
   } else {
-    if (full) acc_foldseg_tile<false, true>(env, out, p, sh_first, sh_wave, sh_rake, sh_pend, sh_pend_at);
-    else acc_foldseg_tile<false, false>(env, out, p, sh_first, sh_wave, sh_rake, sh_pend, sh_pend_at);
+    if (full) acc_foldseg_tile_fast<false, true>(env, out, p, j0, j1, sh_first, sh_head, sh_wave, sh_rake, sh_pend, sh_pend_at, sh_stage, sh_staged);
+    else acc_foldseg_tile_fast<false, false>(env, out, p, j0, j1, sh_first, sh_head, sh_wave, sh_rake, sh_pend, sh_pend_at, sh_stage, sh_staged);
   }
 }
 
