@@ -17,7 +17,8 @@ struct acchip_ctx {
 struct acchip_program {
   std::shared_ptr<Context> keep;  // declared first: destroyed after prog
   Program prog;
-  acchip_program(acchip_ctx* c, const char* t, size_t n) : keep(c->ctx), prog(*c->ctx, t, n) {}
+  std::vector<std::string> keys;
+  acchip_program(acchip_ctx* c, const char* t, size_t n) : keep(c->ctx), prog(*c->ctx, t, n), keys(prog.kernelKeys()) {}
 };
 struct acchip_array {
   AValP v;
@@ -308,6 +309,9 @@ int acchip_compile(acchip_ctx* ctx, const char* program_text, size_t length, acc
 void acchip_program_release(acchip_program* p) { delete p; }
 int acchip_program_arity(const acchip_program* p) { return (int)p->prog.argTypes.size(); }
 int acchip_program_num_kernels(const acchip_program* p) { return (int)p->prog.kernelCount(); }
+const char* acchip_program_kernel_key(const acchip_program* p, int k) {
+  return k >= 0 && k < (int)p->keys.size() ? p->keys[k].c_str() : nullptr;
+}
 
 int acchip_sha3_256(const void* data, size_t length, uint8_t digest[32]) {
   ACCHIP_TRY

@@ -368,6 +368,14 @@ Program::Program(Context& ctx, const char* text, size_t len) : ctx_(ctx) {
   }
 }
 
+std::vector<std::string> Program::kernelKeys() const {
+  std::vector<std::string> keys;
+  for (auto& kv : plans_)
+    if (kv.second.k) keys.push_back(kv.second.k->hash);
+  std::sort(keys.begin(), keys.end());
+  return keys;
+}
+
 std::vector<ArrayR> Program::aenvOf(const TEnv& tenv) {
   std::vector<ArrayR> a(tenv.rbegin(), tenv.rend());  // index 0 = most recently bound
   return a;

@@ -94,6 +94,8 @@ class Program {
   std::vector<ATyP> argTypes;
   ATyP resultType;
   size_t kernelCount() const { return plans_.size(); }
+  // cache keys of the kernels the nodes launch (main variants), sorted
+  std::vector<std::string> kernelKeys() const;
 
  private:
   Context& ctx_;

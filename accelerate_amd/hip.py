@@ -77,6 +77,7 @@ def lib():
         "acchip_program_release": (None, [vp]),
         "acchip_program_arity": (C.c_int, [vp]),
         "acchip_program_num_kernels": (C.c_int, [vp]),
+        "acchip_program_kernel_key": (C.c_char_p, [vp, C.c_int]),
         "acchip_sha3_256": (C.c_int, [vp, C.c_size_t, C.c_char_p]),
         "acchip_set_trace": (C.c_int, [vp, vp, vp]),
         "acchip_execute": (C.c_int, [vp, vp, C.POINTER(vp), C.c_int, C.POINTER(vp), C.c_int, C.POINTER(vp)]),
@@ -327,6 +328,17 @@ class Program:
     @property
     def num_kernels(self):
         return lib().acchip_program_num_kernels(self._h)
+
+    @property
+    def kernel_keys(self):
+        """Cache keys (hex SHA3-256) of the program's kernels, sorted."""
+        out, k = [], 0
+        while True:
+            key = lib().acchip_program_kernel_key(self._h, k)
+            if key is None:
+                return out
+            out.append(key.decode())
+            k += 1
 
     def _arg(self, ty, v, keep):
         if isinstance(v, DeviceArray):

@@ -1,18 +1,27 @@
 #!/usr/bin/env python3
-"""Benchmark of the MI355X Accelerate backend on its headline workload.
+"""Benchmark of the MI355X Accelerate backend.
 
-One step = one application of the prepared program `runN (scanl1 (+))` to a device-resident
-Int64 vector of 2^28 elements (one launch of the single-pass scan kernel), through the C
-ABI.  Prints one JSON line.  The other four configurations and the 2^28 fold / map are
-timed once each and reported under "skeletons" in the same line (skip with --quick).
+Headline (the JSON line's `value`, `roofline`, `cpu_baseline`): one step = one application of the
+prepared program `runN (scanl1 (+))` to a device-resident Int64 vector of 2^28 elements (one
+launch of the single-pass scan kernel), through the C ABI.  The same line carries, under
+"configs", every benchmark configuration (dotp, both scans, foldSeg, histogram, Jacobi) and the
+2^28 map / dotp the bandwidth target is stated for, each with its own roofline entry (median of
+the per-step times between HIP events on the library's stream) and the CPU figures of the same
+workload on one core and on all host cores.
 
-  python bench.py [--gpus 1] [--steps K] [--warmup W] [--quick] [--no-cpu]
+  python bench.py [--gpus 1] [--steps K] [--warmup W] [--quick] [--no-cpu] [--only ID]
+
+--only ID runs one workload and nothing else (the form profiles are taken in); --quick the
+headline only.  HBM traffic per launch comes from profiles/traffic.json, which records what
+rocprofv3 counted for the kernels with the cache keys named there; a figure recorded for other
+code is reported as null.
 """
 from __future__ import annotations
 
 import argparse
 import json
 import os
+import statistics
 import sys
 import time
 
@@ -22,38 +31,187 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0   # MI355X HBM3E, published peak
-# HBM bytes one launch of the headline kernel moves, from the rocprofv3 FETCH_SIZE and
-# WRITE_SIZE passes over this same program (profiles/acc_scan_scanl1_int64_2p28.md: 2.0047 GiB
-# read + 2.0016 GiB written, counters scaled by a copy kernel of known size); a counter pass
-# cannot run inside the timed process, so the figure is carried here.
-SCAN_TRAFFIC_BYTES = 4299695478
+TRAFFIC_FILE = os.path.join(ROOT, "profiles", "traffic.json")
 
 
 def log(*a):
     print(*a, file=sys.stderr, flush=True)
 
 
-def time_program(ctx, run, args, steps, warmup):
-    """Returns (wall ms per step, event ms per step) over exactly `steps` applications."""
+def time_steps(ctx, run, args, steps, warmup):
+    """(wall ms per step over exactly `steps` applications, list of per-step ms between events)"""
+    res = None
     for _ in range(warmup):
         res = run.execute(*args)
     ctx.sync()
-    e0 = ctx.event()
+    ev = [ctx.event()]
     t0 = time.perf_counter()
     for _ in range(steps):
         res = run.execute(*args)
-    e1 = ctx.event()
+        ev.append(ctx.event())
     ctx.sync()
     wall = (time.perf_counter() - t0) * 1e3 / steps
-    ev = e0.elapsed_ms(e1) / steps
+    per = [ev[k].elapsed_ms(ev[k + 1]) for k in range(steps)]
     del res
-    return wall, ev
+    return wall, per
 
 
-def entry(name, n, nbytes, ev_ms):
-    gbs = nbytes / ev_ms / 1e6
-    return {"workload": name, "elements": n, "algorithmic_bytes": nbytes, "us": round(ev_ms * 1e3, 2),
-            "gelem_per_s": round(n / ev_ms / 1e6, 2), "gb_per_s": round(gbs, 1), "frac_of_hbm_peak": round(gbs / HBM_PEAK_GBS, 4)}
+def cpu_time(fn, reps):
+    fn()
+    best = []
+    for _ in range(reps):
+        t0 = time.perf_counter()
+        fn()
+        best.append(time.perf_counter() - t0)
+    return statistics.median(best)
+
+
+def traffic_for(workload, keys):
+    """HBM bytes per launch recorded for this workload's kernels, or None when the record was
+    taken on kernels with other cache keys (stale) or is absent."""
+    try:
+        rec = json.load(open(TRAFFIC_FILE))["workloads"].get(workload)
+    except (OSError, ValueError, KeyError):
+        return None
+    if not rec or sorted(rec.get("kernel_keys", [])) != sorted(keys):
+        return None
+    return int(rec["fetch_bytes"] + rec["write_bytes"])
+
+
+class Workloads:
+    """The configurations: program, seeded inputs, algorithmic bytes, CPU loops."""
+
+    def __init__(self):
+        from accelerate_amd import ir as A, programs as P, workloads as W
+        self.A, self.P, self.W = A, P, W
+        self._cache = {}
+
+    def ids(self):
+        return ["scan_i64", "scan_f32", "map_f32", "dotp_2p28", "dotp_2p24", "foldseg", "histogram", "jacobi"]
+
+    def vec(self, kind, n, seed):
+        key = (kind, n, seed)
+        if key not in self._cache:
+            W = self.W
+            self._cache[key] = {"i64": lambda: W.uniform_int(n, seed), "f01": lambda: W.uniform_f32(n, seed, 0.0, 1.0),
+                                "f11": lambda: W.uniform_f32(n, seed)}[kind]()
+        return self._cache[key]
+
+    def drop(self):
+        self._cache.clear()
+
+    def make(self, wid):
+        """dict(name, program, arg types, host args, elements, bytes, kernel, cpu(seq, omp) closures)"""
+        A, P, W = self.A, self.P, self.W
+        from oracle import c as OC
+        n28 = 1 << 28
+        if wid == "scan_i64":
+            x = self.vec("i64", n28, 20240601)
+            return dict(name="scanl1 (+) Int64 n=2^28", prog=P.scanl1_sum(A.i64), tys=[A.tarray(1, A.i64)], args=[x],
+                        n=n28, bytes=16 * n28, kernel="acc_scan", unit="Gelem/s",
+                        seq=lambda: OC.scanl1_i64(x), omp=lambda: OC.omp_scanl1(x), sample="full workload")
+        if wid == "scan_f32":
+            x = self.vec("f01", n28, 11)
+            return dict(name="scanl1 (+) Float32 n=2^28", prog=P.scanl1_sum(A.f32), tys=[A.tarray(1, A.f32)], args=[x],
+                        n=n28, bytes=8 * n28, kernel="acc_scan", unit="Gelem/s",
+                        seq=lambda: OC.scanl1_f32(x), omp=lambda: OC.omp_scanl1(x), sample="full workload")
+        if wid == "map_f32":
+            x = self.vec("f01", n28, 11)
+            return dict(name="map (\\x -> 2*x+1) Float32 n=2^28", prog=P.map_affine(), tys=[A.tarray(1, A.f32)], args=[x],
+                        n=n28, bytes=8 * n28, kernel="acc_map_stream", unit="Gelem/s",
+                        seq=lambda: np.add(np.multiply(x, np.float32(2)), np.float32(1)), omp=None,
+                        sample="full workload (numpy, one core)")
+        if wid in ("dotp_2p28", "dotp_2p24"):
+            n = n28 if wid == "dotp_2p28" else 1 << 24
+            x, y = self.vec("f01", n28, 11)[:n], self.vec("f11", n28, 12)[:n]
+            return dict(name="dotp Float32 n=2^%d" % (28 if n == n28 else 24), prog=P.dotp(),
+                        tys=[A.tarray(1, A.f32)] * 2, args=[x, y], n=n, bytes=8 * n + 4,
+                        kernel="acc_fold_main_stream" if n == n28 else "acc_fold_main", unit="Gelem/s",
+                        seq=lambda: OC.dotp_f32(x, y), omp=lambda: OC.omp_dotp_f32(x, y), sample="full workload")
+        if wid == "foldseg":
+            nseg, total = 1 << 20, 1 << 27
+            vals, lens = W.uniform_int(total, 13, dtype=np.int32), W.segment_lengths(nseg, total, 14)
+            offs = OC.offsets_i32(lens)
+            return dict(name="foldSeg (+) 0 Int32, 2^27 values / 2^20 segments (offsets scan included)",
+                        prog=P.foldseg_sum(), tys=[A.tarray(1, A.i32), A.tarray(1, A.i32)], args=[vals, lens], n=total,
+                        bytes=4 * total + 4 * (nseg + 1) + 4 * nseg + 8 * nseg + 4, kernel="acc_foldseg", unit="Gelem/s",
+                        seq=lambda: OC.foldseg_i32(vals, lens), omp=lambda: OC.omp_foldseg_i32(vals, OC.offsets_i32(lens)),
+                        sample="full workload", check=lambda got: np.array_equal(got, OC.seq_foldseg_offsets_i32(vals, offs)))
+        if wid == "histogram":
+            nk, nb = 1 << 26, 1 << 16
+            keys = W.zipf_keys(nk, nb, 15)
+            return dict(name="histogram: permute (+) of 2^26 Zipf(1.1) keys into 2^16 Int32 bins", prog=P.histogram(nb),
+                        tys=[A.tarray(1, A.i32)], args=[keys], n=nk, bytes=4 * nk + 8 * nb, kernel="acc_permute_count",
+                        unit="Gelem/s", seq=lambda: OC.histogram_i32(keys, nb), omp=lambda: OC.omp_histogram_i32(keys, nb),
+                        sample="full workload", check=lambda got: np.array_equal(got, np.bincount(keys, minlength=nb)))
+        if wid == "jacobi":
+            side = 8192
+            g = W.uniform_f32(side * side, 16, 0.0, 1.0).reshape(side, side)
+            return dict(name="Jacobi 3x3 cross, clamp, 8192x8192 Float32, per sweep of 100", prog=P.jacobi_step(),
+                        tys=[A.tarray(2, A.f32)], args=[g], n=side * side, bytes=8 * side * side, kernel="acc_stencil2d",
+                        unit="Gcell/s", iterate=100, seq=lambda: OC.jacobi_f32(g, 2), omp=lambda: OC.omp_jacobi_f32(g, 4),
+                        seq_units=2, omp_units=4, sample="2 (one core) / 4 (all cores) sweeps of the 100")
+        raise KeyError(wid)
+
+
+def run_workload(ctx, wl, steps, warmup, with_cpu, cpu_reps=3):
+    """Time one workload on the GPU (and the CPU); returns (entry, wall ms per step, mean event ms)."""
+    from accelerate_amd import hip  # noqa: F401
+    run = ctx.compile(wl["prog"])
+    dev = [ctx.to_device(a, t) for a, t in zip(wl["args"], wl["tys"])]
+    if wl.get("iterate"):
+        # the stencil configuration: `iterate` sweeps, each fed with the previous one's result
+        it = wl["iterate"]
+        g = dev[0]
+        for _ in range(5):
+            g = run.execute(g)
+        ctx.sync()
+        per = []
+        t0 = time.perf_counter()
+        for _ in range(max(1, steps // 10)):
+            g = dev[0]
+            ev = [ctx.event()]
+            for _ in range(it):
+                g = run.execute(g)
+                ev.append(ctx.event())
+            ctx.sync()
+            per += [ev[k].elapsed_ms(ev[k + 1]) for k in range(it)]
+        wall = (time.perf_counter() - t0) * 1e3 / len(per)
+        del g
+    else:
+        wall, per = time_steps(ctx, run, dev, steps, warmup)
+    if "check" in wl:
+        assert wl["check"](run.execute(*dev).to_host()), "result of %s differs from the oracle" % wl["name"]
+    med, mean = statistics.median(per), sum(per) / len(per)
+    gbs = wl["bytes"] / med / 1e6
+    entry = {"workload": wl["name"], "elements": wl["n"], "algorithmic_bytes": wl["bytes"], "us": round(med * 1e3, 2),
+             "steps_timed": len(per), "value": round(wl["n"] / med / 1e6, 2), "unit": wl["unit"],
+             "roofline": {"bound": "hbm", "kernel": wl["kernel"], "achieved": round(gbs, 1), "peak": HBM_PEAK_GBS,
+                          "unit": "GB/s", "frac": round(gbs / HBM_PEAK_GBS, 4),
+                          "traffic": traffic_for(wl["name"], run.kernel_keys)},
+             "kernel_keys": run.kernel_keys}
+    del dev
+    if with_cpu:
+        from oracle import c as OC
+        su, ou = wl.get("seq_units", 1), wl.get("omp_units", 1)
+        dt = cpu_time(wl["seq"], cpu_reps)
+        entry["cpu_seq"] = {"value": round(wl["n"] * su / dt / 1e9, 4), "unit": wl["unit"], "cores": 1, "kind": "port",
+                            "sample": wl["sample"]}
+        if wl["omp"] is not None:
+            dt = cpu_time(wl["omp"], cpu_reps)
+            entry["cpu_omp"] = {"value": round(wl["n"] * ou / dt / 1e9, 4), "unit": wl["unit"], "cores": OC.omp_threads(),
+                                "kind": "port", "sample": wl["sample"]}
+    return entry, wall, mean
+
+
+def cpu_model():
+    try:
+        for line in open("/proc/cpuinfo"):
+            if line.startswith("model name"):
+                return line.split(":", 1)[1].strip()
+    except OSError:
+        pass
+    return "unknown"
 
 
 def main():
@@ -62,105 +220,60 @@ def main():
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--quick", action="store_true", help="headline workload only")
-    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baselines")
+    ap.add_argument("--only", default=None, help="run one workload (an id of Workloads.ids()) and print its entry")
     a = ap.parse_args()
     if a.gpus != 1:
         sys.exit("bench.py: this backend runs on one GPU per process and has no multi-GPU path; "
                  "run with --gpus 1 (the per-GPU figure is the whole-job figure)")
 
-    from accelerate_amd import hip, ir as A, programs as P, workloads as W
+    from accelerate_amd import hip
     ctx = hip.Context(0)   # fails loudly without the HIP library or a GPU: there is no fallback
+    wls = Workloads()
+
+    if a.only:
+        entry, _, _ = run_workload(ctx, wls.make(a.only), a.steps, a.warmup, not a.no_cpu)
+        print(json.dumps(entry), flush=True)
+        return
 
     # ---- headline: scanl1 (+) on Int64, n = 2^28 -------------------------------------------
-    n = 1 << 28
-    log("generating 2^28 Int64 input ...")
-    x = W.uniform_int(n, 20240601)
-    run = ctx.compile(P.scanl1_sum(A.i64))
-    dx = ctx.to_device(x, A.tarray(1, A.i64))
-    wall, ev = time_program(ctx, run, [dx], a.steps, a.warmup)
-    alg_bytes = 16 * n          # 8 B read + 8 B written per element
-    achieved = alg_bytes / ev / 1e6
-    # cheap integrity check of the timed path: last element equals the total
-    last = run.execute(dx).to_host()[-1]
-    assert int(last) == int(x.sum()), "scan result does not match the input's total"
-
+    log("headline: scanl1 (+) Int64 n=2^28 ...")
+    wl = wls.make("scan_i64")
+    x = wl["args"][0]
+    wl["check"] = lambda got: int(got[-1]) == int(x.sum())     # cheap integrity check of the timed path
+    head, wall, mean = run_workload(ctx, wl, a.steps, a.warmup, not a.no_cpu)
+    achieved = wl["bytes"] / mean / 1e6       # average launch duration over the timed region
     cpu = None
     if not a.no_cpu:
-        from oracle import c as OC
-        reps = 3
-        OC.scanl1_i64(x[: 1 << 20])
-        t0 = time.perf_counter()
-        for _ in range(reps):
-            ref = OC.scanl1_i64(x)
-        dt = (time.perf_counter() - t0) / reps
-        assert int(ref[-1]) == int(last)
-        cpu = {"value": round(n / dt / 1e9, 4), "unit": "Gelem/s", "cores": 1, "kind": "port",
-               "sample": "full workload (2^28 Int64), %d repetitions of oracle/configs.c oracle_scanl1_i64, "
-                         "sequential as the reference interpreter's loop" % reps}
-        del ref
-    del dx
-
+        cpu = dict(head["cpu_omp"])
+        cpu["sample"] = ("full workload (2^28 Int64), median of 3 runs of oracle/configs_omp.c oracle_omp_scanl1_i64 on %d "
+                         "threads (%s); one core, oracle/configs.c: %s Gelem/s" % (cpu["cores"], cpu_model(),
+                                                                                 head["cpu_seq"]["value"]))
+        cpu["seq_value"] = head["cpu_seq"]["value"]
     out = {
         "metric": "Gelem/s + HBM GB/s (% peak) per skeleton: fold, scan, foldSeg, permute, stencil",
-        "value": round(n / wall / 1e6, 3), "unit": "Gelem/s", "n_gpus": 1, "steps": a.steps, "warmup": a.warmup,
+        "value": round(wl["n"] / wall / 1e6, 3), "unit": "Gelem/s", "n_gpus": 1, "steps": a.steps, "warmup": a.warmup,
         "ms_per_step": round(wall, 5), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "int64", "data": "synthetic",
         "config": {"workload": "scanl1 (+) on an Int64 vector, n=2^28, uniform integers in [-1000,1000]",
                    "program": "Scan LeftToRight (+) Nothing (Manifest (Avar a0))", "kernel": "acc_scan"},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": SCAN_TRAFFIC_BYTES},
+                     "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": head["roofline"]["traffic"]},
         "cpu_baseline": cpu,
     }
 
-    # ---- the other configurations, once each ------------------------------------------------
+    # ---- every configuration, with its own roofline and CPU figures -------------------------
     if not a.quick:
-        sk = []
-        k, w = max(5, a.steps // 2), 3
-        x32 = W.uniform_f32(n, 11, 0.0, 1.0)
-        d = ctx.to_device(x32, A.tarray(1, A.f32))
-        _, ev = time_program(ctx, ctx.compile(P.scanl1_sum(A.f32)), [d], k, w)
-        sk.append(entry("scanl1 (+) Float32 n=2^28", n, 8 * n, ev))
-        _, ev = time_program(ctx, ctx.compile(P.map_affine()), [d], k, w)
-        sk.append(entry("map (\\x -> 2*x+1) Float32 n=2^28", n, 8 * n, ev))
-        y32 = W.uniform_f32(n, 12)
-        d2 = ctx.to_device(y32, A.tarray(1, A.f32))
-        dot = ctx.compile(P.dotp())
-        _, ev = time_program(ctx, dot, [d, d2], k, w)
-        sk.append(entry("dotp Float32 n=2^28", n, 8 * n, ev))
-        del d, d2
-        m = 1 << 24
-        da, db = ctx.to_device(x32[:m], A.tarray(1, A.f32)), ctx.to_device(y32[:m], A.tarray(1, A.f32))
-        _, ev = time_program(ctx, dot, [da, db], 50, 10)
-        sk.append(entry("dotp Float32 n=2^24 (fits the last-level cache)", m, 8 * m, ev))
-        del da, db, x32, y32
-        nseg, total = 1 << 20, 1 << 27
-        dv = ctx.to_device(W.uniform_int(total, 13, dtype=np.int32), A.tarray(1, A.i32))
-        dl = ctx.to_device(W.segment_lengths(nseg, total, 14), A.tarray(1, A.i32))
-        _, ev = time_program(ctx, ctx.compile(P.foldseg_sum()), [dv, dl], k, w)
-        sk.append(entry("foldSeg (+) 0 Int32, 2^27 values / 2^20 segments (offsets scan included)",
-                        total, 4 * total + 4 * (nseg + 1) + 4 * nseg + 8 * nseg + 4, ev))
-        del dv, dl
-        nk, nb = 1 << 26, 1 << 16
-        dk = ctx.to_device(W.zipf_keys(nk, nb, 15), A.tarray(1, A.i32))
-        _, ev = time_program(ctx, ctx.compile(P.histogram(nb)), [dk], 20, 5)
-        sk.append(entry("histogram: permute (+) of 2^26 Zipf(1.1) keys into 2^16 Int32 bins", nk, 4 * nk + 8 * nb, ev))
-        del dk
-        side = 8192
-        dg = ctx.to_device(W.uniform_f32(side * side, 16, 0.0, 1.0).reshape(side, side), A.tarray(2, A.f32))
-        step = ctx.compile(P.jacobi_step())
-        g = dg
-        for _ in range(5):
-            g = step.execute(g)
-        ctx.sync()
-        e0 = ctx.event()
-        g = dg
-        for _ in range(100):
-            g = step.execute(g)
-        e1 = ctx.event()
-        e1.sync()
-        ev = e0.elapsed_ms(e1) / 100
-        sk.append(entry("Jacobi 3x3 cross, clamp, 8192x8192 Float32, per iteration of 100", side * side, 8 * side * side, ev))
-        out["skeletons"] = sk
+        entries = [head]
+        for wid in wls.ids()[1:]:
+            log(wid, "...")
+            steps = 50 if wid == "dotp_2p24" else max(20, a.steps)
+            e, _, _ = run_workload(ctx, wls.make(wid), steps, a.warmup, not a.no_cpu)
+            entries.append(e)
+            if wid in ("dotp_2p24",):
+                wls.drop()
+        out["configs"] = entries
+        out["host"] = {"cpu": cpu_model(), "threads": os.cpu_count()}
 
     print(json.dumps(out), flush=True)
 

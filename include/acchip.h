@@ -132,6 +132,12 @@ int acchip_compile(acchip_ctx* ctx, const char* program_text, size_t length, acc
 void acchip_program_release(acchip_program* p);
 int acchip_program_arity(const acchip_program* p);
 int acchip_program_num_kernels(const acchip_program* p);
+/* Cache key of the program's k-th kernel, k = 0 .. num_kernels - 1: the hexadecimal SHA3-256 of
+ * its generated source, compile options and hipRTC version (the counterpart of the reference's
+ * hashPreOpenAccWith, Analysis/Hash.hs:107-111, which names the kernels of accelerate-llvm's
+ * cache).  NULL beyond the last kernel; valid while the program lives.  Profiles refer to
+ * kernels by this key, so a figure measured on other code is recognised as stale. */
+const char* acchip_program_kernel_key(const acchip_program* p, int k);
 
 /* SHA3-256 digest used for kernel cache keys; same function as the reference's
  * Crypto.Hash.XKCP (src/Crypto/Hash/XKCP.hs:93-170, cbits/xkcp SHA3_256). */

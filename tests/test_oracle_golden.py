@@ -251,6 +251,25 @@ def test_c_loops_match_interpreter():
     assert same(OC.fold_sum_i32(m, 42), O.run_n(P.fold_sum(A.i32, 2, 42).text(), m))
 
 
+def test_all_cores_loops_agree_with_the_sequential_ones():
+    # the OpenMP versions only serve as a timing baseline; integer results must still be the same
+    # bits, Float32 sums the same within the benchmark's tolerance
+    xi = W.uniform_int(100003, 3)
+    assert same(OC.omp_scanl1(xi), OC.scanl1_i64(xi))
+    xf = W.uniform_f32(100003, 4, 0, 1)
+    assert np.all(np.abs(OC.omp_scanl1(xf) - np.cumsum(xf.astype(np.float64))) <= 1e-4 * np.cumsum(np.abs(xf.astype(np.float64))))
+    x, y = W.uniform_f32(70001, 1), W.uniform_f32(70001, 2)
+    assert abs(float(OC.omp_dotp_f32(x, y)) - float(np.dot(x.astype(np.float64), y))) <= 1e-4 * float(np.sum(np.abs(x * y)))
+    lens = W.segment_lengths(400, 50000, 5)
+    vals = W.uniform_int(50000, 6, dtype=np.int32)
+    assert same(OC.omp_foldseg_i32(vals, OC.offsets_i32(lens)), OC.foldseg_i32(vals, lens))
+    keys = W.zipf_keys(200000, 1000, 8)
+    assert same(OC.omp_histogram_i32(keys, 1000), OC.histogram_i32(keys, 1000))
+    g = W.uniform_f32(37 * 53, 9, 0, 1).reshape(37, 53)
+    assert same(OC.omp_jacobi_f32(g, 5), OC.jacobi_f32(g, 5))
+    assert OC.omp_threads() >= 1
+
+
 def test_workload_generators_are_seeded_and_shaped():
     lens = W.segment_lengths(1 << 12, 1 << 19, 3)
     assert lens.sum() == 1 << 19 and lens.min() >= 0 and same(lens, W.segment_lengths(1 << 12, 1 << 19, 3))
