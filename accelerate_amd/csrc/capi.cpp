@@ -114,6 +114,59 @@ int acchip_peek(acchip_ctx* ctx, void* host, const void* devptr, size_t bytes) {
   ACCHIP_END
 }
 
+int acchip_table_malloc(acchip_ctx* ctx, uint64_t id, void* host, size_t bytes, int frozen, int* allocated) {
+  ACCHIP_TRY
+  const bool fresh = ctx->ctx->tableMalloc(id, host, bytes, frozen != 0);
+  if (allocated) *allocated = fresh ? 1 : 0;
+  return ACCHIP_OK;
+  ACCHIP_END
+}
+int acchip_table_use(acchip_ctx* ctx, uint64_t id, void** devptr) {
+  ACCHIP_TRY
+  if (!devptr) return failMsg("null output pointer");
+  *devptr = ctx->ctx->tableUse(id);
+  return ACCHIP_OK;
+  ACCHIP_END
+}
+int acchip_table_release(acchip_ctx* ctx, uint64_t id) {
+  ACCHIP_TRY
+  ctx->ctx->tableRelease(id);
+  return ACCHIP_OK;
+  ACCHIP_END
+}
+void acchip_table_free(acchip_ctx* ctx, uint64_t id) {
+  try {
+    ctx->ctx->tableFree(id);
+  } catch (...) {
+  }
+}
+int acchip_table_insert_unmanaged(acchip_ctx* ctx, uint64_t id, void* devptr) {
+  ACCHIP_TRY
+  ctx->ctx->tableInsertUnmanaged(id, devptr);
+  return ACCHIP_OK;
+  ACCHIP_END
+}
+void acchip_table_reclaim(acchip_ctx* ctx) {
+  try {
+    ctx->ctx->tableReclaim();
+  } catch (...) {
+  }
+}
+int acchip_table_status(acchip_ctx* ctx, uint64_t id) {
+  try {
+    return ctx->ctx->tableStatus(id);
+  } catch (...) {
+    return -1;
+  }
+}
+int acchip_set_clean_hook(acchip_ctx* ctx, acchip_clean_fn fn, void* user) {
+  ACCHIP_TRY
+  if (!fn) ctx->ctx->cleanHook = nullptr;
+  else ctx->ctx->cleanHook = [fn, user]() { fn(user); };
+  return ACCHIP_OK;
+  ACCHIP_END
+}
+
 long long acchip_stat(acchip_ctx* ctx, const char* name) {
   Stats& s = ctx->ctx->stats;
   std::string n = name ? name : "";
@@ -127,6 +180,7 @@ long long acchip_stat(acchip_ctx* ctx, const char* name) {
   if (n == "launches") return s.launches;
   if (n == "pool_hits") return s.poolHits;
   if (n == "pool_misses") return s.poolMisses;
+  if (n == "arrays_evicted") return s.arraysEvicted;
   return -1;
 }
 

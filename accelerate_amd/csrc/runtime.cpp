@@ -44,6 +44,11 @@ Context::Context(int device) : device_(device) {
     dumpExec = f.find("dump-exec") != std::string::npos;
     forceRecomp = f.find("force-recomp") != std::string::npos;
   }
+  if (device_ == -2) {
+    fakeMemory_ = true;
+    device_ = -1;
+  }
+  if (const char* pl = std::getenv("ACCHIP_POOL_LIMIT")) limit_ = (size_t)std::strtoull(pl, nullptr, 0);
   if (device_ >= 0) {
     hipCheck(hipSetDevice(device_), "hipSetDevice");
     hipCheck(hipStreamCreateWithFlags(&stream_, hipStreamNonBlocking), "hipStreamCreate");
@@ -59,14 +64,23 @@ Context::~Context() {
     } catch (...) {
     }
   }
-  if (device_ < 0) return;
+  if (device_ < 0) {
+    purge();
+    for (auto& kv : live_) rawFree(kv.first, kv.second);
+    return;
+  }
   (void)hipSetDevice(device_);
   (void)hipStreamSynchronize(stream_);
   for (auto& kv : kernels_)
     if (kv.second->module) (void)hipModuleUnload(kv.second->module);
+  for (auto& kv : table_)
+    if (kv.second.task) (void)hipEventDestroy(kv.second.task);
   purge();
-  for (auto& kv : live_) (void)hipFree(kv.first);
-  if (staging_) (void)hipHostFree(staging_);
+  for (auto& kv : live_) rawFree(kv.first, kv.second);
+  for (int b = 0; b < 2; ++b) {
+    if (staging_[b]) (void)hipHostFree(staging_[b]);
+    if (stagingDone_[b]) (void)hipEventDestroy(stagingDone_[b]);
+  }
   if (errHost_) (void)hipHostFree(errHost_);
   if (scan_.desc) (void)hipFree(scan_.desc);
   if (scan_.ticket) (void)hipFree(scan_.ticket);
@@ -76,45 +90,93 @@ Context::~Context() {
 // ------------------------------------------------------------------------------------
 // memory
 
+static const size_t kStagePiece = (size_t)32 << 20;
+
 static size_t roundUp(size_t bytes) {
   const size_t chunk = 1024;  // remoteAllocationSize default (Array/Remote/Table.hs:180-190)
   if (bytes == 0) bytes = 1;
   return (bytes + chunk - 1) / chunk * chunk;
 }
 
-void* Context::malloc(size_t bytes) {
-  if (device_ < 0) return nullptr;
-  size_t n = roundUp(bytes);
+void* Context::rawMalloc(size_t n) {
   {
     std::lock_guard<std::mutex> g(mu_);
-    auto it = nursery_.find(n);
-    if (it != nursery_.end() && !it->second.empty()) {
-      void* p = it->second.back();
-      it->second.pop_back();
-      live_[p] = n;
-      stats.poolHits++;
-      return p;
+    if (limit_ && rawBytes_ + n > limit_) return nullptr;  // the budget stands in for a full device
+    rawBytes_ += n;
+  }
+  void* p = nullptr;
+  if (fakeMemory_) {
+    p = std::malloc(n);
+  } else {
+    (void)hipSetDevice(device_);
+    if (hipMalloc(&p, n) != hipSuccess) {
+      (void)hipGetLastError();
+      p = nullptr;
     }
+  }
+  if (!p) {
+    std::lock_guard<std::mutex> g(mu_);
+    rawBytes_ -= n;
+  }
+  return p;
+}
+
+void Context::rawFree(void* p, size_t n) {
+  if (fakeMemory_) std::free(p);
+  else (void)hipFree(p);
+  std::lock_guard<std::mutex> g(mu_);
+  rawBytes_ -= n;
+}
+
+void* Context::malloc(size_t bytes) { return poolMalloc(bytes, true); }
+
+void* Context::poolMalloc(size_t bytes, bool mayEvict) {
+  if (!hasMemory()) return nullptr;
+  const size_t n = roundUp(bytes);
+  auto fromNursery = [&]() -> void* {
+    std::lock_guard<std::mutex> g(mu_);
+    auto it = nursery_.find(n);
+    if (it == nursery_.end() || it->second.empty()) return nullptr;
+    void* p = it->second.back();
+    it->second.pop_back();
+    live_[p] = n;
+    return p;
+  };
+  auto fresh = [&]() -> void* {
+    void* p = rawMalloc(n);
+    if (p) {
+      stats.bytesAllocated += (long long)n;
+      std::lock_guard<std::mutex> g(mu_);
+      live_[p] = n;
+    }
+    return p;
+  };
+  if (void* p = fromNursery()) {
+    stats.poolHits++;
+    return p;
   }
   stats.poolMisses++;
-  void* p = nullptr;
-  (void)hipSetDevice(device_);
-  hipError_t e = hipMalloc(&p, n);
-  if (e != hipSuccess) {
-    (void)hipGetLastError();
-    // work queued on the stream may still use blocks waiting in the free lists
-    (void)hipStreamSynchronize(stream_);
-    purge();
-    e = hipMalloc(&p, n);
-    if (e != hipSuccess) {
-      (void)hipGetLastError();
-      return nullptr;
-    }
+  if (void* p = fresh()) return p;
+  // the caller's collector may find dead host arrays, whose blocks then wait in the free lists
+  if (cleanHook) {
+    cleanHook();
+    if (void* p = fromNursery()) return p;
   }
-  stats.bytesAllocated += (long long)n;
-  std::lock_guard<std::mutex> g(mu_);
-  live_[p] = n;
-  return p;
+  // work queued on the stream may still use blocks waiting in the free lists
+  if (device_ >= 0) (void)hipStreamSynchronize(stream_);
+  purge();
+  if (void* p = fresh()) return p;
+  // evict unused arrays of the table, eldest first, until the block fits or nothing is left
+  while (mayEvict) {
+    {
+      std::lock_guard<std::mutex> g(tableMu_);
+      if (!evictEldest()) break;
+    }
+    if (void* p = fromNursery()) return p;
+    purge();
+    if (void* p = fresh()) return p;
+  }
+  return nullptr;
 }
 
 void Context::free(void* p) {
@@ -134,7 +196,7 @@ void Context::purge() {
   }
   for (auto& kv : take)
     for (void* p : kv.second) {
-      (void)hipFree(p);
+      rawFree(p, kv.first);
       stats.bytesEvicted += (long long)kv.first;
     }
 }
@@ -147,54 +209,222 @@ size_t Context::blockSize(void* p) {
 
 void Context::memInfo(size_t* total, size_t* avail) {
   *total = *avail = 0;
-  if (device_ < 0) return;
-  hipCheck(hipMemGetInfo(avail, total), "hipMemGetInfo");
+  if (!hasMemory()) return;
+  if (device_ >= 0) hipCheck(hipMemGetInfo(avail, total), "hipMemGetInfo");
   std::lock_guard<std::mutex> g(mu_);
+  if (limit_) {
+    *total = limit_;
+    *avail = limit_ > rawBytes_ ? limit_ - rawBytes_ : 0;
+  } else if (fakeMemory_) {
+    *total = *avail = (size_t)1 << 40;
+  }
   for (auto& kv : nursery_) *avail += kv.first * kv.second.size();  // reusable without asking the driver
 }
 
-void* Context::staging(size_t bytes) {
-  if (bytes > stagingBytes_) {
-    if (staging_) {
-      hipCheck(hipStreamSynchronize(stream_), "hipStreamSynchronize");
-      (void)hipHostFree(staging_);
-      staging_ = nullptr;
-    }
-    hipCheck(hipHostMalloc(&staging_, bytes, hipHostMallocDefault), "hipHostMalloc");
-    stagingBytes_ = bytes;
+// ------------------------------------------------------------------------------------
+// array table
+
+bool Context::taskDone(Entry& e) {
+  if (!e.task) return true;
+  const hipError_t r = hipEventQuery(e.task);
+  if (r == hipErrorNotReady) {
+    (void)hipGetLastError();
+    return false;
   }
-  return staging_;
+  return true;
 }
 
+// LRU.evictLRU (LRU.hs:273-303): the eldest array that nobody uses and whose last task has
+// finished gives up its device block; a Dirty one is copied back to its host array first.
+bool Context::evictEldest() {
+  uint64_t best = 0;
+  Entry* pick = nullptr;
+  for (auto& kv : table_) {
+    Entry& e = kv.second;
+    if (e.count != 0 || !e.dev || (e.st != Status::Clean && e.st != Status::Dirty) || !taskDone(e)) continue;
+    if (!pick || e.stamp < best) {
+      pick = &e;
+      best = e.stamp;
+    }
+  }
+  if (!pick) return false;
+  if (pick->st == Status::Dirty && pick->host) peek(pick->host, pick->dev, pick->bytes);
+  free(pick->dev);
+  stats.arraysEvicted++;
+  pick->dev = nullptr;
+  pick->st = Status::Evicted;
+  return true;
+}
+
+bool Context::tableMalloc(uint64_t id, void* host, size_t bytes, bool frozen) {
+  if (!hasMemory()) throw Error("no device");
+  {
+    std::lock_guard<std::mutex> g(tableMu_);
+    if (table_.count(id)) return false;
+  }
+  void* dev = poolMalloc(bytes, true);  // (not under the table's lock: eviction takes it)
+  if (!dev) throw Error("Remote memory exhausted");
+  std::lock_guard<std::mutex> g(tableMu_);
+  Entry e;
+  e.dev = dev;
+  e.bytes = bytes;
+  e.host = host;
+  e.st = frozen ? Status::Clean : Status::Dirty;
+  e.stamp = ++clock_;
+  if (!table_.emplace(id, e).second) {  // someone else was quicker
+    free(dev);
+    return false;
+  }
+  return true;
+}
+
+void* Context::tableUse(uint64_t id) {
+  {
+    std::lock_guard<std::mutex> g(tableMu_);
+    auto it = table_.find(id);
+    if (it == table_.end()) return nullptr;
+    Entry& e = it->second;
+    ++e.count;  // from here on it cannot be evicted
+    if (e.dev) return e.dev;
+    if (e.st != Status::Evicted) throw Error("internal error: non-evicted array has been lost");
+  }
+  // evicted: a new block, filled from the host array, which holds the current contents
+  // (withRemote / copyBack, LRU.hs:140-186)
+  size_t bytes;
+  void* host;
+  {
+    std::lock_guard<std::mutex> g(tableMu_);
+    Entry& e = table_.at(id);
+    bytes = e.bytes;
+    host = e.host;
+  }
+  void* dev = poolMalloc(bytes, true);
+  if (!dev) {
+    std::lock_guard<std::mutex> g(tableMu_);
+    --table_.at(id).count;
+    throw Error("Remote memory exhausted");
+  }
+  if (host) poke(dev, host, bytes);
+  std::lock_guard<std::mutex> g(tableMu_);
+  Entry& e = table_.at(id);
+  if (e.dev) {  // a concurrent use uploaded it meanwhile
+    free(dev);
+    return e.dev;
+  }
+  e.dev = dev;
+  e.st = Status::Clean;
+  return dev;
+}
+
+void Context::tableRelease(uint64_t id) {
+  std::lock_guard<std::mutex> g(tableMu_);
+  auto it = table_.find(id);
+  if (it == table_.end()) return;
+  Entry& e = it->second;
+  if (e.count > 0) --e.count;
+  e.stamp = ++clock_;
+  if (device_ >= 0) {  // everything queued so far may still read or write the block
+    if (!e.task) hipCheck(hipEventCreateWithFlags(&e.task, hipEventDisableTiming), "hipEventCreate");
+    hipCheck(hipEventRecord(e.task, stream_), "hipEventRecord");
+  }
+}
+
+void Context::tableFree(uint64_t id) {
+  std::lock_guard<std::mutex> g(tableMu_);
+  auto it = table_.find(id);
+  if (it == table_.end()) return;
+  Entry& e = it->second;
+  if (e.dev && e.st != Status::Unmanaged) free(e.dev);  // to the free list of its size (one stream: reuse is ordered)
+  if (e.task) (void)hipEventDestroy(e.task);
+  table_.erase(it);
+}
+
+void Context::tableInsertUnmanaged(uint64_t id, void* dev) {
+  std::lock_guard<std::mutex> g(tableMu_);
+  Entry e;
+  e.dev = dev;
+  e.st = Status::Unmanaged;
+  e.stamp = ++clock_;
+  table_[id] = e;
+}
+
+void Context::tableReclaim() {
+  if (cleanHook) cleanHook();
+  if (device_ >= 0) (void)hipStreamSynchronize(stream_);
+  purge();
+}
+
+int Context::tableStatus(uint64_t id) {
+  std::lock_guard<std::mutex> g(tableMu_);
+  auto it = table_.find(id);
+  return it == table_.end() ? -1 : (int)it->second.st;
+}
+
+// ------------------------------------------------------------------------------------
+// transfers
+
+void Context::ensureStaging() {
+  if (staging_[0]) return;
+  for (int b = 0; b < 2; ++b) {
+    hipCheck(hipHostMalloc(&staging_[b], kStagePiece, hipHostMallocDefault), "hipHostMalloc");
+    hipCheck(hipEventCreateWithFlags(&stagingDone_[b], hipEventDisableTiming), "hipEventCreate");
+  }
+}
+
+// Pageable host memory goes through two pinned buffers of 32 MiB in turn: while one piece is
+// on the wire the host copies the next one into (or the previous one out of) the other buffer.
 void Context::poke(void* dev, const void* host, size_t bytes) {
   if (bytes == 0) return;
+  if (fakeMemory_) {
+    std::memcpy(dev, host, bytes);
+    stats.bytesCopiedToRemote += (long long)bytes;
+    return;
+  }
   if (device_ < 0) throw Error("no device");
-  // Pageable host memory is staged through a pinned buffer in 64 MiB pieces.
-  const size_t piece = 64u << 20;
+  std::lock_guard<std::mutex> g(stagingMu_);
+  ensureStaging();
   const char* src = static_cast<const char*>(host);
   char* dst = static_cast<char*>(dev);
-  for (size_t off = 0; off < bytes; off += piece) {
-    size_t n = bytes - off < piece ? bytes - off : piece;
-    void* st = staging(n < piece ? n : piece);
-    std::memcpy(st, src + off, n);
-    hipCheck(hipMemcpyAsync(dst + off, st, n, hipMemcpyHostToDevice, stream_), "hipMemcpyAsync(H2D)");
-    hipCheck(hipStreamSynchronize(stream_), "hipStreamSynchronize");  // staging buffer is reused
+  int b = 0;
+  bool used[2] = {false, false};
+  for (size_t off = 0; off < bytes; off += kStagePiece, b ^= 1) {
+    const size_t n = bytes - off < kStagePiece ? bytes - off : kStagePiece;
+    if (used[b]) hipCheck(hipEventSynchronize(stagingDone_[b]), "hipEventSynchronize");  // its last copy has left
+    std::memcpy(staging_[b], src + off, n);
+    hipCheck(hipMemcpyAsync(dst + off, staging_[b], n, hipMemcpyHostToDevice, stream_), "hipMemcpyAsync(H2D)");
+    hipCheck(hipEventRecord(stagingDone_[b], stream_), "hipEventRecord");
+    used[b] = true;
   }
+  for (int k = 0; k < 2; ++k)
+    if (used[k]) hipCheck(hipEventSynchronize(stagingDone_[k]), "hipEventSynchronize");  // the buffers are free again
   stats.bytesCopiedToRemote += (long long)bytes;
 }
 
 void Context::peek(void* host, const void* dev, size_t bytes) {
   if (bytes == 0) return;
+  if (fakeMemory_) {
+    std::memcpy(host, dev, bytes);
+    stats.bytesCopiedFromRemote += (long long)bytes;
+    return;
+  }
   if (device_ < 0) throw Error("no device");
-  const size_t piece = 64u << 20;
-  char* dst = static_cast<char*>(host);
-  const char* src = static_cast<const char*>(dev);
-  for (size_t off = 0; off < bytes; off += piece) {
-    size_t n = bytes - off < piece ? bytes - off : piece;
-    void* st = staging(n < piece ? n : piece);
-    hipCheck(hipMemcpyAsync(st, src + off, n, hipMemcpyDeviceToHost, stream_), "hipMemcpyAsync(D2H)");
-    hipCheck(hipStreamSynchronize(stream_), "hipStreamSynchronize");
-    std::memcpy(dst + off, st, n);
+  {
+    std::lock_guard<std::mutex> g(stagingMu_);
+    ensureStaging();
+    char* dst = static_cast<char*>(host);
+    const char* src = static_cast<const char*>(dev);
+    const size_t pieces = (bytes + kStagePiece - 1) / kStagePiece;
+    auto len = [&](size_t k) { return bytes - k * kStagePiece < kStagePiece ? bytes - k * kStagePiece : kStagePiece; };
+    auto start = [&](size_t k) {
+      hipCheck(hipMemcpyAsync(staging_[k & 1], src + k * kStagePiece, len(k), hipMemcpyDeviceToHost, stream_), "hipMemcpyAsync(D2H)");
+      hipCheck(hipEventRecord(stagingDone_[k & 1], stream_), "hipEventRecord");
+    };
+    start(0);
+    for (size_t k = 0; k < pieces; ++k) {
+      if (k + 1 < pieces) start(k + 1);  // the next piece travels while this one is copied out
+      hipCheck(hipEventSynchronize(stagingDone_[k & 1]), "hipEventSynchronize");
+      std::memcpy(dst + k * kStagePiece, staging_[k & 1], len(k));
+    }
   }
   stats.bytesCopiedFromRemote += (long long)bytes;
   raiseDeviceError();

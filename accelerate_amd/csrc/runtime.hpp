@@ -35,7 +35,8 @@ using KernelP = std::shared_ptr<Kernel>;
 // Counters with the meaning of the reference's cbits/monitoring.c:26-32.
 struct Stats {
   std::atomic<long long> bytesAllocated{0}, bytesCopiedToRemote{0}, bytesCopiedFromRemote{0}, bytesEvicted{0},
-      kernelsCompiled{0}, kernelsFromDisk{0}, kernelsFromMemory{0}, launches{0}, poolHits{0}, poolMisses{0};
+      kernelsCompiled{0}, kernelsFromDisk{0}, kernelsFromMemory{0}, launches{0}, poolHits{0}, poolMisses{0},
+      arraysEvicted{0};
 };
 
 // Always owned by a std::shared_ptr: device buffers, programs and events keep their
@@ -47,6 +48,9 @@ class Context : public std::enable_shared_from_this<Context> {
   ~Context();
 
   bool hasDevice() const { return device_ >= 0; }
+  // device == -2: no GPU, but host memory stands in for device memory, so that the memory
+  // manager (pool, table, eviction) can be driven without one; programs still cannot run
+  bool hasMemory() const { return device_ >= 0 || fakeMemory_; }
   int device() const { return device_; }
   hipStream_t stream() const { return stream_; }
 
@@ -59,6 +63,25 @@ class Context : public std::enable_shared_from_this<Context> {
   void purge();
   size_t blockSize(void* p);
   void memInfo(size_t* total, size_t* avail);
+
+  // Array table (counterpart of Array/Remote/LRU.hs + Table.hs): host arrays, named by an id
+  // the caller chooses (the reference's StableArray / Unique), and the device blocks that
+  // mirror them.  An array in use (between tableUse and tableRelease) stays where it is; any
+  // other may be evicted when memory runs out -- copied back to its host array first if the
+  // device copy is the newer one (Dirty) -- and is uploaded again by the next tableUse.
+  // Allocation ladder (Table.hs:194-206, LRU.hs:258-303): free list of the size class, the
+  // device, the clean hook (the caller's garbage collector, whose finalisers call tableFree)
+  // and the free list again, purge + the device, then eviction of the eldest unused arrays
+  // one at a time, and only then failure.
+  enum class Status { Clean, Dirty, Unmanaged, Evicted };
+  bool tableMalloc(uint64_t id, void* host, size_t bytes, bool frozen);  // false: already known
+  void* tableUse(uint64_t id);                 // nullptr: never allocated (LRU.withRemote -> Nothing)
+  void tableRelease(uint64_t id);              // end of the use; work queued so far may still touch it
+  void tableFree(uint64_t id);                 // the host array died
+  void tableInsertUnmanaged(uint64_t id, void* dev);
+  void tableReclaim();                         // LRU.reclaim: clean + purge
+  int tableStatus(uint64_t id);                // -1 unknown, else a Status
+  std::function<void()> cleanHook;
 
   void poke(void* dev, const void* host, size_t bytes);   // H->D through pinned staging, stream-ordered
   void peek(void* host, const void* dev, size_t bytes);   // D->H, synchronises the stream
@@ -100,13 +123,37 @@ class Context : public std::enable_shared_from_this<Context> {
   std::unordered_map<void*, size_t> live_;                  // block -> rounded size
   std::map<size_t, std::vector<void*>> nursery_;            // rounded size -> free blocks
   std::unordered_map<std::string, KernelP> kernels_;
-  void* staging_ = nullptr;
   unsigned* errHost_ = nullptr;  // pinned, mapped: written by kernels, read here
   unsigned* errDev_ = nullptr;
-  size_t stagingBytes_ = 0;
+  // two pinned staging buffers: the host copies into / out of one while the other is on the wire
+  std::mutex stagingMu_;
+  void* staging_[2] = {nullptr, nullptr};
+  hipEvent_t stagingDone_[2] = {nullptr, nullptr};
   ScanState scan_;
   void ensureLoaded(const KernelP& k);
-  void* staging(size_t bytes);
+  void ensureStaging();
+
+  // raw device memory under the byte budget (ACCHIP_POOL_LIMIT; 0 = whatever the device has)
+  bool fakeMemory_ = false;
+  size_t limit_ = 0, rawBytes_ = 0;
+  void* rawMalloc(size_t n);
+  void rawFree(void* p, size_t n);
+  void* poolMalloc(size_t bytes, bool mayEvict);
+
+  struct Entry {
+    void* dev = nullptr;
+    size_t bytes = 0;       // of the host array
+    void* host = nullptr;
+    Status st = Status::Clean;
+    int count = 0;          // uses in progress
+    uint64_t stamp = 0;     // time of the last release
+    hipEvent_t task = nullptr;  // recorded at the last release: work queued until then
+  };
+  std::mutex tableMu_;
+  std::unordered_map<uint64_t, Entry> table_;
+  uint64_t clock_ = 0;
+  bool evictEldest();       // tableMu_ held
+  bool taskDone(Entry& e);
 };
 
 void hipCheck(hipError_t e, const char* what);

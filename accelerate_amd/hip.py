@@ -53,6 +53,14 @@ def lib():
         "acchip_poke": (C.c_int, [vp, vp, vp, C.c_size_t]),
         "acchip_peek": (C.c_int, [vp, vp, vp, C.c_size_t]),
         "acchip_stat": (C.c_longlong, [vp, C.c_char_p]),
+        "acchip_table_malloc": (C.c_int, [vp, C.c_uint64, vp, C.c_size_t, C.c_int, C.POINTER(C.c_int)]),
+        "acchip_table_use": (C.c_int, [vp, C.c_uint64, C.POINTER(vp)]),
+        "acchip_table_release": (C.c_int, [vp, C.c_uint64]),
+        "acchip_table_free": (None, [vp, C.c_uint64]),
+        "acchip_table_insert_unmanaged": (C.c_int, [vp, C.c_uint64, vp]),
+        "acchip_table_reclaim": (None, [vp]),
+        "acchip_table_status": (C.c_int, [vp, C.c_uint64]),
+        "acchip_set_clean_hook": (C.c_int, [vp, vp, vp]),
         "acchip_event_record": (C.c_int, [vp, C.POINTER(vp)]),
         "acchip_event_query": (C.c_int, [vp, C.POINTER(C.c_int)]),
         "acchip_event_sync": (C.c_int, [vp]),
@@ -115,6 +123,7 @@ def _parse_type(text):
 
 
 TRACE_FN = C.CFUNCTYPE(None, C.c_void_p, C.c_char_p, C.c_void_p)
+CLEAN_FN = C.CFUNCTYPE(None, C.c_void_p)
 
 
 class Context:
@@ -171,6 +180,44 @@ class Context:
 
     def stat(self, name):
         return lib().acchip_stat(self._h, name.encode())
+
+    # array table (Array/Remote/LRU.hs): host arrays named by an id, mirrored on the device
+    def table_malloc(self, ident, host, frozen=False):
+        """host: a C-contiguous numpy array the caller keeps alive until table_free."""
+        fresh = C.c_int()
+        _check(lib().acchip_table_malloc(self._h, ident, host.ctypes.data, host.nbytes, int(frozen), C.byref(fresh)))
+        return bool(fresh.value)
+
+    def table_use(self, ident):
+        p = C.c_void_p()
+        _check(lib().acchip_table_use(self._h, ident, C.byref(p)))
+        return p.value
+
+    def table_release(self, ident):
+        _check(lib().acchip_table_release(self._h, ident))
+
+    def table_free(self, ident):
+        lib().acchip_table_free(self._h, ident)
+
+    def table_status(self, ident):
+        return lib().acchip_table_status(self._h, ident)
+
+    def table_reclaim(self):
+        lib().acchip_table_reclaim(self._h)
+
+    def set_clean_hook(self, fn):
+        if fn is None:
+            self._clean_cb = None
+            _check(lib().acchip_set_clean_hook(self._h, None, None))
+            return
+        self._clean_cb = CLEAN_FN(lambda _user: fn())
+        _check(lib().acchip_set_clean_hook(self._h, C.cast(self._clean_cb, C.c_void_p), None))
+
+    def poke(self, devptr, host):
+        _check(lib().acchip_poke(self._h, devptr, host.ctypes.data, host.nbytes))
+
+    def peek(self, host, devptr):
+        _check(lib().acchip_peek(self._h, host.ctypes.data, devptr, host.nbytes))
 
     def sync(self):
         _check(lib().acchip_sync(self._h))

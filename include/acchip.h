@@ -44,9 +44,13 @@ const char* acchip_last_error(void);
 
 /* --- context ---------------------------------------------------------------------- */
 
-/* Create a context on HIP device `device` (one stream, default priority).  device < 0
- * creates a compile-only context.  Replaces the implicit global state of the reference
- * interpreter; a compiling backend creates this once per process. */
+/* Create a context on HIP device `device` (one stream, default priority).  device = -1
+ * creates a compile-only context.  device = -2 creates a compile-only context in which host
+ * memory stands in for device memory, so that the memory manager below (pool, array table,
+ * eviction) can be exercised without a GPU; it cannot run programs either.  Replaces the
+ * implicit global state of the reference interpreter; a compiling backend creates this once
+ * per process.  ACCHIP_POOL_LIMIT=<bytes> in the environment caps what a context takes from
+ * its device, as if the device were that small. */
 int acchip_init(int device, acchip_ctx** out);
 /* Gives up the caller's handle.  Arrays, programs and events made in the context keep it
  * alive and may be released afterwards, in any order (GHC finalisers run in any order,
@@ -67,15 +71,54 @@ void acchip_free(acchip_ctx* ctx, void* devptr);
 void acchip_purge(acchip_ctx* ctx);
 
 /* pokeRemote / peekRemote (Array/Remote/Class.hs:56-62): host <-> device copies through
- * a pinned staging buffer on the context's stream.  poke is stream-ordered and returns
+ * two pinned staging buffers in turn on the context's stream.  poke is stream-ordered and returns
  * once the host buffer may be reused; peek returns once the data is in `host`. */
 int acchip_poke(acchip_ctx* ctx, void* devptr, const void* host, size_t bytes);
 int acchip_peek(acchip_ctx* ctx, void* host, const void* devptr, size_t bytes);
 
+/* --- array table: Array/Remote/LRU.hs (on top of Table.hs and Nursery.hs) ------------- */
+
+/* The reference keeps, per host array, the device block that mirrors it, evicts the least
+ * recently used ones when the device is full and uploads them again on their next use.  Here
+ * the host array is named by an id the caller chooses (the reference's StableArray is the
+ * array's Unique, Array/Unique.hs:48-51) and described by its pinned host address and size.
+ *
+ * acchip_table_malloc: LRU.malloc (LRU.hs:207-243).  Allocates the block if the id is new
+ * (*allocated = 1) and is a no-op otherwise (*allocated = 0).  frozen != 0: the host copy
+ * stays valid (Clean), so eviction just drops the block; otherwise the device copy is taken
+ * to be the newer one (Dirty) and eviction copies it back to `host` first.  When memory runs
+ * out the ladder of Table.hs:194-206 and LRU.hs:258-303 runs: free list, device, clean hook
+ * + free list, purge + device, then eviction of the eldest arrays not in use, one by one;
+ * ACCHIP_OUT_OF_MEMORY ("Remote memory exhausted") only when all of that fails. */
+int acchip_table_malloc(acchip_ctx* ctx, uint64_t id, void* host, size_t bytes, int frozen, int* allocated);
+/* LRU.withRemote (LRU.hs:140-205), split in two: acchip_table_use pins the array and yields
+ * its device pointer, uploading the host copy again if it had been evicted (*devptr = NULL
+ * with ACCHIP_OK: the id was never allocated -- withRemote's Nothing); acchip_table_release
+ * ends the use, stamps the array as most recently used and remembers the point the stream
+ * has reached (the `Task` of LRU.hs:105-110): the array cannot be evicted before that work
+ * has finished. */
+int acchip_table_use(acchip_ctx* ctx, uint64_t id, void** devptr);
+int acchip_table_release(acchip_ctx* ctx, uint64_t id);
+/* The host array died (the finaliser of Table.insert, Table.hs:247-264): its block goes to
+ * the free list of its size.  Thread-safe; may be called from finaliser threads. */
+void acchip_table_free(acchip_ctx* ctx, uint64_t id);
+/* Table.insertUnmanaged (Table.hs:266-284): memory the caller owns; never evicted or freed. */
+int acchip_table_insert_unmanaged(acchip_ctx* ctx, uint64_t id, void* devptr);
+/* LRU.reclaim / Table.reclaim: run the clean hook and release the free lists. */
+void acchip_table_reclaim(acchip_ctx* ctx);
+/* -1: unknown id; 0 Clean, 1 Dirty, 2 Unmanaged, 3 Evicted (data Status, LRU.hs:84-89). */
+int acchip_table_status(acchip_ctx* ctx, uint64_t id);
+/* Table.clean (Table.hs:209-245) needs the caller's garbage collector: the hook is called when
+ * the device is full, before anything is purged or evicted; a Haskell caller passes performGC,
+ * whose finalisers then call acchip_table_free. */
+typedef void (*acchip_clean_fn)(void* user);
+int acchip_set_clean_hook(acchip_ctx* ctx, acchip_clean_fn fn, void* user);
+
 /* Counters with the meaning of cbits/monitoring.c:26-32 plus kernel-cache statistics.
  * names: "bytes_allocated_remote", "bytes_copied_to_remote", "bytes_copied_from_remote",
  * "bytes_evicted_from_remote", "kernels_compiled", "kernels_from_disk",
- * "kernels_from_memory", "launches", "pool_hits", "pool_misses".  Unknown name: -1. */
+ * "kernels_from_memory", "launches", "pool_hits", "pool_misses", "arrays_evicted".  Unknown
+ * name: -1. */
 long long acchip_stat(acchip_ctx* ctx, const char* name);
 
 /* --- events: `Task` of Array/Remote/LRU.hs:105-110 --------------------------------- */

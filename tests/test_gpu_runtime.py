@@ -1,5 +1,7 @@
 """Array-level control flow (evalOpenAcc, Interpreter.hs:175-259) and the device memory
 manager behind the C ABI, on the GPU."""
+import ctypes as C
+
 import numpy as np
 import pytest
 
@@ -221,3 +223,61 @@ def test_handles_may_be_released_after_shutdown():
     del ev
     del res
     assert np.array_equal(host, 2 * x + 1)
+
+
+def test_array_table_evicts_and_uploads_again_on_a_real_device(monkeypatch):
+    # the ladder of tests/test_memory_manager.py against the GPU, the budget standing in for a
+    # full device: 5 arrays of 96 MiB under 256 MiB, each read by a program between use and release
+    # (its transfers take several pieces of the staging buffers)
+    monkeypatch.setenv("ACCHIP_POOL_LIMIT", str(256 << 20))
+    ctx = hip.Context(0)
+    try:
+        n = 24 << 20
+        V = A.tarray(1, A.i32)
+        total = ctx.compile(P.fold_sum(A.i32, 1, 0))
+        host = {k: np.full(n, k, np.int32) for k in range(1, 6)}
+        lib = hip.lib()
+
+        def fold_of(k):
+            ptr = ctx.table_use(k)
+            h = C.c_void_p()
+            shp = (C.c_int64 * 1)(n)
+            bufs = (C.c_void_p * 1)(ptr)
+            hip._check(lib.acchip_array_wrap(ctx._h, 1, shp, b"i32", bufs, 1, C.byref(h)))
+            arr = hip.DeviceArray(ctx, h)
+            res = total.execute(arr)
+            ctx.table_release(k)                      # the fold may still be running: the event guards the block
+            return int(res.to_host())
+
+        for k in host:
+            assert ctx.table_malloc(k, host[k], frozen=True)
+            ctx.poke(ctx.table_use(k), host[k])
+            ctx.table_release(k)
+        # 5 x 96 MiB do not fit 256 MiB: the eldest were evicted on the way
+        assert ctx.stat("arrays_evicted") >= 3
+        assert sorted(ctx.table_status(k) for k in host).count(3) >= 3
+        for k in (1, 2, 3, 4, 5, 1, 3, 5):           # every use of an evicted array uploads it again
+            assert fold_of(k) == k * n
+        total_avail = ctx.mem_info()
+        assert total_avail[0] == 256 << 20
+        # the budget also binds what programs allocate themselves: a map over 96 MiB needs a second block of
+        # 96 MiB, which evicts table arrays; one over 200 MiB cannot be served at all
+        ptr = ctx.table_use(2)
+        ctx.table_release(2)
+        big = ctx.compile(P.map_affine())
+        with pytest.raises(hip.AccError, match="Remote memory exhausted") as e:
+            big(np.zeros(50 << 20, np.float32))
+        assert e.value.code == 3
+    finally:
+        ctx.close()
+
+
+def test_transfers_of_many_pieces_round_trip(gpu_ctx):
+    # 200 MiB + 12 bytes through the two 32 MiB staging buffers, both directions
+    x = np.random.default_rng(5).integers(0, 255, (200 << 20) + 12).astype(np.uint8)
+    p = gpu_ctx.malloc(x.nbytes)
+    gpu_ctx.poke(p, x)
+    y = np.empty_like(x)
+    gpu_ctx.peek(y, p)
+    gpu_ctx.free(p)
+    assert np.array_equal(x, y)
