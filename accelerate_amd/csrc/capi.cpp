@@ -146,6 +146,19 @@ int acchip_table_insert_unmanaged(acchip_ctx* ctx, uint64_t id, void* devptr) {
   return ACCHIP_OK;
   ACCHIP_END
 }
+int acchip_table_adopt(acchip_ctx* ctx, uint64_t id, void* host, size_t bytes, acchip_array* a, int leaf, int clean) {
+  ACCHIP_TRY
+  if (!a || a->v->k != AVal::Arr || leaf < 0 || leaf >= (int)a->v->arr->bufs.size())
+    throw Error("table adopt: no such buffer");
+  Buffer& b = *a->v->arr->bufs[leaf];
+  // a buffer the handle does not own (wrapped, or adopted before through another handle) stays
+  // where it is: the caller copies instead
+  if (!b.owned || b.ctx != ctx->ctx) throw Error("table adopt: the array does not own this buffer");
+  ctx->ctx->tableAdopt(id, host, bytes, b.p, clean != 0);
+  b.owned = false;  // from here on the table frees the block
+  return ACCHIP_OK;
+  ACCHIP_END
+}
 void acchip_table_reclaim(acchip_ctx* ctx) {
   try {
     ctx->ctx->tableReclaim();
@@ -280,7 +293,7 @@ int acchip_array_wrap(acchip_ctx* ctx, int rank, const int64_t* shape, const cha
 
 int acchip_array_new(acchip_ctx* ctx, int rank, const int64_t* shape, const char* elt_type, acchip_array** out) {
   ACCHIP_TRY
-  if (!ctx->ctx->hasDevice()) throw Error("no device");
+  if (!ctx->ctx->hasMemory()) throw Error("no device");
   DArrayP d = describe(rank, shape, elt_type);
   int64_t n = d->size();
   for (ST st : typeLeaves(d->r.elt)) {

@@ -343,6 +343,12 @@ static HValP hostEval(const Sx& e, std::vector<HValP> env, const std::vector<DAr
 Program::Program(Context& ctx, const char* text, size_t len) : ctx_(ctx) {
   root_ = parseSx(text, len);
   const Sx* f = &root_;
+  // (acchip-ir VERSION afun): the version of the term grammar; a bare term is read as version 1
+  if (f->is("acchip-ir")) {
+    if (f->size() != 3 || !f->at(1).atom) throw Error("malformed program header");
+    if (f->at(1).s != "1") throw Error("unsupported wire format version " + f->at(1).s + " (this library reads version 1)");
+    f = &f->at(2);
+  }
   TEnv tenv;
   while (f->is("alam")) {
     argTypes.push_back(lhsType(f->at(1)));

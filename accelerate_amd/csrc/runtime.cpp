@@ -348,6 +348,19 @@ void Context::tableInsertUnmanaged(uint64_t id, void* dev) {
   table_[id] = e;
 }
 
+void Context::tableAdopt(uint64_t id, void* host, size_t bytes, void* dev, bool clean) {
+  if (blockSize(dev) < bytes) throw Error("table adopt: not a live block of this context's pool, or too small");
+  std::lock_guard<std::mutex> g(tableMu_);
+  if (table_.count(id)) throw Error("table adopt: the id is already in the table");
+  Entry e;
+  e.dev = dev;
+  e.bytes = bytes;
+  e.host = host;
+  e.st = clean ? Status::Clean : Status::Dirty;
+  e.stamp = ++clock_;
+  table_.emplace(id, e);
+}
+
 void Context::tableReclaim() {
   if (cleanHook) cleanHook();
   if (device_ >= 0) (void)hipStreamSynchronize(stream_);

@@ -79,6 +79,8 @@ class Context : public std::enable_shared_from_this<Context> {
   void tableRelease(uint64_t id);              // end of the use; work queued so far may still touch it
   void tableFree(uint64_t id);                 // the host array died
   void tableInsertUnmanaged(uint64_t id, void* dev);
+  // a block of the pool (e.g. a program's result) becomes the device copy of host array `id`
+  void tableAdopt(uint64_t id, void* host, size_t bytes, void* dev, bool clean);
   void tableReclaim();                         // LRU.reclaim: clean + purge
   int tableStatus(uint64_t id);                // -1 unknown, else a Status
   std::function<void()> cleanHook;

@@ -59,6 +59,7 @@ def lib():
         "acchip_table_free": (None, [vp, C.c_uint64]),
         "acchip_table_insert_unmanaged": (C.c_int, [vp, C.c_uint64, vp]),
         "acchip_table_reclaim": (None, [vp]),
+        "acchip_table_adopt": (C.c_int, [vp, C.c_uint64, vp, C.c_size_t, vp, C.c_int, C.c_int]),
         "acchip_table_status": (C.c_int, [vp, C.c_uint64]),
         "acchip_set_clean_hook": (C.c_int, [vp, vp, vp]),
         "acchip_event_record": (C.c_int, [vp, C.POINTER(vp)]),
@@ -201,6 +202,9 @@ class Context:
 
     def table_status(self, ident):
         return lib().acchip_table_status(self._h, ident)
+
+    def table_adopt(self, ident, host, array, leaf=0, clean=False):
+        _check(lib().acchip_table_adopt(self._h, ident, host.ctypes.data, host.nbytes, array._h, leaf, int(clean)))
 
     def table_reclaim(self):
         lib().acchip_table_reclaim(self._h)
@@ -367,6 +371,8 @@ class Program:
         _check(lib().acchip_compile(ctx._h, raw, len(raw), C.byref(self._h)))
         # the library accepted the text, so it is well formed: read the argument types off it
         sx = _parse_type(self.text)
+        if isinstance(sx, tuple) and sx and sx[0] == "acchip-ir":
+            sx = sx[2]
         self.arg_types = []
         while isinstance(sx, tuple) and sx and sx[0] == "alam":
             self.arg_types.append(_lhs_type(sx[1]))

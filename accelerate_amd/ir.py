@@ -10,6 +10,9 @@ S-expression per constructor, de Bruijn indices kept exactly as in the reference
 such text from Python so that tests and benchmarks can state programs the way the
 reference's own tests do; it contains no evaluation logic.
 
+A program is wrapped as ``(acchip-ir 1 AFUN)``: the number is the version of this grammar
+(docs/WIRE.md is its normative statement; the library refuses versions it does not know).
+
 Grammar (atoms are bare words; every list starts with its constructor name):
 
   scalar type   i8 i16 i32 i64 u8 u16 u32 u64 f16 f32 f64   (Int = i64, Word = u64,
@@ -42,6 +45,8 @@ from __future__ import annotations
 import math
 import struct
 import threading
+
+WIRE_VERSION = 1   # of the grammar above; the library refuses any other
 
 # --------------------------------------------------------------------------------------
 # types
@@ -144,7 +149,8 @@ class Node:
         raise NotImplementedError
 
     def text(self):
-        return render(self.sx(0, 0))
+        """The program as it crosses the C boundary: (acchip-ir VERSION term)."""
+        return "(acchip-ir %d %s)" % (WIRE_VERSION, render(self.sx(0, 0)))
 
 
 class Raw(Node):

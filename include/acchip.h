@@ -104,6 +104,14 @@ int acchip_table_release(acchip_ctx* ctx, uint64_t id);
 void acchip_table_free(acchip_ctx* ctx, uint64_t id);
 /* Table.insertUnmanaged (Table.hs:266-284): memory the caller owns; never evicted or freed. */
 int acchip_table_insert_unmanaged(acchip_ctx* ctx, uint64_t id, void* devptr);
+/* A buffer the library allocated (leaf `leaf` of a result of acchip_execute, or of an array made
+ * by acchip_array_new) becomes the device copy of host array `id`: what a backend does when it
+ * hands a result to the caller without copying it back at once, or after it has (the reference
+ * keeps results in its table the same way, LRU.malloc followed by the kernel's writes).
+ * clean != 0: `host` already holds the same data; otherwise the device copy is the newer one and
+ * eviction writes it to `host`.  The handle stops owning the buffer and may be released; fails if
+ * it does not own it (wrapped memory, or adopted before). */
+int acchip_table_adopt(acchip_ctx* ctx, uint64_t id, void* host, size_t bytes, acchip_array* a, int leaf, int clean);
 /* LRU.reclaim / Table.reclaim: run the clean hook and release the free lists. */
 void acchip_table_reclaim(acchip_ctx* ctx);
 /* -1: unknown id; 0 Clean, 1 Dirty, 2 Unmanaged, 3 Evicted (data Status, LRU.hs:84-89). */

@@ -83,6 +83,11 @@ def parse(text):
 
     x = rd()
     assert pos == len(toks), "trailing input"
+    # a program travels as (acchip-ir VERSION afun); scalar and array terms inside tests come bare
+    if isinstance(x, list) and x and x[0] == "acchip-ir":
+        if x[1] != "1":
+            raise OracleError("unsupported wire format version " + str(x[1]))
+        x = x[2]
     return x
 
 

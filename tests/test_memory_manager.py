@@ -151,6 +151,28 @@ def test_unmanaged_arrays_are_never_evicted(small):
     assert ctx.table_status(1) == UNMANAGED
 
 
+def test_adopted_results_live_in_the_table(small):
+    # a buffer the library allocated (a program's result) becomes the device copy of a host array:
+    # the handle may go, the block stays, is evicted with copy-back like any dirty array, and comes back
+    from accelerate_amd import ir as A
+    ctx = small
+    res = ctx.empty((4 * KIB,), A.tarray(1, A.i32))                  # 16 KiB, stands for a result
+    p = hip.lib().acchip_array_buffer(res._h, 0)
+    ctx.poke(p, np.full(4 * KIB, 7, np.int32))
+    host = np.zeros(4 * KIB, np.int32)
+    ctx.table_adopt(5, host, res)
+    with pytest.raises(hip.AccError, match="does not own"):
+        ctx.table_adopt(6, host, res)                                 # once only
+    res.release()
+    assert ctx.table_use(5) == p and ctx.table_status(5) == DIRTY
+    ctx.table_release(5)
+    filler = np.zeros(14 * KIB, np.int32)                             # 56 KiB: only fits if the adopted block goes
+    ctx.table_malloc(1, filler)
+    assert ctx.table_status(5) == EVICTED and np.all(host == 7)       # its contents reached the host array
+    ctx.table_free(1)
+    assert np.all(_read(ctx, ctx.table_use(5), host) == 7)
+
+
 def test_contexts_without_memory_refuse(cc_ctx):
     assert cc_ctx.malloc(100) is None
     with pytest.raises(hip.AccError, match="no device"):

@@ -48,3 +48,27 @@ def test_all_runtime_programs_compile_and_oracle_evaluates_them(cc_ctx):
             O.run_n(prog.text(), *args, uses=[O.to_arr(u, t) for u, t in uses])
         except Exception as e:
             pytest.fail("oracle on %s: %r" % (cid, e))
+
+
+def test_benchmark_programs_print_to_the_committed_term_texts():
+    # tests/golden/terms/*.sx are the exact texts of the five configurations' terms: the golden
+    # files of any printer of the wire format (the Haskell serialiser must produce these bytes
+    # for the same programs), so the Python builder must not drift from them either
+    import os
+    from accelerate_amd import ir as A, programs as P
+    here = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "terms")
+    progs = {"c1_dotp": P.dotp(), "c2_scanl1_i64": P.scanl1_sum(A.i64), "c2_scanl1_f32": P.scanl1_sum(A.f32),
+             "c3_foldseg": P.foldseg_sum(), "c4_histogram": P.histogram(1 << 16), "c5_jacobi_step": P.jacobi_step()}
+    assert sorted(f[:-3] for f in os.listdir(here) if f.endswith(".sx")) == sorted(progs)
+    for name, prog in progs.items():
+        assert open(os.path.join(here, name + ".sx")).read() == prog.text() + "\n", name
+
+
+def test_unknown_wire_version_is_refused(cc_ctx):
+    from accelerate_amd import hip, ir as A, programs as P
+    text = P.scanl1_sum(A.i64).text()
+    assert text.startswith("(acchip-ir 1 ")
+    bare = text[len("(acchip-ir 1 "):-1]
+    assert cc_ctx.compile(bare).num_kernels == 1               # a bare term is version 1
+    with pytest.raises(hip.AccError, match="wire format version 2"):
+        cc_ctx.compile("(acchip-ir 2 " + bare + ")")
