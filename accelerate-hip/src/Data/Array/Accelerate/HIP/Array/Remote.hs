@@ -11,7 +11,7 @@
 -- by the 'Unique' of each 'UniqueArray', so that eviction, copy-back and the allocation ladder
 -- run below the C boundary.  What stays in Haskell: taking the pinned host pointer, attaching
 -- the finaliser that tells the table an array has died, and 'performGC' as the table's clean
--- hook (Table.clean, Array/Remote/Table.hs:209-245).
+-- hook (Table.clean, Array/Remote/Table.hs:313-339).
 --
 -- For code written against 'RemoteMemory' (Array/Remote/Class.hs:47-73) the instance is given
 -- as well, over a reader of the context.
@@ -62,6 +62,9 @@ theContext = unsafePerformIO $ alloca $ \out -> do
   ctx  <- peek out
   hook <- mkCleanHook (\_ -> performGC)
   check "acchip_set_clean_hook" =<< c_set_clean_hook ctx hook nullPtr
+  -- -fno-inplace, -ffast-math, -fno-fast-permute-const, -fforce-recomp, -ddump-cc / -exec / -gc reach
+  -- the library as the reference's own bit layout (cbits/flags.h:19-49)
+  check "acchip_set_flags" =<< c_set_flags ctx =<< peek cmdLineFlags
   return (Context ctx)
 
 withContext :: (Ptr Ctx -> IO a) -> IO a
@@ -78,7 +81,7 @@ check what _ = do
 ident :: UniqueArray e -> Word64
 ident = fromIntegral . hash . uniqueArrayId
 
--- | Run an action with the device copy of one host buffer (LRU.withRemote, LRU.hs:140-205).  The
+-- | Run an action with the device copy of one host buffer (LRU.withRemote, LRU.hs:140-207).  The
 -- first use allocates the block, uploads the host data and attaches the finaliser; a buffer that
 -- was evicted since is uploaded again by the table.  The block stays pinned for the duration of
 -- the action and, through the table's task, until the work queued in it has finished.

@@ -43,6 +43,13 @@ foreign import ccall unsafe "acchip_table_status"      c_table_status      :: Pt
 foreign import ccall safe   "acchip_set_clean_hook"    c_set_clean_hook    :: Ptr Ctx -> FunPtr (Ptr () -> IO ()) -> Ptr () -> IO CInt
 foreign import ccall "wrapper"                         mkCleanHook         :: (Ptr () -> IO ()) -> IO (FunPtr (Ptr () -> IO ()))
 
+foreign import ccall unsafe "acchip_set_flags"         c_set_flags         :: Ptr Ctx -> Word32 -> IO CInt
+foreign import ccall unsafe "acchip_get_flags"         c_get_flags         :: Ptr Ctx -> IO Word32
+-- the option word that accelerate's own cbits parse from the command line and $ACCELERATE_FLAGS (cbits/flags.c:44)
+foreign import ccall        "&__cmd_line_flags"        cmdLineFlags        :: Ptr Word32
+foreign import ccall unsafe "acchip_set_knob"          c_set_knob          :: Ptr Ctx -> CString -> CLLong -> IO CInt
+foreign import ccall unsafe "acchip_get_knob"          c_get_knob          :: Ptr Ctx -> CString -> Ptr CLLong -> IO CInt
+
 foreign import ccall unsafe "acchip_event_record"      c_event_record      :: Ptr Ctx -> Ptr (Ptr Event) -> IO CInt
 foreign import ccall unsafe "acchip_event_query"       c_event_query       :: Ptr Event -> Ptr CInt -> IO CInt
 foreign import ccall safe   "acchip_event_sync"        c_event_sync        :: Ptr Event -> IO CInt

@@ -180,6 +180,26 @@ int acchip_set_clean_hook(acchip_ctx* ctx, acchip_clean_fn fn, void* user) {
   ACCHIP_END
 }
 
+int acchip_set_knob(acchip_ctx* ctx, const char* name, long long value) {
+  ACCHIP_TRY
+  if (!name || !ctx->ctx->knobs.set(name, value)) throw Error(std::string("no such knob: ") + (name ? name : "(null)"));
+  return ACCHIP_OK;
+  ACCHIP_END
+}
+int acchip_get_knob(acchip_ctx* ctx, const char* name, long long* value) {
+  ACCHIP_TRY
+  if (!name || !value || !ctx->ctx->knobs.get(name, *value)) throw Error(std::string("no such knob: ") + (name ? name : "(null)"));
+  return ACCHIP_OK;
+  ACCHIP_END
+}
+int acchip_set_flags(acchip_ctx* ctx, uint32_t bitfield) {
+  ACCHIP_TRY
+  ctx->ctx->flags = bitfield;
+  return ACCHIP_OK;
+  ACCHIP_END
+}
+uint32_t acchip_get_flags(acchip_ctx* ctx) { return ctx->ctx->flags; }
+
 long long acchip_stat(acchip_ctx* ctx, const char* name) {
   Stats& s = ctx->ctx->stats;
   std::string n = name ? name : "";

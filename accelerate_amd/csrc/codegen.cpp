@@ -1381,7 +1381,7 @@ KernelSource Codegen::permute(const Sx& f, const ArrayR& dst, const Sx& p, const
   ST st = ST::I32;
   const bool single = leaves.size() == 1;
   const bool wide = single && !stIsVec(leaves[0]) && (stSize(leaves[0]) == 4 || stSize(leaves[0]) == 8);
-  if (ignoresSecond(f)) mode = "store";
+  if (ignoresSecond(f) && (fastPermuteConst || wide)) mode = "store";
   else if (wide && isCommutative(f, &op, &st) && st == leaves[0] &&
            (op == "add" ? (st != ST::F16) : (op != "mul" && stIsInt(st))))
     mode = "atomic";

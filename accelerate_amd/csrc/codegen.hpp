@@ -64,6 +64,10 @@ class Codegen {
   // aenv[i] is the type of array variable with de Bruijn index i at this node
   explicit Codegen(std::vector<ArrayR> aenv) : aenv_(std::move(aenv)) {}
 
+  // off: a permute with `const` as its combination over a product type goes through the
+  // per-element locks, so that no element mixes two sources (Language.hs:786-790)
+  bool fastPermuteConst = true;
+
   std::string addTemp(const ArrayR& r);  // returns slot name for a materialised operand
 
   KernelSource fold(const Sx& f, const Sx* seed, const Operand& src);

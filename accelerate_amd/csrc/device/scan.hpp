@@ -152,14 +152,12 @@ ACC_DEV void acc_window(const typename S::Env& env, const u64* rowDesc, i64 look
     first = mEnd ? __builtin_ctzll(mEnd) : ACC_WAVE;
     const u64 need = first >= 63 ? ~0ull : ((2ull << first) - 1);
     if ((mInv & need) == 0) break;
-#ifndef ACC_SCAN_AB_UNBOUNDED
     if (++polls >= limit) {
       if (lane == 0) __hip_atomic_store(err, 3u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
       nv = 0;
       terminal = true;
       return;
     }
-#endif
     __builtin_amdgcn_s_sleep(ACC_SCAN_SLEEP);
   }
   nv = ACC_WAVE;

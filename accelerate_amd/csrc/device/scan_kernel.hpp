@@ -8,12 +8,10 @@ acc_scan(Spec::Env env, Spec::Out out, Spec::Out tot, ScanParams p) {
   const int W = AccScanCfg<S>::W;
   const i64 gtile = acc_take_ticket(p.ticket, p.ticket_base);
   // a ticket outside the launch means that the host's count of tickets is off: touch nothing
-#ifndef ACC_SCAN_AB_NORANGE
   if (gtile < 0 || gtile >= p.rows * p.tpr) {
     if (threadIdx.x == 0) __hip_atomic_store(p.err, 3u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
     return;
   }
-#endif
   const i64 row = gtile / p.tpr;
   const i64 tile = gtile - row * p.tpr;
   const i64 n = p.n;

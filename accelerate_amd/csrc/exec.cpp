@@ -489,6 +489,7 @@ ATyP Program::prepare(const Sx& n, TEnv& tenv) {
 
   Plan& plan = plans_[&n];
   Codegen cg(aenvOf(tenv));
+  cg.fastPermuteConst = ctx_.flag(Context::kFastPermuteConst);
   auto done = [&](const ArrayR& r) {
     plan.ty = atArr(r);
     return plan.ty;
@@ -595,10 +596,10 @@ ATyP Program::prepare(const Sx& n, TEnv& tenv) {
     for (ST st : typeLeaves(srcs[0].r.elt)) simd = simd || stIsVec(st);
     if (simd) {
       plan.k = ctx_.kernel(cg.stencil(pats, outElt, *f, bnds, srcs));
-    } else if (!two && srcs[0].r.rank == 2 && !std::getenv("ACCHIP_STENCIL_NO2D")) {
+    } else if (!two && srcs[0].r.rank == 2 && !ctx_.knobs.stencil_no2d) {
       plan.k = ctx_.kernel(cg.stencil2d(pats[0], outElt, *f, bnds[0], srcs[0]));
       plan.mode = "lds2d";
-    } else if (!two && srcs[0].r.rank == 3 && !std::getenv("ACCHIP_STENCIL_NO3D")) {
+    } else if (!two && srcs[0].r.rank == 3 && !ctx_.knobs.stencil_no3d) {
       plan.k = ctx_.kernel(cg.stencil3d(pats[0], outElt, *f, bnds[0], srcs[0]));
       plan.mode = "lds3d";
     } else {
@@ -672,7 +673,7 @@ DArrayP Program::alloc(const ArrayR& r, const std::vector<int64_t>& shape) {
     b->ctx = ctx_.shared_from_this();
     b->bytes = (size_t)n * stSize(st);
     b->p = ctx_.malloc(b->bytes);
-    if (!b->p) throw Error("Remote memory exhausted");  // Array/Remote/LRU.hs:258-303
+    if (!b->p) throw Error("Remote memory exhausted");  // Array/Remote/LRU.hs:250-341
     b->owned = true;
     a->bufs.push_back(b);
   }
@@ -766,8 +767,7 @@ bool Program::streams(const KernelSource& ks, const AEnv& aenv, const std::vecto
   if (!ks.streaming) return false;
   // Measured on MI355X (256 MiB last-level cache): the non-temporal variants win once a launch
   // moves more than about twice that, and lose below.
-  const char* e = std::getenv("ACCHIP_STREAM_BYTES");  // override, for tests and tuning
-  const int64_t threshold = e ? (int64_t)std::atoll(e) : (int64_t)512 << 20;
+  const int64_t threshold = ctx_.knobs.stream_bytes;
   int64_t bytes = more;
   for (const ArraySlot& s : ks.arrays) {
     if (s.name == "out") continue;
@@ -876,8 +876,8 @@ void Program::launchMap(const KernelP& k, const AEnv& aenv, const std::vector<DA
   int64_t per = (int64_t)256 * k->meta.vec;
   const bool st = streams(k->meta, aenv, temps, arrayBytes(out));
   // a launch holds fewer than 2^32 threads: larger index spaces take several
-  const char* me = std::getenv("ACCHIP_MAP_MAX_BLOCKS");  // for tests: several launches over a small index space
-  const int64_t blocks = (n + per - 1) / per, most = me && std::atoll(me) > 0 ? std::atoll(me) : (int64_t)1 << 23;
+  // (the knob lets tests cover an index space with several launches at a small size)
+  const int64_t blocks = (n + per - 1) / per, most = std::max<int64_t>(1, ctx_.knobs.map_max_blocks);
   for (int64_t base = 0; base < blocks; base += most) {
     args.back() = (uint64_t)base;
     ctx_.launch(k, st ? "acc_map_stream" : "acc_map", (uint64_t)std::min(most, blocks - base), 256, args);
@@ -1066,9 +1066,9 @@ AValP Program::eval(const Sx& n, AEnv& aenv) {
     // (acc_map_tiled): a transposition then uses whole cache lines of its source
     const int64_t w = r.rank >= 2 ? out->shape.back() : 0;
     const int64_t cols = 8 * (int64_t)plan.k->meta.vec;
-    const char* te = std::getenv("ACCHIP_MAP_TILED");  // "0" / "1": override, for tests
+    const long long te = ctx_.knobs.map_tiled;  // 0 / 1: override, for tests
     bool tiled = h != "generate" && r.rank >= 2 && w >= cols && out->size() / w >= 32;
-    if (tiled && !te) {
+    if (tiled && te < 0) {
       // Tiles pay off only when neighbouring results read far-apart sources.  Where the index
       // function is pure index arithmetic it is evaluated here at two neighbouring result
       // indices; one that reads index arrays (a gather) keeps the linear order.
@@ -1101,8 +1101,8 @@ AValP Program::eval(const Sx& n, AEnv& aenv) {
         }
       }
     }
-    if (te && te[0] == '0') tiled = false;
-    if (te && te[0] == '1') tiled = h != "generate" && r.rank >= 2 && out->size() > 0;
+    if (te == 0) tiled = false;
+    if (te == 1) tiled = h != "generate" && r.rank >= 2 && out->size() > 0;
     if (tiled) {
       const int64_t rows = out->size() / w;
       const int64_t tilesX = (w + cols - 1) / cols, tilesY = (rows + 31) / 32;
@@ -1150,10 +1150,10 @@ AValP Program::eval(const Sx& n, AEnv& aenv) {
       // many short rows: several whole rows per workgroup (acc_fold_rows)
       const KernelSource& m = plan.k->meta;
       const int64_t rowsTile = (int64_t)m.block * m.group * m.vec;
-      const char* fr = std::getenv("ACCHIP_FOLD_ROWS");  // "0" / "1": override, for tests
+      const long long fr = ctx_.knobs.fold_rows;  // 0 / 1: override, for tests
       bool useRows = len >= 1 && rows >= 64 && 4 * len <= rowsTile;
-      if (fr && fr[0] == '0') useRows = false;
-      if (fr && fr[0] == '1') useRows = len >= 1 && len <= rowsTile;
+      if (fr == 0) useRows = false;
+      if (fr == 1) useRows = len >= 1 && len <= rowsTile;
       if (useRows) {
         const int64_t rpt = rowsTile / len;
         const int64_t groups = (rows + rpt - 1) / rpt;
@@ -1170,8 +1170,7 @@ AValP Program::eval(const Sx& n, AEnv& aenv) {
     }
     // geometry: enough workgroups to fill the chip, each with at least a few tiles of work
     const int64_t tile = (int64_t)4 * 64 * plan.k->meta.vec;
-    const char* ft = std::getenv("ACCHIP_FOLD_TARGET");  // workgroups aimed at (tuning knob)
-    const int64_t target = ft ? std::max<int64_t>(1, std::atoll(ft)) : 2048;
+    const int64_t target = std::max<int64_t>(1, ctx_.knobs.fold_target);  // workgroups aimed at
     int64_t bpr = 1;
     if (rows < target && len > 8 * tile)
       bpr = std::min((target + rows - 1) / rows, (len + 8 * tile - 1) / (8 * tile));
@@ -1208,6 +1207,7 @@ AValP Program::eval(const Sx& n, AEnv& aenv) {
                                   "scan", "permute", "stencil", "stencil2", "unit"};
     bool inPlace = false;
     for (const char* k : fresh) inPlace = inPlace || n.at(2).is(k);
+    inPlace = inPlace && ctx_.flag(Context::kInplace);  // -fno-inplace: always a copy (cbits/flags.h:25)
     if (!inPlace) {
       out = alloc(dv->arr->r, dv->arr->shape);
       for (size_t k = 0; k < out->bufs.size(); ++k) ctx_.copy(out->bufs[k]->p, dv->arr->bufs[k]->p, out->bufs[k]->bytes);
@@ -1236,20 +1236,18 @@ AValP Program::eval(const Sx& n, AEnv& aenv) {
     // Up to 128 LDS-fuls: every share re-reads the sources (from its XCD's L2), so the cost grows
     // with the destination -- 2^26 keys into 2^20 / 2^22 Int32 bins take 0.5 / 2.0 ms, which is
     // where plain global atomics are for uniform keys (2.5 ms); for Zipf keys those take 110 ms.
-    const char* pe = std::getenv("ACCHIP_PERMUTE_PARTS");
-    const int64_t maxParts = pe ? std::atoll(pe) : 128;
+    const int64_t maxParts = ctx_.knobs.permute_parts;
     // From 2^20 sources on, and from 2^12 on when every destination element receives several of
     // them (few destinations under many sources contend in the memory-side atomic units: 2^16
     // keys into 256 bins take 33 us through global atomics, 2^14 keys into 16 bins 47 us,
     // against 9 us this way).
     const bool many = cnt >= (1 << 20) || (cnt >= (1 << 12) && cnt >= 4 * out->size());
-    const char* ce = std::getenv("ACCHIP_PERMUTE_COUNT");  // "0": never take the counting kernel (tests, tuning)
-    if (plan.k->meta.permuteCount && many && out->size() <= maxParts * 65536 && !(ce && ce[0] == '0')) {
+    if (plan.k->meta.permuteCount && many && out->size() <= maxParts * 65536 && ctx_.knobs.permute_count != 0) {
       // a sum of one constant per source: 16-bit counters, 65536 destination elements per LDS-ful
       const int64_t nparts = (out->size() + 65535) / 65536;
       const int64_t part = nparts == 1 ? out->size() : 65536;
-      const char* ge = std::getenv("ACCHIP_PERMUTE_GROUPS");
-      int64_t groups = ge ? std::atoll(ge) : std::min<int64_t>(256 / nparts, cnt / 16384);
+      const long long ge = ctx_.knobs.permute_groups;
+      int64_t groups = ge > 0 ? ge : std::min<int64_t>(256 / nparts, cnt / 16384);
       groups = std::max<int64_t>(8, groups / 8 * 8);
       int64_t chunk = ((cnt + groups - 1) / groups + 3) / 4 * 4;
       args.push_back((uint64_t)cnt);
@@ -1260,9 +1258,8 @@ AValP Program::eval(const Sx& n, AEnv& aenv) {
       args.push_back((uint64_t)(uintptr_t)ctx_.errorWord());
       // The workgroups leave their counters in memory and a second launch sums them, unless there
       // are so few workgroups that adding them to the destination directly is as cheap.
-      const char* pe2 = std::getenv("ACCHIP_PERMUTE_PARTIALS");  // "0" / "1": override, for tests
       bool viaPartials = groups >= 32;
-      if (pe2) viaPartials = pe2[0] != '0';
+      if (ctx_.knobs.permute_partials >= 0) viaPartials = ctx_.knobs.permute_partials != 0;
       DArrayP partials;
       int64_t slices = 1;
       if (viaPartials) {
@@ -1285,8 +1282,8 @@ AValP Program::eval(const Sx& n, AEnv& aenv) {
       // one workgroup per CU in total (each holds 128 KiB of LDS): fewer, longer workgroups
       // mean fewer private copies to add into the destination at the end; at least 16 Ki
       // sources per workgroup
-      const char* ge = std::getenv("ACCHIP_PERMUTE_GROUPS");
-      int64_t groups = ge ? std::atoll(ge) : std::min<int64_t>(256 / nparts, cnt / 16384);
+      const long long ge = ctx_.knobs.permute_groups;
+      int64_t groups = ge > 0 ? ge : std::min<int64_t>(256 / nparts, cnt / 16384);
       groups = std::max<int64_t>(8, groups / 8 * 8);
       int64_t chunk = ((cnt + groups - 1) / groups + 3) / 4 * 4;
       args.push_back((uint64_t)cnt);
@@ -1354,8 +1351,8 @@ AValP Program::eval(const Sx& n, AEnv& aenv) {
       // a workgroup can chain several tiles down a column, prefetching the next one; with
       // 128-bit staging one tile per workgroup measured best (92 us against 103 / 107 us for
       // chains of 2 / 4 on the 8192 x 8192 Jacobi sweep), so chains are only a knob
-      const char* ce = std::getenv("ACCHIP_STENCIL_CHAIN");
-      int64_t chain = ce ? std::atoll(ce) : 1;
+      const long long ce = ctx_.knobs.stencil_chain;
+      int64_t chain = ce > 0 ? ce : 1;
       chain = std::max<int64_t>(1, std::min(chain, tilesY));
       args.push_back((uint64_t)chain);
       const int64_t chunksY = (tilesY + chain - 1) / chain;
@@ -1368,9 +1365,9 @@ AValP Program::eval(const Sx& n, AEnv& aenv) {
       const int64_t tilesY = (ext[1] + th - 1) / th, tilesX = (ext[2] + tw - 1) / tw;
       // planes per workgroup: long enough to amortise the 2*HZ planes staged before the first
       // result, short enough that the grid fills the device
-      const char* ce = std::getenv("ACCHIP_STENCIL_CHAIN");
-      int64_t chain = ce ? std::atoll(ce) : 16;  // measured on 512^3: 8..32 planes within 5 %
-      while (!ce && chain > 4 && tilesX * tilesY * ((ext[0] + chain - 1) / chain) < 2048) chain /= 2;
+      const long long ce = ctx_.knobs.stencil_chain;
+      int64_t chain = ce > 0 ? ce : 16;  // measured on 512^3: 8..32 planes within 5 %
+      while (ce <= 0 && chain > 4 && tilesX * tilesY * ((ext[0] + chain - 1) / chain) < 2048) chain /= 2;
       chain = std::max<int64_t>(1, std::min(chain, ext[0]));
       const int64_t chunksZ = (ext[0] + chain - 1) / chain;
       if (tilesX * tilesY * chunksZ > 0x7fffffffLL) throw Error("stencil: too many tiles for one launch");
@@ -1457,17 +1454,15 @@ AValP Program::eval(const Sx& n, AEnv& aenv) {
       const int64_t smallTile = (int64_t)sm.block * sm.group * sm.vec;
       small = rows * ((len + bigTile - 1) / bigTile) < 80 || len <= 2 * smallTile;
     }
-    if (const char* v = std::getenv("ACCHIP_SCAN_TILES")) {  // "large" / "small": override, for tests
-      if (std::string(v) == "large") small = false;
-      if (std::string(v) == "small" && plan.k2) small = true;
-    }
+    const long long forcedTiles = ctx_.knobs.scan_tiles;  // 1 large / 2 small / 3 rows: override, for tests
+    if (forcedTiles == 1) small = false;
+    if (forcedTiles == 2 && plan.k2) small = true;
     if (plan.k2 && len >= 1) {
       // many short rows: several whole rows per workgroup (acc_scan_rows)
       const KernelSource& sm = plan.k2->meta;
       const int64_t rowsTile = (int64_t)sm.block * sm.group * sm.vec;
-      const char* v = std::getenv("ACCHIP_SCAN_TILES");
-      const bool forced = v && std::string(v) == "rows";
-      if ((forced && len <= rowsTile) || (!v && rows >= 2 && 2 * len <= rowsTile)) {
+      const bool forced = forcedTiles == 3;
+      if ((forced && len <= rowsTile) || (forcedTiles == 0 && rows >= 2 && 2 * len <= rowsTile)) {
         const int64_t rpt = rowsTile / len;
         const int64_t groups = (rows + rpt - 1) / rpt;
         if (groups > 0x7fffffffLL) throw Error("scan: too many rows for one launch");
@@ -1500,11 +1495,9 @@ AValP Program::eval(const Sx& n, AEnv& aenv) {
     // fault injection for the test of the bounded look-back wait: a ticket base that lags the
     // counter by `skew` gives every tile a number `skew` too high, so the first tiles wait for
     // predecessors that never run, give up after `spin` polls and report
-    const char* sk = std::getenv("ACCHIP_SCAN_TEST_SKEW");
-    const char* sp = std::getenv("ACCHIP_SCAN_SPIN_LIMIT");
-    const uint64_t skew = sk ? (uint64_t)std::atoll(sk) : 0;
+    const uint64_t skew = (uint64_t)std::max<long long>(0, ctx_.knobs.scan_test_skew);
     // a legitimate wait lasts microseconds; 2^22 polls are several seconds
-    const uint64_t spin = sp && std::atoll(sp) > 0 ? (uint64_t)std::atoll(sp) : (uint64_t)1 << 22;
+    const uint64_t spin = (uint64_t)std::max<long long>(1, ctx_.knobs.scan_spin_limit);
     args.push_back((uint64_t)(st.ticketBase - skew));
     args.push_back((uint64_t)st.epoch);
     args.push_back(spin);

@@ -137,7 +137,7 @@ class Program {
   static void packOut(std::vector<uint64_t>& args, const DArray& a);
   // does a launch of ks move so much more than the last-level cache holds that its
   // streaming variant pays?  (the whole of every array it reads, plus `more` bytes)
-  static bool streams(const KernelSource& ks, const AEnv& aenv, const std::vector<DArrayP>& temps, int64_t more);
+  bool streams(const KernelSource& ks, const AEnv& aenv, const std::vector<DArrayP>& temps, int64_t more);
   void launchMap(const KernelP& k, const AEnv& aenv, const std::vector<DArrayP>& temps, DArray& out);
 };
 

@@ -5,6 +5,7 @@
 #include <sys/stat.h>
 #include <unistd.h>
 
+#include <cctype>
 #include <cstdio>
 #include <cstdlib>
 #include <cstring>
@@ -28,21 +29,99 @@ std::string libraryDir() {
   return ".";
 }
 
-static const char* kCompileOptions[] = {
-    "--offload-arch=gfx950", "-O3", "-std=c++17", "-ffp-contract=off",
-    // packed fp32 instructions are kept out of generated code on this target
-    "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"};
-static const int kNumCompileOptions = sizeof(kCompileOptions) / sizeof(kCompileOptions[0]);
+// Without fast-math a kernel computes what the scalar language says, operation by operation
+// (no contraction into fused multiply-adds), which is what bit-wise parity with a CPU needs; with
+// it the compiler may contract, reassociate and use reciprocals, as the reference's LLVM backends
+// do under -ffast-math (cbits/flags.h:26), NaN and infinity still honoured.
+static std::vector<const char*> compileOptions(bool fastMath) {
+  std::vector<const char*> o = {"--offload-arch=gfx950", "-O3", "-std=c++17",
+                                // packed fp32 instructions are kept out of generated code on this target
+                                "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"};
+  if (fastMath) {
+    for (const char* x : {"-ffp-contract=fast", "-fno-math-errno", "-fno-trapping-math", "-fno-signed-zeros",
+                          "-fassociative-math", "-freciprocal-math"})
+      o.push_back(x);
+  } else {
+    o.push_back("-ffp-contract=off");
+  }
+  return o;
+}
+
+namespace {
+struct KnobName {
+  const char* name;
+  long long Knobs::*field;
+};
+const KnobName kKnobs[] = {
+    {"stream_bytes", &Knobs::stream_bytes},       {"map_max_blocks", &Knobs::map_max_blocks},
+    {"map_tiled", &Knobs::map_tiled},             {"fold_rows", &Knobs::fold_rows},
+    {"fold_target", &Knobs::fold_target},         {"permute_parts", &Knobs::permute_parts},
+    {"permute_count", &Knobs::permute_count},     {"permute_groups", &Knobs::permute_groups},
+    {"permute_partials", &Knobs::permute_partials}, {"stencil_chain", &Knobs::stencil_chain},
+    {"stencil_no2d", &Knobs::stencil_no2d},       {"stencil_no3d", &Knobs::stencil_no3d},
+    {"scan_tiles", &Knobs::scan_tiles},           {"scan_spin_limit", &Knobs::scan_spin_limit},
+    {"scan_test_skew", &Knobs::scan_test_skew},
+};
+}  // namespace
+
+bool Knobs::set(const std::string& name, long long value) {
+  for (const KnobName& k : kKnobs)
+    if (name == k.name) {
+      this->*k.field = value;
+      return true;
+    }
+  return false;
+}
+
+bool Knobs::get(const std::string& name, long long& value) const {
+  for (const KnobName& k : kKnobs)
+    if (name == k.name) {
+      value = this->*k.field;
+      return true;
+    }
+  return false;
+}
+
+void Knobs::fromEnv() {
+  for (const KnobName& k : kKnobs) {
+    std::string env = "ACCHIP_";
+    for (const char* c = k.name; *c; ++c) env += (char)std::toupper((unsigned char)*c);
+    const char* v = std::getenv(env.c_str());
+    if (!v || !*v) continue;
+    const std::string sv = v;
+    if (sv == "large") this->*k.field = 1;  // ACCHIP_SCAN_TILES also takes the variants' names
+    else if (sv == "small") this->*k.field = 2;
+    else if (sv == "rows") this->*k.field = 3;
+    else this->*k.field = std::atoll(v);
+  }
+}
 
 Context::Context(int device) : device_(device) {
+  knobs.fromEnv();
   const char* cd = std::getenv("ACCHIP_CACHE_DIR");
   cacheDir = cd ? cd : libraryDir() + "/kcache";
   const char* fl = std::getenv("ACCHIP_FLAGS");
   if (fl) {
-    std::string f = fl;
-    dumpCC = f.find("dump-cc") != std::string::npos;
-    dumpExec = f.find("dump-exec") != std::string::npos;
-    forceRecomp = f.find("force-recomp") != std::string::npos;
+    // names as the reference spells them after -f / -d (Debug/Internal/Flags.hs:70-105)
+    static const struct { const char* name; uint32_t bit; } names[] = {
+        {"inplace", kInplace}, {"fast-math", kFastMath}, {"fast-permute-const", kFastPermuteConst},
+        {"force-recomp", kForceRecomp}, {"dump-gc", kDumpGc}, {"dump-cc", kDumpCc}, {"dump-exec", kDumpExec}};
+    // tokens separated by blanks or commas; "-f" / "-d" in front as on the reference's command
+    // line are accepted, "no-" clears the bit, unknown tokens are ignored
+    const std::string f = std::string(fl) + " ";
+    std::string tok;
+    for (char ch : f) {
+      if (ch != ' ' && ch != ',' && ch != '\t') {
+        tok += ch;
+        continue;
+      }
+      if (tok.size() > 2 && tok[0] == '-' && (tok[1] == 'f' || tok[1] == 'd')) tok = tok.substr(2);
+      const bool no = tok.compare(0, 3, "no-") == 0;
+      if (no) tok = tok.substr(3);
+      for (const auto& nm : names)
+        if (tok == nm.name) flags = no ? flags & ~nm.bit : flags | nm.bit;
+      tok.clear();
+    }
   }
   if (device_ == -2) {
     fakeMemory_ = true;
@@ -234,7 +313,7 @@ bool Context::taskDone(Entry& e) {
   return true;
 }
 
-// LRU.evictLRU (LRU.hs:273-303): the eldest array that nobody uses and whose last task has
+// LRU.evictLRU (LRU.hs:273-337): the eldest array that nobody uses and whose last task has
 // finished gives up its device block; a Dirty one is copied back to its host array first.
 bool Context::evictEldest() {
   uint64_t best = 0;
@@ -249,6 +328,8 @@ bool Context::evictEldest() {
   }
   if (!pick) return false;
   if (pick->st == Status::Dirty && pick->host) peek(pick->host, pick->dev, pick->bytes);
+  if (flag(kDumpGc))
+    fprintf(stderr, "[acchip] gc: evict %zu bytes (%s)\n", pick->bytes, pick->st == Status::Dirty ? "copied back" : "clean");
   free(pick->dev);
   stats.arraysEvicted++;
   pick->dev = nullptr;
@@ -289,7 +370,7 @@ void* Context::tableUse(uint64_t id) {
     if (e.st != Status::Evicted) throw Error("internal error: non-evicted array has been lost");
   }
   // evicted: a new block, filled from the host array, which holds the current contents
-  // (withRemote / copyBack, LRU.hs:140-186)
+  // (withRemote / copyBack, LRU.hs:140-207)
   size_t bytes;
   void* host;
   {
@@ -524,11 +605,12 @@ static void writeFile(const std::string& path, const std::string& data) {
   std::rename(tmp.c_str(), path.c_str());
 }
 
-static std::string compileHipRTC(const std::string& source, std::string& log) {
+static std::string compileHipRTC(const std::string& source, bool fastMath, std::string& log) {
+  const std::vector<const char*> opts = compileOptions(fastMath);
   hiprtcProgram prog;
   if (hiprtcCreateProgram(&prog, source.c_str(), "acchip_kernel.hip", 0, nullptr, nullptr) != HIPRTC_SUCCESS)
     throw Error("hiprtcCreateProgram failed");
-  hiprtcResult r = hiprtcCompileProgram(prog, kNumCompileOptions, kCompileOptions);
+  hiprtcResult r = hiprtcCompileProgram(prog, (int)opts.size(), const_cast<const char**>(opts.data()));
   size_t ls = 0;
   hiprtcGetProgramLogSize(prog, &ls);
   log.assign(ls, '\0');
@@ -599,7 +681,8 @@ KernelP Context::kernel(const KernelSource& ks0) {
   KernelSource ks = ks0;
   ks.source = definesPrefix() + ks0.source;
   std::string keyText = ks.source;
-  for (int i = 0; i < kNumCompileOptions; ++i) keyText += std::string("\n//opt ") + kCompileOptions[i];
+  const bool fastMath = flag(kFastMath);
+  for (const char* o : compileOptions(fastMath)) keyText += std::string("\n//opt ") + o;
   int major = 0, minor = 0;
   hiprtcVersion(&major, &minor);
   keyText += "\n//hiprtc " + std::to_string(major) + "." + std::to_string(minor);
@@ -617,10 +700,10 @@ KernelP Context::kernel(const KernelSource& ks0) {
   k->meta = ks;
   k->meta.source.clear();
   std::string path = cacheDir + "/" + hash + ".hsaco";
-  if (dumpCC) fprintf(stderr, "[acchip] kernel %s\n%s\n", hash.c_str(), ks.source.c_str());
+  if (flag(kDumpCc)) fprintf(stderr, "[acchip] kernel %s\n%s\n", hash.c_str(), ks.source.c_str());
   // a cached code object must at least look like one (an ELF image); anything else is compiled anew
   const bool fromDisk =
-      !forceRecomp && readFile(path, k->code) && k->code.size() > 64 && k->code.compare(0, 4, "\177ELF") == 0;
+      !flag(kForceRecomp) && readFile(path, k->code) && k->code.size() > 64 && k->code.compare(0, 4, "\177ELF") == 0;
   // Two threads may miss on the same key: the one that enters the table first owns the
   // compilation, the other takes its kernel.  The worker is started under the lock, after the
   // entry is in the table, so no kernel with a worker attached is ever dropped.
@@ -635,14 +718,14 @@ KernelP Context::kernel(const KernelSource& ks0) {
   } else {
     // compile on a worker thread, at most as many at once as there are cores
     stats.kernelsCompiled++;
-    const bool dump = dumpCC;
+    const bool dump = flag(kDumpCc);
     const std::string dir = cacheDir;
     k->code.clear();
     Kernel* raw = k.get();  // kept alive by kernels_ until the context goes, which waits
-    k->ready = std::async(std::launch::async, [raw, src = ks.source, path, dir, dump]() {
+    k->ready = std::async(std::launch::async, [raw, src = ks.source, path, dir, dump, fastMath]() {
                  CompileSlot slot;
                  std::string log;
-                 raw->code = compileHipRTC(src, log);
+                 raw->code = compileHipRTC(src, fastMath, log);
                  if (dump && !log.empty()) fprintf(stderr, "[acchip] hipRTC log:\n%s\n", log.c_str());
                  ::mkdir(dir.c_str(), 0777);
                  writeFile(path, raw->code);
@@ -695,7 +778,7 @@ void Context::launch(const KernelP& k, const char* fn, uint64_t grid, unsigned b
   size_t size = args.size() * sizeof(uint64_t);
   void* config[] = {HIP_LAUNCH_PARAM_BUFFER_POINTER, (void*)args.data(), HIP_LAUNCH_PARAM_BUFFER_SIZE, &size,
                     HIP_LAUNCH_PARAM_END};
-  if (dumpExec) fprintf(stderr, "[acchip] launch %s<<<%llu,%u>>> %s (%zu arg bytes)\n", fn, (unsigned long long)grid, block, k->hash.substr(0, 12).c_str(), size);
+  if (flag(kDumpExec)) fprintf(stderr, "[acchip] launch %s<<<%llu,%u>>> %s (%zu arg bytes)\n", fn, (unsigned long long)grid, block, k->hash.substr(0, 12).c_str(), size);
   hipCheck(hipModuleLaunchKernel(f, (unsigned)grid, 1, 1, block, 1, 1, 0, stream_, nullptr, config), "hipModuleLaunchKernel");
   stats.launches++;
 }

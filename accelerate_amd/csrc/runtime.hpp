@@ -39,6 +39,29 @@ struct Stats {
       arraysEvicted{0};
 };
 
+// Launch-time choices that tests and tuning override.  Read from the environment once, when
+// the context is made (ACCHIP_<NAME IN CAPITALS>), and changed afterwards only through set():
+// no launch looks at the environment.
+struct Knobs {
+  long long stream_bytes = (long long)512 << 20;  // bytes a launch must move before the non-temporal variants are taken
+  long long map_max_blocks = (long long)1 << 23;  // workgroups per launch of the map skeleton
+  long long map_tiled = -1;         // -1: decide per launch, 0 / 1: never / always tile index-permuting producers
+  long long fold_rows = -1;         // -1 / 0 / 1: the several-rows-per-workgroup fold
+  long long fold_target = 2048;     // workgroups a fold aims at
+  long long permute_parts = 128;    // LDS-fuls of destination the privatised permute accepts
+  long long permute_count = 1;      // 0: never take the counting kernel
+  long long permute_groups = 0;     // 0: decide per launch
+  long long permute_partials = -1;  // -1 / 0 / 1: counters summed by a second launch
+  long long stencil_chain = 0;      // 0: decide per launch; tiles (rank 2) or planes (rank 3) per workgroup
+  long long stencil_no2d = 0, stencil_no3d = 0;  // 1: rank-2 / rank-3 stencils through the generic skeleton
+  long long scan_tiles = 0;         // 0: decide per launch, 1 large, 2 small, 3 rows
+  long long scan_spin_limit = (long long)1 << 22;  // polls after which a tile stops waiting (seconds)
+  long long scan_test_skew = 0;     // fault injection: the ticket base passed to the kernel lags by this much
+  void fromEnv();
+  bool set(const std::string& name, long long value);  // false: no such knob
+  bool get(const std::string& name, long long& value) const;
+};
+
 // Always owned by a std::shared_ptr: device buffers, programs and events keep their
 // context alive, so handles may be released in any order (finalisers run in any order).
 class Context : public std::enable_shared_from_this<Context> {
@@ -69,7 +92,7 @@ class Context : public std::enable_shared_from_this<Context> {
   // mirror them.  An array in use (between tableUse and tableRelease) stays where it is; any
   // other may be evicted when memory runs out -- copied back to its host array first if the
   // device copy is the newer one (Dirty) -- and is uploaded again by the next tableUse.
-  // Allocation ladder (Table.hs:194-206, LRU.hs:258-303): free list of the size class, the
+  // Allocation ladder (Table.hs:194-211, LRU.hs:250-341): free list of the size class, the
   // device, the clean hook (the caller's garbage collector, whose finalisers call tableFree)
   // and the free list again, purge + the device, then eviction of the eldest unused arrays
   // one at a time, and only then failure.
@@ -115,8 +138,15 @@ class Context : public std::enable_shared_from_this<Context> {
   void preload(const KernelP& k, std::initializer_list<const char*> fns);
 
   Stats stats;
+  Knobs knobs;
   std::string cacheDir;
-  bool dumpCC = false, dumpExec = false, forceRecomp = false;
+  // The reference's option word (cbits/flags.h:19-49); only the bits below change anything here.
+  enum Flag : uint32_t {
+    kInplace = 1u << 4, kFastMath = 1u << 5, kFastPermuteConst = 1u << 6, kForceRecomp = 1u << 7,
+    kDumpGc = 1u << 18, kDumpCc = 1u << 20, kDumpExec = 1u << 23,
+  };
+  uint32_t flags = kInplace | kFastPermuteConst;
+  bool flag(Flag f) const { return (flags & f) != 0; }
 
  private:
   int device_ = -1;

@@ -62,6 +62,10 @@ def lib():
         "acchip_table_adopt": (C.c_int, [vp, C.c_uint64, vp, C.c_size_t, vp, C.c_int, C.c_int]),
         "acchip_table_status": (C.c_int, [vp, C.c_uint64]),
         "acchip_set_clean_hook": (C.c_int, [vp, vp, vp]),
+        "acchip_set_knob": (C.c_int, [vp, C.c_char_p, C.c_longlong]),
+        "acchip_get_knob": (C.c_int, [vp, C.c_char_p, C.POINTER(C.c_longlong)]),
+        "acchip_set_flags": (C.c_int, [vp, C.c_uint32]),
+        "acchip_get_flags": (C.c_uint32, [vp]),
         "acchip_event_record": (C.c_int, [vp, C.POINTER(vp)]),
         "acchip_event_query": (C.c_int, [vp, C.POINTER(C.c_int)]),
         "acchip_event_sync": (C.c_int, [vp]),
@@ -208,6 +212,29 @@ class Context:
 
     def table_reclaim(self):
         lib().acchip_table_reclaim(self._h)
+
+    # bits of the reference's option word that this backend honours (cbits/flags.h:19-49)
+    FLAG_INPLACE, FLAG_FAST_MATH, FLAG_FAST_PERMUTE_CONST, FLAG_FORCE_RECOMP = 1 << 4, 1 << 5, 1 << 6, 1 << 7
+    FLAG_DUMP_GC, FLAG_DUMP_CC, FLAG_DUMP_EXEC = 1 << 18, 1 << 20, 1 << 23
+
+    def set_knob(self, name, value):
+        """Override one launch-time choice (see acchip_set_knob); returns the previous value."""
+        old = self.knob(name)
+        _check(lib().acchip_set_knob(self._h, name.encode(), int(value)))
+        return old
+
+    def knob(self, name):
+        v = C.c_longlong(0)
+        _check(lib().acchip_get_knob(self._h, name.encode(), C.byref(v)))
+        return v.value
+
+    @property
+    def flags(self):
+        return lib().acchip_get_flags(self._h)
+
+    @flags.setter
+    def flags(self, bitfield):
+        _check(lib().acchip_set_flags(self._h, int(bitfield) & 0xFFFFFFFF))
 
     def set_clean_hook(self, fn):
         if fn is None:

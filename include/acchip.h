@@ -35,7 +35,7 @@ enum {
   ACCHIP_OK = 0,
   ACCHIP_ERROR = 1,          /* malformed program, type error, internal error: see last_error */
   ACCHIP_NO_DEVICE = 2,      /* the context owns no GPU */
-  ACCHIP_OUT_OF_MEMORY = 3,  /* "Remote memory exhausted", Array/Remote/LRU.hs:258-303 */
+  ACCHIP_OUT_OF_MEMORY = 3,  /* "Remote memory exhausted", Array/Remote/LRU.hs:250-341 */
   ACCHIP_BOUNDS = 4          /* a condition the reference reports via boundsCheck (Error.hs:33-62):
                                 empty fold1, shape mismatch in reshape, empty segment descriptor */
 };
@@ -54,20 +54,20 @@ const char* acchip_last_error(void);
 int acchip_init(int device, acchip_ctx** out);
 /* Gives up the caller's handle.  Arrays, programs and events made in the context keep it
  * alive and may be released afterwards, in any order (GHC finalisers run in any order,
- * Array/Remote/Table.hs:116-121); the device resources go with the last of them. */
+ * Array/Remote/Table.hs:116-128); the device resources go with the last of them. */
 void acchip_shutdown(acchip_ctx* ctx);
 
 /* totalRemoteMem / availableRemoteMem of class RemoteMemory (Array/Remote/Class.hs:47-73). */
 int acchip_mem_info(acchip_ctx* ctx, size_t* total, size_t* available);
 
 /* mallocRemote (Array/Remote/Class.hs:52-54): returns NULL when the device is exhausted
- * even after releasing the pool's free lists (Array/Remote/Table.hs:194-206); never
+ * even after releasing the pool's free lists (Array/Remote/Table.hs:194-211); never
  * aborts.  Thread-safe; may be called from finaliser threads. */
 void* acchip_malloc(acchip_ctx* ctx, size_t bytes);
 /* freeRemote; the block returns to the pool's free list of its size class
  * (Array/Remote/Nursery.hs:43-113). */
 void acchip_free(acchip_ctx* ctx, void* devptr);
-/* Release every block waiting in the free lists (Table.purge, Table.hs:247-284). */
+/* Release every block waiting in the free lists (Table.purge, Table.hs:341-348). */
 void acchip_purge(acchip_ctx* ctx);
 
 /* pokeRemote / peekRemote (Array/Remote/Class.hs:56-62): host <-> device copies through
@@ -83,15 +83,15 @@ int acchip_peek(acchip_ctx* ctx, void* host, const void* devptr, size_t bytes);
  * the host array is named by an id the caller chooses (the reference's StableArray is the
  * array's Unique, Array/Unique.hs:48-51) and described by its pinned host address and size.
  *
- * acchip_table_malloc: LRU.malloc (LRU.hs:207-243).  Allocates the block if the id is new
+ * acchip_table_malloc: LRU.malloc (LRU.hs:225-248).  Allocates the block if the id is new
  * (*allocated = 1) and is a no-op otherwise (*allocated = 0).  frozen != 0: the host copy
  * stays valid (Clean), so eviction just drops the block; otherwise the device copy is taken
  * to be the newer one (Dirty) and eviction copies it back to `host` first.  When memory runs
- * out the ladder of Table.hs:194-206 and LRU.hs:258-303 runs: free list, device, clean hook
+ * out the ladder of Table.hs:194-211 and LRU.hs:250-341 runs: free list, device, clean hook
  * + free list, purge + device, then eviction of the eldest arrays not in use, one by one;
  * ACCHIP_OUT_OF_MEMORY ("Remote memory exhausted") only when all of that fails. */
 int acchip_table_malloc(acchip_ctx* ctx, uint64_t id, void* host, size_t bytes, int frozen, int* allocated);
-/* LRU.withRemote (LRU.hs:140-205), split in two: acchip_table_use pins the array and yields
+/* LRU.withRemote (LRU.hs:140-207), split in two: acchip_table_use pins the array and yields
  * its device pointer, uploading the host copy again if it had been evicted (*devptr = NULL
  * with ACCHIP_OK: the id was never allocated -- withRemote's Nothing); acchip_table_release
  * ends the use, stamps the array as most recently used and remembers the point the stream
@@ -99,10 +99,10 @@ int acchip_table_malloc(acchip_ctx* ctx, uint64_t id, void* host, size_t bytes, 
  * has finished. */
 int acchip_table_use(acchip_ctx* ctx, uint64_t id, void** devptr);
 int acchip_table_release(acchip_ctx* ctx, uint64_t id);
-/* The host array died (the finaliser of Table.insert, Table.hs:247-264): its block goes to
+/* The host array died (the finaliser of Table.insert, Table.hs:247-265): its block goes to
  * the free list of its size.  Thread-safe; may be called from finaliser threads. */
 void acchip_table_free(acchip_ctx* ctx, uint64_t id);
-/* Table.insertUnmanaged (Table.hs:266-284): memory the caller owns; never evicted or freed. */
+/* Table.insertUnmanaged (Table.hs:293-311): memory the caller owns; never evicted or freed. */
 int acchip_table_insert_unmanaged(acchip_ctx* ctx, uint64_t id, void* devptr);
 /* A buffer the library allocated (leaf `leaf` of a result of acchip_execute, or of an array made
  * by acchip_array_new) becomes the device copy of host array `id`: what a backend does when it
@@ -114,13 +114,35 @@ int acchip_table_insert_unmanaged(acchip_ctx* ctx, uint64_t id, void* devptr);
 int acchip_table_adopt(acchip_ctx* ctx, uint64_t id, void* host, size_t bytes, acchip_array* a, int leaf, int clean);
 /* LRU.reclaim / Table.reclaim: run the clean hook and release the free lists. */
 void acchip_table_reclaim(acchip_ctx* ctx);
-/* -1: unknown id; 0 Clean, 1 Dirty, 2 Unmanaged, 3 Evicted (data Status, LRU.hs:84-89). */
+/* -1: unknown id; 0 Clean, 1 Dirty, 2 Unmanaged, 3 Evicted (data Status, LRU.hs:81-86). */
 int acchip_table_status(acchip_ctx* ctx, uint64_t id);
-/* Table.clean (Table.hs:209-245) needs the caller's garbage collector: the hook is called when
+/* Table.clean (Table.hs:313-339) needs the caller's garbage collector: the hook is called when
  * the device is full, before anything is purged or evicted; a Haskell caller passes performGC,
  * whose finalisers then call acchip_table_free. */
 typedef void (*acchip_clean_fn)(void* user);
 int acchip_set_clean_hook(acchip_ctx* ctx, acchip_clean_fn fn, void* user);
+
+/* Launch-time choices (kernel variant selection, thresholds) that tests and tuning override:
+ * read from the environment once, when the context is made (ACCHIP_STREAM_BYTES, ACCHIP_SCAN_TILES,
+ * ...: the name in capitals), and changed afterwards only here.  Names: stream_bytes,
+ * map_max_blocks, map_tiled, fold_rows, fold_target, permute_parts, permute_count, permute_groups,
+ * permute_partials, stencil_chain, stencil_no2d, stencil_no3d (these two take effect for programs
+ * compiled afterwards), scan_tiles (0 automatic, 1 large, 2 small, 3 rows), scan_spin_limit,
+ * scan_test_skew.  Fails for a name it does not know.  No counterpart in the reference. */
+int acchip_set_knob(acchip_ctx* ctx, const char* name, long long value);
+int acchip_get_knob(acchip_ctx* ctx, const char* name, long long* value);
+/* The reference's option word (cbits/flags.h:19-49: `__cmd_line_flags.bitfield`), of which a
+ * backend honours: inplace (bit 4: off = permute always copies its defaults), fast_math (bit 5: on =
+ * kernels compiled afterwards may contract and reassociate floating point), fast_permute_const
+ * (bit 6: see below), force_recomp (bit 7), dump_gc (bit 18), dump_cc (bit 20), dump_exec (bit 23).
+ * A context starts from the defaults of cbits/flags.c:37 (inplace and fast_permute_const on,
+ * fast_math off for bit-wise parity) adjusted by the names in $ACCHIP_FLAGS (dump-cc, dump-exec,
+ * dump-gc, force-recomp, fast-math, no-inplace, no-fast-permute-const).  fast_permute_const: a
+ * permute whose combination ignores the old value (`const`) is written with plain stores; off, its
+ * targets are taken to collide and the stores go through per-element locks, so that every element
+ * holds one complete source value (Language.hs:786-790). */
+int acchip_set_flags(acchip_ctx* ctx, uint32_t bitfield);
+uint32_t acchip_get_flags(acchip_ctx* ctx);
 
 /* Counters with the meaning of cbits/monitoring.c:26-32 plus kernel-cache statistics.
  * names: "bytes_allocated_remote", "bytes_copied_to_remote", "bytes_copied_from_remote",

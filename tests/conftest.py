@@ -29,3 +29,18 @@ def cc_ctx():
     ctx = hip.Context(-1)
     yield ctx
     ctx.close()
+
+
+@pytest.fixture
+def knobs(gpu_ctx):
+    """knobs(name, value) overrides one launch-time choice of the session's context for the
+    duration of the test."""
+    before = {}
+
+    def put(name, value):
+        old = gpu_ctx.set_knob(name, value)
+        before.setdefault(name, old)
+
+    yield put
+    for name, old in before.items():
+        gpu_ctx.set_knob(name, old)

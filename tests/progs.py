@@ -117,7 +117,7 @@ def scatter(ty=Int):
             A.min_(Int, A.untup(s1)[0], A.untup(s0)[0]))))
         src = A.delayed(A.tarray(1, ty), ext, A.lam([sh1], lambda ix: A.index(xs, A.vexp(ix))),
                         A.lam([Int], lambda i: A.linearindex(xs, i)))
-        return A.permute(A.lam([ty, A.wild(ty)], lambda x, _: x), over,
+        return A.permute(A.lam([ty, A.wild(ty)], lambda x, _: A.vexp(x)), over,
                          A.lam([sh1], lambda ix: A.just(A.sh(A.index(to, A.vexp(ix))))), src)
 
     return A.alam([A.tarray(1, Int), A.tarray(1, ty), A.tarray(1, ty)], body)

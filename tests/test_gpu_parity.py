@@ -50,11 +50,11 @@ SCANS = [(c, g) for cs, g in ((GOLDEN, True), (PARITY, False)) for c in cs if "s
 
 @pytest.mark.parametrize("tiles", ["large", "small", "rows"])
 @pytest.mark.parametrize("case", SCANS, ids=[c[0][0] for c in SCANS])
-def test_scans_with_either_tile_size(gpu_ctx, monkeypatch, case, tiles):
+def test_scans_with_either_tile_size(gpu_ctx, knobs, case, tiles):
     # rows this short take the small-tile kernel or, several rows per workgroup, the rows
     # kernel by default; every variant must agree with the reference's known answers and with
     # the oracle on every case ("rows" falls back to tiles where a row exceeds a tile)
-    monkeypatch.setenv("ACCHIP_SCAN_TILES", tiles)
+    knobs("scan_tiles", {"large": 1, "small": 2, "rows": 3}[tiles])
     (_, prog, args, last), golden = case
     got = gpu_ctx.compile(prog)(*args)
     if golden:
@@ -71,9 +71,9 @@ FOLDS = [(c, g) for cs, g in ((GOLDEN, True), (PARITY, False)) for c in cs
 
 @pytest.mark.parametrize("rows_kernel", ["0", "1"])
 @pytest.mark.parametrize("case", FOLDS, ids=[c[0][0] for c in FOLDS])
-def test_folds_with_and_without_the_rows_kernel(gpu_ctx, monkeypatch, case, rows_kernel):
+def test_folds_with_and_without_the_rows_kernel(gpu_ctx, knobs, case, rows_kernel):
     # short rows are reduced several per workgroup; both paths must give the same answers
-    monkeypatch.setenv("ACCHIP_FOLD_ROWS", rows_kernel)
+    knobs("fold_rows", int(rows_kernel))
     (_, prog, args, last), golden = case
     got = gpu_ctx.compile(prog)(*args)
     if golden:
@@ -91,11 +91,11 @@ ELEMENTWISE = [(c, g) for cs, g in ((GOLDEN, True), (PARITY, False)) for c in cs
 
 
 @pytest.mark.parametrize("case", ELEMENTWISE, ids=[c[0][0] for c in ELEMENTWISE])
-def test_streaming_variants_of_map_and_fold(gpu_ctx, monkeypatch, case):
+def test_streaming_variants_of_map_and_fold(gpu_ctx, knobs, case):
     # launches that move far more than the last-level cache holds use kernels with
     # non-temporal accesses; forced here at every size, the answers must not change
-    monkeypatch.setenv("ACCHIP_STREAM_BYTES", "0")
-    monkeypatch.setenv("ACCHIP_FOLD_ROWS", "0")
+    knobs("stream_bytes", 0)
+    knobs("fold_rows", 0)
     (_, prog, args, last), golden = case
     got = gpu_ctx.compile(prog)(*args)
     if golden:
@@ -180,12 +180,12 @@ def test_histogram_2pow26_bit_exact(gpu_ctx):
     assert got.sum(dtype=np.int64) == n and np.array_equal(got, np.bincount(keys, minlength=nbins))
 
 
-def test_map_over_several_launches(gpu_ctx, monkeypatch):
+def test_map_over_several_launches(gpu_ctx, knobs):
     # index spaces of 2^32 threads and more are covered by several launches of the map skeleton;
     # here the limit is lowered to 3 workgroups so that small arrays take that path: a plain map,
     # an indexed generate of rank 3 and a directly evaluated stencil (XCD-contiguous numbering)
-    monkeypatch.setenv("ACCHIP_MAP_MAX_BLOCKS", "3")
-    monkeypatch.setenv("ACCHIP_STENCIL_NO2D", "1")
+    knobs("map_max_blocks", 3)
+    knobs("stencil_no2d", 1)
     rng = np.random.default_rng(5)
     x = rng.standard_normal(50001).astype(np.float32)
     assert np.array_equal(gpu_ctx.compile(P.map_affine())(x), x * np.float32(2) + np.float32(1))
@@ -213,10 +213,10 @@ TILE_EDGES = sorted({t * k + d for t in (4096, 8192, 12288, 24576, 49152) for k 
 
 @pytest.mark.parametrize("tiles", ["large", "small"])
 @pytest.mark.parametrize("ty", [A.i32, A.i64])
-def test_scans_and_folds_at_tile_borders(gpu_ctx, monkeypatch, ty, tiles):
+def test_scans_and_folds_at_tile_borders(gpu_ctx, knobs, ty, tiles):
     # lengths one short of, equal to and one beyond multiples of every tile size the scans use,
     # through both tile variants: left, right and exclusive scans and the fold, against numpy
-    monkeypatch.setenv("ACCHIP_SCAN_TILES", tiles)
+    knobs("scan_tiles", {"large": 1, "small": 2, "rows": 3}[tiles])
     dt = np.int32 if ty == A.i32 else np.int64
     rng = np.random.default_rng(77)
     progs = {"scanl1": gpu_ctx.compile(P.scanl1_sum(ty)), "scanl'": gpu_ctx.compile(P.scan_prime_sum("l", ty, 1, 3)),
@@ -233,12 +233,12 @@ def test_scans_and_folds_at_tile_borders(gpu_ctx, monkeypatch, ty, tiles):
 
 
 @pytest.mark.parametrize("tiles", ["large", "small", "rows"])
-def test_scan_whose_function_indexes_a_table_at_tile_borders(gpu_ctx, monkeypatch, tiles):
+def test_scan_whose_function_indexes_a_table_at_tile_borders(gpu_ctx, knobs, tiles):
     # composition of finite-state transitions: the combination function reads tbl[a * k + b].  The
     # kernels apply it to every lane of a tile, also to lanes past the end of a row, so those lanes
     # must hold values of the array: anything else indexes outside the table.  Lengths around
     # the multiples of every tile size, against a sequential fold of the same table.
-    monkeypatch.setenv("ACCHIP_SCAN_TILES", tiles)
+    knobs("scan_tiles", {"large": 1, "small": 2, "rows": 3}[tiles])
     k = 7
     rng = np.random.default_rng(123)
     tbl = rng.integers(0, k, k * k).astype(np.int64)
@@ -272,14 +272,14 @@ def test_many_short_rows_of_a_table_scan(gpu_ctx):
 
 
 @pytest.mark.parametrize("nbins", [1 << 20, (1 << 21) + 12345, 1 << 22])
-def test_histogram_over_many_lds_fuls(gpu_ctx, monkeypatch, nbins):
+def test_histogram_over_many_lds_fuls(gpu_ctx, knobs, nbins):
     # destinations of up to 128 LDS-fuls are still combined in workgroup-private copies, one
     # range of the destination per pass; against numpy and against the plain global atomics
     keys = W.zipf_keys(1 << 22, nbins, 5)
     ref = np.bincount(keys, minlength=nbins)
     run = gpu_ctx.compile(P.histogram(nbins))
     assert np.array_equal(run(keys), ref)
-    monkeypatch.setenv("ACCHIP_PERMUTE_PARTS", "0")
+    knobs("permute_parts", 0)
     assert np.array_equal(run(keys), ref)
 
 
@@ -318,10 +318,10 @@ def test_jacobi_100_iterations_small_grid_bit_equal(gpu_ctx):
 
 @pytest.mark.parametrize("chain", [2, 3, 7])
 @pytest.mark.parametrize("bname", ["clamp", "mirror", "wrap", "constant", "function"])
-def test_stencil_tile_chains_match_oracle(gpu_ctx, monkeypatch, bname, chain):
+def test_stencil_tile_chains_match_oracle(gpu_ctx, knobs, bname, chain):
     # a workgroup that walks down several tiles of a column (forced here; by default only
     # large arrays do that), on extents that leave ragged tiles at the right and bottom edge
-    monkeypatch.setenv("ACCHIP_STENCIL_CHAIN", str(chain))
+    knobs("stencil_chain", chain)
     rng = np.random.default_rng(1000 + chain)
     b = {"constant": A.constant(A.i64, -3), "function": Q.boundary_function(A.i64, 2)}.get(bname, bname)
     for widths, shp in [([3, 3], (150, 70)), ([5, 3], (97, 130)), ([3, 5], (33, 64))]:
@@ -335,10 +335,10 @@ _ORACLE_3D = {}
 
 @pytest.mark.parametrize("chain", [1, 3, 32])
 @pytest.mark.parametrize("bname", ["clamp", "mirror", "wrap", "constant", "function"])
-def test_stencil3d_plane_ring_matches_oracle(gpu_ctx, monkeypatch, bname, chain):
+def test_stencil3d_plane_ring_matches_oracle(gpu_ctx, knobs, bname, chain):
     # rank 3: columns that march along z over a ring of planes in LDS; chains shorter than,
     # equal to and longer than the array, ragged columns at the y and x edges
-    monkeypatch.setenv("ACCHIP_STENCIL_CHAIN", str(chain))
+    knobs("stencil_chain", chain)
     b = {"constant": A.constant(A.i64, -3), "function": Q.boundary_function(A.i64, 3)}.get(bname, bname)
     for n, (widths, shp) in enumerate([([3, 3, 3], (7, 11, 140)), ([5, 3, 3], (6, 8, 128)), ([3, 5, 7], (4, 19, 30))]):
         prog = Q.stencil_weighted(A.i64, widths, b)
@@ -348,11 +348,11 @@ def test_stencil3d_plane_ring_matches_oracle(gpu_ctx, monkeypatch, bname, chain)
         assert same(gpu_ctx.compile(prog)(x), _ORACLE_3D[(bname, n)])
 
 
-def test_stencil2d_direct_evaluation_matches_oracle(monkeypatch):
+def test_stencil2d_direct_evaluation_matches_oracle():
     # the same direct evaluation forced for rank 2: rows long enough for threads whose results
     # and taps all lie inside a row (evaluated without tests) next to threads at the borders
-    monkeypatch.setenv("ACCHIP_STENCIL_NO2D", "1")
     ctx = hip.Context(0)
+    ctx.set_knob("stencil_no2d", 1)
     rng = np.random.default_rng(32)
     for bname in ("clamp", "mirror", "wrap", "constant", "function"):
         for ty, widths in ((A.i64, [3, 5]), (A.i32, [5, 3])):
@@ -363,11 +363,11 @@ def test_stencil2d_direct_evaluation_matches_oracle(monkeypatch):
     ctx.close()
 
 
-def test_stencil3d_direct_evaluation_matches_oracle(monkeypatch):
+def test_stencil3d_direct_evaluation_matches_oracle():
     # the direct (one thread per result) evaluation that ranks other than 2 and 3 use, forced
     # here for rank 3
-    monkeypatch.setenv("ACCHIP_STENCIL_NO3D", "1")
     ctx = hip.Context(0)
+    ctx.set_knob("stencil_no3d", 1)
     rng = np.random.default_rng(31)
     for bname in ("clamp", "wrap", "constant"):
         b = {"constant": A.constant(A.i64, -3)}.get(bname, bname)
@@ -378,13 +378,11 @@ def test_stencil3d_direct_evaluation_matches_oracle(monkeypatch):
 
 
 @pytest.mark.parametrize("tiled", ["0", "1", None])
-def test_transposes_with_and_without_tiles(gpu_ctx, monkeypatch, tiled):
+def test_transposes_with_and_without_tiles(gpu_ctx, knobs, tiled):
     # index-permuting producers go over 32 x 8V tiles of the result when it is large enough;
     # forced on and off here, ragged tiles included
-    if tiled is None:
-        monkeypatch.delenv("ACCHIP_MAP_TILED", raising=False)
-    else:
-        monkeypatch.setenv("ACCHIP_MAP_TILED", tiled)
+    if tiled is not None:
+        knobs("map_tiled", int(tiled))
     rng = np.random.default_rng(5)
     for ty, npt in ((A.i32, np.int32), (A.i64, np.int64)):
         run = gpu_ctx.compile(Q.transpose(ty))
@@ -433,7 +431,7 @@ def test_stencil_extent_too_short_for_its_boundary_is_a_bounds_error(gpu_ctx, ki
     assert same(gpu_ctx.compile(prog)(y), O.run_n(prog.text(), y))
 
 
-def test_lookback_wait_is_bounded_and_reported(gpu_ctx, monkeypatch):
+def test_lookback_wait_is_bounded_and_reported(gpu_ctx, knobs):
     # Fault injection from the host: the launch is told a ticket count that lags the device's by
     # 3, so its tiles take numbers 3 too high -- the first ones wait for predecessors that never
     # run, the last ones fall outside the launch.  With a poll limit of 50 every workgroup still
@@ -442,14 +440,14 @@ def test_lookback_wait_is_bounded_and_reported(gpu_ctx, monkeypatch):
     x = W.uniform_int(400_000, 3)
     run = gpu_ctx.compile(P.scanl1_sum(A.i64))
     assert np.array_equal(run(x), np.cumsum(x))
-    monkeypatch.setenv("ACCHIP_SCAN_TEST_SKEW", "3")
-    monkeypatch.setenv("ACCHIP_SCAN_SPIN_LIMIT", "50")
+    knobs("scan_test_skew", 3)
+    knobs("scan_spin_limit", 50)
     res = run.execute(gpu_ctx.to_device(x, A.tarray(1, A.i64)))
     with pytest.raises(hip.AccError, match="gave up waiting"):
         gpu_ctx.sync()
     res.release()
-    monkeypatch.delenv("ACCHIP_SCAN_TEST_SKEW")
-    monkeypatch.delenv("ACCHIP_SCAN_SPIN_LIMIT")
+    knobs("scan_test_skew", 0)
+    knobs("scan_spin_limit", 1 << 22)
     assert np.array_equal(run(x), np.cumsum(x))
 
 

@@ -127,11 +127,11 @@ def test_counting_permute_matches_bincount(gpu_ctx, keys_kind, nbins, ty, value)
 
 
 @pytest.mark.gpu
-def test_counting_permute_agrees_with_the_atomic_paths(gpu_ctx, monkeypatch):
+def test_counting_permute_agrees_with_the_atomic_paths(gpu_ctx, knobs):
     rng = np.random.default_rng(3)
     keys = np.minimum(rng.zipf(1.1, 1 << 22) - 1, 65535).astype(np.int64)
     prog = _histogram_with_drops(1 << 16)
     a = gpu_ctx.compile(prog)(keys)
-    monkeypatch.setenv("ACCHIP_PERMUTE_COUNT", "0")
+    knobs("permute_count", 0)
     b = gpu_ctx.compile(prog)(keys)
     assert np.array_equal(a, b) and np.array_equal(a, np.bincount(keys, minlength=1 << 16))

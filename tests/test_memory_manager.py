@@ -4,7 +4,7 @@ A context made with device = -2 takes host memory for device memory; ACCHIP_POOL
 it may take, so every rung of the reference's allocation ladder can be forced: free list of the
 size class, fresh block, clean hook, purge, eviction of the eldest unused array with copy-back
 of dirty data, re-upload on the next use, and failure only when everything is in use
-(Array/Remote/Table.hs:170-211, Nursery.hs:43-113, LRU.hs:140-303).  The reference ships no such
+(Array/Remote/Table.hs:170-211, Nursery.hs:43-113, LRU.hs:140-341).  The reference ships no such
 test; the same entry points run against a real device in tests/test_gpu_runtime.py.
 """
 import ctypes as C
@@ -117,7 +117,7 @@ def test_freed_arrays_feed_the_free_lists_and_unknown_ids_are_nothing(small):
     ctx.table_malloc(2, a)
     assert ctx.table_use(2) == first and ctx.stat("bytes_allocated_remote") == 32 * KIB
     ctx.table_free(2)
-    ctx.table_free(2)                                                 # twice: ignored (Table.hs:226-229)
+    ctx.table_free(2)                                                 # twice: ignored (Table.hs:253-258)
 
 
 def test_clean_hook_runs_before_anything_is_purged_or_evicted(small):
