@@ -444,13 +444,17 @@ ACC_DEV void acc_foldseg_tile_fast(const Spec::Env& env, const Spec::Out& out, c
   // the run (starting afresh at every head), bits[g] = boundaries at the run's V + 1 positions
   u32 bits[C::G];
   P agg[C::G];
+  S::Elt firstEnd[C::G];  // running value at the run's first boundary that lies behind an element
+#pragma unroll
+  for (int g = 0; g < G; ++g) {  // (all reads of the bitmap in flight together)
+    const int rel0 = (int)(wlo - tlo) + (g * ACC_WAVE + lane) * V;
+    const u32 w0 = sh_head[rel0 >> 5], w1 = sh_head[(rel0 >> 5) + 1];
+    bits[g] = (u32)((((u64)w1 << 32) | (u64)w0) >> (rel0 & 31)) & ((2u << V) - 1u);
+  }
 #pragma unroll
   for (int g = 0; g < G; ++g) {
     const i64 t0 = wlo + ((i64)g * ACC_WAVE + lane) * V;
-    const int rel0 = (int)(t0 - tlo);
-    const u32 w0 = sh_head[rel0 >> 5], w1 = sh_head[(rel0 >> 5) + 1];
-    const u32 b = (u32)((((u64)w1 << 32) | (u64)w0) >> (rel0 & 31)) & ((2u << V) - 1u);
-    bits[g] = b;
+    const u32 b = bits[g];
     i64 c = n - t0;
     c = c < 0 ? 0 : (c > V ? V : c);
     S::Elt* e = x[g];
@@ -467,18 +471,25 @@ ACC_DEV void acc_foldseg_tile_fast(const Spec::Env& env, const Spec::Out& out, c
       for (int k = 1; k < V; ++k) v = S::combine(env, v, e[k]);
       agg[g].v = v;
       agg[g].f = 0u;
+      firstEnd[g] = v;
     } else {
 #pragma unroll
       for (int k = 1; k < V; ++k) {
         if (FULL || k < c) {
           const S::Elt joined = S::combine(env, e[k - 1], e[k]);
-          if (!((b >> k) & 1u)) e[k] = joined;
+          if (!((b >> k) & 1u)) e[k] = joined;  // a head starts afresh
         } else {
           e[k] = e[k - 1];
         }
       }
       agg[g].v = e[V - 1];
       agg[g].f = (b & ((1u << V) - 1u)) != 0u ? 1u : 0u;
+      const u32 eb = b >> 1, lowest = eb & (0u - eb);  // the first end, one bit
+      S::Elt fe = e[0];
+#pragma unroll
+      for (int k = 1; k < V; ++k)
+        if ((lowest >> k) & 1u) fe = e[k];
+      firstEnd[g] = fe;
     }
   }
   // prefixes of the runs inside the wave by raking, wave totals through LDS
@@ -496,15 +507,13 @@ ACC_DEV void acc_foldseg_tile_fast(const Spec::Env& env, const Spec::Out& out, c
   const i64 perWave = (i64)G * C::GROUP;
   i64 wd = tcnt <= 0 ? 0 : (tcnt + perWave - 1) / perWave;
   const int wavesWithData = wd > ACC_SCAN_WAVES ? ACC_SCAN_WAVES : (int)wd;
-  if (w == 0) {
-    P t = sh_wave[lane < ACC_SCAN_WAVES ? lane : 0];
-    t = acc_wave_scan<SS>(env, t, lane);
-    if (lane < ACC_SCAN_WAVES) sh_wave[lane] = t;
-    if (lane == wavesWithData - 1) reinterpret_cast<P*>(p.carry)[tile] = t;
-  }
-  __syncthreads();
+  // every wave joins the totals of the waves in front of it by itself (a few combinations,
+  // the same in all lanes): a second barrier with one wave scanning in between costs more
   const bool hasWavePre = w > 0 && w <= wavesWithData;
-  const P wavePre = sh_wave[w > 0 ? w - 1 : 0];
+  P wavePre = sh_wave[0];
+  for (int i = 1; i < w; ++i) wavePre = SS::combine(env, wavePre, sh_wave[i]);
+  if (w == wavesWithData - 1 && lane == 0)
+    reinterpret_cast<P*>(p.carry)[tile] = w > 0 ? SS::combine(env, wavePre, waveTot) : waveTot;
 
   auto write = [&](int idx, const S::Elt& v) {
     const i64 j = j0 + idx;
@@ -512,33 +521,57 @@ ACC_DEV void acc_foldseg_tile_fast(const Spec::Env& env, const Spec::Out& out, c
     if (s == 0) return;  // what precedes a row's first boundary belongs to no segment
     S::store(out, row * p.nseg + s - 1, S::kSeeded ? S::combine(env, S::seed(env), v) : v);
   };
-  // the segment ends
+  // The segment ends.  Nearly every wave has, in each of its groups, a few lanes whose run
+  // holds a boundary, and hardly any lane has two: the first end of every run is therefore
+  // prepared by all lanes without a branch (the G reads of boundary numbers are in flight
+  // together; a lane without an end reads the tile's first mark and ignores it), and what is
+  // rare -- further ends in the same run, an end nothing of the tile precedes, a boundary
+  // number beyond the staging area -- goes through a branch afterwards.
+  int endIdx[C::G];
 #pragma unroll
   for (int g = 0; g < G; ++g) {
-    const u32 b = bits[g];
-    if ((b >> 1) != 0u) {  // a boundary behind one of the run's elements
-      const int rel0 = (int)(wlo - tlo) + (g * ACC_WAVE + lane) * V;
-      // everything of the tile in front of the run
-      P fore;
-      const bool hasFore = acc_join<SS>(env, hasWavePre, wavePre, g * ACC_WAVE + lane > 0, pre[g], fore);
+    const u32 eb = bits[g] >> 1;
+    const int rel0 = (int)(wlo - tlo) + (g * ACC_WAVE + lane) * V;
+    endIdx[g] = sh_first[eb != 0u ? rel0 + __builtin_ctz(eb) + 1 : 0];
+  }
 #pragma unroll
-      for (int k = 0; k < V; ++k) {
-        if ((b >> (k + 1)) & 1u) {
-          const int idx = sh_first[rel0 + k + 1];
-          const bool local = (b & ((2u << k) - 1u)) != 0u;  // the segment's head lies in this run
-          const S::Elt v = !local && hasFore ? S::combine(env, fore.v, x[g][k]) : x[g][k];
-          if (local || (hasFore && fore.f)) {
-            // finished: it waits in LDS under its boundary's number and is written with its
-            // neighbours; boundaries beyond the staging area are written at once
-            if (idx < ACC_FOLDSEG_STAGE) {
-              sh_stage[idx] = v;
-              (void)__hip_atomic_fetch_or(&sh_staged[idx >> 5], 1u << (idx & 31), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
-            } else {
-              write(idx, v);
-            }
+  for (int g = 0; g < G; ++g) {
+    const u32 b = bits[g], eb = b >> 1;
+    const bool has = eb != 0u;
+    // everything of the tile in front of the run
+    P fore;
+    const bool hasFore = acc_join<SS>(env, hasWavePre, wavePre, g * ACC_WAVE + lane > 0, pre[g], fore);
+    const bool local = (b & 1u) != 0u;  // the segment's head is the run's first position
+    const S::Elt v = !local && hasFore ? S::combine(env, fore.v, firstEnd[g]) : firstEnd[g];
+    const bool finished = local || (hasFore && fore.f);
+    const int idx = endIdx[g];
+    // finished: it waits in LDS under its boundary's number and is written with its neighbours
+    const bool stage = has && finished && idx < ACC_FOLDSEG_STAGE;
+    if (stage) {
+      sh_stage[idx] = v;
+      (void)__hip_atomic_fetch_or(&sh_staged[idx >> 5], 1u << (idx & 31), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+    }
+    if (has && (!stage || (eb & (eb - 1u)) != 0u)) {
+      if (!stage) {
+        if (finished) {
+          write(idx, v);  // beyond the staging area: written at once
+        } else {
+          sh_pend_at = idx;  // no head of the tile precedes it: at most one such end per tile
+          sh_pend = v;
+        }
+      }
+      // the run's further ends: their segments began in the run
+      const int rel0 = (int)(wlo - tlo) + (g * ACC_WAVE + lane) * V;
+      const u32 rest = eb & (eb - 1u);
+#pragma unroll
+      for (int k = 1; k < V; ++k) {
+        if ((rest >> k) & 1u) {
+          const int idx2 = sh_first[rel0 + k + 1];
+          if (idx2 < ACC_FOLDSEG_STAGE) {
+            sh_stage[idx2] = x[g][k];
+            (void)__hip_atomic_fetch_or(&sh_staged[idx2 >> 5], 1u << (idx2 & 31), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
           } else {
-            sh_pend_at = idx;  // no head of the tile precedes it: at most one such end per tile
-            sh_pend = v;
+            write(idx2, x[g][k]);
           }
         }
       }
