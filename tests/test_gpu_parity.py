@@ -84,6 +84,25 @@ def test_folds_with_and_without_the_rows_kernel(gpu_ctx, knobs, case, rows_kerne
         assert same(got, O.run_n(prog.text(), *args), exact=False, atol=last)
 
 
+def test_rows_split_over_workgroups_are_combined_in_order(gpu_ctx):
+    # rows long enough for several workgroups each, whose partial results a second launch
+    # combines: a non-commutative operator (the maximum segment sum's) shows a partial out of
+    # place; pinned by a numpy restatement
+    rng = np.random.default_rng(77)
+    for shp in [(3, 300_000), (1, 2_000_001), (17, 70_000)]:
+        x = rng.integers(-50, 50, shp).astype(np.int64)
+        run = gpu_ctx.compile(Q.mss(A.Int, 2))
+        want = []
+        for row in x:                      # Kadane's maximum segment sum, empty segment allowed
+            c = np.concatenate(([0], np.cumsum(row)))
+            want.append(int((c - np.minimum.accumulate(c)).max()))
+        for _ in range(2):
+            assert same(run(x), np.array(want, np.int64))
+    y = rng.random((2, 1 << 20), dtype=np.float32)
+    got = gpu_ctx.compile(P.fold_sum(A.f32, 2))(y)
+    assert np.allclose(got, y.astype(np.float64).sum(axis=1), rtol=1e-5)
+
+
 ELEMENTWISE = [(c, g) for cs, g in ((GOLDEN, True), (PARITY, False)) for c in cs
                if c[0].startswith(("map", "transpose", "gather", "identity", "issue185", "misc", "filter", "smvm",
                                    "radix", "fold", "dotp", "mss", "issue228"))
