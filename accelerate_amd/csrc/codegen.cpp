@@ -462,7 +462,12 @@ ValP Codegen::prim(const std::string& name, const std::vector<ST>& tys, const Va
     a = un();
     ST to = tys[1];
     if (to == ST::F16 && stIsInt(tys[0])) return bindLeaf(to, "(f16)(f32)" + a, em);  // Half goes through Float
-    return bindLeaf(to, "(" + T(to) + ")" + a, em);
+    ValP r = bindLeaf(to, "(" + T(to) + ")" + a, em);
+    if (stIsInt(tys[0]) && !stIsVec(tys[0]) && stSize(tys[0]) <= 4 && stIsInt(to) && !stIsVec(to) && stSize(to) == 8) {
+      r->narrowEx = a;
+      r->narrowSt = tys[0];
+    }
+    return r;
   }
   throw Error("unknown primitive '" + name + "'");
 }
@@ -1346,6 +1351,7 @@ KernelSource Codegen::permute(const Sx& f, const ArrayR& dst, const Sx& p, const
     if (!typeEq(valType(v), elt)) throw Error("permute: fused producer does not return the element type");
     body += fnHead("Elt", "in_linear", "const Env& env, i64 i") + returnElt(v, em) + "  }\n";
   }
+  std::string target32, preamble;
   {
     // source index -> PrimMaybe destination index = (tag, ((), dst))  (AST.hs:202)
     Emit em;
@@ -1371,10 +1377,25 @@ KernelSource Codegen::permute(const Sx& f, const ArrayR& dst, const Sx& p, const
       for (size_t d = 0; d < dd.size(); ++d)
         bad += (bad.empty() ? "" : " | ") + std::string("((u64)") + ii[d] + " >= (u64)" + dd[d] + ")";
       if (bad.empty()) bad = "false";
+      preamble = em.code;
       em.line("j = " + toIndex(shapeOf(o), m->b->b, em) + ";");
       em.line("return " + tag + " == 0 ? 0 : ((" + bad + ") ? 2 : 1);");
     }
     body += fnHead("int", "target", "const Env& env, i64 i, i64& j") + em.code + "  }\n";
+    // The same for a destination of rank 1 and fewer than 2^31 elements (the caller's to check)
+    // whose index was widened from an integer of at most 32 bits: the test stays in 32 bits.  An
+    // index below zero wraps to a number no such destination has.
+    std::vector<ValP> il;
+    valLeaves(m->b->b, il);
+    if (il.size() == 1 && !il[0]->narrowEx.empty()) {
+      std::vector<std::string> dd;
+      shapeDims(shapeOf(o), dd);
+      const ST ns = il[0]->narrowSt;
+      const std::string widened = stIsSigned(ns) ? "(u32)(i32)(" + il[0]->narrowEx + ")" : "(u32)(" + il[0]->narrowEx + ")";
+      target32 = "#define ACC_PERMUTE_TARGET32 1\n" + fnHead("int", "target32", "const Env& env, i64 i, u32& j") + preamble +
+                 "    j = " + widened + ";\n    return " + tag + " == 0 ? 0 : (j >= (u32)" + dd[0] + " ? 2 : 1);\n  }\n";
+      body += target32;
+    }
   }
   // how to combine into the destination
   std::string mode = "lock", op;
@@ -1502,6 +1523,7 @@ KernelSource Codegen::permute(const Sx& f, const ArrayR& dst, const Sx& p, const
   ks.source.insert(endSpec, u);
   ks.permuteMode = mode;
   ks.permuteCount = countable;
+  ks.permuteTarget32 = !target32.empty();
   return ks;
 }
 

@@ -20,6 +20,10 @@ struct Val {
   ST st = ST::I64;
   std::string ex;
   ValP a, b;
+  // set on a 64-bit integer leaf that is the widening of an integer of at most 32 bits: the
+  // expression and type it was widened from (a permute's index test can then stay in 32 bits)
+  std::string narrowEx;
+  ST narrowSt = ST::I64;
 };
 ValP vUnit();
 ValP vLeaf(ST st, const std::string& ex);
@@ -57,6 +61,7 @@ struct KernelSource {
   bool streaming = false;             // has acc_*_stream entry points (non-temporal variant)
   std::string permuteMode;            // permute only: "atomic", "cas", "lock", "store"
   bool permuteCount = false;          // permute only: has acc_permute_count (sum of a constant per source)
+  bool permuteTarget32 = false;       // permute only: has target32 (rank-1 destination, index widened from <= 32 bits)
 };
 
 class Codegen {

@@ -5,6 +5,7 @@ the Float32 case sums multiples of 1/4, which are exact in any order."""
 import numpy as np
 import pytest
 
+from accelerate_amd import hip
 from accelerate_amd import ir as A
 
 from . import progs as Q
@@ -135,3 +136,60 @@ def test_counting_permute_agrees_with_the_atomic_paths(gpu_ctx, knobs):
     knobs("permute_count", 0)
     b = gpu_ctx.compile(prog)(keys)
     assert np.array_equal(a, b) and np.array_equal(a, np.bincount(keys, minlength=1 << 16))
+
+
+def _histogram_of_narrow_keys(nbins, key_ty, drop_negative):
+    """The same with keys of at most 32 bits widened by fromIntegral: the index test of the
+    counting kernel then stays in 32 bits."""
+    sh1 = A.tshape(1)
+
+    def target(ix, keys):
+        k = A.index(keys, A.vexp(ix))
+        wide = A.fromintegral(key_ty, A.Int, k)
+        if not drop_negative:
+            return A.just(A.sh(wide))
+        return A.let(A.Int, wide, lambda t: A.cond(A.lt(A.Int, t, A.constI(0)), A.nothing(sh1), A.just(A.sh(t))))
+
+    return A.alam([A.tarray(1, key_ty)], lambda keys: A.permute(
+        Q.binop(A.add, A.i32),
+        A.generate(A.tarray(1, A.i32), A.sh(nbins), A.lam([sh1], lambda ix: A.const(A.i32, 0))),
+        A.lam([sh1], lambda ix: target(ix, keys)),
+        A.delayed(A.tarray(1, A.i32), A.shape(keys), A.lam([sh1], lambda ix: A.const(A.i32, 1)),
+                  A.lam([A.Int], lambda i: A.const(A.i32, 1)))))
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("key_ty,npt", [(A.i32, np.int32), (A.u32, np.uint32), (A.i16, np.int16), (A.u8, np.uint8)])
+@pytest.mark.parametrize("nbins", [200, 1 << 16, 3 * 65536 + 5])
+def test_counting_permute_with_narrow_keys(gpu_ctx, key_ty, npt, nbins):
+    # targets inside one and several ranges, in the last element, and (signed keys, dropped by the
+    # index function) below zero; pinned by numpy's bincount
+    n = (1 << 21) + 77
+    rng = np.random.default_rng(nbins + np.dtype(npt).itemsize)
+    top = min(nbins, int(np.iinfo(npt).max) + 1)
+    keys = rng.integers(0, top, n).astype(npt)
+    keys[::1000] = top - 1
+    signed = np.iinfo(npt).min < 0
+    if signed:
+        keys[rng.random(n) < 0.2] = -1
+        keys[5] = np.iinfo(npt).min
+    got = gpu_ctx.compile(_histogram_of_narrow_keys(nbins, key_ty, signed))(keys)
+    k64 = keys.astype(np.int64)
+    assert np.array_equal(got, np.bincount(k64[k64 >= 0], minlength=nbins).astype(np.int32))
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("key_ty,npt,bad", [(A.i32, np.int32, -1), (A.i32, np.int32, 1 << 16), (A.u32, np.uint32, 0xffffffff),
+                                            (A.i32, np.int32, -(1 << 31))])
+def test_narrow_key_outside_the_destination_is_an_error(gpu_ctx, key_ty, npt, bad):
+    # toIndex's bounds check (Shape.hs:98-106): reported by the next wait, nothing written for it
+    keys = np.random.default_rng(4).integers(0, 1 << 16, 1 << 21).astype(npt)
+    keys[12345] = npt(bad) if bad >= 0 else np.array(bad, np.int64).astype(npt)
+    run = gpu_ctx.compile(_histogram_of_narrow_keys(1 << 16, key_ty, False))
+    res = run.execute(gpu_ctx.to_device(keys, A.tarray(1, key_ty)))
+    with pytest.raises(hip.AccError, match="index out of bounds"):
+        gpu_ctx.sync()
+    res.release()
+    good = keys.copy()
+    good[12345] = 7
+    assert np.array_equal(run(good), np.bincount(good.astype(np.int64), minlength=1 << 16).astype(np.int32))
