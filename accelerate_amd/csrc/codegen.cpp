@@ -1382,9 +1382,10 @@ KernelSource Codegen::permute(const Sx& f, const ArrayR& dst, const Sx& p, const
       em.line("return " + tag + " == 0 ? 0 : ((" + bad + ") ? 2 : 1);");
     }
     body += fnHead("int", "target", "const Env& env, i64 i, i64& j") + em.code + "  }\n";
-    // The same for a destination of rank 1 and fewer than 2^31 elements (the caller's to check)
-    // whose index was widened from an integer of at most 32 bits: the test stays in 32 bits.  An
-    // index below zero wraps to a number no such destination has.
+    // For a destination of rank 1 and fewer than 2^31 elements (the caller's to check) whose index
+    // was widened from an integer of at most 32 bits: the index in 32 bits, untested (the skeleton
+    // compares it with the extent when it uses it, not when it is loaded); returns the Maybe's
+    // tag.  An index below zero wraps to a number no such destination has.
     std::vector<ValP> il;
     valLeaves(m->b->b, il);
     if (il.size() == 1 && !il[0]->narrowEx.empty()) {
@@ -1393,7 +1394,7 @@ KernelSource Codegen::permute(const Sx& f, const ArrayR& dst, const Sx& p, const
       const ST ns = il[0]->narrowSt;
       const std::string widened = stIsSigned(ns) ? "(u32)(i32)(" + il[0]->narrowEx + ")" : "(u32)(" + il[0]->narrowEx + ")";
       target32 = "#define ACC_PERMUTE_TARGET32 1\n" + fnHead("int", "target32", "const Env& env, i64 i, u32& j") + preamble +
-                 "    j = " + widened + ";\n    return " + tag + " == 0 ? 0 : (j >= (u32)" + dd[0] + " ? 2 : 1);\n  }\n";
+                 "    j = " + widened + ";\n    return " + tag + " != 0 ? 1 : 0;\n  }\n";
       body += target32;
     }
   }

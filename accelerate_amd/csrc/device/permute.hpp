@@ -158,6 +158,9 @@ acc_permute_lds(Spec::Env env, Spec::Out out, PermuteLdsParams p) {
 #ifndef ACC_COUNT_UNROLL
 #define ACC_COUNT_UNROLL 4
 #endif
+#ifndef ACC_COUNT_DEPTH
+#define ACC_COUNT_DEPTH 2
+#endif
 #define ACC_COUNT_WORDS 32768
 #define ACC_COUNT_T 32768u
 
@@ -186,40 +189,46 @@ ACC_DEV void acc_permute_count_body(const Spec::Env& env, const Spec::Out& out, 
   // outside either is at least span away from the range's first element.  A source that does not
   // count adds 0 to whatever word its number falls on.  (The 64-bit version below spends 17
   // vector instructions per source, this one 10: 23.8 M against 15.5 M wave instructions for 2^26
-  // sources, 58 against 54 us.)
+  // sources, 58 against 54 us.)  What is fetched is kept as it comes from the index function and
+  // examined only when it is counted: a comparison at fetch time is a wait for the load.
   (void)spare;
-  auto locate = [&](i64 i) -> u32 {
+  const u32 dstN = (u32)p.dst_n;
+  auto locate = [&](i64 i, bool& tag) -> u32 {
     u32 j;
-    const int t = S::target32(env, i, j);
-    bad = bad || t == 2;
-    return t == 0 ? NONE : (ONE ? j : j - (u32)lo);
+    tag = S::target32(env, i, j) != 0;
+    return j;
   };
-  auto bump = [&](u32 e, u32& sh) -> bool {
-    const bool valid = e < (u32)span;  // (NONE is beyond every span)
+  auto bump = [&](u32 j, bool tag, u32& sh) -> bool {
+    const u32 e = ONE ? j : j - (u32)lo;
+    const bool valid = tag && e < (u32)span;
+    bad = bad || (tag && (ONE ? e >= (u32)span : j >= dstN));
     sh = (e >> 11) & 16u;
     const u32 old = __hip_atomic_fetch_add(&cnt[e & (ACC_COUNT_WORDS - 1)], valid ? 1u << sh : 0u, __ATOMIC_RELAXED,
                                            __HIP_MEMORY_SCOPE_WORKGROUP);
     return valid && ((old >> sh) & 0xffffu) == ACC_COUNT_T - 1u;
   };
+#define ACC_COUNT_ELEMENT(j) (ONE ? (j) : (j) - (u32)lo)
 #else
   // the element of this range a source goes to, or NONE
-  auto locate = [&](i64 i) -> u32 {
+  auto locate = [&](i64 i, bool& tag) -> u32 {
     i64 j;
     const int t = S::target(env, i, j);
     bad = bad || t == 2;
+    tag = true;
     // t == 1 says 0 <= j < dst_n, which fits 32 bits (at most 128 ranges of 65536): a target below
     // this range wraps to something far beyond span
     const u32 e = (u32)j - (u32)lo;
     return t == 1 && e < (u32)span ? e : NONE;
   };
   // one more source for element e (or none, for NONE): returns whether this lane took the counter to T
-  auto bump = [&](u32 e, u32& sh) -> bool {
+  auto bump = [&](u32 e, bool, u32& sh) -> bool {
     const bool valid = e != NONE;
     sh = (e >> 11) & 16u;
     const u32 old = __hip_atomic_fetch_add(&cnt[valid ? (e & (ACC_COUNT_WORDS - 1)) : spare], valid ? 1u << sh : 0u,
                                            __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
     return ((old >> sh) & 0xffffu) == ACC_COUNT_T - 1u;  // (a spare word reads 0)
   };
+#define ACC_COUNT_ELEMENT(e) (e)
 #endif
   auto relieve = [&](u32 e, u32 sh) {
     (void)__hip_atomic_fetch_sub(&cnt[e & (ACC_COUNT_WORDS - 1)], ACC_COUNT_T << sh, __ATOMIC_RELAXED,
@@ -234,23 +243,27 @@ ACC_DEV void acc_permute_count_body(const Spec::Env& env, const Spec::Out& out, 
   // steps between two barriers: as many as handle at most T sources (a power of two)
   constexpr int kSync = ACC_COUNT_T / (ACC_PERMUTE_LDS_BLOCK * 4 * ACC_COUNT_UNROLL);
   static_assert(kSync >= 1 && (kSync & (kSync - 1)) == 0, "a step must not handle more than T sources");
-  u32 cur[ACC_COUNT_UNROLL][4], nxt[ACC_COUNT_UNROLL][4];
-  auto fetch = [&](i64 base, u32 (&e)[ACC_COUNT_UNROLL][4]) {
+  struct Batch {
+    u32 e[ACC_COUNT_UNROLL][4];
+    bool tag[ACC_COUNT_UNROLL][4];
+  };
+  Batch batch[ACC_COUNT_DEPTH];
+  auto fetch = [&](i64 base, Batch& b) {
 #pragma unroll
     for (int g = 0; g < ACC_COUNT_UNROLL; ++g) {
       const i64 i0 = base + ((i64)g * ACC_PERMUTE_LDS_BLOCK + threadIdx.x) * 4;
 #pragma unroll
-      for (int k = 0; k < 4; ++k) e[g][k] = locate(i0 + k);
+      for (int k = 0; k < 4; ++k) b.e[g][k] = locate(i0 + k, b.tag[g][k]);
     }
   };
-  auto countAll = [&](const u32 (&e)[ACC_COUNT_UNROLL][4]) {
+  auto countAll = [&](const Batch& b) {
     u32 sh[ACC_COUNT_UNROLL][4];
     bool hit[ACC_COUNT_UNROLL][4];
     bool any = false;
 #pragma unroll
     for (int g = 0; g < ACC_COUNT_UNROLL; ++g)
 #pragma unroll
-      for (int k = 0; k < 4; ++k) hit[g][k] = bump(e[g][k], sh[g][k]);
+      for (int k = 0; k < 4; ++k) hit[g][k] = bump(b.e[g][k], b.tag[g][k], sh[g][k]);
 #pragma unroll
     for (int g = 0; g < ACC_COUNT_UNROLL; ++g)
 #pragma unroll
@@ -260,27 +273,33 @@ ACC_DEV void acc_permute_count_body(const Spec::Env& env, const Spec::Out& out, 
       for (int g = 0; g < ACC_COUNT_UNROLL; ++g)
 #pragma unroll
         for (int k = 0; k < 4; ++k)
-          if (hit[g][k]) relieve(e[g][k], sh[g][k]);
+          if (hit[g][k]) relieve(ACC_COUNT_ELEMENT(b.e[g][k]), sh[g][k]);
     }
   };
   const i64 nsteps = end > begin ? (end - begin) / step : 0;  // whole steps of the chunk
-  if (nsteps > 0) fetch(begin, cur);
-  for (i64 s = 0; s < nsteps; ++s) {
-    // (the last step fetches its own sources again instead of branching around the fetch)
-    fetch(begin + (s + 1 < nsteps ? s + 1 : s) * step, nxt);
-    countAll(cur);
-    if ((s & (kSync - 1)) == kSync - 1) __syncthreads();  // (uniform: begin and end are the workgroup's)
+  auto stepBase = [&](i64 s) { return begin + (s < nsteps ? s : nsteps - 1) * step; };
+  if (nsteps > 0) {
 #pragma unroll
-    for (int g = 0; g < ACC_COUNT_UNROLL; ++g)
+    for (int d = 0; d < ACC_COUNT_DEPTH - 1; ++d) fetch(stepBase(d), batch[d]);
+  }
+  for (i64 s0 = 0; s0 < nsteps; s0 += ACC_COUNT_DEPTH) {
 #pragma unroll
-      for (int k = 0; k < 4; ++k) cur[g][k] = nxt[g][k];
+    for (int d = 0; d < ACC_COUNT_DEPTH; ++d) {
+      const i64 s = s0 + d;
+      if (s < nsteps) {  // (uniform: begin and end are the workgroup's)
+        fetch(stepBase(s + ACC_COUNT_DEPTH - 1), batch[(d + ACC_COUNT_DEPTH - 1) % ACC_COUNT_DEPTH]);
+        countAll(batch[d]);
+        if ((s & (kSync - 1)) == kSync - 1) __syncthreads();
+      }
+    }
   }
   // what is left of the chunk: fewer sources than a step, an interval of its own
   __syncthreads();
   for (i64 i = begin + nsteps * step + threadIdx.x; i < end; i += ACC_PERMUTE_LDS_BLOCK) {
     u32 sh;
-    const u32 e = locate(i);
-    if (bump(e, sh)) relieve(e, sh);
+    bool tag;
+    const u32 e = locate(i, tag);
+    if (bump(e, tag, sh)) relieve(ACC_COUNT_ELEMENT(e), sh);
   }
   __syncthreads();
   if (p.partials) {
