@@ -22,6 +22,7 @@ struct FoldParams {
   i64 n;      // extent of the innermost dimension
   i64 bpr;    // workgroups per row
   i64 chunk;  // elements per workgroup (multiple of ACC_WAVES * 64 * V)
+  i64 first;  // number of the launch's first workgroup: more workgroups than a launch holds take several
 };
 
 template <class S, class Src>
@@ -162,7 +163,7 @@ ACC_DEV void acc_fold_finish(const typename S::Env& env, const typename S::Out& 
 template <bool NT>
 ACC_DEV void acc_fold_main_body(const Spec::Env& env, const Spec::Out& out, const Spec::Out& tmp, const FoldParams& p) {
   typedef Spec S;
-  i64 bid = (i64)blockIdx.x;
+  i64 bid = p.first + (i64)blockIdx.x;
   i64 row = bid / p.bpr;
   i64 b = bid - row * p.bpr;
   i64 lo = b * p.chunk;

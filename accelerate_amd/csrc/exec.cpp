@@ -1177,7 +1177,6 @@ AValP Program::eval(const Sx& n, AEnv& aenv) {
     int64_t chunk = ((len + bpr - 1) / bpr + tile - 1) / tile * tile;
     if (chunk == 0) chunk = tile;
     bpr = std::max<int64_t>(1, (len + chunk - 1) / chunk);
-    if (rows * bpr > 0x7fffffffLL) throw Error("fold: too many rows for one launch");
     DArrayP tmp = out;
     if (bpr > 1) {
       ArrayR tr = plan.ty->r;
@@ -1191,8 +1190,15 @@ AValP Program::eval(const Sx& n, AEnv& aenv) {
     args.push_back((uint64_t)len);
     args.push_back((uint64_t)bpr);
     args.push_back((uint64_t)chunk);
+    args.push_back(0);  // FoldParams::first
     const bool st = streams(plan.k->meta, aenv, temps, 0);
-    ctx_.launch(plan.k, st ? "acc_fold_main_stream" : "acc_fold_main", (uint64_t)(rows * bpr), 256, args);
+    // a launch holds fewer than 2^32 threads: more rows than that many workgroups take several launches
+    const int64_t most = std::max<int64_t>(1, std::min<int64_t>(ctx_.knobs.fold_max_blocks, 0xffffffffLL / 256));
+    for (int64_t first = 0; first < rows * bpr; first += most) {
+      args.back() = (uint64_t)first;
+      ctx_.launch(plan.k, st ? "acc_fold_main_stream" : "acc_fold_main", (uint64_t)std::min(most, rows * bpr - first), 256, args);
+    }
+    args.back() = 0;
     if (bpr > 1) ctx_.launch(plan.k, "acc_fold_final", (uint64_t)rows, 256, args);
     return avArr(out);
   }

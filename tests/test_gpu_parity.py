@@ -84,6 +84,18 @@ def test_folds_with_and_without_the_rows_kernel(gpu_ctx, knobs, case, rows_kerne
         assert same(got, O.run_n(prog.text(), *args), exact=False, atol=last)
 
 
+def test_fold_over_several_launches(gpu_ctx, knobs):
+    # more rows than one launch holds workgroups (2^24 at 256 threads) take several launches;
+    # forced here at a small size: 1000 rows, 7 workgroups per launch, with and without rows that
+    # are split over workgroups
+    knobs("fold_max_blocks", 7)
+    knobs("fold_rows", 0)
+    rng = np.random.default_rng(78)
+    for shp in [(1000, 33), (5, 100_000)]:
+        x = rng.integers(-50, 50, shp).astype(np.int64)
+        assert same(gpu_ctx.compile(P.fold_sum(A.i64, 2))(x), x.sum(axis=1))
+
+
 def test_rows_split_over_workgroups_are_combined_in_order(gpu_ctx):
     # rows long enough for several workgroups each, whose partial results a second launch
     # combines: a non-commutative operator (the maximum segment sum's) shows a partial out of
