@@ -55,6 +55,30 @@ def counters(d):
     return {k: {c: sum(v) / len(v) for c, v in cs.items()} for k, cs in acc.items()}
 
 
+def derived(others, avg_ns, elements):
+    """What the counters say about where a kernel's time goes, per kernel that runs for at least
+    10 us: the share of their life the waves spend waiting (SQ_WAIT_ANY / SQ_WAVE_CYCLES) and
+    waiting for LDS, vector instructions per element of the workload, the time the vector
+    instructions alone would take on 1024 SIMDs at 4 cycles each and 2.4 GHz, and the share of
+    LDS cycles lost to bank conflicts."""
+    out = ["## Derived", "", "| kernel | waves waiting | waiting for LDS | VALU instr / element | VALU issue time | LDS cycles in conflict |",
+           "|---|---|---|---|---|---|"]
+    rows = 0
+    for k in sorted(others):
+        c = others[k]
+        if avg_ns.get(k, 0.0) < 10e3 or not c.get("SQ_WAVE_CYCLES"):
+            continue
+        valu = c.get("SQ_INSTS_VALU", 0.0)
+        issue_us = valu / 1024.0 * 4.0 / 2400.0
+        conflict = c.get("SQ_LDS_BANK_CONFLICT", 0.0) / c["SQ_LDS_IDX_ACTIVE"] if c.get("SQ_LDS_IDX_ACTIVE") else 0.0
+        out.append("| `%s` | %.0f %% | %.0f %% | %.1f | %.0f us of %.0f us | %.0f %% |"
+                   % (k, 100.0 * c.get("SQ_WAIT_ANY", 0.0) / c["SQ_WAVE_CYCLES"],
+                      100.0 * c.get("SQ_WAIT_INST_LDS", 0.0) / c["SQ_WAVE_CYCLES"], valu * 64.0 / elements, issue_us,
+                      avg_ns[k] / 1e3, 100.0 * conflict))
+        rows += 1
+    return out + [""] if rows else []
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("run_dir")
@@ -112,6 +136,7 @@ def main():
             for k in sorted(others):
                 lines.append("`%s`: " % k + ", ".join("%s %d" % (c, round(v)) for c, v in sorted(others[k].items())))
                 lines.append("")
+            lines += derived(others, {name: avg for name, _, avg, _, _ in ks}, e["elements"])
         if commands:
             lines += ["## Commands", "", "```", commands.replace("$ID", wid).rstrip(), "```", ""]
         open(os.path.join(a.out, wid + ".md"), "w").write("\n".join(lines))
