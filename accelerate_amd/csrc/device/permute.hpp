@@ -188,8 +188,8 @@ ACC_DEV void acc_permute_count_body(const Spec::Env& env, const Spec::Out& out, 
   // comparison decides both "inside the destination" and "inside this range", because a target
   // outside either is at least span away from the range's first element.  A source that does not
   // count adds 0 to whatever word its number falls on.  (The 64-bit version below spends 17
-  // vector instructions per source, this one 10: 23.8 M against 15.5 M wave instructions for 2^26
-  // sources, 58 against 54 us.)  What is fetched is kept as it comes from the index function and
+  // vector instructions per source, this one 10: 23.8 M against 11.7 M wave instructions for 2^26
+  // sources, 58 against 52 us.)  What is fetched is kept as it comes from the index function and
   // examined only when it is counted: a comparison at fetch time is a wait for the load.
   (void)spare;
   const u32 dstN = (u32)p.dst_n;
