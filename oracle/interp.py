@@ -17,7 +17,12 @@ What it follows (paths relative to the reference's src/Data/Array/Accelerate):
   fromFunction traversal (row-major)          Representation/Array.hs:102-122
 
 Pinned by tests/test_oracle_golden.py against the reference's own doctest outputs and
-issue regression vectors (tests/golden/*.json) and against closed forms.
+issue regression vectors (tests/golden/*.json) and against closed forms, and by
+tests/test_oracle_pins.py for what those vectors leave open: every scalar primitive on every
+type against Python's unbounded integers, numpy and struct; stencils of ranks 1-4 and stencil2
+by brute force; fold1Seg against foldl1 over split places; transform; SIMD pack / unpack.
+Parity unpinned: the last-ulp behaviour of transcendental primitives (libm here, GHC's in the
+reference), and the exact shapes of the terms the reference's fusion emits.
 
 Value representation: unit is (), pairs are 2-tuples, shapes are nested pairs
 (((), d_outer), d_inner) exactly as in the reference.  Integers are Python ints
