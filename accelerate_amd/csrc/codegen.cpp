@@ -1332,7 +1332,7 @@ static bool ignoresSecond(const Sx& f) {
   return W::allWild(g.at(1));
 }
 
-KernelSource Codegen::permute(const Sx& f, const ArrayR& dst, const Sx& p, const Operand& src) {
+KernelSource Codegen::permute(const Sx& f, const ArrayR& dst, const Sx& p, const Operand& src, const Sx* freshInit) {
   const TypeP elt = dst.elt;
   if (!typeEq(elt, src.r.elt)) throw Error("permute: source and defaults have different element types");
   auto leaves = typeLeaves(elt);
@@ -1503,7 +1503,7 @@ KernelSource Codegen::permute(const Sx& f, const ArrayR& dst, const Sx& p, const
   // A sum of one and the same constant per source (a histogram: `permute (+) zeros p ones`, the ones
   // fused into a constant producer): the skeleton only counts, in 16-bit LDS counters, and adds
   // count * constant (acc_permute_count).
-  bool countable = false;
+  bool countable = false, countSet = false;
   if (mode == "atomic" && op == "add" && stIsInt(st) && src.delayed && src.linearD.is("lam") &&
       src.linearD.at(2).is("const") && isST(src.linearD.at(2).at(1)) && parseST(src.linearD.at(2).at(1)) == st) {
     countable = true;
@@ -1512,6 +1512,13 @@ KernelSource Codegen::permute(const Sx& f, const ArrayR& dst, const Sx& p, const
     lds += "  ACC_DEV void count_flush(const Out& out, i64 j, u32 n) {\n    (void)__hip_atomic_fetch_add(&out.o0[j], (" + T +
            ")((" + U + ")n * (" + U + ")(" + literalText(st, src.linearD.at(2).at(2).s) +
            ")), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);\n  }\n";
+    if (freshInit && freshInit->is("const") && isST(freshInit->at(1)) && parseST(freshInit->at(1)) == st) {
+      countSet = true;
+      lds += "#define ACC_PERMUTE_COUNT_SET 1\n";
+      lds += "  ACC_DEV void count_set(const Out& out, i64 j, u32 n) {\n    out.o0[j] = (" + T + ")((" + U + ")(" +
+             literalText(st, freshInit->at(2).s) + ") + (" + U + ")n * (" + U + ")(" + literalText(st, src.linearD.at(2).at(2).s) +
+             "));\n  }\n";
+    }
   }
   u += "  }\n" + lds;
   // update() uses store()/combine(): it must come after them, and finish() appends load/store
@@ -1524,6 +1531,7 @@ KernelSource Codegen::permute(const Sx& f, const ArrayR& dst, const Sx& p, const
   ks.source.insert(endSpec, u);
   ks.permuteMode = mode;
   ks.permuteCount = countable;
+  ks.permuteCountSet = countSet;
   ks.permuteTarget32 = !target32.empty();
   return ks;
 }

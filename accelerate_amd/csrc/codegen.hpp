@@ -61,6 +61,7 @@ struct KernelSource {
   bool streaming = false;             // has acc_*_stream entry points (non-temporal variant)
   std::string permuteMode;            // permute only: "atomic", "cas", "lock", "store"
   bool permuteCount = false;          // permute only: has acc_permute_count (sum of a constant per source)
+  bool permuteCountSet = false;       // permute only: has count_set (defaults of one constant, written with the counts)
   bool permuteTarget32 = false;       // permute only: has target32 (rank-1 destination, index widened from <= 32 bits)
 };
 
@@ -84,7 +85,9 @@ class Codegen {
   // small: the variant for short rows (256-thread workgroups)
   KernelSource scan(const Sx& f, const Sx* seed, const Operand& src, bool right, int kind, bool small = false);
   KernelSource foldSeg(const Sx& f, const Sx* seed, const Operand& src, const Operand& seg, ST segType);
-  KernelSource permute(const Sx& f, const ArrayR& dst, const Sx& p, const Operand& src);
+  // freshInit: the literal every element of the defaults holds when they are `generate sh (\_ -> c)`
+  // (the counting variant can then write defaults and counts together), else null
+  KernelSource permute(const Sx& f, const ArrayR& dst, const Sx& p, const Operand& src, const Sx* freshInit = nullptr);
   KernelSource stencil(const std::vector<Sx>& patterns, const TypeP& outElt, const Sx& f,
                        const std::vector<Sx>& boundaries, const std::vector<Operand>& srcs);
   // rank-2 single-source stencil through LDS halo tiles

@@ -73,10 +73,13 @@ struct PermuteLdsParams {
   i64 dst_n;   // destination elements
   u32* err;    // host-visible word: 2 = a target outside the destination, 4 = a lock never came free
   // counting variant only: where the workgroups leave their counters for acc_permute_count_reduce,
-  // [nparts][groups][32768] words (null: every workgroup adds its counters to the destination itself)
+  // [nparts][groups][32768 + 16] words (null: every workgroup adds its counters to the destination itself)
   u32* partials;
   i64 groups;  // source chunks
-  i64 slices;  // the reduction sums the groups in this many slices
+  // != 0: the destination holds nothing yet; its elements all start from one constant, which
+  // acc_permute_count_reduce writes together with the counts (Spec::count_set), and nothing else
+  // may touch it
+  i64 fresh;
 };
 
 extern "C" __global__ void __launch_bounds__(ACC_PERMUTE_LDS_BLOCK)
@@ -162,6 +165,9 @@ acc_permute_lds(Spec::Env env, Spec::Out out, PermuteLdsParams p) {
 #define ACC_COUNT_DEPTH 2
 #endif
 #define ACC_COUNT_WORDS 32768
+// words a workgroup leaves for acc_permute_count_reduce: its counters, then the list of the
+// elements whose counter it relieved of ACC_COUNT_T (their number first, at most 15 of them)
+#define ACC_COUNT_STRIDE (ACC_COUNT_WORDS + 16)
 #define ACC_COUNT_T 32768u
 
 // ONE: the destination is one range (range 0 starts at element 0 and covers all of it)
@@ -174,8 +180,10 @@ ACC_DEV void acc_permute_count_body(const Spec::Env& env, const Spec::Out& out, 
   const i64 lo = range * p.part;
   const i64 hi = lo + p.part < p.dst_n ? lo + p.part : p.dst_n;
   const u64 span = (u64)(hi - lo);  // <= 65536
+  __shared__ u32 relieved[16];  // [0]: how many elements follow
   for (int i = threadIdx.x; i < (ACC_COUNT_WORDS + ACC_WAVE) / 4; i += ACC_PERMUTE_LDS_BLOCK)
     reinterpret_cast<uint4*>(cnt)[i] = make_uint4(0u, 0u, 0u, 0u);
+  if (threadIdx.x < 16) relieved[threadIdx.x] = 0u;
   __syncthreads();
   const i64 begin = chunkId * p.chunk;
   const i64 end = begin + p.chunk < p.n ? begin + p.chunk : p.n;
@@ -230,10 +238,19 @@ ACC_DEV void acc_permute_count_body(const Spec::Env& env, const Spec::Out& out, 
   };
 #define ACC_COUNT_ELEMENT(e) (e)
 #endif
+  // A destination that holds nothing yet cannot take the relief: the element is noted in the
+  // workgroup's list instead (a relief uses up ACC_COUNT_T of the workgroup's sources, and the host
+  // gives a workgroup fewer than 15 * ACC_COUNT_T), for acc_permute_count_reduce to add.
   auto relieve = [&](u32 e, u32 sh) {
     (void)__hip_atomic_fetch_sub(&cnt[e & (ACC_COUNT_WORDS - 1)], ACC_COUNT_T << sh, __ATOMIC_RELAXED,
                                  __HIP_MEMORY_SCOPE_WORKGROUP);
-    S::count_flush(out, lo + (i64)e, ACC_COUNT_T);
+    if (p.fresh) {
+      const u32 at = __hip_atomic_fetch_add(&relieved[0], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP) + 1u;
+      if (at < 16u) relieved[at] = e;
+      else __hip_atomic_store(p.err, 5u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+    } else {
+      S::count_flush(out, lo + (i64)e, ACC_COUNT_T);
+    }
   };
   // ACC_COUNT_UNROLL groups of 4 consecutive sources per thread and step.  The loop body is free
   // of branches up to the rare relief of a counter: the targets of the next step are computed
@@ -307,8 +324,10 @@ ACC_DEV void acc_permute_count_body(const Spec::Env& env, const Spec::Out& out, 
     // (2^16 counters in each of 256 workgroups: 58 us against 52 us for the counting itself); the
     // counters are left in memory as they are, 128 KiB of coalesced stores per workgroup, and summed by
     // acc_permute_count_reduce.
-    uint4* dst = reinterpret_cast<uint4*>(p.partials + ((u64)range * (u64)p.groups + (u64)chunkId) * ACC_COUNT_WORDS);
+    u32* mine = p.partials + ((u64)range * (u64)p.groups + (u64)chunkId) * ACC_COUNT_STRIDE;
+    uint4* dst = reinterpret_cast<uint4*>(mine);
     for (int i = threadIdx.x; i < ACC_COUNT_WORDS / 4; i += ACC_PERMUTE_LDS_BLOCK) dst[i] = reinterpret_cast<const uint4*>(cnt)[i];
+    if (threadIdx.x < 16) mine[ACC_COUNT_WORDS + threadIdx.x] = relieved[threadIdx.x];
   } else {
     for (int i = threadIdx.x; i < ACC_COUNT_WORDS; i += ACC_PERMUTE_LDS_BLOCK) {
       const u32 w = cnt[i];
@@ -342,8 +361,8 @@ acc_permute_count_reduce(Spec::Env env, Spec::Out out, PermuteLdsParams p) {
   const int wbase = (int)(b % blocksPerPart) * 128;
   const i64 lo = range * p.part;
   const int col = (int)threadIdx.x & 31, sl = (int)threadIdx.x >> 5;
-  const uint4* src =
-      reinterpret_cast<const uint4*>(p.partials + (u64)range * (u64)p.groups * ACC_COUNT_WORDS + wbase + col * 4);
+  const u32* mine0 = p.partials + (u64)range * (u64)p.groups * ACC_COUNT_STRIDE;
+  const uint4* src = reinterpret_cast<const uint4*>(mine0 + wbase + col * 4);
   u32 sum[8] = {0, 0, 0, 0, 0, 0, 0, 0};  // low halves of the 4 words, then their high halves
   auto take = [&](const uint4& v) {
     const u32 w[4] = {v.x, v.y, v.z, v.w};
@@ -357,11 +376,11 @@ acc_permute_count_reduce(Spec::Env env, Spec::Out out, PermuteLdsParams p) {
   for (; g + 24 < p.groups; g += 32) {
     uint4 v[4];
 #pragma unroll
-    for (int u = 0; u < 4; ++u) v[u] = src[(u64)(g + 8 * u) * (ACC_COUNT_WORDS / 4)];
+    for (int u = 0; u < 4; ++u) v[u] = src[(u64)(g + 8 * u) * (ACC_COUNT_STRIDE / 4)];
 #pragma unroll
     for (int u = 0; u < 4; ++u) take(v[u]);
   }
-  for (; g < p.groups; g += 8) take(src[(u64)g * (ACC_COUNT_WORDS / 4)]);
+  for (; g < p.groups; g += 8) take(src[(u64)g * (ACC_COUNT_STRIDE / 4)]);
   uint4* mine = reinterpret_cast<uint4*>(part + sl * 256 + col * 8);
   mine[0] = make_uint4(sum[0], sum[1], sum[2], sum[3]);
   mine[1] = make_uint4(sum[4], sum[5], sum[6], sum[7]);
@@ -370,6 +389,37 @@ acc_permute_count_reduce(Spec::Env env, Spec::Out out, PermuteLdsParams p) {
 #pragma unroll
   for (int q = 0; q < 8; ++q) total += part[q * 256 + threadIdx.x];
   const int c2 = (int)threadIdx.x >> 3, v = (int)threadIdx.x & 7;
-  if (total) S::count_flush(out, lo + (v >> 2) * ACC_COUNT_WORDS + wbase + c2 * 4 + (v & 3), total);
+  const u32 e = (u32)((v >> 2) * ACC_COUNT_WORDS + wbase + c2 * 4 + (v & 3));  // this thread's element of the range
+#ifdef ACC_PERMUTE_COUNT_SET
+  if (p.fresh) {
+    // what the workgroups relieved their counters of: a thread reads the list of one workgroup
+    // (of every 256th) and adds, in LDS, for each of its entries that falls among this
+    // workgroup's 256 elements
+    __shared__ u32 extra[256];
+    extra[threadIdx.x] = 0u;
+    __syncthreads();
+    for (i64 g = threadIdx.x; g < p.groups; g += ACC_BLOCK) {
+      const uint4* l = reinterpret_cast<const uint4*>(mine0 + (u64)g * ACC_COUNT_STRIDE + ACC_COUNT_WORDS);
+      uint4 q[4];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) q[i] = l[i];
+      const u32 w[16] = {q[0].x, q[0].y, q[0].z, q[0].w, q[1].x, q[1].y, q[1].z, q[1].w,
+                         q[2].x, q[2].y, q[2].z, q[2].w, q[3].x, q[3].y, q[3].z, q[3].w};
+#pragma unroll
+      for (int k = 1; k < 16; ++k) {
+        const u32 rel = (w[k] & (ACC_COUNT_WORDS - 1)) - (u32)wbase;  // (an element's word, from this workgroup's first)
+        if ((u32)k <= w[0] && rel < 128u)
+          (void)__hip_atomic_fetch_add(&extra[(rel >> 2) * 8 + ((w[k] >> 15) << 2) + (rel & 3u)], ACC_COUNT_T, __ATOMIC_RELAXED,
+                                       __HIP_MEMORY_SCOPE_WORKGROUP);
+      }
+    }
+    __syncthreads();
+    total += extra[threadIdx.x];
+    const i64 j = lo + (i64)e;
+    if ((i64)e < p.part && j < p.dst_n) S::count_set(out, j, total);
+    return;
+  }
+#endif
+  if (total) S::count_flush(out, lo + (i64)e, total);
 }
 #endif

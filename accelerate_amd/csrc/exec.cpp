@@ -564,7 +564,10 @@ ATyP Program::prepare(const Sx& n, TEnv& tenv) {
     ATyP dt = prepare(n.at(2), tenv);
     ArrayR dr = oneArray(dt, "permute defaults");
     Operand src = operandOf(n.at(4), cg, tenv, plan);
-    KernelSource ks = cg.permute(n.at(1), dr, n.at(3), src);
+    // defaults that are one constant everywhere (`generate sh (\_ -> c)`, what `fill` becomes)
+    const Sx* freshInit = nullptr;
+    if (n.at(2).is("generate") && n.at(2).at(3).is("lam") && n.at(2).at(3).at(2).is("const")) freshInit = &n.at(2).at(3).at(2);
+    KernelSource ks = cg.permute(n.at(1), dr, n.at(3), src, freshInit);
     plan.mode = ks.permuteMode;
     plan.k = ctx_.kernel(ks);
     return done(dr);
@@ -1205,24 +1208,65 @@ AValP Program::eval(const Sx& n, AEnv& aenv) {
   if (h == "permute") {
     // the destination starts as the defaults; a defaults operand that is not a variable is
     // a fresh array nobody else can see and is updated in place (Trafo/Fusion.hs:559-566)
-    AValP dv = eval(n.at(2), aenv);
-    if (dv->k != AVal::Arr) throw Error("permute: defaults must be a single array");
-    materialize(*dv->arr);
-    DArrayP out = dv->arr;
-    static const char* fresh[] = {"generate", "map", "zipwith", "transform", "backpermute", "fold", "foldseg",
-                                  "scan", "permute", "stencil", "stencil2", "unit"};
-    bool inPlace = false;
-    for (const char* k : fresh) inPlace = inPlace || n.at(2).is(k);
-    inPlace = inPlace && ctx_.flag(Context::kInplace);  // -fno-inplace: always a copy (cbits/flags.h:25)
-    if (!inPlace) {
-      out = alloc(dv->arr->r, dv->arr->shape);
-      for (size_t k = 0; k < out->bufs.size(); ++k) ctx_.copy(out->bufs[k]->p, dv->arr->bufs[k]->p, out->bufs[k]->bytes);
-    }
     std::vector<DArrayP> temps = evalTemps(plan.temps, aenv);
     size_t cur = 0;
     std::vector<int64_t> ext = operandExtent(n.at(4), aenv, plan, temps, cur);
     int64_t cnt = 1;
     for (int64_t d : ext) cnt *= std::max<int64_t>(d, 0);
+    // the counting kernels' launch geometry for a destination of `size` elements (false: they do not apply)
+    struct CountGeometry {
+      int64_t nparts, part, groups, chunk;
+      bool viaPartials;
+    };
+    auto countGeometry = [&](int64_t size, CountGeometry& g) {
+      const int64_t maxParts = ctx_.knobs.permute_parts;
+      const bool many = cnt >= (1 << 20) || (cnt >= (1 << 12) && cnt >= 4 * size);
+      if (!(plan.k->meta.permuteCount && many && size > 0 && size <= maxParts * 65536 && ctx_.knobs.permute_count != 0)) return false;
+      g.nparts = (size + 65535) / 65536;
+      g.part = g.nparts == 1 ? size : 65536;
+      const long long ge = ctx_.knobs.permute_groups;
+      g.groups = ge > 0 ? ge : std::min<int64_t>(256 / g.nparts, cnt / 16384);
+      g.groups = std::max<int64_t>(8, g.groups / 8 * 8);
+      g.chunk = ((cnt + g.groups - 1) / g.groups + 3) / 4 * 4;
+      // The workgroups leave their counters in memory and a second launch sums them, unless there
+      // are so few workgroups that adding them to the destination directly is as cheap.
+      g.viaPartials = g.groups >= 32;
+      if (ctx_.knobs.permute_partials >= 0) g.viaPartials = ctx_.knobs.permute_partials != 0;
+      return true;
+    };
+    // Defaults of one constant under the counting kernels with a second launch: that launch
+    // writes constant + count to every element, and the defaults are never materialised (a
+    // workgroup must then note its reliefs in a list of 15 entries: chunk < 15 * 32768).
+    DArrayP out;
+    bool freshDefaults = false;
+    if (plan.k->meta.permuteCountSet && ctx_.flag(Context::kInplace) && ctx_.knobs.permute_fresh != 0) {
+      const Sx& gen = n.at(2);
+      const Plan& gp = plans_.at(&gen);
+      const ArrayR& gr = gp.ty->r;
+      std::vector<int64_t> shp = hostShape(gen.at(2), aenv, gp, gr.rank);
+      int64_t size = 1;
+      for (int64_t d : shp) size *= std::max<int64_t>(d, 0);
+      CountGeometry g;
+      if (cnt > 0 && countGeometry(size, g) && g.viaPartials && g.chunk < 15 * 32768) {
+        out = alloc(gr, shp);
+        freshDefaults = true;
+      }
+    }
+    if (!out) {
+      AValP dv = eval(n.at(2), aenv);
+      if (dv->k != AVal::Arr) throw Error("permute: defaults must be a single array");
+      materialize(*dv->arr);
+      out = dv->arr;
+      static const char* fresh[] = {"generate", "map", "zipwith", "transform", "backpermute", "fold", "foldseg",
+                                    "scan", "permute", "stencil", "stencil2", "unit"};
+      bool inPlace = false;
+      for (const char* k : fresh) inPlace = inPlace || n.at(2).is(k);
+      inPlace = inPlace && ctx_.flag(Context::kInplace);  // -fno-inplace: always a copy (cbits/flags.h:25)
+      if (!inPlace) {
+        out = alloc(dv->arr->r, dv->arr->shape);
+        for (size_t k = 0; k < out->bufs.size(); ++k) ctx_.copy(out->bufs[k]->p, dv->arr->bufs[k]->p, out->bufs[k]->bytes);
+      }
+    }
     if (cnt == 0 || out->size() == 0) return avArr(out);
     DArrayP locks;
     if (plan.mode == "lock") {
@@ -1248,36 +1292,26 @@ AValP Program::eval(const Sx& n, AEnv& aenv) {
     // keys into 256 bins take 33 us through global atomics, 2^14 keys into 16 bins 47 us,
     // against 9 us this way).
     const bool many = cnt >= (1 << 20) || (cnt >= (1 << 12) && cnt >= 4 * out->size());
-    if (plan.k->meta.permuteCount && many && out->size() <= maxParts * 65536 && ctx_.knobs.permute_count != 0) {
+    CountGeometry cg;
+    if (countGeometry(out->size(), cg)) {
       // a sum of one constant per source: 16-bit counters, 65536 destination elements per LDS-ful
-      const int64_t nparts = (out->size() + 65535) / 65536;
-      const int64_t part = nparts == 1 ? out->size() : 65536;
-      const long long ge = ctx_.knobs.permute_groups;
-      int64_t groups = ge > 0 ? ge : std::min<int64_t>(256 / nparts, cnt / 16384);
-      groups = std::max<int64_t>(8, groups / 8 * 8);
-      int64_t chunk = ((cnt + groups - 1) / groups + 3) / 4 * 4;
+      const int64_t nparts = cg.nparts, groups = cg.groups;
       args.push_back((uint64_t)cnt);
-      args.push_back((uint64_t)chunk);
+      args.push_back((uint64_t)cg.chunk);
       args.push_back((uint64_t)nparts);
-      args.push_back((uint64_t)part);
+      args.push_back((uint64_t)cg.part);
       args.push_back((uint64_t)out->size());
       args.push_back((uint64_t)(uintptr_t)ctx_.errorWord());
-      // The workgroups leave their counters in memory and a second launch sums them, unless there
-      // are so few workgroups that adding them to the destination directly is as cheap.
-      bool viaPartials = groups >= 32;
-      if (ctx_.knobs.permute_partials >= 0) viaPartials = ctx_.knobs.permute_partials != 0;
       DArrayP partials;
-      int64_t slices = 1;
-      if (viaPartials) {
+      if (cg.viaPartials) {
         ArrayR pr;
         pr.rank = 1;
         pr.elt = tScalar(ST::U32);
-        partials = alloc(pr, {nparts * groups * 32768});
-        slices = std::max<int64_t>(1, std::min<int64_t>(16, groups / 16));
+        partials = alloc(pr, {nparts * groups * (32768 + 16)});  // ACC_COUNT_STRIDE words per workgroup
       }
       args.push_back(partials ? (uint64_t)(uintptr_t)partials->bufs[0]->p : 0);
       args.push_back((uint64_t)groups);
-      args.push_back((uint64_t)slices);
+      args.push_back(freshDefaults ? 1 : 0);
       ctx_.launch(plan.k, "acc_permute_count", (uint64_t)(groups * nparts), 1024, args);
       if (partials) ctx_.launch(plan.k, "acc_permute_count_reduce", (uint64_t)(nparts * (32768 / 128)), 256, args);
       return avArr(out);
@@ -1300,7 +1334,7 @@ AValP Program::eval(const Sx& n, AEnv& aenv) {
       args.push_back((uint64_t)(uintptr_t)ctx_.errorWord());
       args.push_back(0);  // (fields of the counting variant)
       args.push_back((uint64_t)groups);
-      args.push_back(1);
+      args.push_back(0);
       ctx_.launch(plan.k, "acc_permute_lds", (uint64_t)(groups * nparts), 1024, args);
       return avArr(out);
     }

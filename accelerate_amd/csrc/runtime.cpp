@@ -57,7 +57,7 @@ const KnobName kKnobs[] = {
     {"map_tiled", &Knobs::map_tiled},             {"fold_rows", &Knobs::fold_rows},
     {"fold_target", &Knobs::fold_target},         {"fold_max_blocks", &Knobs::fold_max_blocks},         {"permute_parts", &Knobs::permute_parts},
     {"permute_count", &Knobs::permute_count},     {"permute_groups", &Knobs::permute_groups},
-    {"permute_partials", &Knobs::permute_partials}, {"stencil_chain", &Knobs::stencil_chain},
+    {"permute_partials", &Knobs::permute_partials}, {"permute_fresh", &Knobs::permute_fresh}, {"stencil_chain", &Knobs::stencil_chain},
     {"stencil_no2d", &Knobs::stencil_no2d},       {"stencil_no3d", &Knobs::stencil_no3d},
     {"scan_tiles", &Knobs::scan_tiles},           {"scan_spin_limit", &Knobs::scan_spin_limit},
     {"scan_test_skew", &Knobs::scan_test_skew},
@@ -556,6 +556,7 @@ void Context::raiseDeviceError() {
   if (code == 2) throw Error("index out of bounds");  // permute target, Shape.hs:98-106
   if (code == 3) throw Error("internal error: a scan tile gave up waiting for its predecessors (ticket count out of step)");
   if (code == 4) throw Error("internal error: a permute update gave up waiting for its destination's lock");
+  if (code == 5) throw Error("internal error: a counting permute relieved more counters than its list holds");
   if (code != 0) throw Error("a kernel reported error " + std::to_string(code));
 }
 

@@ -53,6 +53,7 @@ struct Knobs {
   long long permute_count = 1;      // 0: never take the counting kernel
   long long permute_groups = 0;     // 0: decide per launch
   long long permute_partials = -1;  // -1 / 0 / 1: counters summed by a second launch
+  long long permute_fresh = 1;      // 0: constant defaults are materialised also where the counting kernels could write them
   long long stencil_chain = 0;      // 0: decide per launch; tiles (rank 2) or planes (rank 3) per workgroup
   long long stencil_no2d = 0, stencil_no3d = 0;  // 1: rank-2 / rank-3 stencils through the generic skeleton
   long long scan_tiles = 0;         // 0: decide per launch, 1 large, 2 small, 3 rows

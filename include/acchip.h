@@ -126,7 +126,7 @@ int acchip_set_clean_hook(acchip_ctx* ctx, acchip_clean_fn fn, void* user);
  * read from the environment once, when the context is made (ACCHIP_STREAM_BYTES, ACCHIP_SCAN_TILES,
  * ...: the name in capitals), and changed afterwards only here.  Names: stream_bytes,
  * map_max_blocks, map_tiled, fold_rows, fold_target, fold_max_blocks, permute_parts, permute_count, permute_groups,
- * permute_partials, stencil_chain, stencil_no2d, stencil_no3d (these two take effect for programs
+ * permute_partials, permute_fresh, stencil_chain, stencil_no2d, stencil_no3d (these two take effect for programs
  * compiled afterwards), scan_tiles (0 automatic, 1 large, 2 small, 3 rows), scan_spin_limit,
  * scan_test_skew.  Fails for a name it does not know.  No counterpart in the reference. */
 int acchip_set_knob(acchip_ctx* ctx, const char* name, long long value);

@@ -193,3 +193,45 @@ def test_narrow_key_outside_the_destination_is_an_error(gpu_ctx, key_ty, npt, ba
     good = keys.copy()
     good[12345] = 7
     assert np.array_equal(run(good), np.bincount(good.astype(np.int64), minlength=1 << 16).astype(np.int32))
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("fresh", [1, 0])
+@pytest.mark.parametrize("keys_kind", ["one_key", "two_keys_one_word", "last_bin"])
+@pytest.mark.parametrize("nbins", [1 << 16, 65537])
+def test_counting_permute_relieves_counters_several_times(gpu_ctx, knobs, keys_kind, nbins, fresh):
+    # 32 workgroups of 2^17 keys each: a counter that takes all of a workgroup's keys passes
+    # 32768 four times.  With the defaults written by the summing kernel (fresh) the workgroup
+    # notes each relief in its list; otherwise the relief goes to the destination at once.
+    knobs("permute_groups", 32)
+    knobs("permute_fresh", fresh)
+    n = 1 << 22
+    rng = np.random.default_rng(nbins + fresh)
+    if keys_kind == "one_key":
+        keys = np.full(n, 12345, np.int32)
+    elif keys_kind == "two_keys_one_word":
+        keys = np.where(rng.random(n) < 0.5, 77, 77 + 32768).astype(np.int32)
+    else:
+        keys = np.where(rng.random(n) < 0.7, nbins - 1, 65535).astype(np.int32)
+    got = gpu_ctx.compile(_histogram_of_narrow_keys(nbins, A.i32, False))(keys)
+    assert np.array_equal(got, np.bincount(keys, minlength=nbins).astype(np.int32))
+
+
+@pytest.mark.gpu
+def test_counting_permute_writes_constant_defaults_itself(gpu_ctx, knobs):
+    # defaults of one constant other than zero, a constant other than one per source, a
+    # destination that is not a whole number of ranges: every element must come out as
+    # default + count * constant, also those no key points at
+    sh1 = A.tshape(1)
+    nbins, n = 70001, 1 << 21
+    prog = A.alam([A.tarray(1, A.i32)], lambda keys: A.permute(
+        Q.binop(A.add, A.i64),
+        A.generate(A.tarray(1, A.i64), A.sh(nbins), A.lam([sh1], lambda ix: A.const(A.i64, -5))),
+        A.lam([sh1], lambda ix: A.just(A.sh(A.fromintegral(A.i32, A.Int, A.index(keys, A.vexp(ix)))))),
+        A.delayed(A.tarray(1, A.i64), A.shape(keys), A.lam([sh1], lambda ix: A.const(A.i64, 3)),
+                  A.lam([A.Int], lambda i: A.const(A.i64, 3)))))
+    keys = np.random.default_rng(9).integers(0, nbins - 1000, n).astype(np.int32)   # the last 1000 bins stay at the default
+    want = np.bincount(keys, minlength=nbins).astype(np.int64) * 3 - 5
+    for fresh in (1, 0):
+        knobs("permute_fresh", fresh)
+        assert np.array_equal(gpu_ctx.compile(prog)(keys), want)
