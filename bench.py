@@ -217,8 +217,10 @@ def cpu_model():
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=20)
-    ap.add_argument("--warmup", type=int, default=5)
+    # (the first half dozen launches after an idle period run 3-5 % slower than the rest: the
+    # default warm-up covers them; a step takes under a millisecond)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--quick", action="store_true", help="headline workload only")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baselines")
     ap.add_argument("--only", default=None, help="run one workload (an id of Workloads.ids()) and print its entry")
