@@ -1110,8 +1110,19 @@ KernelSource Codegen::foldSeg(const Sx& f, const Sx* seed, const Operand& src, c
   return ks;
 }
 
-KernelSource Codegen::scan(const Sx& f, const Sx* seed, const Operand& src, bool right, int kind, bool small) {
+// The pipelined scan moves its input with direct global -> LDS loads: the operand must be an
+// array in memory (nothing fused into it) whose elements are one scalar of 4 or 8 bytes, read
+// left to right.
+bool Codegen::scanPipeable(const Operand& src, bool right) {
+  if (src.delayed || right) return false;
+  auto leaves = typeLeaves(src.r.elt);
+  return leaves.size() == 1 && !stIsVec(leaves[0]) && (stSize(leaves[0]) == 4 || stSize(leaves[0]) == 8);
+}
+
+KernelSource Codegen::scan(const Sx& f, const Sx* seed, const Operand& src, bool right, int kind, int variant) {
   const TypeP elt = src.r.elt;
+  const bool small = variant == 1, pipe = variant == 2;
+  if (pipe && !scanPipeable(src, right)) throw Error("scan: this operand cannot take the pipelined kernel");
   if (kind != 0 && !seed) throw Error("scan: this variant needs a seed");
   std::string body;
   body += std::string("  static constexpr bool kSeeded = ") + (seed ? "true" : "false") + ";\n";
@@ -1155,6 +1166,7 @@ KernelSource Codegen::scan(const Sx& f, const Sx* seed, const Operand& src, bool
   std::vector<ArraySlot> tmpOrder;
   for (auto& kv : used_) tmpOrder.push_back(kv.second);
   int vec = vecFor(leaves, tmpOrder);
+  if (pipe) vec = 16 / stSize(leaves[0]);  // a lane's share of a row is one 128-bit load
   // Large tiles keep the number of look-back steps on the critical path small, but a row of
   // a few tiles cannot fill 256 CUs and a row shorter than a tile leaves most of a large
   // workgroup idle: short rows get 256-thread workgroups with 128 bytes per lane (one row
@@ -1168,9 +1180,22 @@ KernelSource Codegen::scan(const Sx& f, const Sx* seed, const Operand& src, bool
     g = std::max(1, std::min(16, bytes / std::max(1, vec * std::max(1, eltBytes))));
     body += "#define ACC_SCAN_LBWAVES " + std::to_string(sl ? std::max(1, std::min(4, std::atoi(sl))) : 1) + "\n";
   }
+  if (pipe) {
+    // bytes of elements a lane holds per tile of the pipelined kernel (ACCHIP_SCAN_PIPE_BYTES)
+    const char* pb = std::getenv("ACCHIP_SCAN_PIPE_BYTES");
+    const int bytes = pb ? std::atoi(pb) : 128;
+    g = std::max(2, std::min(9, bytes / 16));
+    const std::string T = stName(leaves[0]);
+    const std::string at = "env." + slotByName(src.slot).name + "_0";
+    body += "  typedef " + T + " Raw;\n";
+    body += "  ACC_DEV const Raw* in_base(const Env& env) { return " + at + "; }\n";
+    body += "  ACC_DEV Raw* out_base(const Out& o) { return o.o0; }\n";
+    body += "  ACC_DEV Elt from_raw(Raw v) {\n    Elt r_;\n    r_.c0 = v;\n    return r_;\n  }\n";
+    body += "  ACC_DEV Raw to_raw(const Elt& e) { return e.c0; }\n";
+  }
   body += "  static constexpr int G = " + std::to_string(g) + ";\n";
-  body += "#define ACC_SCAN_BLOCK " + std::to_string(block) + "\n";
-  {
+  body += "#define ACC_SCAN_BLOCK " + std::to_string(pipe ? 1024 : block) + "\n";
+  if (!pipe) {
     // prefixes of the lane totals by raking through LDS, when the totals of a workgroup fit
     int sz = 0, al = 1;
     structLayout(leaves, sz, al);
@@ -1184,8 +1209,8 @@ KernelSource Codegen::scan(const Sx& f, const Sx* seed, const Operand& src, bool
     if (small && g > 1 && (long)(block / 64) * (64 * (g + 1) + 1) * sz <= 64 * 1024 && !(re && re[0] == '0'))
       body += "#define ACC_ROWS_RAKE 1\n";
   }
-  KernelSource ks = finish(body, elt, leaves, "scan.hpp+scan_kernel.hpp", vec);
-  ks.block = block;
+  KernelSource ks = finish(body, elt, leaves, pipe ? "scan.hpp+scan_pipe.hpp" : "scan.hpp+scan_kernel.hpp", vec);
+  ks.block = pipe ? 1024 : block;
   ks.group = g;
   ks.words = structWords(leaves);
   return ks;

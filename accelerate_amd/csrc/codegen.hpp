@@ -83,7 +83,10 @@ class Codegen {
   KernelSource backpermute(int outRank, const Sx& p, const Sx* f, const TypeP& outElt, const Operand& src);
   // kind 0: scanl1/scanr1, 1: scanl/scanr, 2: scanl'/scanr' (seed required for 1 and 2)
   // small: the variant for short rows (256-thread workgroups)
-  KernelSource scan(const Sx& f, const Sx* seed, const Operand& src, bool right, int kind, bool small = false);
+  // variant 0: large tiles, 1: small tiles (short rows), 2: persistent pipeline for long rows of a plain array
+  // (only where scanPipeable holds)
+  KernelSource scan(const Sx& f, const Sx* seed, const Operand& src, bool right, int kind, int variant = 0);
+  static bool scanPipeable(const Operand& src, bool right);
   KernelSource foldSeg(const Sx& f, const Sx* seed, const Operand& src, const Operand& seg, ST segType);
   // freshInit: the literal every element of the defaults holds when they are `generate sh (\_ -> c)`
   // (the counting variant can then write defaults and counts together), else null

@@ -45,6 +45,7 @@ struct ScanParams {
   u64 epoch;        // tag of this launch, 1 .. 2^30 - 1
   u64 spin_limit;   // polls of one window after which a tile stops waiting for its predecessors
   u32* err;         // host-visible word: 3 = a tile gave up waiting, or took a ticket outside the launch
+  i64 tpr_full;     // tiles per row that lie completely inside the row (the pipelined kernel's share)
 };
 
 #ifndef ACC_SCAN_BLOCK

@@ -363,6 +363,7 @@ Program::Program(Context& ctx, const char* text, size_t len) : ctx_(ctx) {
   for (auto& kv : plans_) {
     ctx_.wait(kv.second.k);
     ctx_.wait(kv.second.k2);
+    ctx_.wait(kv.second.k3);
     for (auto& sk : kv.second.scalarKernels) ctx_.wait(sk.second);
   }
   // a program that is one scan can be run without allocating (runInto): its code objects are
@@ -371,6 +372,7 @@ Program::Program(Context& ctx, const char* text, size_t len) : ctx_(ctx) {
     const Plan& plan = plans_.at(body_);
     ctx_.preload(plan.k, {"acc_scan", "acc_scan_rows"});
     ctx_.preload(plan.k2, {"acc_scan", "acc_scan_rows"});
+    if (plan.k3) ctx_.preload(plan.k3, {"acc_scan_pipe", "acc_scan_pipe_tail"});
   }
 }
 
@@ -636,7 +638,14 @@ ATyP Program::prepare(const Sx& n, TEnv& tenv) {
       Codegen cgs(aenvOf(tenv));
       Plan scratch;
       Operand srcS = operandOf(n.at(4), cgs, tenv, scratch);
-      plan.k2 = ctx_.kernel(cgs.scan(n.at(2), z, srcS, dir == "r", kind, true));
+      plan.k2 = ctx_.kernel(cgs.scan(n.at(2), z, srcS, dir == "r", kind, 1));
+    }
+    if (Codegen::scanPipeable(src, dir == "r")) {
+      // and as a pipeline in persistent workgroups, chosen at launch for long rows
+      Codegen cgp(aenvOf(tenv));
+      Plan scratch;
+      Operand srcP = operandOf(n.at(4), cgp, tenv, scratch);
+      plan.k3 = ctx_.kernel(cgp.scan(n.at(2), z, srcP, false, kind, 2));
     }
     if (prime) {
       ArrayR tr = src.r;
@@ -1516,7 +1525,25 @@ AValP Program::eval(const Sx& n, AEnv& aenv) {
         return result;
       }
     }
-    const KernelP& kern = small ? plan.k2 : plan.k;
+    // Long rows of a plain array: the pipelined kernel (persistent workgroups, one per CU).  Its
+    // direct global -> LDS loads move 16 bytes per lane from 16-byte aligned addresses.
+    bool pipe = false;
+    if (plan.k3 && !small) {
+      const KernelSource& pm = plan.k3->meta;
+      const int64_t pipeTile = (int64_t)pm.block * pm.group * pm.vec;
+      const int64_t eltBytes = 16 / pm.vec;
+      const Sx& so = n.at(4);
+      DArrayP srcArr = so.is("avar") ? aenv[aenv.size() - 1 - (size_t)so.at(1).asInt()] : (temps.empty() ? DArrayP() : temps[0]);
+      const bool aligned = srcArr && !srcArr->bufs.empty() && ((uintptr_t)srcArr->bufs[0]->p & 15) == 0 &&
+                           (rows == 1 || (len * eltBytes) % 16 == 0);
+      const int64_t tprP = (len + pipeTile - 1) / pipeTile;
+      // measured on 2^28 elements: Float32 363 us against 396 us for a workgroup per tile; Int64 775
+      // against 760 (two descriptor words per tile make its look-back dearer), so elements of 8 bytes
+      // take it only when forced
+      pipe = aligned && (forcedTiles == 4 ? len >= pipeTile
+                                          : (forcedTiles == 0 && eltBytes == 4 && tprP >= 16 && rows * tprP >= 4 * ctx_.computeUnits()));
+    }
+    const KernelP& kern = pipe ? plan.k3 : (small ? plan.k2 : plan.k);
     const KernelSource& m = kern->meta;
     const int64_t tile = (int64_t)m.block * m.group * m.vec;
     const int64_t tpr = std::max<int64_t>(1, (len + tile - 1) / tile);
@@ -1542,6 +1569,18 @@ AValP Program::eval(const Sx& n, AEnv& aenv) {
     args.push_back((uint64_t)st.epoch);
     args.push_back(spin);
     args.push_back((uint64_t)(uintptr_t)ctx_.errorWord());
+    const int64_t tprFull = len / tile;
+    args.push_back((uint64_t)tprFull);
+    if (pipe) {
+      // the full tiles of every row; every workgroup takes tickets until it meets the first one
+      // beyond them.  Then, with the same epoch, the rows' last tiles where they are partial.
+      const int64_t fullTiles = rows * tprFull;
+      const uint64_t groups = (uint64_t)std::min<int64_t>(fullTiles, ctx_.computeUnits());
+      ctx_.launch(kern, "acc_scan_pipe", groups, (unsigned)m.block, args);
+      st.ticketBase += (uint64_t)fullTiles + groups;
+      if (tprFull < tpr) ctx_.launch(kern, "acc_scan_pipe_tail", (uint64_t)rows, (unsigned)m.block, args);
+      return result;
+    }
     ctx_.launch(kern, "acc_scan", (uint64_t)tiles, (unsigned)m.block, args);
     st.ticketBase += (uint64_t)tiles;
     return result;

@@ -72,7 +72,7 @@ struct HVal {
 };
 
 struct Plan {
-  KernelP k, k2;
+  KernelP k, k2, k3;                             // k3: scans only, the pipelined kernel for long rows of a plain array
   std::vector<const Sx*> temps;                  // nested manifest operands, in slot order
   std::map<const Sx*, KernelP> scalarKernels;    // expressions evaluated by a one-thread kernel
   std::map<const Sx*, std::vector<const Sx*>> scalarTemps;

@@ -136,6 +136,17 @@ Context::Context(int device) : device_(device) {
   }
 }
 
+int Context::computeUnits() {
+  if (cus_ == 0) {
+    cus_ = 256;
+    if (device_ >= 0) {
+      int v = 0;
+      if (hipDeviceGetAttribute(&v, hipDeviceAttributeMultiprocessorCount, device_) == hipSuccess && v > 0) cus_ = v;
+    }
+  }
+  return cus_;
+}
+
 Context::~Context() {
   for (auto& kv : kernels_) {
     try {

@@ -56,7 +56,7 @@ struct Knobs {
   long long permute_fresh = 1;      // 0: constant defaults are materialised also where the counting kernels could write them
   long long stencil_chain = 0;      // 0: decide per launch; tiles (rank 2) or planes (rank 3) per workgroup
   long long stencil_no2d = 0, stencil_no3d = 0;  // 1: rank-2 / rank-3 stencils through the generic skeleton
-  long long scan_tiles = 0;         // 0: decide per launch, 1 large, 2 small, 3 rows
+  long long scan_tiles = 0;         // 0: decide per launch, 1 large, 2 small, 3 rows, 4 pipelined (where the operand allows)
   long long scan_spin_limit = (long long)1 << 22;  // polls after which a tile stops waiting (seconds)
   long long scan_test_skew = 0;     // fault injection: the ticket base passed to the kernel lags by this much
   void fromEnv();
@@ -77,6 +77,7 @@ class Context : public std::enable_shared_from_this<Context> {
   // manager (pool, table, eviction) can be driven without one; programs still cannot run
   bool hasMemory() const { return device_ >= 0 || fakeMemory_; }
   int device() const { return device_; }
+  int computeUnits();  // of the device (256 on MI355X); 256 for a context without one
   hipStream_t stream() const { return stream_; }
 
   // memory pool (counterpart of Array/Remote/Table.hs:170-211 + Nursery.hs:43-113):
@@ -152,6 +153,7 @@ class Context : public std::enable_shared_from_this<Context> {
 
  private:
   int device_ = -1;
+  int cus_ = 0;
   hipStream_t stream_ = nullptr;
   std::mutex mu_;
   std::unordered_map<void*, size_t> live_;                  // block -> rounded size
