@@ -20,7 +20,11 @@ Pinned by tests/test_oracle_golden.py against the reference's own doctest output
 issue regression vectors (tests/golden/*.json) and against closed forms, and by
 tests/test_oracle_pins.py for what those vectors leave open: every scalar primitive on every
 type against Python's unbounded integers, numpy and struct; stencils of ranks 1-4 and stencil2
-by brute force; fold1Seg against foldl1 over split places; transform; SIMD pack / unpack.
+by brute force; fold1Seg against foldl1 over split places; transform; SIMD pack / unpack; and by
+tests/test_oracle_control_pins.py for the array-level control flow (alet, apair, apply, aforeign,
+acond, awhile, atrace, use, unit, reshape: every program the GPU suite runs through these branches
+against the same computation in numpy, plus while-before-step, closed fallbacks, slot numbers and
+de Bruijn levels).  No branch of eval_acc that a GPU test reaches is without such a pin.
 Parity unpinned: the last-ulp behaviour of transcendental primitives (libm here, GHC's in the
 reference), and the exact shapes of the terms the reference's fusion emits.
 
