@@ -336,6 +336,16 @@ def test_jacobi_8192_100_iterations_bit_equal(gpu_ctx):
     assert np.array_equal(got, OC.jacobi_f32(g, 100))
 
 
+def test_jacobi_8192_100_iterations_under_awhile_bit_equal(gpu_ctx):
+    # the same configuration driven by awhile instead of repeated run1 (the configuration allows
+    # either): the loop state is (grid, counter), the counter is followed on the host
+    from .runtime_cases import jacobi_awhile
+    g = W.uniform_f32(8192 * 8192, 8, 0.0, 1.0).reshape(8192, 8192)
+    run = gpu_ctx.compile(jacobi_awhile(100))
+    got = run.execute(gpu_ctx.to_device(g, A.tarray(2, A.f32))).to_host()
+    assert np.array_equal(got, OC.jacobi_f32(g, 100))
+
+
 def test_jacobi_100_iterations_small_grid_bit_equal(gpu_ctx):
     g = W.uniform_f32(96 * 160, 9, 0.0, 1.0).reshape(96, 160)
     step = gpu_ctx.compile(P.jacobi_step())
