@@ -884,7 +884,25 @@ KernelSource Codegen::finish(const std::string& specBody, const TypeP& elt, cons
   std::string envS = envStruct(ks.arrays);
   ks.outLeaves = outLeaves;
   ks.vec = vec > 0 ? vec : vecFor(outLeaves, ks.arrays);
-  std::string s = deviceHeader("prelude.hpp");
+  // ACCHIP_KERNEL_DEFINES="NAME=VALUE ...": macros put in front of every generated translation unit
+  // (the skeletons' tuning constants are #ifndef-guarded); part of the source, hence of the cache key
+  std::string s;
+  if (const char* defs = std::getenv("ACCHIP_KERNEL_DEFINES")) {
+    std::string tok;
+    for (const char* c = defs;; ++c) {
+      if (*c && *c != ' ' && *c != ',') {
+        tok += *c;
+        continue;
+      }
+      if (!tok.empty()) {
+        const size_t eq = tok.find('=');
+        s += "#define " + (eq == std::string::npos ? tok + " 1" : tok.substr(0, eq) + " " + tok.substr(eq + 1)) + "\n";
+        tok.clear();
+      }
+      if (!*c) break;
+    }
+  }
+  s += deviceHeader("prelude.hpp");
   s += "\n" + envS + eltStruct(elt, "Elt") + outStruct(outLeaves);
   s += "struct Spec {\n  typedef ::Env Env;\n  typedef ::Elt Elt;\n  typedef ::Out Out;\n";
   s += "  static constexpr int V = " + std::to_string(ks.vec) + ";\n";
