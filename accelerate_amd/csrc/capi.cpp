@@ -214,6 +214,8 @@ long long acchip_stat(acchip_ctx* ctx, const char* name) {
   if (n == "pool_hits") return s.poolHits;
   if (n == "pool_misses") return s.poolMisses;
   if (n == "arrays_evicted") return s.arraysEvicted;
+  if (n == "raw_allocs") return s.rawAllocs;
+  if (n == "modules_loaded") return s.modulesLoaded;
   return -1;
 }
 
@@ -395,7 +397,7 @@ int acchip_compile(acchip_ctx* ctx, const char* program_text, size_t length, acc
 }
 void acchip_program_release(acchip_program* p) { delete p; }
 int acchip_program_arity(const acchip_program* p) { return (int)p->prog.argTypes.size(); }
-int acchip_program_num_kernels(const acchip_program* p) { return (int)p->prog.kernelCount(); }
+int acchip_program_num_kernels(const acchip_program* p) { return (int)p->keys.size(); }
 const char* acchip_program_kernel_key(const acchip_program* p, int k) {
   return k >= 0 && k < (int)p->keys.size() ? p->keys[k].c_str() : nullptr;
 }

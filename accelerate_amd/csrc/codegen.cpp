@@ -1485,11 +1485,16 @@ KernelSource Codegen::permute(const Sx& f, const ArrayR& dst, const Sx& p, const
     // ballot).  With a per-lane exit the compiler may move the critical section behind the
     // loop, where a lane that won the lock waits for the lanes still spinning on it: two
     // lanes of one wave with the same destination then never finish.
-    // The wait for a lock is bounded (ACC_LOCK_SPIN_LIMIT rounds, seconds): a lane that never
-    // gets its lock reports through err and drops its update, so that the kernel always ends.
+    // The wait for a lock is bounded: a wave that sees none of its lanes win a lock for
+    // ACC_LOCK_SPIN_LIMIT rounds in a row (many seconds) reports through err and drops the updates
+    // still waiting, so that the kernel always ends.  The count starts again whenever a lane of
+    // the wave wins, so heavy but legitimate contention -- millions of sources for one cell -- is
+    // slow, not an error, as long as the wave's own updates keep landing.
     u += "    u32* lk_ = locks + j;\n    bool done_ = false;\n    u32 rounds_ = 0;\n    while (__ballot(!done_) != 0ull) {\n";
     u += "      if (++rounds_ > ACC_LOCK_SPIN_LIMIT) {\n        if (!done_) __hip_atomic_store(err, 4u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);\n        break;\n      }\n";
-    u += "      if (!done_ && __hip_atomic_exchange(lk_, 1u, __ATOMIC_ACQUIRE, __HIP_MEMORY_SCOPE_AGENT) == 0u) {\n        Elt y_;\n";
+    u += "      const bool won_ = !done_ && __hip_atomic_exchange(lk_, 1u, __ATOMIC_ACQUIRE, __HIP_MEMORY_SCOPE_AGENT) == 0u;\n";
+    u += "      if (__ballot(won_) != 0ull) rounds_ = 0;\n";
+    u += "      if (won_) {\n        Elt y_;\n";
     // leaf by leaf (component by component for SIMD vector leaves) through relaxed atomics
     auto each = [&](size_t k, const std::function<void(const std::string& cell, const std::string& field)>& fn) {
       const std::string cell = "out.o" + std::to_string(k) + "[j]", field = ".c" + std::to_string(k);

@@ -30,7 +30,7 @@ template <class T, int N> struct __attribute__((packed, aligned(alignof(T)))) ac
 #define ACC_DEV static __device__ __forceinline__
 #define ACC_WAVE 64
 #ifndef ACC_LOCK_SPIN_LIMIT
-#define ACC_LOCK_SPIN_LIMIT (1u << 24)  // rounds a lane of a locked permute tries for its destination's lock
+#define ACC_LOCK_SPIN_LIMIT (1u << 26)  // rounds in a row without any lane of the wave winning its lock, after which a locked permute gives up
 #endif
 #define ACC_BLOCK 256
 #define ACC_WAVES (ACC_BLOCK / ACC_WAVE)

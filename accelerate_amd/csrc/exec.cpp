@@ -378,9 +378,14 @@ Program::Program(Context& ctx, const char* text, size_t len) : ctx_(ctx) {
 
 std::vector<std::string> Program::kernelKeys() const {
   std::vector<std::string> keys;
-  for (auto& kv : plans_)
-    if (kv.second.k) keys.push_back(kv.second.k->hash);
+  for (auto& kv : plans_) {
+    for (const KernelP& k : {kv.second.k, kv.second.k2, kv.second.k3})
+      if (k) keys.push_back(k->hash);
+    for (auto& sk : kv.second.scalarKernels)
+      if (sk.second) keys.push_back(sk.second->hash);
+  }
   std::sort(keys.begin(), keys.end());
+  keys.erase(std::unique(keys.begin(), keys.end()), keys.end());
   return keys;
 }
 

@@ -94,7 +94,7 @@ class Program {
   std::vector<ATyP> argTypes;
   ATyP resultType;
   size_t kernelCount() const { return plans_.size(); }
-  // cache keys of the kernels the nodes launch (main variants), sorted
+  // cache keys of every kernel the program may launch (all variants of every node, scalar kernels), sorted, distinct
   std::vector<std::string> kernelKeys() const;
 
  private:

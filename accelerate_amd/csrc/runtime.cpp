@@ -58,6 +58,7 @@ const KnobName kKnobs[] = {
     {"fold_target", &Knobs::fold_target},         {"fold_max_blocks", &Knobs::fold_max_blocks},         {"permute_parts", &Knobs::permute_parts},
     {"permute_count", &Knobs::permute_count},     {"permute_groups", &Knobs::permute_groups},
     {"permute_partials", &Knobs::permute_partials}, {"permute_fresh", &Knobs::permute_fresh}, {"stencil_chain", &Knobs::stencil_chain},
+    {"pool_async", &Knobs::pool_async},
     {"stencil_no2d", &Knobs::stencil_no2d},       {"stencil_no3d", &Knobs::stencil_no3d},
     {"scan_tiles", &Knobs::scan_tiles},           {"scan_spin_limit", &Knobs::scan_spin_limit},
     {"scan_test_skew", &Knobs::scan_test_skew},
@@ -174,6 +175,7 @@ Context::~Context() {
   if (errHost_) (void)hipHostFree(errHost_);
   if (scan_.desc) (void)hipFree(scan_.desc);
   if (scan_.ticket) (void)hipFree(scan_.ticket);
+  (void)hipStreamSynchronize(stream_);  // the stream-ordered frees above
   (void)hipStreamDestroy(stream_);
 }
 
@@ -198,10 +200,28 @@ void* Context::rawMalloc(size_t n) {
   if (fakeMemory_) {
     p = std::malloc(n);
   } else {
+    // Stream-ordered underneath (the reference's ladder, Array/Remote/Table.hs:194-211, sits on
+    // top): a block freed behind queued work needs no synchronisation, the runtime's pool keeps
+    // what is freed (release threshold = everything) and hands it out again in stream order.
     (void)hipSetDevice(device_);
-    if (hipMalloc(&p, n) != hipSuccess) {
+    const bool async = knobs.pool_async != 0;
+    if (async && !asyncPoolReady_) {
+      hipMemPool_t mp = nullptr;
+      if (hipDeviceGetDefaultMemPool(&mp, device_) == hipSuccess && mp) {
+        uint64_t keep = ~(uint64_t)0;
+        (void)hipMemPoolSetAttribute(mp, hipMemPoolAttrReleaseThreshold, &keep);
+      }
+      (void)hipGetLastError();
+      asyncPoolReady_ = true;
+    }
+    const hipError_t e = async ? hipMallocAsync(&p, n, stream_) : hipMalloc(&p, n);
+    if (e != hipSuccess) {
       (void)hipGetLastError();
       p = nullptr;
+    } else {
+      stats.rawAllocs++;
+      std::lock_guard<std::mutex> g(mu_);
+      if (async) asyncBlocks_.insert(p);
     }
   }
   if (!p) {
@@ -212,10 +232,15 @@ void* Context::rawMalloc(size_t n) {
 }
 
 void Context::rawFree(void* p, size_t n) {
+  bool async = false;
+  {
+    std::lock_guard<std::mutex> g(mu_);
+    async = asyncBlocks_.erase(p) > 0;
+    rawBytes_ -= n;
+  }
   if (fakeMemory_) std::free(p);
+  else if (async) (void)hipFreeAsync(p, stream_);   // ordered behind whatever the stream still does with the block
   else (void)hipFree(p);
-  std::lock_guard<std::mutex> g(mu_);
-  rawBytes_ -= n;
 }
 
 void* Context::malloc(size_t bytes) { return poolMalloc(bytes, true); }
@@ -252,8 +277,9 @@ void* Context::poolMalloc(size_t bytes, bool mayEvict) {
     cleanHook();
     if (void* p = fromNursery()) return p;
   }
-  // work queued on the stream may still use blocks waiting in the free lists
-  if (device_ >= 0) (void)hipStreamSynchronize(stream_);
+  // work queued on the stream may still use blocks waiting in the free lists: blocks of the
+  // stream-ordered allocator are freed behind it, others only once the stream has drained
+  if (device_ >= 0 && knobs.pool_async == 0) (void)hipStreamSynchronize(stream_);
   purge();
   if (void* p = fresh()) return p;
   // evict unused arrays of the table, eldest first, until the block fits or nothing is left
@@ -300,7 +326,17 @@ size_t Context::blockSize(void* p) {
 void Context::memInfo(size_t* total, size_t* avail) {
   *total = *avail = 0;
   if (!hasMemory()) return;
-  if (device_ >= 0) hipCheck(hipMemGetInfo(avail, total), "hipMemGetInfo");
+  if (device_ >= 0) {
+    hipCheck(hipMemGetInfo(avail, total), "hipMemGetInfo");
+    // what the stream-ordered allocator keeps for reuse is not in use
+    hipMemPool_t mp = nullptr;
+    uint64_t reserved = 0, used = 0;
+    if (asyncPoolReady_ && hipDeviceGetDefaultMemPool(&mp, device_) == hipSuccess && mp &&
+        hipMemPoolGetAttribute(mp, hipMemPoolAttrReservedMemCurrent, &reserved) == hipSuccess &&
+        hipMemPoolGetAttribute(mp, hipMemPoolAttrUsedMemCurrent, &used) == hipSuccess && reserved > used)
+      *avail += (size_t)(reserved - used);
+    (void)hipGetLastError();
+  }
   std::lock_guard<std::mutex> g(mu_);
   if (limit_) {
     *total = limit_;
@@ -338,7 +374,7 @@ bool Context::evictEldest() {
     }
   }
   if (!pick) return false;
-  if (pick->st == Status::Dirty && pick->host) peek(pick->host, pick->dev, pick->bytes);
+  if (pick->st == Status::Dirty && pick->host) copyFromDevice(pick->host, pick->dev, pick->bytes);
   if (flag(kDumpGc))
     fprintf(stderr, "[acchip] gc: evict %zu bytes (%s)\n", pick->bytes, pick->st == Status::Dirty ? "copied back" : "clean");
   free(pick->dev);
@@ -472,6 +508,7 @@ void Context::ensureStaging() {
   if (staging_[0]) return;
   for (int b = 0; b < 2; ++b) {
     hipCheck(hipHostMalloc(&staging_[b], kStagePiece, hipHostMallocDefault), "hipHostMalloc");
+    stats.rawAllocs++;
     hipCheck(hipEventCreateWithFlags(&stagingDone_[b], hipEventDisableTiming), "hipEventCreate");
   }
 }
@@ -506,6 +543,14 @@ void Context::poke(void* dev, const void* host, size_t bytes) {
 }
 
 void Context::peek(void* host, const void* dev, size_t bytes) {
+  copyFromDevice(host, dev, bytes);
+  raiseDeviceError();
+}
+
+// The copy alone: what eviction uses to write a Dirty block back.  An error that an earlier
+// kernel left in the error word stays there for the next call that waits for the stream on the
+// caller's behalf -- raised from inside an allocation it would come back as "out of memory".
+void Context::copyFromDevice(void* host, const void* dev, size_t bytes) {
   if (bytes == 0) return;
   if (fakeMemory_) {
     std::memcpy(host, dev, bytes);
@@ -532,7 +577,6 @@ void Context::peek(void* host, const void* dev, size_t bytes) {
     }
   }
   stats.bytesCopiedFromRemote += (long long)bytes;
-  raiseDeviceError();
 }
 
 void Context::copy(void* dst, const void* src, size_t bytes) {
@@ -553,6 +597,7 @@ void Context::sync() {
 unsigned* Context::errorWord() {
   if (!errDev_) {
     hipCheck(hipHostMalloc((void**)&errHost_, 64, hipHostMallocMapped), "hipHostMalloc(error word)");
+    stats.rawAllocs++;
     *errHost_ = 0;
     hipCheck(hipHostGetDevicePointer((void**)&errDev_, errHost_, 0), "hipHostGetDevicePointer");
   }
@@ -574,6 +619,7 @@ void Context::raiseDeviceError() {
 ScanState& Context::scanState(size_t descBytes) {
   if (!scan_.ticket) {
     hipCheck(hipMalloc((void**)&scan_.ticket, 256), "hipMalloc(scan ticket)");
+    stats.rawAllocs++;
     hipCheck(hipMemsetAsync(scan_.ticket, 0, 256, stream_), "hipMemsetAsync");
     scan_.ticketBase = 0;
   }
@@ -584,6 +630,7 @@ ScanState& Context::scanState(size_t descBytes) {
     }
     size_t n = std::max(descBytes, (size_t)4 << 20);
     hipCheck(hipMalloc(&scan_.desc, n), "hipMalloc(scan descriptors)");
+    stats.rawAllocs++;
     hipCheck(hipMemsetAsync(scan_.desc, 0, n, stream_), "hipMemsetAsync");
     scan_.descBytes = n;
     scan_.epoch = 0;
@@ -755,6 +802,7 @@ void Context::ensureLoaded(const KernelP& k) {
   wait(k);
   if (device_ < 0) throw Error("this context has no device: programs can be compiled but not executed");
   hipCheck(hipModuleLoadData(&k->module, k->code.data()), "hipModuleLoadData");
+  stats.modulesLoaded++;
 }
 
 void Context::preload(const KernelP& k, std::initializer_list<const char*> fns) {

@@ -8,6 +8,7 @@
 #include <functional>
 #include <future>
 #include <map>
+#include <unordered_set>
 #include <memory>
 #include <mutex>
 #include <string>
@@ -36,7 +37,9 @@ using KernelP = std::shared_ptr<Kernel>;
 struct Stats {
   std::atomic<long long> bytesAllocated{0}, bytesCopiedToRemote{0}, bytesCopiedFromRemote{0}, bytesEvicted{0},
       kernelsCompiled{0}, kernelsFromDisk{0}, kernelsFromMemory{0}, launches{0}, poolHits{0}, poolMisses{0},
-      arraysEvicted{0};
+      arraysEvicted{0},
+      rawAllocs{0},      // device or pinned host allocations of any kind the library asked the runtime for
+      modulesLoaded{0};  // code objects loaded onto the device
 };
 
 // Launch-time choices that tests and tuning override.  Read from the environment once, when
@@ -56,6 +59,7 @@ struct Knobs {
   long long permute_fresh = 1;      // 0: constant defaults are materialised also where the counting kernels could write them
   long long stencil_chain = 0;      // 0: decide per launch; tiles (rank 2) or planes (rank 3) per workgroup
   long long stencil_no2d = 0, stencil_no3d = 0;  // 1: rank-2 / rank-3 stencils through the generic skeleton
+  long long pool_async = 1;         // 1: device blocks come from the stream-ordered allocator (hipMallocAsync), 0: hipMalloc
   long long scan_tiles = 0;         // 0: decide per launch, 1 large, 2 small, 3 rows, 4 pipelined (where the operand allows)
   long long scan_spin_limit = (long long)1 << 22;  // polls after which a tile stops waiting (seconds)
   long long scan_test_skew = 0;     // fault injection: the ticket base passed to the kernel lags by this much
@@ -112,7 +116,8 @@ class Context : public std::enable_shared_from_this<Context> {
   std::function<void()> cleanHook;
 
   void poke(void* dev, const void* host, size_t bytes);   // H->D through pinned staging, stream-ordered
-  void peek(void* host, const void* dev, size_t bytes);   // D->H, synchronises the stream
+  void peek(void* host, const void* dev, size_t bytes);   // D->H, synchronises the stream, raises what kernels reported
+  void copyFromDevice(void* host, const void* dev, size_t bytes);  // the same without looking at the error word
   void copy(void* dst, const void* src, size_t bytes);    // D->D
   void fill0(void* dev, size_t bytes);
   void sync();
@@ -157,6 +162,8 @@ class Context : public std::enable_shared_from_this<Context> {
   hipStream_t stream_ = nullptr;
   std::mutex mu_;
   std::unordered_map<void*, size_t> live_;                  // block -> rounded size
+  std::unordered_set<void*> asyncBlocks_;                   // blocks that came from the stream-ordered allocator
+  bool asyncPoolReady_ = false;
   std::map<size_t, std::vector<void*>> nursery_;            // rounded size -> free blocks
   std::unordered_map<std::string, KernelP> kernels_;
   unsigned* errHost_ = nullptr;  // pinned, mapped: written by kernels, read here

@@ -5,9 +5,12 @@ Headline (the JSON line's `value`, `roofline`, `cpu_baseline`): one step = one a
 prepared program `runN (scanl1 (+))` to a device-resident Int64 vector of 2^28 elements (one
 launch of the single-pass scan kernel), through the C ABI.  The same line carries, under
 "configs", every benchmark configuration (dotp, both scans, foldSeg, histogram, Jacobi) and the
-2^28 map / dotp the bandwidth target is stated for, each with its own roofline entry (median of
-the per-step times between HIP events on the library's stream) and the CPU figures of the same
-workload on one core and on all host cores.
+2^28 map / dotp the bandwidth target is stated for, each with its own roofline entry and the CPU
+figures of the same workload on one core and on all host cores.  Every roofline figure, the
+headline's and the configurations', is algorithmic bytes / the MEAN time of a step over the timed
+region, between HIP events recorded on the library's stream; the median is reported next to it
+("us_median").  "transfer" gives what acchip_poke / acchip_peek move per second for the headline's
+2 GiB input (never part of `value`).
 
   python bench.py [--gpus 1] [--steps K] [--warmup W] [--quick] [--no-cpu] [--only ID]
 
@@ -31,6 +34,7 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0   # MI355X HBM3E, published peak
+LLC_BYTES = 256 << 20   # MI355X last-level (memory-side) cache
 TRAFFIC_FILE = os.path.join(ROOT, "profiles", "traffic.json")
 
 
@@ -113,7 +117,7 @@ class Workloads:
         if wid == "scan_f32":
             x = self.vec("f01", n28, 11)
             return dict(name="scanl1 (+) Float32 n=2^28", prog=P.scanl1_sum(A.f32), tys=[A.tarray(1, A.f32)], args=[x],
-                        n=n28, bytes=8 * n28, kernel="acc_scan", unit="Gelem/s",
+                        n=n28, bytes=8 * n28, kernel="acc_scan_pipe", unit="Gelem/s",
                         seq=lambda: OC.scanl1_f32(x), omp=lambda: OC.omp_scanl1(x), sample="full workload")
         if wid == "map_f32":
             x = self.vec("f01", n28, 11)
@@ -140,7 +144,9 @@ class Workloads:
         if wid == "histogram":
             nk, nb = 1 << 26, 1 << 16
             keys = W.zipf_keys(nk, nb, 15)
-            return dict(name="histogram: permute (+) of 2^26 Zipf(1.1) keys into 2^16 Int32 bins", prog=P.histogram(nb),
+            counts = np.bincount(keys, minlength=nb)
+            return dict(hot=(int(counts.max()), float(counts.max()) / nk),
+                        name="histogram: permute (+) of 2^26 Zipf(1.1) keys into 2^16 Int32 bins", prog=P.histogram(nb),
                         tys=[A.tarray(1, A.i32)], args=[keys], n=nk, bytes=4 * nk + 8 * nb, kernel="acc_permute_count",
                         unit="Gelem/s", seq=lambda: OC.histogram_i32(keys, nb), omp=lambda: OC.omp_histogram_i32(keys, nb),
                         sample="full workload", check=lambda got: np.array_equal(got, np.bincount(keys, minlength=nb)))
@@ -149,7 +155,7 @@ class Workloads:
             g = W.uniform_f32(side * side, 16, 0.0, 1.0).reshape(side, side)
             return dict(name="Jacobi 3x3 cross, clamp, 8192x8192 Float32, per sweep of 100", prog=P.jacobi_step(),
                         tys=[A.tarray(2, A.f32)], args=[g], n=side * side, bytes=8 * side * side, kernel="acc_stencil2d",
-                        unit="Gcell/s", iterate=100, seq=lambda: OC.jacobi_f32(g, 2), omp=lambda: OC.omp_jacobi_f32(g, 4),
+                        unit="Gcell/s", iterate=100, resident=True,   # a sweep reads what the previous one wrote (256 MiB) seq=lambda: OC.jacobi_f32(g, 2), omp=lambda: OC.omp_jacobi_f32(g, 4),
                         seq_units=2, omp_units=4, sample="2 (one core) / 4 (all cores) sweeps of the 100")
         raise KeyError(wid)
 
@@ -183,13 +189,23 @@ def run_workload(ctx, wl, steps, warmup, with_cpu, cpu_reps=3):
     if "check" in wl:
         assert wl["check"](run.execute(*dev).to_host()), "result of %s differs from the oracle" % wl["name"]
     med, mean = statistics.median(per), sum(per) / len(per)
-    gbs = wl["bytes"] / med / 1e6
-    entry = {"workload": wl["name"], "elements": wl["n"], "algorithmic_bytes": wl["bytes"], "us": round(med * 1e3, 2),
-             "steps_timed": len(per), "value": round(wl["n"] / med / 1e6, 2), "unit": wl["unit"],
+    gbs = wl["bytes"] / mean / 1e6
+    ws = wl.get("working_set", wl["bytes"])
+    entry = {"workload": wl["name"], "elements": wl["n"], "algorithmic_bytes": wl["bytes"], "us": round(mean * 1e3, 2),
+             "us_median": round(med * 1e3, 2), "steps_timed": len(per), "value": round(wl["n"] / mean / 1e6, 2),
+             "unit": wl["unit"],
              "roofline": {"bound": "hbm", "kernel": wl["kernel"], "achieved": round(gbs, 1), "peak": HBM_PEAK_GBS,
                           "unit": "GB/s", "frac": round(gbs / HBM_PEAK_GBS, 4),
                           "traffic": traffic_for(wl["name"], run.kernel_keys)},
+             # what a step touches against the 256 MiB last-level cache: a resident working set is
+             # served by the cache from the second step on, and its figure says nothing about HBM
+             "working_set_bytes": ws, "cache_resident": bool(ws <= LLC_BYTES or wl.get("resident")),
              "kernel_keys": run.kernel_keys}
+    if "hot" in wl:
+        keys_hot, share = wl["hot"]
+        entry["hottest_bin"] = {"updates_per_launch": keys_hot, "share_of_keys": round(share, 4),
+                                "updates_per_s": round(keys_hot / (mean * 1e-3), 1),
+                                "note": "updates of the most popular bin's counters per second of the whole step"}
     del dev
     if with_cpu:
         from oracle import c as OC
@@ -202,6 +218,23 @@ def run_workload(ctx, wl, steps, warmup, with_cpu, cpu_reps=3):
             entry["cpu_omp"] = {"value": round(wl["n"] * ou / dt / 1e9, 4), "unit": wl["unit"], "cores": OC.omp_threads(),
                                 "kind": "port", "sample": wl["sample"]}
     return entry, wall, mean
+
+
+def measure_transfer(ctx, x, aty):
+    """Host <-> device rates of the boundary's copies (acchip_poke / acchip_peek through pinned
+    staging buffers) for one array, from and to pageable numpy memory; the second of two rounds."""
+    out = {}
+    for _ in range(2):
+        t0 = time.perf_counter()
+        d = ctx.to_device(x, aty)
+        ctx.sync()
+        t1 = time.perf_counter()
+        h = d.to_host()
+        t2 = time.perf_counter()
+        out = {"bytes": int(x.nbytes), "h2d_GBs": round(x.nbytes / (t1 - t0) / 1e9, 2), "d2h_GBs": round(x.nbytes / (t2 - t1) / 1e9, 2),
+               "note": "acchip_poke / acchip_peek of the headline's input, pageable host memory; not part of `value`"}
+        del d, h
+    return out
 
 
 def cpu_model():
@@ -245,6 +278,7 @@ def main():
     wl["check"] = lambda got: int(got[-1]) == int(x.sum())     # cheap integrity check of the timed path
     head, wall, mean = run_workload(ctx, wl, a.steps, a.warmup, not a.no_cpu)
     achieved = wl["bytes"] / mean / 1e6       # average launch duration over the timed region
+    transfer = measure_transfer(ctx, x, wl["tys"][0])
     cpu = None
     if not a.no_cpu:
         cpu = dict(head["cpu_omp"])
@@ -262,6 +296,7 @@ def main():
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": head["roofline"]["traffic"]},
         "cpu_baseline": cpu,
+        "transfer": transfer,
     }
 
     # ---- every configuration, with its own roofline and CPU figures -------------------------

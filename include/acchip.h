@@ -204,8 +204,11 @@ void acchip_array_release(acchip_array* a);
 int acchip_compile(acchip_ctx* ctx, const char* program_text, size_t length, acchip_program** out);
 void acchip_program_release(acchip_program* p);
 int acchip_program_arity(const acchip_program* p);
+/* Number of distinct compiled kernels behind the program: every variant of every array node
+ * (a scan has up to three: large tiles, small tiles, the pipelined kernel) and the one-thread
+ * kernels that evaluate scalar expressions for the host. */
 int acchip_program_num_kernels(const acchip_program* p);
-/* Cache key of the program's k-th kernel, k = 0 .. num_kernels - 1: the hexadecimal SHA3-256 of
+/* Cache key of the program's k-th kernel, k = 0 .. num_kernels - 1 (sorted): the hexadecimal SHA3-256 of
  * its generated source, compile options and hipRTC version (the counterpart of the reference's
  * hashPreOpenAccWith, Analysis/Hash.hs:107-111, which names the kernels of accelerate-llvm's
  * cache).  NULL beyond the last kernel; valid while the program lives.  Profiles refer to
@@ -234,15 +237,19 @@ int acchip_execute(acchip_ctx* ctx, acchip_program* p, acchip_array* const* args
                    acchip_array* const* uses, int n_uses, acchip_array** result);
 
 /* No counterpart in the reference: a variant of acchip_execute for callers that cannot allocate
- * device memory (code under HIP graph capture, tight serving loops, harnesses that forbid
- * hipMalloc).  The program's body must be a single scan (any of the six) whose operand is an
+ * device memory (tight serving loops, harnesses that forbid hipMalloc).  It is NOT meant for
+ * recording into a HIP graph: the ticket base and the epoch of a launch are kernel arguments that
+ * the host advances per call, so a recorded launch replayed later would carry stale ones (every
+ * tile would then refuse its ticket and report an error), and the context's stream is not
+ * exposed for capture.  The program's body must be a single scan (any of the six) whose operand is an
  * array variable or a fused producer with a host-computable extent; `result` is an array the
  * caller made (acchip_array_wrap / acchip_array_new) with the type and extents of the
  * program's result -- for scanl' / scanr' the pair (array, totals) built with
  * acchip_array_pair.  The tile descriptors and the ticket counter that acchip_execute keeps in
  * pool memory live in a static device array of 1 MiB + 256 B per GPU instead (131072 descriptor
- * words: a scan may have at most 131072 / ceil(element bytes / 4) tiles, e.g. 2^28 Int64 or
- * Float32 elements in one row take 10923 or 5462 tiles); larger scans fail with an error and
+ * words: a scan may have at most 131072 / ceil(element bytes / 4) tiles, e.g. 2^28 Int64
+ * elements in one row take 10923 tiles of two words, 2^28 Float32 elements 8192 tiles of one);
+ * larger scans fail with an error and
  * nothing is launched.  The call performs no hipMalloc / hipFree and clears nothing with memset
  * nodes; code objects were loaded by acchip_compile.  All contexts on one GPU share the array:
  * calls of this entry point that overlap on one GPU (two streams, two threads) race. */

@@ -21,10 +21,13 @@ def _both(ctx, prog, x, aty, out_shape, pair_shape=None):
     if pair_shape is not None:
         tot = ctx.empty(pair_shape, ("array", len(pair_shape), aty[2]))
         dest = ctx.pair(dest, tot)
-    before = ctx.stat("bytes_allocated_remote"), ctx.stat("pool_hits"), ctx.stat("pool_misses")
+    # the pool's counters, and the library's count of every allocation it asks the runtime for
+    # outside the pool (hipMalloc, hipMallocAsync, hipHostMalloc) and of code objects it loads
+    names = ("bytes_allocated_remote", "pool_hits", "pool_misses", "raw_allocs", "modules_loaded")
+    before = [ctx.stat(n) for n in names]
     prog.execute_into(dest, d)
-    after = ctx.stat("bytes_allocated_remote"), ctx.stat("pool_hits"), ctx.stat("pool_misses")
-    assert before == after, "acchip_execute_into went to the memory pool"
+    after = [ctx.stat(n) for n in names]
+    assert before == after, "acchip_execute_into allocated or loaded something: %s" % dict(zip(names, zip(before, after)))
     got = dest.to_host()
     return want, got
 
@@ -80,6 +83,18 @@ def test_scanl1_float32_within_tolerance(gpu_ctx):
         bound = 1e-4 * np.cumsum(np.abs(x.astype(np.float64)))
         assert np.all(np.abs(got - ref) <= bound)
         assert np.all(np.abs(got - want) <= bound)
+
+
+def test_long_float32_row_takes_the_pipelined_kernel(gpu_ctx):
+    # long rows of 4-byte elements run the persistent pipelined kernel in both entry points (its
+    # code object is loaded at compile time like the others); a second, shorter call follows
+    aty = A.tarray(1, A.f32)
+    prog = gpu_ctx.compile(P.scanl1_sum(A.f32))
+    for k, n in enumerate(((1 << 26) + 5, 40_000_003)):
+        x = W.uniform_f32(n, 61 + k, 0.0, 1.0)
+        want, got = _both(gpu_ctx, prog, x, aty, (n,))
+        ref = np.cumsum(x.astype(np.float64))
+        assert np.all(np.abs(got - ref) <= 1e-4 * ref) and np.all(np.abs(got - want) <= 1e-4 * ref)
 
 
 def test_refusals_launch_nothing(gpu_ctx):
