@@ -21,7 +21,7 @@
 module Data.Array.Accelerate.HIP.Array.Remote (
 
   Context(..), theContext, withContext, check,
-  withLeaf, withArrayData, adoptLeaf, HIP(..), StreamEvent(..),
+  withLeaf, withArrayData, adoptLeaf, HIP(..), StreamEvent(..), mirrorCounters,
 
 ) where
 
@@ -77,6 +77,26 @@ check what _ = do
   msg <- peekCString =<< c_last_error
   internalError (what ++ ": " ++ msg)
 
+-- | The reference's monitoring counters (cbits/monitoring.c:26-32, read by its @-ddump-gc@ report and
+-- by the Tracy plots): the library keeps the same quantities per context, and they are copied
+-- over after every program and collection, so that tools written against the reference's
+-- counters see this backend's remote memory.  This backend is the only user of the remote
+-- counters in a process, hence totals are stored, not added.
+foreign import ccall "&__total_bytes_allocated_remote"    total_bytes_allocated_remote    :: Ptr Int64
+foreign import ccall "&__total_bytes_copied_to_remote"    total_bytes_copied_to_remote    :: Ptr Int64
+foreign import ccall "&__total_bytes_copied_from_remote"  total_bytes_copied_from_remote  :: Ptr Int64
+foreign import ccall "&__total_bytes_evicted_from_remote" total_bytes_evicted_from_remote :: Ptr Int64
+foreign import ccall "&__num_evictions"                   num_evictions                   :: Ptr Int64
+
+mirrorCounters :: IO ()
+mirrorCounters = withContext $ \ctx -> do
+  let copy name dst = withCString name $ \n -> poke dst . fromIntegral =<< c_stat ctx n
+  copy "bytes_allocated_remote"    total_bytes_allocated_remote
+  copy "bytes_copied_to_remote"    total_bytes_copied_to_remote
+  copy "bytes_copied_from_remote"  total_bytes_copied_from_remote
+  copy "bytes_evicted_from_remote" total_bytes_evicted_from_remote
+  copy "arrays_evicted"            num_evictions
+
 -- the table's name for a host buffer
 ident :: UniqueArray e -> Word64
 ident = fromIntegral . hash . uniqueArrayId
@@ -101,6 +121,7 @@ withLeaf ua n k = withContext $ \ctx -> withUniqueArrayPtr ua $ \host -> do
     check "acchip_poke" =<< c_poke ctx dev host bytes
   r <- k dev
   check "acchip_table_release" =<< c_table_release ctx key
+  mirrorCounters
   return r
 
 -- | The same for all buffers of an array's payload, left to right (the struct-of-arrays order of
