@@ -50,18 +50,32 @@ def test_all_runtime_programs_compile_and_oracle_evaluates_them(cc_ctx):
             pytest.fail("oracle on %s: %r" % (cid, e))
 
 
-def test_benchmark_programs_print_to_the_committed_term_texts():
-    # tests/golden/terms/*.sx are the exact texts of the five configurations' terms: the golden
-    # files of any printer of the wire format (the Haskell serialiser must produce these bytes
-    # for the same programs), so the Python builder must not drift from them either
+def test_programs_print_to_the_committed_term_texts():
+    # tests/golden/terms/*.sx are the exact texts of every named program of the suite -- the five
+    # configurations, the reference's doctest and issue programs, the control-flow programs, the
+    # property-shaped cases and whole programs: the golden files of any printer of the wire format
+    # (the Haskell serialiser must produce these bytes for the same programs), so the Python
+    # builder must not drift from them either.  tests/golden/make_terms.py writes them.
     import os
-    from accelerate_amd import ir as A, programs as P
+    from .golden.make_terms import named_terms
     here = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "terms")
-    progs = {"c1_dotp": P.dotp(), "c2_scanl1_i64": P.scanl1_sum(A.i64), "c2_scanl1_f32": P.scanl1_sum(A.f32),
-             "c3_foldseg": P.foldseg_sum(), "c4_histogram": P.histogram(1 << 16), "c5_jacobi_step": P.jacobi_step()}
-    assert sorted(f[:-3] for f in os.listdir(here) if f.endswith(".sx")) == sorted(progs)
-    for name, prog in progs.items():
-        assert open(os.path.join(here, name + ".sx")).read() == prog.text() + "\n", name
+    terms = named_terms()
+    assert {"c1_dotp", "c2_scanl1_i64", "c2_scanl1_f32", "c3_foldseg", "c4_histogram", "c5_jacobi_step"} <= set(terms)
+    assert sorted(f[:-3] for f in os.listdir(here) if f.endswith(".sx")) == sorted(terms)
+    for name, text in terms.items():
+        assert open(os.path.join(here, name + ".sx")).read() == text + "\n", name
+
+
+def test_committed_term_texts_are_accepted_by_the_library(cc_ctx):
+    # and the library reads every one of them as it stands in the file
+    import os
+    here = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "terms")
+    for f in sorted(os.listdir(here)):
+        if f.endswith(".sx"):
+            try:
+                assert cc_ctx.compile(open(os.path.join(here, f)).read().rstrip("\n")).num_kernels >= 0
+            except Exception as e:
+                pytest.fail("%s: %s" % (f, e))
 
 
 def test_unknown_wire_version_is_refused(cc_ctx):
