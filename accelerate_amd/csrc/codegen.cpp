@@ -952,6 +952,8 @@ static std::string streamHead(const char* ret, const char* name, const char* par
 
 static void structLayout(const std::vector<ST>& leaves, int& size, int& align);
 
+static int structWords(const std::vector<ST>& leaves);
+
 KernelSource Codegen::fold(const Sx& f, const Sx* seed, const Operand& src) {
   const TypeP elt = src.r.elt;
   std::string body;
@@ -1010,6 +1012,7 @@ KernelSource Codegen::fold(const Sx& f, const Sx* seed, const Operand& src) {
   }
   KernelSource ks = finish(body, elt, leaves, "scan.hpp+fold.hpp", vec);
   ks.commutative = comm;
+  ks.words = structWords(leaves);
   ks.group = g;
   ks.block = 256;
   ks.streaming = true;

@@ -12,10 +12,17 @@
 //     which keeps operands strictly left to right (associativity only).
 // Wave results meet in LDS and are combined in wave order.  With bpr > 1 the chunk
 // results go to `tmp` (rows x bpr) and acc_fold_final reduces them, again in order, and
-// applies the seed exactly once on the left.  (Letting the workgroup that delivers a row's
-// last partial do that reduction saves the second launch but needs device-wide fences around
-// the count, which write back and invalidate the XCD's whole L2 under the streaming
-// workgroups: dotp over 2^28 elements went from 0.37 to 0.44 ms, over 2^24 from 23 to 86 us.)
+// applies the seed exactly once on the left.
+// A fold of a single row needs no second launch: every workgroup publishes its chunk's result
+// as self-validating words (acc_publish of scan.hpp: value and the launch's tag in one relaxed
+// 64-bit store, no fence); the workgroup of the row's last chunk, which the hardware starts last,
+// then reads the others' words -- valid exactly when they carry this launch's tag, polled under
+// the same bounded wait as the scans' look-back -- and reduces them in order.  It waits for
+// nobody who needs its place: a fold launches at most `fold_target` workgroups.  (Measured and
+// rejected: a counter of finished workgroups, whose last increment elects the reducer -- 2048
+// atomics on one address cost more than the launch they save, dotp over 2^24 elements 23 -> 40
+// us; and before that a release / acquire pair around such a count: the fences write back and
+// invalidate the XCD's whole L2 under the streaming workgroups, 2^28 elements 0.37 -> 0.44 ms.)
 
 struct FoldParams {
   i64 rows;   // number of outer rows
@@ -23,6 +30,11 @@ struct FoldParams {
   i64 bpr;    // workgroups per row
   i64 chunk;  // elements per workgroup (multiple of ACC_WAVES * 64 * V)
   i64 first;  // number of the launch's first workgroup: more workgroups than a launch holds take several
+  // one launch for a single row (null desc: chunk results go to tmp for acc_fold_final)
+  u64* desc;        // bpr descriptors of AccWords<Elt>::N words
+  u64 epoch;        // tag of this launch
+  u64 spin_limit;   // polls after which the last workgroup stops waiting for a chunk's words
+  u32* err;         // host-visible word: 3 = it gave up
 };
 
 template <class S, class Src>
@@ -148,6 +160,25 @@ template <class S> struct AccFoldSrcTmp {
   __device__ __forceinline__ typename S::Elt operator()(i64 i) const { return S::load(tmp, i); }
 };
 
+// chunk results published by the workgroups of this launch: waits (bounded) until the words carry the launch's tag
+template <class S> struct AccFoldSrcDesc {
+  const u64* desc;
+  u64 epoch, limit;
+  u32* err;
+  __device__ __forceinline__ typename S::Elt operator()(i64 i) const {
+    typename S::Elt v;
+    u64 polls = 0;
+    while (acc_try_read<typename S::Elt>(desc + i * AccWords<typename S::Elt>::N, v, epoch) == 0) {
+      if (++polls >= limit) {
+        __hip_atomic_store(err, 3u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+        break;
+      }
+      __builtin_amdgcn_s_sleep(8);
+    }
+    return v;
+  }
+};
+
 template <class S>
 ACC_DEV void acc_fold_finish(const typename S::Env& env, const typename S::Out& out, i64 row, bool have,
                              const typename S::Elt& r) {
@@ -173,6 +204,17 @@ ACC_DEV void acc_fold_main_body(const Spec::Env& env, const Spec::Out& out, cons
   bool have = acc_fold_block<S>(env, src, row * p.n, lo, hi, r);
   if (p.bpr == 1) {
     acc_fold_finish<S>(env, out, row, have, r);
+  } else if (p.desc) {
+    // a single row, one launch (every chunk holds elements: `have` is true in thread 0)
+    const int W = AccWords<S::Elt>::N;
+    if (threadIdx.x == 0) acc_publish<S::Elt>(p.desc + b * W, r, p.epoch, 1);
+    if (b == p.bpr - 1) {
+      __syncthreads();  // (the reduction below reuses the LDS of the one above)
+      AccFoldSrcDesc<S> parts{p.desc, p.epoch, p.spin_limit, p.err};
+      S::Elt t;
+      const bool any = acc_fold_block<S>(env, parts, 0, 0, p.bpr, t);
+      acc_fold_finish<S>(env, out, row, any, t);
+    }
   } else if (threadIdx.x == 0 && have) {
     S::store(tmp, bid, r);
   }

@@ -1194,8 +1194,12 @@ AValP Program::eval(const Sx& n, AEnv& aenv) {
     int64_t chunk = ((len + bpr - 1) / bpr + tile - 1) / tile * tile;
     if (chunk == 0) chunk = tile;
     bpr = std::max<int64_t>(1, (len + chunk - 1) / chunk);
+    const int64_t most = std::max<int64_t>(1, std::min<int64_t>(ctx_.knobs.fold_max_blocks, 0xffffffffLL / 256));
+    // A single row cut into chunks is finished by the workgroup that publishes last (no second
+    // launch): the chunk results travel as tagged words in the scans' descriptor memory.
+    const bool oneLaunch = rows == 1 && bpr > 1 && bpr <= most && ctx_.knobs.fold_one_launch != 0;
     DArrayP tmp = out;
-    if (bpr > 1) {
+    if (bpr > 1 && !oneLaunch) {
       ArrayR tr = plan.ty->r;
       tr.rank = 1;
       tmp = alloc(tr, {rows * bpr});
@@ -1208,15 +1212,24 @@ AValP Program::eval(const Sx& n, AEnv& aenv) {
     args.push_back((uint64_t)bpr);
     args.push_back((uint64_t)chunk);
     args.push_back(0);  // FoldParams::first
+    const size_t firstAt = args.size() - 1;
+    if (oneLaunch) {
+      ScanState& ss = ctx_.scanState((size_t)bpr * plan.k->meta.words * sizeof(uint64_t));
+      args.push_back((uint64_t)(uintptr_t)ss.desc);
+      args.push_back((uint64_t)ss.epoch);
+      args.push_back((uint64_t)std::max<long long>(1, ctx_.knobs.scan_spin_limit));
+      args.push_back((uint64_t)(uintptr_t)ctx_.errorWord());
+    } else {
+      for (int k = 0; k < 4; ++k) args.push_back(0);
+    }
     const bool st = streams(plan.k->meta, aenv, temps, 0);
     // a launch holds fewer than 2^32 threads: more rows than that many workgroups take several launches
-    const int64_t most = std::max<int64_t>(1, std::min<int64_t>(ctx_.knobs.fold_max_blocks, 0xffffffffLL / 256));
     for (int64_t first = 0; first < rows * bpr; first += most) {
-      args.back() = (uint64_t)first;
+      args[firstAt] = (uint64_t)first;
       ctx_.launch(plan.k, st ? "acc_fold_main_stream" : "acc_fold_main", (uint64_t)std::min(most, rows * bpr - first), 256, args);
     }
-    args.back() = 0;
-    if (bpr > 1) ctx_.launch(plan.k, "acc_fold_final", (uint64_t)rows, 256, args);
+    args[firstAt] = 0;
+    if (bpr > 1 && !oneLaunch) ctx_.launch(plan.k, "acc_fold_final", (uint64_t)rows, 256, args);
     return avArr(out);
   }
   if (h == "permute") {

@@ -58,7 +58,7 @@ const KnobName kKnobs[] = {
     {"fold_target", &Knobs::fold_target},         {"fold_max_blocks", &Knobs::fold_max_blocks},         {"permute_parts", &Knobs::permute_parts},
     {"permute_count", &Knobs::permute_count},     {"permute_groups", &Knobs::permute_groups},
     {"permute_partials", &Knobs::permute_partials}, {"permute_fresh", &Knobs::permute_fresh}, {"stencil_chain", &Knobs::stencil_chain},
-    {"pool_async", &Knobs::pool_async},
+    {"pool_async", &Knobs::pool_async}, {"fold_one_launch", &Knobs::fold_one_launch},
     {"stencil_no2d", &Knobs::stencil_no2d},       {"stencil_no3d", &Knobs::stencil_no3d},
     {"scan_tiles", &Knobs::scan_tiles},           {"scan_spin_limit", &Knobs::scan_spin_limit},
     {"scan_test_skew", &Knobs::scan_test_skew},

@@ -96,6 +96,27 @@ def test_fold_over_several_launches(gpu_ctx, knobs):
         assert same(gpu_ctx.compile(P.fold_sum(A.i64, 2))(x), x.sum(axis=1))
 
 
+@pytest.mark.parametrize("one_launch", [0, 1])
+def test_single_row_with_and_without_the_second_launch(gpu_ctx, knobs, one_launch):
+    # a single row cut into chunks: either a second launch combines the chunk results, or the
+    # workgroup of the last chunk does, reading the others' results as tagged words; both in order
+    # (the maximum segment sum's operator is not commutative), several calls in a row so that
+    # words left by one call are met by the next, and at lengths where the last chunk is ragged
+    knobs("fold_one_launch", one_launch)
+    rng = np.random.default_rng(79)
+    run = gpu_ctx.compile(Q.mss(A.Int, 1))
+    total = gpu_ctx.compile(P.fold_sum(A.i64, 1, 7))
+    for n in (2_000_001, 300_000, 5_000_017, 70_001):
+        x = rng.integers(-50, 50, n).astype(np.int64)
+        c = np.concatenate(([0], np.cumsum(x)))
+        assert int(run(x)) == int((c - np.minimum.accumulate(c)).max()), n
+        assert int(total(x)) == 7 + int(x.sum()), n
+    a, b = W.uniform_f32(1 << 24, 11, 0.0, 1.0), W.uniform_f32(1 << 24, 12)
+    got = float(gpu_ctx.compile(P.dotp())(a, b))
+    ref = float(np.dot(a.astype(np.float64), b.astype(np.float64)))
+    assert abs(got - ref) <= 1e-4 * float(np.sum(np.abs(a.astype(np.float64) * b)))
+
+
 def test_rows_split_over_workgroups_are_combined_in_order(gpu_ctx):
     # rows long enough for several workgroups each, whose partial results a second launch
     # combines: a non-commutative operator (the maximum segment sum's) shows a partial out of
