@@ -155,7 +155,9 @@ class Workloads:
             g = W.uniform_f32(side * side, 16, 0.0, 1.0).reshape(side, side)
             return dict(name="Jacobi 3x3 cross, clamp, 8192x8192 Float32, per sweep of 100", prog=P.jacobi_step(),
                         tys=[A.tarray(2, A.f32)], args=[g], n=side * side, bytes=8 * side * side, kernel="acc_stencil2d",
-                        unit="Gcell/s", iterate=100, resident=True,   # a sweep reads what the previous one wrote (256 MiB) seq=lambda: OC.jacobi_f32(g, 2), omp=lambda: OC.omp_jacobi_f32(g, 4),
+                        unit="Gcell/s", iterate=100,
+                        resident=True,   # a sweep reads the 256 MiB the previous one wrote
+                        seq=lambda: OC.jacobi_f32(g, 2), omp=lambda: OC.omp_jacobi_f32(g, 4),
                         seq_units=2, omp_units=4, sample="2 (one core) / 4 (all cores) sweeps of the 100")
         raise KeyError(wid)
 
