@@ -1555,11 +1555,10 @@ AValP Program::eval(const Sx& n, AEnv& aenv) {
       const bool aligned = srcArr && !srcArr->bufs.empty() && ((uintptr_t)srcArr->bufs[0]->p & 15) == 0 &&
                            (rows == 1 || (len * eltBytes) % 16 == 0);
       const int64_t tprP = (len + pipeTile - 1) / pipeTile;
-      // measured on 2^28 elements: Float32 363 us against 396 us for a workgroup per tile; Int64 775
-      // against 760 (two descriptor words per tile make its look-back dearer), so elements of 8 bytes
-      // take it only when forced
+      // measured on 2^28 elements: Float32 364 us against 404 us for a workgroup per tile, Int64 714
+      // against 745
       pipe = aligned && (forcedTiles == 4 ? len >= pipeTile
-                                          : (forcedTiles == 0 && eltBytes == 4 && tprP >= 16 && rows * tprP >= 4 * ctx_.computeUnits()));
+                                          : (forcedTiles == 0 && tprP >= 16 && rows * tprP >= 4 * ctx_.computeUnits()));
     }
     const KernelP& kern = pipe ? plan.k3 : (small ? plan.k2 : plan.k);
     const KernelSource& m = kern->meta;
