@@ -3,7 +3,7 @@
 
 Headline (the JSON line's `value`, `roofline`, `cpu_baseline`): one step = one application of the
 prepared program `runN (scanl1 (+))` to a device-resident Int64 vector of 2^28 elements (one
-launch of the single-pass scan kernel), through the C ABI.  The same line carries, under
+launch of the pipelined single-pass scan kernel), through the C ABI.  The same line carries, under
 "configs", every benchmark configuration (dotp, both scans, foldSeg, histogram, Jacobi) and the
 2^28 map / dotp the bandwidth target is stated for, each with its own roofline entry and the CPU
 figures of the same workload on one core and on all host cores.  Every roofline figure, the
@@ -112,7 +112,7 @@ class Workloads:
         if wid == "scan_i64":
             x = self.vec("i64", n28, 20240601)
             return dict(name="scanl1 (+) Int64 n=2^28", prog=P.scanl1_sum(A.i64), tys=[A.tarray(1, A.i64)], args=[x],
-                        n=n28, bytes=16 * n28, kernel="acc_scan", unit="Gelem/s",
+                        n=n28, bytes=16 * n28, kernel="acc_scan_pipe", unit="Gelem/s",
                         seq=lambda: OC.scanl1_i64(x), omp=lambda: OC.omp_scanl1(x), sample="full workload")
         if wid == "scan_f32":
             x = self.vec("f01", n28, 11)
@@ -294,7 +294,7 @@ def main():
         "ms_per_step": round(wall, 5), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "int64", "data": "synthetic",
         "config": {"workload": "scanl1 (+) on an Int64 vector, n=2^28, uniform integers in [-1000,1000]",
-                   "program": "Scan LeftToRight (+) Nothing (Manifest (Avar a0))", "kernel": "acc_scan"},
+                   "program": "Scan LeftToRight (+) Nothing (Manifest (Avar a0))", "kernel": "acc_scan_pipe"},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": head["roofline"]["traffic"]},
         "cpu_baseline": cpu,
