@@ -86,3 +86,13 @@ def test_unknown_wire_version_is_refused(cc_ctx):
     assert cc_ctx.compile(bare).num_kernels >= 1               # a bare term is version 1
     with pytest.raises(hip.AccError, match="wire format version 2"):
         cc_ctx.compile("(acchip-ir 2 " + bare + ")")
+
+
+def test_scan_phase_stamps_still_fit_the_kernel():
+    # accelerate_amd/scan_phases.py rebuilds acc_scan_pipe with time stamps put in by text
+    # substitution: building it here shows that every place it names is still there and that the
+    # instrumented kernel compiles for gfx950
+    import os
+    from accelerate_amd import scan_phases
+    exe = scan_phases.build("i64")
+    assert os.path.exists(exe)
