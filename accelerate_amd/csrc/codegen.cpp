@@ -1204,7 +1204,10 @@ KernelSource Codegen::scan(const Sx& f, const Sx* seed, const Operand& src, bool
   if (pipe) {
     // bytes of elements a lane holds per tile of the pipelined kernel (ACCHIP_SCAN_PIPE_BYTES)
     const char* pb = std::getenv("ACCHIP_SCAN_PIPE_BYTES");
-    const int bytes = pb ? std::atoi(pb) : 128;
+    // 4-byte elements: 112 B, so that the rake area (57 KiB) fits beside the load buffer (112 KiB)
+    // and the next tile's loads can leave in the middle of the rake; 8-byte elements would have to
+    // come down to 96 B for that, which gains nothing over 128 B with the rake area over the buffer
+    const int bytes = pb ? std::atoi(pb) : (eltBytes == 4 ? 112 : 128);
     g = std::max(2, std::min(9, bytes / 16));
     const std::string T = stName(leaves[0]);
     const std::string at = "env." + slotByName(src.slot).name + "_0";

@@ -67,6 +67,9 @@ ACC_DEV i64 acc_uniform(i64 v) {
   return (i64)(((u64)hi << 32) | lo);
 }
 
+#ifndef ACC_PIPE_EARLY
+#define ACC_PIPE_EARLY 1      // with the rake area over the load buffer: waves beyond it send the next loads early
+#endif
 #ifndef ACC_PIPE_WINDOW
 #define ACC_PIPE_WINDOW 1     // predecessors a lane of the polling wave looks at per round trip (window = 64 x this)
 #endif
@@ -176,10 +179,18 @@ acc_scan_pipe(Spec::Env env, Spec::Out out, Spec::Out tot, ScanParams p) {
   __shared__ Elt sh_rake[kSep ? (G + 1) * ACC_SCAN_BLOCK : 1];
   static_assert(kSep || sizeof(Elt) * (G + 1) * ACC_SCAN_BLOCK <= sizeof(sh_buf), "rake area must fit the load buffer");
   Elt* const rk = kSep ? sh_rake : (Elt*)sh_buf;
+  // Waves whose part of the load buffer the rake area does not touch send the next tile's loads
+  // in the middle of the rake, as soon as the tile's aggregate has been published (all waves but
+  // the polling one when the rake area has LDS of its own); the others after the prefixes have
+  // been read back.  Sending them before the aggregate is out delays every successor's look-back
+  // (Float32, 112 B per lane: 409 us against 353).
+  constexpr int kRakeBytes = (int)sizeof(Elt) * (G + 1) * ACC_SCAN_BLOCK;
+  constexpr int kFirstEarly = kSep ? 1 : (ACC_PIPE_EARLY ? (kRakeBytes + G * 1024 - 1) / (G * 1024) : NW);
 
   const int tid = (int)threadIdx.x;
   const int lane = acc_lane();
   const int w = __builtin_amdgcn_readfirstlane(acc_wave());
+  const bool early = w >= kFirstEarly;
   const i64 tpf = p.tpr_full;            // full tiles per row: the pipeline's share
   const i64 total = p.rows * tpf;
   const i64 n = p.n;
@@ -243,7 +254,7 @@ acc_scan_pipe(Spec::Env env, Spec::Out out, Spec::Out tot, ScanParams p) {
     u64* rowDesc = p.desc + (u64)row * (u64)p.tpr * W;
     // the tile's elements are in LDS or on their way there; behind them only stores
     if (tailStores) {
-      if (w == 0 || kSep) acc_wait_vm<G>();
+      if (w == 0 || early) acc_wait_vm<G>();
       else acc_wait_vm<G - S2>();
     } else {
       acc_wait_vm<0>();
@@ -260,7 +271,6 @@ acc_scan_pipe(Spec::Env env, Spec::Out out, Spec::Out tot, ScanParams p) {
     // so the round trip is not waited for
     u64 nextRaw;
     if (ticketLane) acc_ticket_send(p.ticket, nextRaw);
-    const bool hadPrev = hasPrev;
     if (!kSep) acc_lds_barrier();  // every wave holds its elements: the buffer becomes the rake area
 
     // rake: entry e = g * 1024 + tid, chunk e / G, a chunk takes G + 1 slots
@@ -278,18 +288,13 @@ acc_scan_pipe(Spec::Env env, Spec::Out out, Spec::Out tot, ScanParams p) {
     Elt ts = acc_wave_scan<S>(env, c[G - 1], lane);
     const Elt chunkPre = acc_prev_lane(ts);  // everything of this wave before the lane's chunk (lane > 0)
     if (lane == ACC_WAVE - 1) sh_wtot[w] = ts;
-    if (kSep && ticketLane) {
+    if (ticketLane) {
       acc_ticket_receive<0>(nextRaw);
       sh_next = (i64)(nextRaw - p.ticket_base);
     }
     acc_lds_barrier();
-    i64 nxt = 0;
-    bool nextLoaded = false;
-    if (kSep) {
-      nxt = acc_uniform(sh_next);
-      nextLoaded = nxt < total;
-      if (w != 0 && nextLoaded) sendLoads(nxt);
-    }
+    const i64 nxt = acc_uniform(sh_next);
+    const bool nextLoaded = nxt < total;
     // every wave scans the 16 wave totals for itself
     Elt wt = sh_wtot[lane & (NW - 1)];
     wt = acc_wave_scan<S>(env, wt, lane);
@@ -312,6 +317,7 @@ acc_scan_pipe(Spec::Env env, Spec::Out out, Spec::Out tot, ScanParams p) {
 #pragma unroll
       for (int j = 1; j < G; ++j) rk[tid * (G + 1) + j] = hasPre ? S::combine(env, pre, c[j - 1]) : c[j - 1];
     }
+    if (early && w != 0 && nextLoaded) sendLoads(nxt);
     if (hasPrev && w != 0) storePrev(0, S1);
     acc_lds_barrier();
 #pragma unroll
@@ -325,15 +331,8 @@ acc_scan_pipe(Spec::Env env, Spec::Out out, Spec::Out tot, ScanParams p) {
     }
     if (hasPrev && w != 0) storePrev(S1, S2);
     if (!kSep) {
-      if (ticketLane) {
-        if (hadPrev) acc_ticket_receive<S2>(nextRaw);
-        else acc_ticket_receive<0>(nextRaw);
-        sh_next = (i64)(nextRaw - p.ticket_base);
-      }
-      acc_lds_barrier();  // the rake area has been read: the buffer may receive the next tile
-      nxt = acc_uniform(sh_next);
-      nextLoaded = nxt < total;
-      if (w != 0 && nextLoaded) sendLoads(nxt);
+      acc_lds_barrier();  // the rake area has been read: the whole buffer may receive the next tile
+      if (!early && w != 0 && nextLoaded) sendLoads(nxt);
     }
     if (w != 0 && hasPrev) storePrev(S2, G);
 

@@ -1,7 +1,8 @@
 """The pipelined scan kernel (persistent workgroups, direct global -> LDS loads; left scans over long
 rows of a plain array with elements of 4 or 8 bytes, Interpreter.hs:427-474), forced onto every
 case through the `scan_tiles` knob and compared with numpy and with the other tile variants.
-A tile of it holds 1024 lanes x 128 bytes: 16384 elements of 8 bytes, 32768 of 4."""
+A tile of it holds 1024 lanes x 128 bytes of 8-byte elements (16384 of them) or x 112 bytes of 4-byte
+elements (28672)."""
 import numpy as np
 import pytest
 
@@ -11,8 +12,8 @@ from . import progs as Q
 
 pytestmark = pytest.mark.gpu
 
-TYPES = [(A.i32, np.int32, 32768), (A.i64, np.int64, 16384), (A.f32, np.float32, 32768), (A.f64, np.float64, 16384),
-         (A.u32, np.uint32, 32768)]
+TYPES = [(A.i32, np.int32, 28672), (A.i64, np.int64, 16384), (A.f32, np.float32, 28672), (A.f64, np.float64, 16384),
+         (A.u32, np.uint32, 28672)]
 
 
 def _lengths(tile):
@@ -62,7 +63,7 @@ def test_several_rows(gpu_ctx, knobs, rows, n):
 
 def test_rows_that_are_not_16_byte_multiples_keep_the_other_kernels(gpu_ctx, knobs):
     knobs("scan_tiles", 4)
-    x = np.random.default_rng(1).integers(-1000, 1000, (3, 32768 * 16 + 3)).astype(np.int32)
+    x = np.random.default_rng(1).integers(-1000, 1000, (3, 28672 * 16 + 3)).astype(np.int32)
     assert np.array_equal(gpu_ctx.compile(P.scanl1_sum(A.i32, 2))(x), np.cumsum(x, axis=1, dtype=np.int32))
 
 
