@@ -6,9 +6,13 @@
 // stream of rows*n elements which is cut into equal tiles, and a tile reduces its elements
 // as (head flag, value) pairs under
 //     (fa, a) (+) (fb, b) = fb ? (1, b) : (fa, a (+) b)
-// which is associative whenever (+) is.  Tiles do not wait for each other: a tile leaves its
-// carry (head seen, value since the last head) and the one segment end that no head of the
-// tile precedes; acc_foldseg_fixup completes those ends from the carries of the tiles before.
+// which is associative whenever (+) is.  Tiles do not wait for each other: a tile publishes its
+// carry (head seen, value since the last head) and the one segment end that no head of the tile
+// precedes as tagged descriptor words.  The launch has a few workgroups more than tiles; they are
+// dispatched last, and complete those ends from the carries of the tiles before (acc_foldseg_fix),
+// most of which were published long before.  (A tile that completes its own end at its close, by
+// looking back itself, keeps its slot on the CU for a further round trip to memory: 134 us against
+// 121 for the benchmark's 2^27 values.)
 //
 // Boundaries: row r contributes S+1 boundaries at stream positions r*n + offs[s],
 // s = 0..S (S segments per row).  Boundary number j = r*(S+1) + s starts segment (r, s)
@@ -29,11 +33,145 @@ struct FoldSegParams {
   i64 total;   // rows * n
   i64 tiles;   // >= 1
   i64* part;   // [tiles + 1]: boundaries before each tile border; part[tiles] = rows * (S + 1)
-  void* carry;    // [tiles] (head seen, value since the last head) of each tile
-  void* pend;     // [tiles] value of the tile's one segment end that precedes all its heads
-  i64* pend_at;   // [tiles] boundary number of that end, or -1
+  u64* desc;   // [tiles] descriptors: a tile's carry, state 2 when the tile holds a head (or is the first), else 1
+  u64 epoch;   // tag of this launch in the descriptors
+  u64 spin_limit;  // polls after which a wait for a predecessor's carry gives up (reported as 3 through err)
   u32* err;       // host-visible word: 1 = "empty segment" (what the reference's boundsCheck reports)
 };
+
+// The carries as a scan sees them: the value since the tile's last head, combined in order; a
+// carry whose tile holds a head ends the walk like an inclusive prefix does.
+struct AccSegCarrySpec {
+  typedef Spec::Env Env;
+  typedef Spec::Elt Elt;
+  enum { V = AccSegSpec<Spec>::V, G = AccSegSpec<Spec>::G };
+  static constexpr bool kSeeded = false;
+  ACC_DEV Elt combine(const Env& env, const Elt& a, const Elt& b) { return Spec::combine(env, a, b); }
+  ACC_DEV Elt seed(const Env&) {
+    Elt r_{};
+    return r_;
+  }
+  ACC_DEV bool stops(const Elt&) { return false; }
+};
+
+ACC_DEV void acc_foldseg_publish(const FoldSegParams& p, i64 tile, const AccSegSpec<Spec>::Elt& carry) {
+  acc_publish<Spec::Elt>(p.desc + tile * AccWords<Spec::Elt>::N, carry.v, p.epoch, carry.f || tile == 0 ? 2 : 1);
+}
+
+// A tile's pending end: boundary number and the tile's share of the value; state 2 when the tile
+// has one, 1 when not.  The records follow the carries in the descriptor memory.
+struct AccSegPend {
+  Spec::Elt v;
+  i64 j;
+};
+ACC_DEV u64* acc_foldseg_pend_desc(const FoldSegParams& p, i64 tile) {
+  const i64 carries = (p.tiles * AccWords<Spec::Elt>::N + 1) & ~(i64)1;  // 16-byte aligned
+  return p.desc + carries + tile * AccWords<AccSegPend>::N;
+}
+ACC_DEV void acc_foldseg_publish_pend(const FoldSegParams& p, i64 tile, bool has, i64 j, const Spec::Elt& v) {
+  AccSegPend r{};
+  if (has) {
+    r.v = v;
+    r.j = j;
+  }
+  acc_publish<AccSegPend>(acc_foldseg_pend_desc(p, tile), r, p.epoch, has ? 2 : 1);
+}
+
+// Completes the end at boundary j whose value so far is v, from the carries of the tiles before
+// `tile`, 64 a step: called by a whole wave.  Those tiles were dispatched before the caller, so
+// their carries arrive without its help; the wait is bounded all the same (acc_window).
+ACC_DEV void acc_foldseg_pending(const Spec::Env& env, const Spec::Out& out, const FoldSegParams& p, i64 tile, i64 j, Spec::Elt v) {
+  typedef Spec S;
+  bool have = false;
+  S::Elt run;
+  i64 look = tile - 1;
+  while (look >= 0) {
+    S::Elt r;
+    int nv;
+    bool term;
+    acc_window<AccSegCarrySpec>(env, p.desc, look, p.epoch, p.spin_limit, p.err, r, nv, term);
+    if (nv > 0) {
+      run = have ? S::combine(env, r, run) : r;
+      have = true;
+    }
+    if (term) break;
+    look -= ACC_WAVE;
+  }
+  if (acc_lane() != 0) return;
+  if (have) v = S::combine(env, run, v);
+  const i64 sp1 = p.nseg + 1;
+  const i64 row = p.rows == 1 ? 0 : acc_quot(j, sp1), s = j - row * sp1;
+  if (s == 0) return;  // what precedes a row's first boundary belongs to no segment
+  S::store(out, row * p.nseg + s - 1, S::kSeeded ? S::combine(env, S::seed(env), v) : v);
+}
+
+// The workgroups behind the tiles: one lane per tile.  Nearly every pending end needs just the
+// carry of the tile before it (that tile holds a head), which the lanes fetch side by side; an
+// end whose segment began further back is walked by the whole wave.
+ACC_DEV void acc_foldseg_fix(const Spec::Env& env, const Spec::Out& out, const FoldSegParams& p, i64 group) {
+  typedef Spec S;
+  enum { NP = AccWords<AccSegPend>::N, NC = AccWords<Spec::Elt>::N };
+  const i64 t = group * (i64)ACC_SCAN_BLOCK + threadIdx.x;
+  const bool valid = t < p.tiles;
+  // the tile's record and the carry of the tile before it are asked for together: one trip to
+  // memory for nearly every lane (each word validates itself, so the words may arrive singly)
+  auto check = [&](const u64* x, int n) -> int {
+    const u64 tag0 = x[0] >> 32;
+    for (int q = 1; q < n; ++q)
+      if ((x[q] >> 32) != tag0) return 0;
+    if ((tag0 >> 2) != p.epoch) return 0;
+    const int st = (int)(tag0 & 3);
+    return st == 1 || st == 2 ? st : 0;
+  };
+  AccSegPend pr{};
+  S::Elt c{};
+  int st = valid ? 0 : 1, sc = 0;
+  for (u64 polls = 0; valid; ) {
+    u64 xa[NP], xb[NC];
+    const u64* pd = acc_foldseg_pend_desc(p, t);
+    const u64* cd = p.desc + (t > 0 ? t - 1 : 0) * NC;
+#pragma unroll
+    for (int q = 0; q < NP; ++q) xa[q] = __hip_atomic_load(pd + q, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+#pragma unroll
+    for (int q = 0; q < NC; ++q) xb[q] = __hip_atomic_load(cd + q, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    st = check(xa, NP);
+    sc = check(xb, NC);
+    if (st == 1 || (st == 2 && (t == 0 || sc != 0))) {
+      u32 wa[NP], wb[NC];
+#pragma unroll
+      for (int q = 0; q < NP; ++q) wa[q] = (u32)xa[q];
+#pragma unroll
+      for (int q = 0; q < NC; ++q) wb[q] = (u32)xb[q];
+      pr = acc_from_words<AccSegPend>(wa);
+      c = acc_from_words<S::Elt>(wb);
+      break;
+    }
+    if (++polls >= p.spin_limit) {
+      __hip_atomic_store(p.err, 3u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+      st = 1;
+      break;
+    }
+    __builtin_amdgcn_s_sleep(4);
+  }
+  const bool has = st == 2;
+  bool done = !has || t == 0;
+  S::Elt v = pr.v;
+  if (has && t > 0) {
+    v = S::combine(env, c, v);
+    done = sc == 2;
+  }
+  if (has && done) {
+    const i64 sp1 = p.nseg + 1;
+    const i64 row = p.rows == 1 ? 0 : acc_quot(pr.j, sp1), s = pr.j - row * sp1;
+    if (s != 0) S::store(out, row * p.nseg + s - 1, S::kSeeded ? S::combine(env, S::seed(env), v) : v);
+  }
+  u64 m = __ballot(has && !done);
+  while (m) {
+    const int src = __builtin_ctzll(m);
+    m &= m - 1;
+    acc_foldseg_pending(env, out, p, acc_shfl(t, src) - 1, acc_shfl(pr.j, src), acc_shfl(v, src));
+  }
+}
 
 // part[t] = number of boundaries that lie before position t * TILE of the stream.  One
 // thread per boundary j: the borders t * TILE in (position of boundary j-1, position of
@@ -310,7 +448,7 @@ ACC_DEV void acc_foldseg_tile(const Spec::Env& env, const Spec::Out& out, const 
     P t = sh_wave[lane < ACC_SCAN_WAVES ? lane : 0];
     t = acc_wave_scan<SS>(env, t, lane);
     if (lane < ACC_SCAN_WAVES) sh_wave[lane] = t;
-    if (lane == wavesWithData - 1) reinterpret_cast<P*>(p.carry)[tile] = t;
+    if (lane == wavesWithData - 1) acc_foldseg_publish(p, tile, t);
   }
   __syncthreads();
 
@@ -331,10 +469,7 @@ ACC_DEV void acc_foldseg_tile(const Spec::Env& env, const Spec::Out& out, const 
     }
   }
   __syncthreads();
-  if (threadIdx.x == 0) {
-    p.pend_at[tile] = sh_pend_at == NOPEND ? (i64)-1 : j0 + sh_pend_at;
-    if (sh_pend_at != NOPEND) reinterpret_cast<P*>(p.pend)[tile].v = sh_pend;
-  }
+  if (threadIdx.x == 0) acc_foldseg_publish_pend(p, tile, sh_pend_at != NOPEND, j0 + sh_pend_at, sh_pend);
   // the staged segments, in the order of their boundaries
   {
     const i64 inTile = jend - j0 + 1;  // boundary numbers the tile can have met, relative to j0
@@ -512,8 +647,7 @@ ACC_DEV void acc_foldseg_tile_fast(const Spec::Env& env, const Spec::Out& out, c
   const bool hasWavePre = w > 0 && w <= wavesWithData;
   P wavePre = sh_wave[0];
   for (int i = 1; i < w; ++i) wavePre = SS::combine(env, wavePre, sh_wave[i]);
-  if (w == wavesWithData - 1 && lane == 0)
-    reinterpret_cast<P*>(p.carry)[tile] = w > 0 ? SS::combine(env, wavePre, waveTot) : waveTot;
+  if (w == wavesWithData - 1 && lane == 0) acc_foldseg_publish(p, tile, w > 0 ? SS::combine(env, wavePre, waveTot) : waveTot);
 
   auto write = [&](int idx, const S::Elt& v) {
     const i64 j = j0 + idx;
@@ -578,10 +712,7 @@ ACC_DEV void acc_foldseg_tile_fast(const Spec::Env& env, const Spec::Out& out, c
     }
   }
   __syncthreads();
-  if (threadIdx.x == 0) {
-    p.pend_at[tile] = sh_pend_at == NOPEND ? (i64)-1 : j0 + sh_pend_at;
-    if (sh_pend_at != NOPEND) reinterpret_cast<P*>(p.pend)[tile].v = sh_pend;
-  }
+  if (threadIdx.x == 0) acc_foldseg_publish_pend(p, tile, sh_pend_at != NOPEND, j0 + sh_pend_at, sh_pend);
   {
     const i64 inTile = jend - j0 + 1;
     const int top = inTile < ACC_FOLDSEG_STAGE ? (int)inTile : ACC_FOLDSEG_STAGE;
@@ -602,6 +733,10 @@ acc_foldseg(Spec::Env env, Spec::Out out, FoldSegParams p) {
   __shared__ int sh_pend_at;
   __shared__ Spec::Elt sh_stage[ACC_FOLDSEG_STAGE];
   __shared__ u32 sh_staged[ACC_FOLDSEG_STAGE / 32];
+  if ((i64)blockIdx.x >= p.tiles) {
+    acc_foldseg_fix(env, out, p, (i64)blockIdx.x - p.tiles);
+    return;
+  }
   const bool full = ((i64)blockIdx.x + 1) * (i64)C::TILE <= p.total;
   // (clamped: offsets that do not ascend leave entries of part unwritten)
   const i64 nb = p.rows * (p.nseg + 1);
@@ -623,73 +758,8 @@ acc_foldseg(Spec::Env env, Spec::Out out, FoldSegParams p) {
   }
 }
 
-// One wave per tile that has a pending end: walk back over the carries of the preceding
-// tiles, a window of 64 at a time, up to the nearest tile that contains a head (or the
-// start of the stream), combine them in order and complete the end.
-extern "C" __global__ void __launch_bounds__(ACC_BLOCK)
+// the same completion as a launch of its own (the knob that compares the two)
+extern "C" __global__ void __launch_bounds__(ACC_SCAN_BLOCK)
 acc_foldseg_fixup(Spec::Env env, Spec::Out out, FoldSegParams p) {
-  typedef Spec S;
-  typedef AccSegSpec<Spec> SS;
-  typedef SS::Elt P;
-  const int lane = acc_lane();
-  const i64 tile = (i64)blockIdx.x * (ACC_BLOCK / ACC_WAVE) + acc_wave();
-  if (tile >= p.tiles) return;
-  const i64 j = p.pend_at[tile];
-  if (j < 0) return;
-  const P* carry = reinterpret_cast<const P*>(p.carry);
-  S::Elt v = reinterpret_cast<const P*>(p.pend)[tile].v;
-  bool have = false;
-  S::Elt run;
-  // one window of 64 carries: returns true when the walk ends in it
-  auto window = [&](i64 look, const P& c) {
-    const i64 idx = look - lane;
-    const u64 mHead = __ballot(idx >= 0 && c.f != 0);
-    const int first = mHead ? __builtin_ctzll(mHead) : ACC_WAVE;
-    const int nvalid = look + 1 < ACC_WAVE ? (int)(look + 1) : ACC_WAVE;
-    const int nv = first < ACC_WAVE ? first + 1 : nvalid;
-    // earlier tiles sit in higher lanes: fold them in from the left
-    S::Elt r = c.v;
-#pragma unroll
-    for (int d = 1; d < ACC_WAVE; d <<= 1) {
-      S::Elt o = acc_shfl_down(r, d);
-      if (lane + d < nv) r = S::combine(env, o, r);
-    }
-    run = have ? S::combine(env, r, run) : r;
-    have = true;
-    return first < ACC_WAVE;
-  };
-  // The nearest window usually ends the walk.  A segment that spans many tiles is walked
-  // eight windows at a time, their loads issued together: one memory round trip per 512
-  // tiles instead of one per 64.
-  enum { U = 8 };
-  i64 look = tile - 1;
-  bool done = look < 0;
-  if (!done) {
-    P c{};
-    if (look - lane >= 0) c = carry[look - lane];
-    done = window(look, c);
-    look -= ACC_WAVE;
-  }
-  while (!done && look >= 0) {
-    P c[U];
-#pragma unroll
-    for (int u = 0; u < U; ++u) {
-      const i64 idx = look - (i64)u * ACC_WAVE - lane;
-      c[u] = P{};
-      if (idx >= 0) c[u] = carry[idx];
-    }
-#pragma unroll
-    for (int u = 0; u < U; ++u) {
-      if (!done && look >= 0) {
-        done = window(look, c[u]);
-        look -= ACC_WAVE;
-      }
-    }
-  }
-  if (lane != 0) return;
-  if (have) v = S::combine(env, run, v);
-  const i64 sp1 = p.nseg + 1;
-  const i64 row = p.rows == 1 ? 0 : acc_quot(j, sp1), s = j - row * sp1;
-  if (s == 0) return;  // what precedes a row's first boundary belongs to no segment
-  S::store(out, row * p.nseg + s - 1, S::kSeeded ? S::combine(env, S::seed(env), v) : v);
+  acc_foldseg_fix(env, out, p, (i64)blockIdx.x);
 }

@@ -1214,7 +1214,8 @@ AValP Program::eval(const Sx& n, AEnv& aenv) {
     args.push_back(0);  // FoldParams::first
     const size_t firstAt = args.size() - 1;
     if (oneLaunch) {
-      ScanState& ss = ctx_.scanState((size_t)bpr * plan.k->meta.words * sizeof(uint64_t));
+      const size_t descBytes = (size_t)bpr * plan.k->meta.words * sizeof(uint64_t);
+      ScanState& ss = noAlloc_ ? staticScanState(ctx_.device(), ctx_.stream(), descBytes) : ctx_.scanState(descBytes);
       args.push_back((uint64_t)(uintptr_t)ss.desc);
       args.push_back((uint64_t)ss.epoch);
       args.push_back((uint64_t)std::max<long long>(1, ctx_.knobs.scan_spin_limit));
@@ -1467,14 +1468,14 @@ AValP Program::eval(const Sx& n, AEnv& aenv) {
     const int64_t tile = (int64_t)m.block * m.group * m.vec;
     const int64_t total = rows * len;
     const int64_t tiles = std::max<int64_t>(1, (total + tile - 1) / tile);
-    if (tiles > 0x7ffffff0LL) throw Error("foldSeg: too many tiles for one launch");
+    if (tiles > 0x7f000000LL) throw Error("foldSeg: too many tiles for one launch");
     ArrayR pr;
     pr.rank = 1;
     pr.elt = tScalar(ST::I64);
     DArrayP part = alloc(pr, {tiles + 1});
-    // per tile: its carry and its pending end, both (value, head flag) records of m.words words
-    const int64_t recs = (tiles * (int64_t)m.words * 4 + 7) / 8;
-    DArrayP carry = alloc(pr, {recs}), pend = alloc(pr, {recs}), pendAt = alloc(pr, {tiles});
+    // per tile a descriptor of its carry and one of its pending end (value + boundary number), in
+    // the scans' descriptor memory
+    ScanState& st = ctx_.scanState((size_t)tiles * (2 * (size_t)m.words + 4) * sizeof(uint64_t));
     std::vector<uint64_t> args = packArgs(m, aenv, temps, {});
     packOut(args, *out);
     args.push_back((uint64_t)rows);
@@ -1483,15 +1484,21 @@ AValP Program::eval(const Sx& n, AEnv& aenv) {
     args.push_back((uint64_t)total);
     args.push_back((uint64_t)tiles);
     args.push_back((uint64_t)(uintptr_t)part->bufs[0]->p);
-    args.push_back((uint64_t)(uintptr_t)carry->bufs[0]->p);
-    args.push_back((uint64_t)(uintptr_t)pend->bufs[0]->p);
-    args.push_back((uint64_t)(uintptr_t)pendAt->bufs[0]->p);
+    args.push_back((uint64_t)(uintptr_t)st.desc);
+    args.push_back((uint64_t)st.epoch);
+    args.push_back((uint64_t)std::max<long long>(1, ctx_.knobs.scan_spin_limit));
     args.push_back((uint64_t)(uintptr_t)ctx_.errorWord());
     const int64_t boundaries = rows * (nseg + 1);
     if ((boundaries + 255) / 256 > 0x7fffffffLL) throw Error("foldSeg: too many segments for one launch");
     ctx_.launch(plan.k, "acc_foldseg_partition", (uint64_t)((boundaries + 255) / 256), 256, args);
-    ctx_.launch(plan.k, "acc_foldseg", (uint64_t)tiles, (unsigned)m.block, args);
-    ctx_.launch(plan.k, "acc_foldseg_fixup", (uint64_t)((tiles + 3) / 4), 256, args);
+    // behind the tiles, the workgroups that complete the segment ends reaching across tile borders
+    const uint64_t fixGroups = (uint64_t)((tiles + m.block - 1) / m.block);
+    if (ctx_.knobs.foldseg_one_launch != 0) {
+      ctx_.launch(plan.k, "acc_foldseg", (uint64_t)tiles + fixGroups, (unsigned)m.block, args);
+    } else {
+      ctx_.launch(plan.k, "acc_foldseg", (uint64_t)tiles, (unsigned)m.block, args);
+      ctx_.launch(plan.k, "acc_foldseg_fixup", fixGroups, (unsigned)m.block, args);
+    }
     return avArr(out);
   }
   if (h == "scan" || h == "scan'") {

@@ -51,6 +51,7 @@ struct Knobs {
   long long map_tiled = -1;         // -1: decide per launch, 0 / 1: never / always tile index-permuting producers
   long long fold_rows = -1;         // -1 / 0 / 1: the several-rows-per-workgroup fold
   long long fold_target = 2048;     // workgroups a fold aims at
+  long long foldseg_one_launch = 1; // 0: the ends that reach across tile borders are completed by a launch of their own
   long long fold_one_launch = 1;    // 0: a single row cut into chunks always takes the second launch (acc_fold_final)
   long long fold_max_blocks = (long long)1 << 24;  // workgroups per launch of the fold skeleton
   long long permute_parts = 128;    // LDS-fuls of destination the privatised permute accepts

@@ -38,6 +38,9 @@ LLC_BYTES = 256 << 20   # MI355X last-level (memory-side) cache
 TRAFFIC_FILE = os.path.join(ROOT, "profiles", "traffic.json")
 
 
+WARMUP_FLOOR_MS = 40.0
+
+
 def log(*a):
     print(*a, file=sys.stderr, flush=True)
 
@@ -45,9 +48,17 @@ def log(*a):
 def time_steps(ctx, run, args, steps, warmup):
     """(wall ms per step over exactly `steps` applications, list of per-step ms between events)"""
     res = None
+    t0 = time.perf_counter()
     for _ in range(warmup):
         res = run.execute(*args)
     ctx.sync()
+    # Short steps: W of them end before the device has settled (foldSeg, 0.12 ms a step: 0.54 of
+    # the roofline after 10 warm-up steps, 0.60 after 200 and after 1000), so the untimed part
+    # lasts WARMUP_FLOOR_MS at least.  The timed part is exactly `steps` steps either way.
+    while warmup > 0 and (time.perf_counter() - t0) * 1e3 < WARMUP_FLOOR_MS:
+        for _ in range(10):
+            res = run.execute(*args)
+        ctx.sync()
     ev = [ctx.event()]
     t0 = time.perf_counter()
     for _ in range(steps):
@@ -299,6 +310,7 @@ def main():
                      "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": head["roofline"]["traffic"]},
         "cpu_baseline": cpu,
         "transfer": transfer,
+        "warmup_floor_ms": WARMUP_FLOOR_MS,
     }
 
     # ---- every configuration, with its own roofline and CPU figures -------------------------

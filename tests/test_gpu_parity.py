@@ -198,11 +198,15 @@ def test_foldseg_2pow27_bit_exact(gpu_ctx):
     assert np.all(got[lens == 0] == 0)
 
 
+@pytest.mark.parametrize("one_launch", [1, 0], ids=["ends completed in the launch", "ends completed by a second launch"])
 @pytest.mark.parametrize("shape", ["one giant segment", "giants and dwarfs", "runs of empty segments",
                                    "empty segments at the end", "single elements"])
-def test_foldseg_segment_shapes_bit_exact(gpu_ctx, shape):
+def test_foldseg_segment_shapes_bit_exact(gpu_ctx, knobs, shape, one_launch):
     # segments that span hundreds of tiles (the carries of many tiles are chained), tiles
-    # with far more boundaries than elements (runs of empty segments), and length-1 segments
+    # with far more boundaries than elements (runs of empty segments), and length-1 segments;
+    # the ends that reach across tile borders completed by the workgroups behind the tiles, or
+    # by the same code as a launch of its own
+    knobs("foldseg_one_launch", one_launch)
     rng = np.random.default_rng(77)
     total = 1 << 23
     if shape == "one giant segment":
@@ -222,6 +226,21 @@ def test_foldseg_segment_shapes_bit_exact(gpu_ctx, shape):
     vals = rng.integers(-1000, 1000, total).astype(np.int32)
     got = gpu_ctx.compile(P.foldseg_sum())(vals, lens)
     assert np.array_equal(got, OC.foldseg_i32(vals, lens))
+
+
+def test_foldseg_calls_in_a_row_do_not_see_each_others_carries(gpu_ctx):
+    # the carries of the tiles travel as tagged words in memory that the next call uses again:
+    # a long call, a shorter one whose tiles end elsewhere, the long one again
+    run = gpu_ctx.compile(P.foldseg_sum())
+    rng = np.random.default_rng(5)
+    cases = []
+    for total, mean in ((1 << 22, 3000), (1 << 20, 70000), (1 << 22, 9000)):
+        lens = rng.integers(0, 2 * mean, total // mean).astype(np.int64)
+        lens = lens[np.cumsum(lens) <= total]
+        lens = np.append(lens, total - lens.sum()).astype(np.int32)
+        cases.append((rng.integers(-1000, 1000, total).astype(np.int32), lens))
+    for vals, lens in cases + cases[::-1]:
+        assert np.array_equal(run(vals, lens), OC.foldseg_i32(vals, lens))
 
 
 def test_histogram_2pow26_bit_exact(gpu_ctx):
