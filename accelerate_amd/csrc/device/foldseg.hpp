@@ -10,9 +10,14 @@
 // carry (head seen, value since the last head) and the one segment end that no head of the tile
 // precedes as tagged descriptor words.  The launch has a few workgroups more than tiles; they are
 // dispatched last, and complete those ends from the carries of the tiles before (acc_foldseg_fix),
-// most of which were published long before.  (A tile that completes its own end at its close, by
-// looking back itself, keeps its slot on the CU for a further round trip to memory: 134 us against
-// 121 for the benchmark's 2^27 values.)
+// most of which were published long before.  Measured on 2^27 values in 2^20 segments, against
+// 111 us for the three launches scan, partition, tiles + completion: a tile that completes its own
+// end at its close, by looking back itself, keeps its slot on the CU for a further round trip to
+// memory (+10 us and more); the borders numbered by workgroups in front of the tiles of the same launch
+// and read by the tiles as tagged words cost every tile a slower first load and a barrier
+// (+3 us); the borders left by the scan that produces the offsets, as it stores them, lengthen
+// that scan, whose few hundred workgroups are one dependent chain each, by as much as the
+// partition kernel takes (8.5 -> 13.7 us).
 //
 // Boundaries: row r contributes S+1 boundaries at stream positions r*n + offs[s],
 // s = 0..S (S segments per row).  Boundary number j = r*(S+1) + s starts segment (r, s)
@@ -151,7 +156,7 @@ ACC_DEV void acc_foldseg_fix(const Spec::Env& env, const Spec::Out& out, const F
       st = 1;
       break;
     }
-    __builtin_amdgcn_s_sleep(4);
+    __builtin_amdgcn_s_sleep(32);  // the last tiles are still at work: ask again in a microsecond
   }
   const bool has = st == 2;
   bool done = !has || t == 0;
