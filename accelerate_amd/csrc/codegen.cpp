@@ -1135,7 +1135,8 @@ KernelSource Codegen::foldSeg(const Sx& f, const Sx* seed, const Operand& src, c
 // array in memory (nothing fused into it) whose elements are one scalar of 4 or 8 bytes, read
 // left to right.
 bool Codegen::scanPipeable(const Operand& src, bool right) {
-  if (src.delayed || right) return false;
+  (void)right;  // both directions: a right scan walks over the row's mirror image
+  if (src.delayed) return false;
   auto leaves = typeLeaves(src.r.elt);
   return leaves.size() == 1 && !stIsVec(leaves[0]) && (stSize(leaves[0]) == 4 || stSize(leaves[0]) == 8);
 }
@@ -1237,6 +1238,7 @@ KernelSource Codegen::scan(const Sx& f, const Sx* seed, const Operand& src, bool
   ks.block = pipe ? 1024 : block;
   ks.group = g;
   ks.words = structWords(leaves);
+  ks.scanRight = right;
   return ks;
 }
 

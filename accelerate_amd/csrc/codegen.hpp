@@ -59,6 +59,7 @@ struct KernelSource {
   int block = 256;                    // threads per workgroup of the main kernel
   bool commutative = false;
   bool streaming = false;             // has acc_*_stream entry points (non-temporal variant)
+  bool scanRight = false;             // scan only: a right scan
   std::string permuteMode;            // permute only: "atomic", "cas", "lock", "store"
   bool permuteCount = false;          // permute only: has acc_permute_count (sum of a constant per source)
   bool permuteCountSet = false;       // permute only: has count_set (defaults of one constant, written with the counts)

@@ -1,4 +1,4 @@
-// Left scans over long rows of a plain array (Interpreter.hs:427-474), as a pipeline inside
+// Scans over long rows of a plain array (Interpreter.hs:427-474, right scans :513-560), as a pipeline inside
 // persistent workgroups: one workgroup of 1024 threads per CU walks over tiles that it takes from
 // the ticket counter, and the three things a tile needs from memory overlap with the phases
 // that need nothing from it.
@@ -14,6 +14,11 @@
 //    that one load or store instruction of the workgroup covers 16 KiB of consecutive
 //    addresses; all accesses carry the non-temporal hint.  A persistent copy of this shape
 //    reaches 6.0 TB/s on MI355X against 5.3 for wave-contiguous rows without the hint.
+//
+// A right scan is the same walk over the row's mirror image: tile t of the walk lies t tiles from
+// the row's end, a lane asks for the 16 bytes at the mirrored place (they arrive in its own
+// stretch of the buffer all the same: the lane's offset into memory is free, its place in LDS is
+// not), reads them back to front, and stores its results reversed.
 //
 // Order inside a tile: position = (g * 1024 + thread) * V + k.  Lane-local scan of the V
 // elements, then the 1024 * G lane totals are raked through LDS by the whole workgroup (every
@@ -49,6 +54,7 @@ ACC_DEV void acc_dma16(const void* g, u32 laneOff, u32 ldsBase) {
 // address = wave-uniform base + a lane's 32-bit byte offset: one register per lane serves every row of a tile
 template <class T> ACC_DEV T* acc_at(T* base, u32 byteOff) { return (T*)((char*)base + byteOff); }
 template <class T> ACC_DEV const T* acc_at(const T* base, u32 byteOff) { return (const T*)((const char*)base + byteOff); }
+template <class T> ACC_DEV T* acc_back(T* base, u32 byteOff) { return (T*)((char*)base - byteOff); }
 // wait until at most N of this wave's vector memory operations are outstanding (they complete in issue order)
 template <int N> ACC_DEV void acc_wait_vm() { asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory"); }
 // workgroup barrier that orders LDS accesses only (a full fence would also wait for loads in flight)
@@ -216,17 +222,21 @@ acc_scan_pipe(Spec::Env env, Spec::Out out, Spec::Out tot, ScanParams p) {
 
   // the lane's 16 bytes of row g lie at element (g * 1024 + tid) * V of the tile: g * 16 KiB + tid * 16 bytes
   const u32 laneOff = (u32)tid * 16u;
+  constexpr bool R = S::kRight;
+  // where the lane's 16 bytes of a row lie in memory, relative to the row's (mirrored: last) 16 KiB
+  const u32 loadOff = R ? (u32)(ACC_SCAN_BLOCK - 1 - tid) * 16u : laneOff;
   auto sendLoads = [&](i64 gt) {
     const i64 row = gt / tpf, tile = gt - row * tpf;
-    const Raw* src = inP + row * n + tile * (i64)C::TILE;
+    const Raw* src = R ? inP + row * n + (n - (tile + 1) * (i64)C::TILE) : inP + row * n + tile * (i64)C::TILE;
 #pragma unroll
-    for (int g = 0; g < G; ++g) acc_dma16(src + (i64)g * ACC_SCAN_BLOCK * V, laneOff, myLds + (u32)g * 1024u);
+    for (int g = 0; g < G; ++g)
+      acc_dma16(src + (i64)(R ? G - 1 - g : g) * ACC_SCAN_BLOCK * V, loadOff, myLds + (u32)g * 1024u);
   };
 
   // the tile whose results wait in registers
   Elt yprev[C::G][C::V];
   bool hasPrev = false;
-  i64 prevOut = 0;      // output position of the previous tile's first value
+  i64 prevOut = 0;      // output position of the previous tile's first value (right scans: of thread 0's first run of V)
   // rows [lo, hi) of it
   auto storePrev = [&](int lo, int hi) {
 #pragma unroll
@@ -234,8 +244,9 @@ acc_scan_pipe(Spec::Env env, Spec::Out out, Spec::Out tot, ScanParams p) {
       if (g < lo || g >= hi) continue;
       RawRun r;
 #pragma unroll
-      for (int k = 0; k < V; ++k) r[k] = S::to_raw(yprev[g][k]);
-      __builtin_nontemporal_store(r, (RawRun*)acc_at(S::out_base(out) + prevOut + (i64)g * ACC_SCAN_BLOCK * V, laneOff));
+      for (int k = 0; k < V; ++k) r[R ? V - 1 - k : k] = S::to_raw(yprev[g][k]);
+      if (R) __builtin_nontemporal_store(r, (RawRun*)acc_back(S::out_base(out) + prevOut - (i64)g * ACC_SCAN_BLOCK * V, laneOff));
+      else __builtin_nontemporal_store(r, (RawRun*)acc_at(S::out_base(out) + prevOut + (i64)g * ACC_SCAN_BLOCK * V, laneOff));
     }
   };
   // The previous tile's values leave in three pieces (a store holds its wave until the memory
@@ -263,9 +274,9 @@ acc_scan_pipe(Spec::Env env, Spec::Out out, Spec::Out tot, ScanParams p) {
 #pragma unroll
     for (int g = 0; g < G; ++g) {
       const RawRow r = *(const RawRow*)(myRows + (size_t)(g * ACC_WAVE + lane) * V);
-      x[g][0] = S::from_raw(r[0]);
+      x[g][0] = S::from_raw(r[R ? V - 1 : 0]);
 #pragma unroll
-      for (int k = 1; k < V; ++k) x[g][k] = S::combine(env, x[g][k - 1], S::from_raw(r[k]));
+      for (int k = 1; k < V; ++k) x[g][k] = S::combine(env, x[g][k - 1], S::from_raw(r[R ? V - 1 - k : k]));
     }
     // ticket of the next tile; nothing looks at the counter's answer before the end of the rake,
     // so the round trip is not waited for
@@ -388,7 +399,7 @@ acc_scan_pipe(Spec::Env env, Spec::Out out, Spec::Out tot, ScanParams p) {
       for (int g = 0; g < G; ++g)
 #pragma unroll
         for (int k = 0; k < V; ++k) yprev[g][k] = hasBase ? S::combine(env, base, x[g][k]) : x[g][k];
-      prevOut = outBase + tile * (i64)C::TILE + shift;
+      prevOut = R ? outBase + m - shift - V - tile * (i64)C::TILE : outBase + tile * (i64)C::TILE + shift;
       hasPrev = true;
     } else {
 #pragma unroll
@@ -399,14 +410,14 @@ acc_scan_pipe(Spec::Env env, Spec::Out out, Spec::Out tot, ScanParams p) {
           const Elt y = hasBase ? S::combine(env, base, x[g][k]) : x[g][k];
           const i64 u = t0 + k + 1;
           if (u == n) S::store(tot, row, y);
-          else S::store(out, outBase + u, y);
+          else S::store(out, outBase + (R ? m - 1 - u : u), y);
         }
       }
       hasPrev = false;
       tailStores = false;  // more than the counted stores lie behind the loads: wait for all
     }
     if (S::kKind != 0 && tile == 0 && tid == 0) {
-      S::store(out, outBase, S::seed(env));
+      S::store(out, outBase + (R ? m - 1 : 0), S::seed(env));
       tailStores = false;
     }
     cur = nxt;
@@ -428,16 +439,26 @@ acc_scan_pipe_tail(Spec::Env env, Spec::Out out, Spec::Out tot, ScanParams p) {
   const i64 m = S::kKind == 1 ? n + 1 : n;
   const i64 inBase = row * n, outBase = row * m;
   u64* rowDesc = p.desc + (u64)row * (u64)p.tpr * W;
-  auto load = [&](i64 t) -> Elt { return S::in_linear(env, inBase + t); };
+  auto load = [&](i64 t) -> Elt { return S::in_linear(env, inBase + (S::kRight ? n - 1 - t : t)); };
   auto store = [&](i64 t, const Elt& y) {
     if (S::kKind == 0) {
-      S::store(out, outBase + t, y);
+      S::store(out, outBase + (S::kRight ? n - 1 - t : t), y);
     } else {
       const i64 u = t + 1;
       if (S::kKind == 2 && u == n) S::store(tot, row, y);
-      else S::store(out, outBase + u, y);
+      else S::store(out, outBase + (S::kRight ? m - 1 - u : u), y);
     }
   };
-  auto storeRun = [&](i64 t0, const Elt* y) { S::store_run(out, outBase + t0 + (S::kKind == 0 ? 0 : 1), y); };
+  auto storeRun = [&](i64 t0, const Elt* y) {
+    const i64 shift = S::kKind == 0 ? 0 : 1;
+    if (!S::kRight) {
+      S::store_run(out, outBase + t0 + shift, y);
+    } else {
+      Elt z[S::V];
+#pragma unroll
+      for (int k = 0; k < S::V; ++k) z[k] = y[S::V - 1 - k];
+      S::store_run(out, outBase + (m - 1 - shift) - (t0 + S::V - 1), z);
+    }
+  };
   acc_scan_tile<S>(env, rowDesc, p.tpr, tile, n, p.epoch, p.spin_limit, p.err, load, store, storeRun, false, false);
 }

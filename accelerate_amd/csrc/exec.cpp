@@ -650,7 +650,7 @@ ATyP Program::prepare(const Sx& n, TEnv& tenv) {
       Codegen cgp(aenvOf(tenv));
       Plan scratch;
       Operand srcP = operandOf(n.at(4), cgp, tenv, scratch);
-      plan.k3 = ctx_.kernel(cgp.scan(n.at(2), z, srcP, false, kind, 2));
+      plan.k3 = ctx_.kernel(cgp.scan(n.at(2), z, srcP, dir == "r", kind, 2));
     }
     if (prime) {
       ArrayR tr = src.r;
@@ -1559,8 +1559,9 @@ AValP Program::eval(const Sx& n, AEnv& aenv) {
       const int64_t eltBytes = 16 / pm.vec;
       const Sx& so = n.at(4);
       DArrayP srcArr = so.is("avar") ? aenv[aenv.size() - 1 - (size_t)so.at(1).asInt()] : (temps.empty() ? DArrayP() : temps[0]);
+      // (a right scan's tiles are counted from the end of each row)
       const bool aligned = srcArr && !srcArr->bufs.empty() && ((uintptr_t)srcArr->bufs[0]->p & 15) == 0 &&
-                           (rows == 1 || (len * eltBytes) % 16 == 0);
+                           ((rows == 1 && !pm.scanRight) || (len * eltBytes) % 16 == 0);
       const int64_t tprP = (len + pipeTile - 1) / pipeTile;
       // measured on 2^28 elements: Float32 364 us against 404 us for a workgroup per tile, Int64 714
       // against 745

@@ -1,4 +1,4 @@
-"""The pipelined scan kernel (persistent workgroups, direct global -> LDS loads; left scans over long
+"""The pipelined scan kernel (persistent workgroups, direct global -> LDS loads; scans over long
 rows of a plain array with elements of 4 or 8 bytes, Interpreter.hs:427-474), forced onto every
 case through the `scan_tiles` knob and compared with numpy and with the other tile variants.
 A tile of it holds 1024 lanes x 128 bytes of 8-byte elements (16384 of them) or x 112 bytes of 4-byte
@@ -45,6 +45,46 @@ def test_left_scans_of_every_kind(gpu_ctx, knobs, ty, npty, tile):
         body, total = [p.to_host() for p in runs[2].execute(dx).parts()]
         assert _close(body, np.concatenate([[3], 3 + inc[:-1]]).astype(npty), npty), ("scanl'", n)
         assert _close(total, np.array(3 + inc[-1]).astype(npty), npty), ("scanl' total", n)
+
+
+@pytest.mark.parametrize("ty,npty,tile", TYPES, ids=[t[0] for t in TYPES])
+def test_right_scans_of_every_kind(gpu_ctx, knobs, ty, npty, tile):
+    # a right scan walks over the row's mirror image; lengths that are not a multiple of 16 bytes
+    # (the last two) take the other kernel, and must give the same
+    knobs("scan_tiles", 4)
+    rng = np.random.default_rng(8)
+    wide = np.float64 if np.dtype(npty).kind == "f" else npty
+    runs = (gpu_ctx.compile(P.scan1_sum("r", ty)), gpu_ctx.compile(P.scan_sum("r", ty, 1, 5)),
+            gpu_ctx.compile(P.scan_prime_sum("r", ty, 1, 3)))
+    for n in [tile, 3 * tile, 3 * tile + 4, 5 * tile - 4, 40 * tile + 12344, 300 * tile, 7 * tile + 1, 9 * tile - 3]:
+        lo = 0 if np.dtype(npty).kind == "u" else -1000
+        x = rng.integers(lo, 1000, n).astype(npty)
+        inc = np.cumsum(x[::-1].astype(wide), dtype=wide)[::-1]      # inc[i] = x[i] + .. + x[n-1]
+        dx = gpu_ctx.to_device(x, A.tarray(1, ty))
+        assert _close(runs[0].execute(dx).to_host(), inc.astype(npty), npty), ("scanr1", n)
+        assert _close(runs[1].execute(dx).to_host(), np.concatenate([5 + inc, [5]]).astype(npty), npty), ("scanr", n)
+        body, total = [p.to_host() for p in runs[2].execute(dx).parts()]
+        assert _close(body, np.concatenate([3 + inc[1:], [3]]).astype(npty), npty), ("scanr'", n)
+        assert _close(total, np.array(3 + inc[0]).astype(npty), npty), ("scanr' total", n)
+
+
+def test_right_scan_of_several_rows_with_an_operator_that_is_not_commutative(gpu_ctx, knobs):
+    # a (+) b = a if a /= 0 else b: associative, not commutative; scanr1 gives every position the
+    # nearest non-zero value at or to the right of it.  Rows of a whole number of 16 bytes.
+    knobs("scan_tiles", 4)
+    rows, n = 3, 16384 * 17 + 6
+    rng = np.random.default_rng(3)
+    x = rng.integers(1, 1 << 40, (rows, n)).astype(np.int64)
+    x[rng.random((rows, n)) < 0.9995] = 0        # long stretches of zeros: values travel across many tiles
+    f = A.lam([A.Int, A.Int], lambda a, b: A.cond(A.neq(A.Int, a, A.constI(0)), a, b))
+    prog = A.alam([A.tarray(2, A.Int)], lambda xs: A.scan("r", f, None, xs))
+    at = np.where(x != 0, np.arange(n)[None, :], n)
+    nxt = np.minimum.accumulate(at[:, ::-1], axis=1)[:, ::-1]
+    want = np.where(nxt < n, np.take_along_axis(x, np.minimum(nxt, n - 1), axis=1), 0)
+    run = gpu_ctx.compile(prog)
+    for tiles in (4, 1):
+        knobs("scan_tiles", tiles)
+        assert np.array_equal(run(x), want), tiles
 
 
 @pytest.mark.parametrize("rows,n", [(3, 16384 * 17), (5, 16384 * 16 + 8), (2, 16384 * 20 + 4)])
