@@ -1563,10 +1563,11 @@ AValP Program::eval(const Sx& n, AEnv& aenv) {
       const bool aligned = srcArr && !srcArr->bufs.empty() && ((uintptr_t)srcArr->bufs[0]->p & 15) == 0 &&
                            ((rows == 1 && !pm.scanRight) || (len * eltBytes) % 16 == 0);
       const int64_t tprP = (len + pipeTile - 1) / pipeTile;
-      // measured on 2^28 elements: Float32 364 us against 404 us for a workgroup per tile, Int64 714
-      // against 745
+      // measured on 2^28 elements: Float32 350 us against 395 us for a workgroup per tile, Int64 706
+      // against 742; from two tiles per CU on it is level or ahead (Int64 2^23, 512 tiles: 27 against
+      // 32 us; Float32 2^24, 585 tiles: 37 against 36; with 256 tiles 18.7 against 18.0)
       pipe = aligned && (forcedTiles == 4 ? len >= pipeTile
-                                          : (forcedTiles == 0 && tprP >= 16 && rows * tprP >= 4 * ctx_.computeUnits()));
+                                          : (forcedTiles == 0 && tprP >= 16 && rows * tprP >= 2 * ctx_.computeUnits()));
     }
     const KernelP& kern = pipe ? plan.k3 : (small ? plan.k2 : plan.k);
     const KernelSource& m = kern->meta;
