@@ -1191,14 +1191,16 @@ KernelSource Codegen::scan(const Sx& f, const Sx* seed, const Operand& src, bool
   if (pipe) vec = 16 / stSize(leaves[0]);  // a lane's share of a row is one 128-bit load
   // Large tiles keep the number of look-back steps on the critical path small, but a row of
   // a few tiles cannot fill 256 CUs and a row shorter than a tile leaves most of a large
-  // workgroup idle: short rows get 256-thread workgroups with 128 bytes per lane (one row
+  // workgroup idle: short rows get 256-thread workgroups with 256 bytes per lane (one row
   // of 2^20 Int32: 8 us against 15 us with the large tiles; the large tiles win from 2^23 on).
   int g = std::max(1, std::min(16, scanBytesPerLane() / std::max(1, vec * std::max(1, eltBytes))));
   const int block = small ? 256 : scanBlock();
   if (small) {
     const char* sb = std::getenv("ACCHIP_SCAN_SMALL_BYTES");
     const char* sl = std::getenv("ACCHIP_SCAN_SMALL_LB");
-    const int bytes = sb ? std::atoi(sb) : 128;
+    // 256 B per lane (64 KiB tiles): 2^21 / 2^22 / 2^23 Float32 in 9.8 / 13.5 / 21.9 us against 10.9 /
+    // 17.7 / 30.8 with 128 B (and 10.7 / 17.3 / 26.7 with the large tiles)
+    const int bytes = sb ? std::atoi(sb) : 256;
     g = std::max(1, std::min(16, bytes / std::max(1, vec * std::max(1, eltBytes))));
     body += "#define ACC_SCAN_LBWAVES " + std::to_string(sl ? std::max(1, std::min(4, std::atoi(sl))) : 1) + "\n";
   }

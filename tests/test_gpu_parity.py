@@ -279,7 +279,7 @@ def test_arrays_of_more_than_2p32_elements(gpu_ctx):
     gpu_ctx.purge()
 
 
-TILE_EDGES = sorted({t * k + d for t in (4096, 8192, 12288, 24576, 49152) for k in (1, 2, 5) for d in (-1, 0, 1)})
+TILE_EDGES = sorted({t * k + d for t in (4096, 8192, 12288, 16384, 24576, 49152) for k in (1, 2, 5) for d in (-1, 0, 1)})
 
 
 @pytest.mark.parametrize("tiles", ["large", "small"])
