@@ -46,7 +46,8 @@ def log(*a):
 
 
 def time_steps(ctx, run, args, steps, warmup):
-    """(wall ms per step over exactly `steps` applications, list of per-step ms between events)"""
+    """(wall ms per step over exactly `steps` applications, list of per-step ms between events of a
+    second pass, mean ms per step between the two events around the first pass)"""
     res = None
     t0 = time.perf_counter()
     for _ in range(warmup):
@@ -59,16 +60,25 @@ def time_steps(ctx, run, args, steps, warmup):
         for _ in range(10):
             res = run.execute(*args)
         ctx.sync()
-    ev = [ctx.event()]
+    # exactly `steps` steps between two events (and two synchronisations): the figure
+    e0 = ctx.event()
     t0 = time.perf_counter()
+    for _ in range(steps):
+        res = run.execute(*args)
+    e1 = ctx.event()
+    ctx.sync()
+    wall = (time.perf_counter() - t0) * 1e3 / steps
+    mean = e0.elapsed_ms(e1) / steps
+    # and once more with an event after every step, for the median: an event between two launches
+    # costs the stream 1 to 3 us, which a step of 20 to 100 us would carry in its mean
+    ev = [ctx.event()]
     for _ in range(steps):
         res = run.execute(*args)
         ev.append(ctx.event())
     ctx.sync()
-    wall = (time.perf_counter() - t0) * 1e3 / steps
     per = [ev[k].elapsed_ms(ev[k + 1]) for k in range(steps)]
     del res
-    return wall, per
+    return wall, per, mean
 
 
 def cpu_time(fn, reps):
@@ -182,12 +192,27 @@ def run_workload(ctx, wl, steps, warmup, with_cpu, cpu_reps=3):
         # the stencil configuration: `iterate` sweeps, each fed with the previous one's result
         it = wl["iterate"]
         g = dev[0]
-        for _ in range(5):
+        tw = time.perf_counter()
+        for _ in range(max(5, warmup)):
             g = run.execute(g)
         ctx.sync()
-        per = []
+        while (time.perf_counter() - tw) * 1e3 < WARMUP_FLOOR_MS:   # as in time_steps
+            for _ in range(10):
+                g = run.execute(g)
+            ctx.sync()
+        per, total, rounds = [], 0.0, max(1, steps // 10)
         t0 = time.perf_counter()
-        for _ in range(max(1, steps // 10)):
+        for _ in range(rounds):   # the figure: `it` sweeps between two events
+            g = dev[0]
+            e0 = ctx.event()
+            for _ in range(it):
+                g = run.execute(g)
+            e1 = ctx.event()
+            ctx.sync()
+            total += e0.elapsed_ms(e1)
+        wall = (time.perf_counter() - t0) * 1e3 / (rounds * it)
+        mean = total / (rounds * it)
+        for _ in range(rounds):   # the median: an event after every sweep (see time_steps)
             g = dev[0]
             ev = [ctx.event()]
             for _ in range(it):
@@ -195,13 +220,12 @@ def run_workload(ctx, wl, steps, warmup, with_cpu, cpu_reps=3):
                 ev.append(ctx.event())
             ctx.sync()
             per += [ev[k].elapsed_ms(ev[k + 1]) for k in range(it)]
-        wall = (time.perf_counter() - t0) * 1e3 / len(per)
         del g
     else:
-        wall, per = time_steps(ctx, run, dev, steps, warmup)
+        wall, per, mean = time_steps(ctx, run, dev, steps, warmup)
     if "check" in wl:
         assert wl["check"](run.execute(*dev).to_host()), "result of %s differs from the oracle" % wl["name"]
-    med, mean = statistics.median(per), sum(per) / len(per)
+    med = statistics.median(per)
     gbs = wl["bytes"] / mean / 1e6
     ws = wl.get("working_set", wl["bytes"])
     entry = {"workload": wl["name"], "elements": wl["n"], "algorithmic_bytes": wl["bytes"], "us": round(mean * 1e3, 2),
