@@ -1184,7 +1184,7 @@ KernelSource Codegen::scan(const Sx& f, const Sx* seed, const Operand& src, bool
     if (!typeEq(valType(v), elt)) throw Error("scan: fused producer does not return the element type");
     body += fnHead("Elt", "in_linear", "const Env& env, i64 i") + returnElt(v, em) + "  }\n";
   }
-  // V from the widest leaf; G so that a lane holds about 128 bytes of elements
+  // V from the widest leaf; G so that a lane holds scanBytesPerLane() bytes of elements (192)
   std::vector<ArraySlot> tmpOrder;
   for (auto& kv : used_) tmpOrder.push_back(kv.second);
   int vec = vecFor(leaves, tmpOrder);
@@ -1192,7 +1192,7 @@ KernelSource Codegen::scan(const Sx& f, const Sx* seed, const Operand& src, bool
   // Large tiles keep the number of look-back steps on the critical path small, but a row of
   // a few tiles cannot fill 256 CUs and a row shorter than a tile leaves most of a large
   // workgroup idle: short rows get 256-thread workgroups with 256 bytes per lane (one row
-  // of 2^20 Int32: 8 us against 15 us with the large tiles; the large tiles win from 2^23 on).
+  // of 2^20 Int32: 8 us against 15 us with the large tiles; the large tiles win from 2^24 on).
   int g = std::max(1, std::min(16, scanBytesPerLane() / std::max(1, vec * std::max(1, eltBytes))));
   const int block = small ? 256 : scanBlock();
   if (small) {

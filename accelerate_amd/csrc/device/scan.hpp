@@ -26,7 +26,7 @@
 // publishes its inclusive prefix.  One round trip to a predecessor's descriptor costs on
 // the order of a microsecond on this part (device-scope loads cross the XCDs), and the
 // prefix can only advance along the row by (descriptors inspected per round trip) per
-// round trip.  Large tiles (1024 threads x 128 bytes) keep the number of tiles, and with it
+// round trip.  Large tiles (1024 threads x 192 bytes) keep the number of tiles, and with it
 // the number of round trips on the critical path, small; with one workgroup resident per
 // CU the nearest inclusive prefix is a few dozen tiles away, so one wave polling a window of
 // 64 predecessors (one lane each) resolves it in one round trip.  ACC_SCAN_LBWAVES waves can
