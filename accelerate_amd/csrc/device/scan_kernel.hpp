@@ -6,7 +6,8 @@ acc_scan(Spec::Env env, Spec::Out out, Spec::Out tot, ScanParams p) {
   typedef Spec S;
   typedef S::Elt Elt;
   const int W = AccScanCfg<S>::W;
-  const i64 gtile = acc_take_ticket(p.ticket, p.ticket_base);
+  // (no counter: the launch holds no more tiles than the device holds workgroups at a time)
+  const i64 gtile = p.ticket ? acc_take_ticket(p.ticket, p.ticket_base) : (i64)blockIdx.x;
   // a ticket outside the launch means that the host's count of tickets is off: touch nothing
   if (gtile < 0 || gtile >= p.rows * p.tpr) {
     if (threadIdx.x == 0) __hip_atomic_store(p.err, 3u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);

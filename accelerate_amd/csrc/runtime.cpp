@@ -59,7 +59,7 @@ const KnobName kKnobs[] = {
     {"permute_count", &Knobs::permute_count},     {"permute_groups", &Knobs::permute_groups},
     {"permute_partials", &Knobs::permute_partials}, {"permute_fresh", &Knobs::permute_fresh}, {"stencil_chain", &Knobs::stencil_chain},
     {"pool_async", &Knobs::pool_async}, {"fold_one_launch", &Knobs::fold_one_launch},
-    {"foldseg_one_launch", &Knobs::foldseg_one_launch},
+    {"foldseg_one_launch", &Knobs::foldseg_one_launch}, {"scan_ticketless", &Knobs::scan_ticketless},
     {"stencil_no2d", &Knobs::stencil_no2d},       {"stencil_no3d", &Knobs::stencil_no3d},
     {"scan_tiles", &Knobs::scan_tiles},           {"scan_spin_limit", &Knobs::scan_spin_limit},
     {"scan_test_skew", &Knobs::scan_test_skew},
@@ -816,6 +816,33 @@ void Context::preload(const KernelP& k, std::initializer_list<const char*> fns) 
     hipCheck(hipModuleGetFunction(&f, k->module, fn), fn);
     k->fns[fn] = f;
   }
+}
+
+int64_t Context::residentGroups(const KernelP& k, const char* fn, unsigned block) {
+  if (device_ < 0) return 0;
+  std::lock_guard<std::mutex> g(mu_);
+  auto it = k->perCu.find(fn);
+  if (it == k->perCu.end()) {
+    ensureLoaded(k);
+    hipFunction_t f;
+    auto fi = k->fns.find(fn);
+    if (fi == k->fns.end()) {
+      hipCheck(hipModuleGetFunction(&f, k->module, fn), fn);
+      k->fns[fn] = f;
+    } else {
+      f = fi->second;
+    }
+    int n = 0;
+    if (hipModuleOccupancyMaxActiveBlocksPerMultiprocessor(&n, f, (int)block, 0) != hipSuccess) n = 0;
+    it = k->perCu.emplace(fn, n).first;
+  }
+  int cus = cus_;
+  if (cus == 0) {
+    cus = 256;
+    int v = 0;
+    if (hipDeviceGetAttribute(&v, hipDeviceAttributeMultiprocessorCount, device_) == hipSuccess && v > 0) cus = v;
+  }
+  return (int64_t)it->second * cus;
 }
 
 void Context::launch(const KernelP& k, const char* fn, uint64_t grid, unsigned block, const std::vector<uint64_t>& args) {

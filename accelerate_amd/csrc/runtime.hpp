@@ -25,6 +25,7 @@ struct Kernel {
   std::string code;                 // code object (hsaco), complete once `ready` is
   hipModule_t module = nullptr;     // loaded lazily, on first launch
   std::map<std::string, hipFunction_t> fns;
+  std::map<std::string, int> perCu;  // workgroups of an entry point that one CU holds at a time (asked once)
   KernelSource meta;                // argument plan (source text dropped after compilation)
   // compilation in flight (valid only when hipRTC had to run).  Declared last: it is destroyed
   // first, and destroying the last reference to an async task waits for the worker, which
@@ -51,6 +52,7 @@ struct Knobs {
   long long map_tiled = -1;         // -1: decide per launch, 0 / 1: never / always tile index-permuting producers
   long long fold_rows = -1;         // -1 / 0 / 1: the several-rows-per-workgroup fold
   long long fold_target = 2048;     // workgroups a fold aims at
+  long long scan_ticketless = 1;    // 0: the tiles of a scan always take their numbers from the ticket counter
   long long foldseg_one_launch = 1; // 0: the ends that reach across tile borders are completed by a launch of their own
   long long fold_one_launch = 1;    // 0: a single row cut into chunks always takes the second launch (acc_fold_final)
   long long fold_max_blocks = (long long)1 << 24;  // workgroups per launch of the fold skeleton
@@ -84,6 +86,8 @@ class Context : public std::enable_shared_from_this<Context> {
   bool hasMemory() const { return device_ >= 0 || fakeMemory_; }
   int device() const { return device_; }
   int computeUnits();  // of the device (256 on MI355X); 256 for a context without one
+  // workgroups of `block` threads of entry point fn that the device holds at the same time (0: unknown)
+  int64_t residentGroups(const KernelP& k, const char* fn, unsigned block);
   hipStream_t stream() const { return stream_; }
 
   // memory pool (counterpart of Array/Remote/Table.hs:170-211 + Nursery.hs:43-113):
