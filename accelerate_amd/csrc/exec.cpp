@@ -1187,7 +1187,10 @@ AValP Program::eval(const Sx& n, AEnv& aenv) {
     }
     // geometry: enough workgroups to fill the chip, each with at least a few tiles of work
     const int64_t tile = (int64_t)4 * 64 * plan.k->meta.vec;
-    const int64_t target = std::max<int64_t>(1, ctx_.knobs.fold_target);  // workgroups aimed at
+    // workgroups aimed at; long rows take a quarter of them (two per CU: dotp over 2^24 / 2^26 / 2^28
+    // elements 21.2 / 80.2 / 306 us against 21.8 / 82.2 / 311; rows of 2^22 would lose with fewer)
+    int64_t target = std::max<int64_t>(1, ctx_.knobs.fold_target);
+    if (rows == 1 && len >= ((int64_t)1 << 23)) target = std::max<int64_t>(1, target / 4);
     int64_t bpr = 1;
     if (rows < target && len > 8 * tile)
       bpr = std::min((target + rows - 1) / rows, (len + 8 * tile - 1) / (8 * tile));
