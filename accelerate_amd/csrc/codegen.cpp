@@ -1222,6 +1222,7 @@ KernelSource Codegen::scan(const Sx& f, const Sx* seed, const Operand& src, bool
   }
   body += "  static constexpr int G = " + std::to_string(g) + ";\n";
   body += "#define ACC_SCAN_BLOCK " + std::to_string(pipe ? 1024 : block) + "\n";
+  int rowsG = g;
   if (!pipe) {
     // prefixes of the lane totals by raking through LDS, when the totals of a workgroup fit
     int sz = 0, al = 1;
@@ -1233,7 +1234,11 @@ KernelSource Codegen::scan(const Sx& f, const Sx* seed, const Operand& src, bool
     std::vector<ST> flagged = leaves;
     flagged.push_back(ST::U32);
     structLayout(flagged, sz, al);
-    if (small && g > 1 && (long)(block / 64) * (64 * (g + 1) + 1) * sz <= 64 * 1024 && !(re && re[0] == '0'))
+    // (the rows kernel keeps 128 B per lane: its values travel with their flags, and 256 B of them
+    // do not fit the registers -- 2^20 rows of 256 Int32: 406 us against 730)
+    rowsG = std::max(1, std::min(g, 128 / std::max(1, vec * std::max(1, eltBytes))));
+    if (small) body += "#define ACC_ROWS_G " + std::to_string(rowsG) + "\n";
+    if (small && rowsG > 1 && (long)(block / 64) * (64 * (rowsG + 1) + 1) * sz <= 64 * 1024 && !(re && re[0] == '0'))
       body += "#define ACC_ROWS_RAKE 1\n";
   }
   KernelSource ks = finish(body, elt, leaves, pipe ? "scan.hpp+scan_pipe.hpp" : "scan.hpp+scan_kernel.hpp", vec);
@@ -1241,6 +1246,7 @@ KernelSource Codegen::scan(const Sx& f, const Sx* seed, const Operand& src, bool
   ks.group = g;
   ks.words = structWords(leaves);
   ks.scanRight = right;
+  ks.rowsGroup = rowsG;
   return ks;
 }
 

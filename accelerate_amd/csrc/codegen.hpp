@@ -60,6 +60,7 @@ struct KernelSource {
   bool commutative = false;
   bool streaming = false;             // has acc_*_stream entry points (non-temporal variant)
   bool scanRight = false;             // scan only: a right scan
+  int rowsGroup = 1;                  // scan only: groups per wave of acc_scan_rows (small-tile variant)
   std::string permuteMode;            // permute only: "atomic", "cas", "lock", "store"
   bool permuteCount = false;          // permute only: has acc_permute_count (sum of a constant per source)
   bool permuteCountSet = false;       // permute only: has count_set (defaults of one constant, written with the counts)

@@ -372,18 +372,30 @@ ACC_DEV void acc_scan_tile(const typename S::Env& env, u64* desc, i64 tiles, i64
     // of waves without data: the wave scans and the raking below apply the combination
     // function to every lane, and that function may only ever see values of the array (it
     // may index a table by its operands, or loop on them).  Nothing of this is stored.
+    // A wave's group that lies inside the sequence is loaded like those of a full tile (the test
+    // is the same for all its lanes): of a row that fills three quarters of its tile, only the
+    // one group that holds the row's end goes element by element.
     filler = tlo < n ? load(tlo) : S::seed(env);
 #pragma unroll
     for (int g = 0; g < G; ++g) {
       const i64 t0 = wlo + ((i64)g * ACC_WAVE + lane) * V;
+      if (wlo + (i64)(g + 1) * C::GROUP <= n) {
+        Elt e[C::V];
 #pragma unroll
-      for (int k = 0; k < V; ++k) {
-        const i64 t = t0 + k;
-        if (t < n) {
-          Elt e = load(t);
-          x[g][k] = k == 0 ? e : S::combine(env, x[g][k - 1], e);
-        } else {
-          x[g][k] = k > 0 ? x[g][k - 1] : filler;
+        for (int k = 0; k < V; ++k) e[k] = load(t0 + k);
+        x[g][0] = e[0];
+#pragma unroll
+        for (int k = 1; k < V; ++k) x[g][k] = S::combine(env, x[g][k - 1], e[k]);
+      } else {
+#pragma unroll
+        for (int k = 0; k < V; ++k) {
+          const i64 t = t0 + k;
+          if (t < n) {
+            Elt e = load(t);
+            x[g][k] = k == 0 ? e : S::combine(env, x[g][k - 1], e);
+          } else {
+            x[g][k] = k > 0 ? x[g][k - 1] : filler;
+          }
         }
       }
     }
@@ -482,7 +494,7 @@ ACC_DEV void acc_scan_tile(const typename S::Env& env, u64* desc, i64 tiles, i64
 #pragma unroll
   for (int g = 0; g < G; ++g) {
     const i64 t0 = wlo + ((i64)g * ACC_WAVE + lane) * V;
-    if (full) {
+    if (full || wlo + (i64)(g + 1) * C::GROUP <= n) {
       Elt y[C::V];
 #pragma unroll
       for (int k = 0; k < V; ++k) y[k] = hasBase ? S::combine(env, base, x[g][k]) : x[g][k];

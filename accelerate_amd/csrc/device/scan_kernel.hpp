@@ -62,6 +62,14 @@ struct ScanRowsParams {
   i64 rpt;  // rows per workgroup
 };
 
+// the rows kernel's own tile size (values carry a head flag there: half the elements per lane)
+#ifndef ACC_ROWS_G
+#define ACC_ROWS_G Spec::G
+#endif
+struct AccRowsSpec : Spec {
+  static constexpr int G = ACC_ROWS_G;
+};
+
 extern "C" __global__ void __launch_bounds__(ACC_SCAN_BLOCK, ACC_SCAN_MINWAVES)
 acc_scan_rows(Spec::Env env, Spec::Out out, Spec::Out tot, ScanRowsParams p) {
   typedef Spec S;
@@ -87,5 +95,5 @@ acc_scan_rows(Spec::Env env, Spec::Out out, Spec::Out tot, ScanRowsParams p) {
       else S::store(out, outBase + (S::kRight ? m - 1 - u : u), y);
     }
   };
-  acc_rows_tile<S>(env, (int)(nrows * p.n), n, load, store);
+  acc_rows_tile<AccRowsSpec>(env, (int)(nrows * p.n), n, load, store);
 }

@@ -1546,9 +1546,11 @@ AValP Program::eval(const Sx& n, AEnv& aenv) {
     if (plan.k2 && len >= 1) {
       // many short rows: several whole rows per workgroup (acc_scan_rows)
       const KernelSource& sm = plan.k2->meta;
-      const int64_t rowsTile = (int64_t)sm.block * sm.group * sm.vec;
+      const int64_t rowsTile = (int64_t)sm.block * sm.rowsGroup * sm.vec;
       const bool forced = forcedTiles == 3;
-      if ((forced && len <= rowsTile) || (forcedTiles == 0 && rows >= 2 && 2 * len <= rowsTile)) {
+      // (up to a whole tile of it: a row alone in its workgroup still moves group by group, while
+      // a tile of acc_scan that its row does not fill goes through the code for ragged ends)
+      if ((forced && len <= rowsTile) || (forcedTiles == 0 && rows >= 2 && len <= rowsTile)) {
         const int64_t rpt = rowsTile / len;
         const int64_t groups = (rows + rpt - 1) / rpt;
         if (groups > 0x7fffffffLL) throw Error("scan: too many rows for one launch");

@@ -111,8 +111,8 @@ def test_refusals_launch_nothing(gpu_ctx):
         scan.execute_into(gpu_ctx.empty((999,), A.tarray(1, A.i64)), xi)
     with pytest.raises(hip.AccError, match="wrong type"):
         scan.execute_into(gpu_ctx.empty((1000,), A.tarray(1, A.i32)), xi)
-    # more tiles than the static array has descriptors for: 70000 rows of one tile each (longer than
-    # half a small tile of 8192, so no workgroup takes several), two descriptor words per Int64 tile,
+    # more tiles than the static array has descriptors for: 70000 rows of one tile each (too long
+    # for a workgroup to take several of them), two descriptor words per Int64 tile,
     # against 131072 words (arrays left uninitialised: the call fails before anything is launched)
     rows = gpu_ctx.compile(P.scanl1_sum(A.i64, rank=2))
     shape = (70_000, 4200)
