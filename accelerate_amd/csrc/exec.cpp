@@ -1118,6 +1118,20 @@ AValP Program::eval(const Sx& n, AEnv& aenv) {
         }
       }
     }
+    // a transposed matrix moves through LDS tiles (map_tiled 0 / 1 take the linear order / the tiles below)
+    if (h == "backpermute" && plan.k->meta.transpose2d && r.rank == 2 && te < 0 && plan.k->meta.words <= 4 && out->size() > 0) {
+      const int64_t oh = out->shape[0], ow = out->shape[1];
+      const int64_t tilesX = (ow + 63) / 64, tilesY = (oh + 63) / 64;
+      if (tilesX * tilesY > 0x7fffffffLL) throw Error("too many tiles for one launch");
+      std::vector<uint64_t> args = packArgs(plan.k->meta, aenv, temps, out->shape);
+      packOut(args, *out);
+      args.push_back((uint64_t)oh);
+      args.push_back((uint64_t)ow);
+      args.push_back((uint64_t)tilesX);
+      args.push_back(2 * arrayBytes(*out) >= ctx_.knobs.stream_bytes ? 1 : 0);
+      ctx_.launch(plan.k, "acc_transpose2d", (uint64_t)(tilesX * tilesY), 256, args);
+      return avArr(out);
+    }
     if (te == 0) tiled = false;
     if (te == 1) tiled = h != "generate" && r.rank >= 2 && out->size() > 0;
     if (tiled) {

@@ -460,15 +460,16 @@ def test_stencil3d_direct_evaluation_matches_oracle():
 
 @pytest.mark.parametrize("tiled", ["0", "1", None])
 def test_transposes_with_and_without_tiles(gpu_ctx, knobs, tiled):
-    # index-permuting producers go over 32 x 8V tiles of the result when it is large enough;
-    # forced on and off here, ragged tiles included
+    # index-permuting producers go over 32 x 8V tiles of the result when it is large enough
+    # (forced on and off here, ragged tiles included); left alone, the transposition of a matrix
+    # moves through 64 x 64 tiles in LDS
     if tiled is not None:
         knobs("map_tiled", int(tiled))
     rng = np.random.default_rng(5)
-    for ty, npt in ((A.i32, np.int32), (A.i64, np.int64)):
+    for ty, npt in ((A.i32, np.int32), (A.i64, np.int64), (A.f32, np.float32), (A.u8, np.uint8)):
         run = gpu_ctx.compile(Q.transpose(ty))
-        for shp in [(33, 17), (100, 300), (64, 64), (5, 1000), (1, 1), (257, 3), (1000, 513)]:
-            x = rng.integers(-1000, 1000, shp).astype(npt)
+        for shp in [(33, 17), (100, 300), (64, 64), (5, 1000), (1, 1), (257, 3), (1000, 513), (4097, 130), (63, 65)]:
+            x = rng.integers(0, 200, shp).astype(npt)
             assert np.array_equal(run(x), x.T)
 
 
