@@ -328,3 +328,164 @@ acc_fold_rows(Spec::Env env, Spec::Out out, Spec::Out tmp, FoldRowsParams p) {
   };
   acc_rows_tile<S>(env, (int)(nrows * p.n), n, load, store);
 }
+
+// Many rows of up to a few thousand elements under a commutative operator: a row belongs to
+// `lanes` neighbouring lanes of a wave (a power of two: as many as the row has runs of V
+// elements, 64 at most), a wave works on 64 / lanes rows at a time and a workgroup on `rpg`
+// rows in all.  A lane adds up its runs (run c of the row goes to lane c mod lanes, so one load
+// instruction of the wave covers consecutive memory, rows following each other as they do in
+// memory), the lanes of a row combine through shuffles, the first one writes.  No LDS, no
+// barrier.  (2^28 Float32 as rows of 4 ... 2048 elements: 3.6 - 5.4 TB/s through acc_fold_rows
+// and acc_fold_main, whose tiles such rows do not fill.)
+struct FoldWaveRowsParams {
+  i64 rows;
+  i64 n;      // elements per row, >= 1
+  i64 lanes;  // lanes per row: 1, 2, 4, .. 64
+  i64 rpg;    // rows per workgroup, a multiple of ACC_WAVES * (64 / lanes)
+};
+
+// a lane's value on its way through the wave: bit 0 of f marks the first lane of a row, bit 1 a
+// lane that holds a value at all (rows of fewer runs than lanes, rows beyond the last one)
+struct AccFoldRowLanes {
+  typedef Spec::Env Env;
+  struct Elt {
+    Spec::Elt v;
+    u32 f;
+  };
+  ACC_DEV Elt combine(const Env& env, const Elt& a, const Elt& b) {
+    if (b.f & 1u) return b;
+    Elt r;
+    if ((a.f & 2u) && (b.f & 2u)) r.v = Spec::combine(env, a.v, b.v);
+    else r.v = (b.f & 2u) ? b.v : a.v;
+    r.f = (a.f & 1u) | ((a.f | b.f) & 2u);
+    return r;
+  }
+};
+
+template <bool NT>
+ACC_DEV void acc_fold_wrows_body(const Spec::Env& env, const Spec::Out& out, const FoldWaveRowsParams& p) {
+  typedef Spec S;
+  const int V = S::V;
+  const int L = (int)p.lanes;
+  const int lane = acc_lane();
+  const int sub = lane & (L - 1), slot = lane / L;
+  const int perStep = ACC_WAVE / L;  // rows a wave works on at a time
+  AccFoldSrcIn<S, NT> src{env};
+  const i64 first = (i64)blockIdx.x * p.rpg;
+  const i64 last = first + p.rpg < p.rows ? first + p.rpg : p.rows;
+  const i64 step = (i64)L * V;
+  // joins the lanes of each row of a step and writes the rows' results
+  auto finishRows = [&](i64 row, bool valid, S::Elt acc, bool have) {
+    if (L > 1) {
+      // through the wave's ordered scan (data-parallel moves only): a row's last lane ends up
+      // with all of it
+      AccFoldRowLanes::Elt t;
+      t.v = acc;
+      t.f = (sub == 0 ? 1u : 0u) | (have ? 2u : 0u);
+      t = acc_wave_scan<AccFoldRowLanes>(env, t, lane);
+      acc = t.v;
+      have = (t.f & 2u) != 0u;
+    }
+    if (valid && sub == L - 1) {
+      if (S::kSeeded) {
+        const S::Elt z = S::seed(env);
+        S::store(out, row, have ? S::combine(env, z, acc) : z);
+      } else if (have) {
+        S::store(out, row, acc);
+      }
+    }
+  };
+  i64 rw = first + (i64)acc_wave() * perStep;
+  if (p.n <= step) {
+    // a row is one run per lane at most: four steps of rows at a time, so that a lane has four
+    // loads in flight
+    const i64 stride = (i64)ACC_WAVES * perStep;
+    const i64 e0 = (i64)sub * V;
+    for (; rw + 3 * stride < last; rw += 4 * stride) {
+      S::Elt acc[4];
+      bool have[4], ok[4];
+#pragma unroll
+      for (int u = 0; u < 4; ++u) ok[u] = rw + u * stride + slot < last;
+      if (e0 + V <= p.n) {
+        S::Elt x[4][S::V];
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+          const i64 off = (ok[u] ? rw + u * stride + slot : first) * p.n;  // (a row that exists, for the lanes beyond the last)
+#pragma unroll
+          for (int k = 0; k < V; ++k) x[u][k] = src(off + e0 + k);
+        }
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+          acc[u] = x[u][0];
+#pragma unroll
+          for (int k = 1; k < V; ++k) acc[u] = S::combine(env, acc[u], x[u][k]);
+          have[u] = ok[u];
+        }
+      } else {
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+          have[u] = false;
+          if (ok[u])
+            for (i64 e = e0; e < p.n; ++e) {
+              const S::Elt y = src((rw + u * stride + slot) * p.n + e);
+              acc[u] = have[u] ? S::combine(env, acc[u], y) : y;
+              have[u] = true;
+            }
+        }
+      }
+      // (all lanes of the wave together: the join moves values between them)
+#pragma unroll
+      for (int u = 0; u < 4; ++u) finishRows(rw + u * stride + slot, ok[u], acc[u], have[u]);
+    }
+  }
+  for (; rw < last; rw += (i64)ACC_WAVES * perStep) {
+    const i64 row = rw + slot;
+    const bool valid = row < last;
+    const i64 off = row * p.n;
+    S::Elt acc;
+    bool have = false;
+    if (valid) {
+      i64 e0 = (i64)sub * V;
+      // four runs at a time, their loads together
+      for (; e0 + 3 * step + V <= p.n; e0 += 4 * step) {
+        S::Elt x[4][S::V];
+#pragma unroll
+        for (int u = 0; u < 4; ++u)
+#pragma unroll
+          for (int k = 0; k < V; ++k) x[u][k] = src(off + e0 + u * step + k);
+#pragma unroll
+        for (int u = 0; u < 4; ++u)
+#pragma unroll
+          for (int k = 0; k < V; ++k) {
+            acc = have ? S::combine(env, acc, x[u][k]) : x[u][k];
+            have = true;
+          }
+      }
+      for (; e0 + V <= p.n; e0 += step) {
+        S::Elt x[S::V];
+#pragma unroll
+        for (int k = 0; k < V; ++k) x[k] = src(off + e0 + k);
+#pragma unroll
+        for (int k = 0; k < V; ++k) {
+          acc = have ? S::combine(env, acc, x[k]) : x[k];
+          have = true;
+        }
+      }
+      for (i64 e = e0; e < p.n; ++e) {  // the row's ragged end, in one lane
+        const S::Elt x = src(off + e);
+        acc = have ? S::combine(env, acc, x) : x;
+        have = true;
+      }
+    }
+    finishRows(row, valid, acc, have);
+  }
+}
+
+extern "C" __global__ void __launch_bounds__(ACC_BLOCK)
+acc_fold_wrows(Spec::Env env, Spec::Out out, Spec::Out tmp, FoldWaveRowsParams p) {
+  if constexpr (Spec::kCommutative) acc_fold_wrows_body<false>(env, out, p);
+}
+extern "C" __global__ void __launch_bounds__(ACC_BLOCK)
+acc_fold_wrows_stream(Spec::Env env, Spec::Out out, Spec::Out tmp, FoldWaveRowsParams p) {
+  if constexpr (Spec::kCommutative) acc_fold_wrows_body<true>(env, out, p);
+}

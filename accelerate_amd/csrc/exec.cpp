@@ -1178,6 +1178,33 @@ AValP Program::eval(const Sx& n, AEnv& aenv) {
     int64_t rows = out->size();
     if (rows == 0) return avArr(out);
     {
+      // many rows of up to a few thousand elements under a commutative operator: a few lanes of
+      // a wave per row (acc_fold_wrows).  fold_rows: 2 forces it, 0 and 1 keep it off.
+      const KernelSource& m = plan.k->meta;
+      const long long fr = ctx_.knobs.fold_rows;
+      const bool wave = m.commutative && len >= 1 && (fr == 2 || (fr < 0 && rows >= 256 && len < 4096));
+      if (wave) {
+        const int64_t runs = (len + m.vec - 1) / m.vec;
+        int64_t lanes = 1;
+        while (lanes < 64 && lanes < runs) lanes *= 2;
+        const int64_t perStep = 4 * (64 / lanes);  // rows the four waves of a workgroup work on at a time
+        // about 32 KiB of 4-byte elements per workgroup
+        const int64_t rpg = std::max<int64_t>(perStep, ((8192 + len - 1) / len + perStep - 1) / perStep * perStep);
+        const int64_t groups = (rows + rpg - 1) / rpg;
+        if (groups > 0x7fffffffLL) throw Error("fold: too many rows for one launch");
+        std::vector<uint64_t> args = packArgs(m, aenv, temps, {});
+        packOut(args, *out);
+        packOut(args, *out);
+        args.push_back((uint64_t)rows);
+        args.push_back((uint64_t)len);
+        args.push_back((uint64_t)lanes);
+        args.push_back((uint64_t)rpg);
+        const bool st = streams(m, aenv, temps, 0);
+        ctx_.launch(plan.k, st ? "acc_fold_wrows_stream" : "acc_fold_wrows", (uint64_t)groups, 256, args);
+        return avArr(out);
+      }
+    }
+    {
       // many short rows: several whole rows per workgroup (acc_fold_rows)
       const KernelSource& m = plan.k->meta;
       const int64_t rowsTile = (int64_t)m.block * m.group * m.vec;

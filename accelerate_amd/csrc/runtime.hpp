@@ -50,7 +50,7 @@ struct Knobs {
   long long stream_bytes = (long long)512 << 20;  // bytes a launch must move before the non-temporal variants are taken
   long long map_max_blocks = (long long)1 << 23;  // workgroups per launch of the map skeleton
   long long map_tiled = -1;         // -1: decide per launch, 0 / 1: never / always tile index-permuting producers
-  long long fold_rows = -1;         // -1 / 0 / 1: the several-rows-per-workgroup fold
+  long long fold_rows = -1;         // -1: decide per launch; 0 / 1: never / always the several-rows-per-workgroup fold; 2: always a few lanes per row
   long long fold_target = 2048;     // workgroups a fold aims at
   long long scan_ticketless = 1;    // 0: the tiles of a scan always take their numbers from the ticket counter
   long long foldseg_one_launch = 1; // 0: the ends that reach across tile borders are completed by a launch of their own

@@ -69,10 +69,11 @@ FOLDS = [(c, g) for cs, g in ((GOLDEN, True), (PARITY, False)) for c in cs
          if c[0].startswith(("fold", "dotp", "mss", "issue228")) and "foldseg" not in c[0]]
 
 
-@pytest.mark.parametrize("rows_kernel", ["0", "1"])
+@pytest.mark.parametrize("rows_kernel", ["0", "1", "2"])
 @pytest.mark.parametrize("case", FOLDS, ids=[c[0][0] for c in FOLDS])
 def test_folds_with_and_without_the_rows_kernel(gpu_ctx, knobs, case, rows_kernel):
-    # short rows are reduced several per workgroup; both paths must give the same answers
+    # short rows are reduced several per workgroup (1), or, under a commutative operator, by a few
+    # lanes of a wave each (2); all paths must give the same answers
     knobs("fold_rows", int(rows_kernel))
     (_, prog, args, last), golden = case
     got = gpu_ctx.compile(prog)(*args)
@@ -94,6 +95,25 @@ def test_fold_over_several_launches(gpu_ctx, knobs):
     for shp in [(1000, 33), (5, 100_000)]:
         x = rng.integers(-50, 50, shp).astype(np.int64)
         assert same(gpu_ctx.compile(P.fold_sum(A.i64, 2))(x), x.sum(axis=1))
+
+
+def test_rows_reduced_by_a_few_lanes_each(gpu_ctx, knobs):
+    # lengths around the powers of two that decide how many lanes a row gets, ragged last runs,
+    # fewer rows than a wave holds, a seed, an operator on pairs of bits, a maximum
+    knobs("fold_rows", 2)
+    rng = np.random.default_rng(31)
+    sums = gpu_ctx.compile(P.fold_sum(A.i32, 2, 7))
+    maxs = gpu_ctx.compile(P.fold1_op(A.max_, A.i64, 2))
+    for rows, n in [(1, 1), (3, 2), (1000, 3), (777, 4), (64, 5), (999, 17), (4096, 64), (100, 255), (100, 256), (100, 257),
+                    (50, 1000), (33, 4095), (7, 10_001), (300_000, 12)]:
+        x = rng.integers(-1000, 1000, (rows, n))
+        assert np.array_equal(sums(x.astype(np.int32)), (7 + x.sum(axis=1)).astype(np.int32)), (rows, n)
+        assert np.array_equal(maxs(x.astype(np.int64)), x.max(axis=1)), (rows, n)
+    x = rng.random((5000, 300), dtype=np.float32)
+    got = gpu_ctx.compile(P.fold_sum(A.f32, 2))(x)
+    assert np.allclose(got, x.astype(np.float64).sum(axis=1), rtol=1e-5)
+    x3 = rng.integers(-5, 5, (20, 30, 40)).astype(np.int64)
+    assert np.array_equal(gpu_ctx.compile(P.fold_sum(A.i64, 3))(x3), x3.sum(axis=2))
 
 
 @pytest.mark.parametrize("one_launch", [0, 1])
