@@ -1291,7 +1291,10 @@ AValP Program::eval(const Sx& n, AEnv& aenv) {
       bool viaPartials;
     };
     auto countGeometry = [&](int64_t size, CountGeometry& g) {
-      const int64_t maxParts = ctx_.knobs.permute_parts;
+      // every range of the destination reads all the sources again (from the XCD's L2), so the
+      // counting kernels lose to plain global atomics beyond about 90 ranges (2^26 keys: 26 us per
+      // range against 2.5 ms)
+      const int64_t maxParts = std::min<int64_t>(ctx_.knobs.permute_parts, 88);
       const bool many = cnt >= (1 << 20) || (cnt >= (1 << 12) && cnt >= 4 * size);
       if (!(plan.k->meta.permuteCount && many && size > 0 && size <= maxParts * 65536 && ctx_.knobs.permute_count != 0)) return false;
       g.nparts = (size + 65535) / 65536;
@@ -1358,7 +1361,8 @@ AValP Program::eval(const Sx& n, AEnv& aenv) {
     // Up to 128 LDS-fuls: every share re-reads the sources (from its XCD's L2), so the cost grows
     // with the destination -- 2^26 keys into 2^20 / 2^22 Int32 bins take 0.5 / 2.0 ms, which is
     // where plain global atomics are for uniform keys (2.5 ms); for Zipf keys those take 110 ms.
-    const int64_t maxParts = ctx_.knobs.permute_parts;
+    // (the privatised permute: 80 us per range for 2^26 sources, against 2.5 - 3.2 ms of global atomics)
+    const int64_t maxParts = std::min<int64_t>(ctx_.knobs.permute_parts, 32);
     // From 2^20 sources on, and from 2^12 on when every destination element receives several of
     // them (few destinations under many sources contend in the memory-side atomic units: 2^16
     // keys into 256 bins take 33 us through global atomics, 2^14 keys into 16 bins 47 us,
