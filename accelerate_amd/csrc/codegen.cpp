@@ -1368,26 +1368,15 @@ KernelSource Codegen::backpermute(int outRank, const Sx& p, const Sx* f, const T
   if (outRank >= 2) {
     std::string body = indexedFns(outRank, o) + fnHead("Elt", "produce_at", "const Env& env, i64 i, const i64* ix") +
                        returnElt(r, em) + "  }\n" + indexedTail(outRank);
-    // A transposition of a matrix, \(y, x) -> (x, y) (Language.hs:821-842), also gets the source
-    // element at a given source position: the skeleton moves tiles through LDS so that both the
-    // reads and the writes run along rows.
-    bool swap = false;
-    if (outRank == 2 && src.r.rank == 2 && p.is("lam") && p.size() == 3) {
-      const std::string want = "(pair (pair nil (var 0)) (var 1))";
-      const Sx& lhs = p.at(1);
-      swap = p.at(2).str() == want && lhs.is("pair") && lhs.at(2).is("single") && lhs.at(1).is("pair") &&
-             lhs.at(1).at(2).is("single");
-    }
-    if (swap) {
-      Emit es;
-      es.ind = 4;
-      ValP at = vPair(vPair(vUnit(), vLeaf(ST::I64, "sy")), vLeaf(ST::I64, "sx"));
-      ValP sv = operandIndex(src, at, es);
-      ValP sr = f ? applyFun(*f, {sv}, {}, es) : sv;
-      body += "#define ACC_MAP_TRANSPOSE 1\n" + fnHead("Elt", "src_at2", "const Env& env, i64 sy, i64 sx") + returnElt(sr, es) + "  }\n";
-    }
+    // Transpositions -- index functions that walk the source along another dimension than the
+    // result's innermost one (Language.hs:821-842) -- can go through tiles in LDS, 64 x 65
+    // elements of up to 16 bytes (acc_map_xpose).
+    int esz = 0, eal = 1;
+    structLayout(typeLeaves(outElt), esz, eal);
+    const bool fits = esz <= 16;
+    if (fits) body += "#define ACC_MAP_XPOSE 1\n";
     KernelSource ks = finish(body, outElt, typeLeaves(outElt), "map.hpp", 0);
-    ks.transpose2d = swap;
+    ks.xpose = fits;
     ks.words = structWords(typeLeaves(outElt));
     return ks;
   }

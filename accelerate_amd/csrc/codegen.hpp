@@ -59,7 +59,7 @@ struct KernelSource {
   int block = 256;                    // threads per workgroup of the main kernel
   bool commutative = false;
   bool streaming = false;             // has acc_*_stream entry points (non-temporal variant)
-  bool transpose2d = false;           // backpermute only: has acc_transpose2d (the index function swaps the two indices of a matrix)
+  bool xpose = false;                 // backpermute / transform of rank >= 2: has acc_map_xpose (tiles through LDS)
   bool scanRight = false;             // scan only: a right scan
   int rowsGroup = 1;                  // scan only: groups per wave of acc_scan_rows (small-tile variant)
   std::string permuteMode;            // permute only: "atomic", "cas", "lock", "store"

@@ -125,45 +125,60 @@ acc_map_tiled(Spec::Env env, Spec::Out out, MapTiledParams p) {
 #endif
 }
 
-#ifdef ACC_MAP_TRANSPOSE
-// Transposition of a matrix (the generated code supplies the source element at a source
-// position, whatever is fused into the source): tiles of 64 x 64 results.  A workgroup reads its
-// tile of the source along the source's rows into LDS and writes it along the result's rows, a
-// wave covering 64 consecutive elements either way; the tile's rows are 65 elements apart in
-// LDS, so that reading it by columns meets every bank once.
-struct MapTransposeParams {
-  i64 h, w;     // extent of the result
-  i64 tilesX;   // tiles per row of tiles
-  i64 nt;       // the result leaves with the non-temporal hint (a launch that moves more than the caches hold:
-                // 8192 x 8192 Float32 125 -> 87 us, Int64 257 -> 253)
+#ifdef ACC_MAP_XPOSE
+// Index-permuting producers whose source runs along another dimension of the result than the
+// innermost one -- transpositions of any rank: the result is seen as [o][a][m][w] (dimension a is
+// the one the source's memory follows; o and m gather the dimensions around it), and a workgroup
+// produces a 64 x 64 tile of the (a, w) plane: evaluated with the lanes along a, which walks
+// the source contiguously, kept in LDS (rows 65 elements apart), written with the lanes along w.
+// The choice of a is the host's guess from two evaluations of the index function and only
+// decides the order of evaluation: every element is produced at its own index.
+struct MapXposeParams {
+  i64 na, nm, nw;   // extents of a, m, w
+  i64 tilesA, tilesW;
+  i64 axis;         // which dimension of the result a is
+  i64 nt;           // the result leaves with the non-temporal hint
 };
 
 extern "C" __global__ void __launch_bounds__(ACC_BLOCK)
-acc_transpose2d(Spec::Env env, Spec::Out out, MapTransposeParams p) {
+acc_map_xpose(Spec::Env env, Spec::Out out, MapXposeParams p) {
   typedef Spec S;
   __shared__ S::Elt tile[64][65];
-  const i64 b = (i64)blockIdx.x;
-  const i64 ty = b / p.tilesX, tx = b - ty * p.tilesX;
-  const i64 y0 = ty * 64, x0 = tx * 64;
+  i64 b = (i64)blockIdx.x;
+  const i64 tw = b % p.tilesW;
+  b /= p.tilesW;
+  const i64 ta = b % p.tilesA;
+  const i64 rest = b / p.tilesA;
+  const i64 o = rest / p.nm, m = rest - o * p.nm;
+  const i64 a0 = ta * 64, w0 = tw * 64;
   const int c = (int)threadIdx.x & 63, r0 = (int)threadIdx.x >> 6;
-  // tile[r][c] = result (y0 + c, x0 + r) = source (x0 + r, y0 + c)
-#pragma unroll 4
+  auto linear = [&](i64 a, i64 w) { return ((o * p.na + a) * p.nm + m) * p.nw + w; };
+  // the index of the tile's first element, split once; an element of the tile differs from it
+  // in dimension a and in the innermost one only
+  i64 ix0[S::kRank];
+  S::from_index(env, linear(a0 < p.na ? a0 : 0, w0 < p.nw ? w0 : 0), ix0);
+#pragma unroll 2
   for (int r = r0; r < 64; r += ACC_BLOCK / 64) {
-    const i64 x = x0 + r, y = y0 + c;
-    if (x < p.w && y < p.h) tile[r][c] = S::src_at2(env, x, y);
+    const i64 a = a0 + c, w = w0 + r;
+    if (a < p.na && w < p.nw) {
+      i64 ix[S::kRank];
+#pragma unroll
+      for (int d = 0; d < S::kRank; ++d) ix[d] = d == S::kRank - 1 ? w : (d == (int)p.axis ? a : ix0[d]);
+      tile[r][c] = S::produce_at(env, linear(a, w), ix);
+    }
   }
   __syncthreads();
   if (p.nt) {
-#pragma unroll 4
+#pragma unroll 2
     for (int r = r0; r < 64; r += ACC_BLOCK / 64) {
-      const i64 y = y0 + r, x = x0 + c;
-      if (y < p.h && x < p.w) S::template store<true>(out, y * p.w + x, tile[c][r]);
+      const i64 a = a0 + r, w = w0 + c;
+      if (a < p.na && w < p.nw) S::template store<true>(out, linear(a, w), tile[c][r]);
     }
   } else {
-#pragma unroll 4
+#pragma unroll 2
     for (int r = r0; r < 64; r += ACC_BLOCK / 64) {
-      const i64 y = y0 + r, x = x0 + c;
-      if (y < p.h && x < p.w) S::store(out, y * p.w + x, tile[c][r]);
+      const i64 a = a0 + r, w = w0 + c;
+      if (a < p.na && w < p.nw) S::store(out, linear(a, w), tile[c][r]);
     }
   }
 }

@@ -1085,6 +1085,7 @@ AValP Program::eval(const Sx& n, AEnv& aenv) {
     const int64_t cols = 8 * (int64_t)plan.k->meta.vec;
     const long long te = ctx_.knobs.map_tiled;  // 0 / 1: override, for tests
     bool tiled = h != "generate" && r.rank >= 2 && w >= cols && out->size() / w >= 32;
+    int xposeAxis = -1;  // a transposition: the dimension of the result that the source's memory follows
     if (tiled && te < 0) {
       // Tiles pay off only when neighbouring results read far-apart sources.  Where the index
       // function is pure index arithmetic it is evaluated here at two neighbouring result
@@ -1111,25 +1112,41 @@ AValP Program::eval(const Sx& n, AEnv& aenv) {
         std::vector<int64_t> b = a;
         b.back() += b.back() + 1 < out->shape.back() ? 1 : -1;
         try {
-          const int64_t step = sourceAt(b) - sourceAt(a);
+          const int64_t at = sourceAt(a);
+          const int64_t step = sourceAt(b) - at;
           tiled = step > 1 || step < -1;
+          // which other dimension of the result walks the source one element at a time?
+          for (int d = r.rank - 2; tiled && d >= 0 && xposeAxis < 0; --d) {
+            if (out->shape[d] < 2) continue;
+            std::vector<int64_t> e = a;
+            e[d] += e[d] + 1 < out->shape[d] ? 1 : -1;
+            const int64_t sd = sourceAt(e) - at;
+            if (sd == 1 || sd == -1) xposeAxis = d;
+          }
         } catch (const Error&) {
           tiled = false;  // the probe is only a hint
+          xposeAxis = -1;
         }
       }
     }
-    // a transposed matrix moves through LDS tiles (map_tiled 0 / 1 take the linear order / the tiles below)
-    if (h == "backpermute" && plan.k->meta.transpose2d && r.rank == 2 && te < 0 && plan.k->meta.words <= 4 && out->size() > 0) {
-      const int64_t oh = out->shape[0], ow = out->shape[1];
-      const int64_t tilesX = (ow + 63) / 64, tilesY = (oh + 63) / 64;
-      if (tilesX * tilesY > 0x7fffffffLL) throw Error("too many tiles for one launch");
+    if (tiled && te < 0 && xposeAxis >= 0 && plan.k->meta.xpose) {
+      // tiles of the (that dimension, innermost dimension) plane through LDS
+      int64_t no = 1, nm = 1;
+      for (int d = 0; d < xposeAxis; ++d) no *= out->shape[d];
+      for (int d = xposeAxis + 1; d + 1 < r.rank; ++d) nm *= out->shape[d];
+      const int64_t na = out->shape[xposeAxis], nw = out->shape.back();
+      const int64_t tilesA = (na + 63) / 64, tilesW = (nw + 63) / 64;
+      if (no * nm * tilesA * tilesW > 0x7fffffffLL) throw Error("too many tiles for one launch");
       std::vector<uint64_t> args = packArgs(plan.k->meta, aenv, temps, out->shape);
       packOut(args, *out);
-      args.push_back((uint64_t)oh);
-      args.push_back((uint64_t)ow);
-      args.push_back((uint64_t)tilesX);
+      args.push_back((uint64_t)na);
+      args.push_back((uint64_t)nm);
+      args.push_back((uint64_t)nw);
+      args.push_back((uint64_t)tilesA);
+      args.push_back((uint64_t)tilesW);
+      args.push_back((uint64_t)xposeAxis);
       args.push_back(2 * arrayBytes(*out) >= ctx_.knobs.stream_bytes ? 1 : 0);
-      ctx_.launch(plan.k, "acc_transpose2d", (uint64_t)(tilesX * tilesY), 256, args);
+      ctx_.launch(plan.k, "acc_map_xpose", (uint64_t)(no * nm * tilesA * tilesW), 256, args);
       return avArr(out);
     }
     if (te == 0) tiled = false;

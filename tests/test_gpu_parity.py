@@ -493,6 +493,31 @@ def test_transposes_with_and_without_tiles(gpu_ctx, knobs, tiled):
             assert np.array_equal(run(x), x.T)
 
 
+@pytest.mark.parametrize("tiled", [None, "1", "0"])
+def test_axis_permutations_of_rank_3_and_mirrored_transposes(gpu_ctx, knobs, tiled):
+    # index-permuting producers whose source runs along another dimension than the result's innermost
+    # one go through LDS tiles of the plane of the two (left alone), 32 x 8V tiles (1) or the linear
+    # order (0); ragged extents, every pair of dimensions swapped, a transposition that also mirrors
+    if tiled is not None:
+        knobs("map_tiled", int(tiled))
+    rng = np.random.default_rng(6)
+    perms = {"inner two": (0, 2, 1), "outer two": (1, 0, 2), "first and last": (2, 1, 0), "rotate": (1, 2, 0)}
+    for ty, npt in ((A.i32, np.int32), (A.i64, np.int64), (A.u8, np.uint8)):
+        for shp in [(3, 70, 130), (65, 64, 63), (2, 300, 5), (40, 33, 257)]:
+            x = rng.integers(0, 200, shp).astype(npt)
+            for name, pm in perms.items():
+                # result dimension d is source dimension pm[d]: result index ix reads source index src with src[pm[d]] = ix[d]
+                inv = [pm.index(k) for k in range(3)]
+                prog = Q.reindex(3, lambda dd, pm=pm: [dd()[pm[0]], dd()[pm[1]], dd()[pm[2]]],
+                                 lambda ix, dd, inv=inv: [ix[inv[0]], ix[inv[1]], ix[inv[2]]], ty)
+                assert np.array_equal(gpu_ctx.compile(prog)(x), x.transpose(pm)), (name, shp)
+    # transposition with the rows mirrored: result (y, x) = source (x, h - 1 - y)
+    m = rng.integers(0, 1000, (300, 517)).astype(np.int32)
+    prog = Q.reindex(2, lambda dd: [dd()[1], dd()[0]],
+                     lambda ix, dd: [ix[1], A.sub(A.Int, A.sub(A.Int, dd()[1], A.constI(1)), ix[0])], A.i32)
+    assert np.array_equal(gpu_ctx.compile(prog)(m), m.T[::-1, :])
+
+
 def test_more_than_2_pow_31_elements(gpu_ctx):
     # linear indices beyond 32 bits: a map, a fold and a scan over 2^31 + 1000 Word8 elements
     n = (1 << 31) + 1000
