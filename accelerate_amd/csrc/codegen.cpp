@@ -5,6 +5,7 @@
 #include <cstdlib>
 #include <cstring>
 #include <functional>
+#include <regex>
 #include <set>
 
 namespace acchip {
@@ -1136,7 +1137,8 @@ KernelSource Codegen::foldSeg(const Sx& f, const Sx* seed, const Operand& src, c
 // left to right.
 bool Codegen::scanPipeable(const Operand& src, bool right) {
   (void)right;  // both directions: a right scan walks over the row's mirror image
-  if (src.delayed) return false;
+  // (a fused producer may still turn out not to be a function of one array's element at the
+  // same place: Codegen::scan then throws ScanNotPipeable)
   auto leaves = typeLeaves(src.r.elt);
   return leaves.size() == 1 && !stIsVec(leaves[0]) && (stSize(leaves[0]) == 4 || stSize(leaves[0]) == 8);
 }
@@ -1145,6 +1147,7 @@ KernelSource Codegen::scan(const Sx& f, const Sx* seed, const Operand& src, bool
   const TypeP elt = src.r.elt;
   const bool small = variant == 1, pipe = variant == 2;
   if (pipe && !scanPipeable(src, right)) throw Error("scan: this operand cannot take the pipelined kernel");
+  std::string pipeSlot;  // the array the pipelined kernel moves
   if (kind != 0 && !seed) throw Error("scan: this variant needs a seed");
   std::string body;
   body += std::string("  static constexpr bool kSeeded = ") + (seed ? "true" : "false") + ";\n";
@@ -1213,12 +1216,41 @@ KernelSource Codegen::scan(const Sx& f, const Sx* seed, const Operand& src, bool
     const int bytes = pb ? std::atoi(pb) : (eltBytes == 4 ? 112 : 128);
     g = std::max(2, std::min(9, bytes / 16));
     const std::string T = stName(leaves[0]);
-    const std::string at = "env." + slotByName(src.slot).name + "_0";
-    body += "  typedef " + T + " Raw;\n";
+    std::string rawT = T, fromRaw = "    Elt r_;\n    r_.c0 = raw_;\n    return r_;\n";
+    if (!src.delayed) {
+      pipeSlot = slotByName(src.slot).name;
+    } else {
+      // A producer fused into the scan (scanl f z (map g xs)) can ride along when it is a
+      // function of the element of one array at the scan's own position: the kernel moves that
+      // array and applies the function to what arrives in LDS.  The function's code is the
+      // producer's with its one load replaced; anything else that depends on the position
+      // (another array read there, the index itself) disqualifies it.
+      Emit em;
+      em.ind = 4;
+      ValP v = operandLinear(src, "i", em);
+      if (!typeEq(valType(v), elt)) throw Error("scan: fused producer does not return the element type");
+      std::string code = returnElt(v, em);
+      static const std::regex load("acc_ld<kStream>\\(&env\\.(\\w+)_0\\[i\\]\\)");
+      for (std::sregex_iterator it(code.begin(), code.end(), load), end; it != end; ++it) {
+        const std::string name = (*it)[1].str();
+        if (!pipeSlot.empty() && pipeSlot != name) throw ScanNotPipeable();
+        pipeSlot = name;
+      }
+      if (pipeSlot.empty()) throw ScanNotPipeable();
+      code = std::regex_replace(code, load, "raw_");
+      if (std::regex_search(code, std::regex("\\bi\\b"))) throw ScanNotPipeable();
+      const ArraySlot& as = slotByName(pipeSlot);
+      auto rl = typeLeaves(as.r.elt);
+      if (rl.size() != 1 || stIsVec(rl[0]) || stSize(rl[0]) != stSize(leaves[0]) || as.r.rank != src.r.rank) throw ScanNotPipeable();
+      rawT = stName(rl[0]);
+      fromRaw = code;
+    }
+    const std::string at = "env." + pipeSlot + "_0";
+    body += "  typedef " + rawT + " Raw;\n  typedef " + T + " RawOut;\n";
     body += "  ACC_DEV const Raw* in_base(const Env& env) { return " + at + "; }\n";
-    body += "  ACC_DEV Raw* out_base(const Out& o) { return o.o0; }\n";
-    body += "  ACC_DEV Elt from_raw(Raw v) {\n    Elt r_;\n    r_.c0 = v;\n    return r_;\n  }\n";
-    body += "  ACC_DEV Raw to_raw(const Elt& e) { return e.c0; }\n";
+    body += "  ACC_DEV RawOut* out_base(const Out& o) { return o.o0; }\n";
+    body += "  ACC_DEV Elt from_raw(const Env& env, Raw raw_) {\n" + fromRaw + "  }\n";
+    body += "  ACC_DEV RawOut to_raw(const Elt& e) { return e.c0; }\n";
   }
   body += "  static constexpr int G = " + std::to_string(g) + ";\n";
   body += "#define ACC_SCAN_BLOCK " + std::to_string(pipe ? 1024 : block) + "\n";
@@ -1246,6 +1278,7 @@ KernelSource Codegen::scan(const Sx& f, const Sx* seed, const Operand& src, bool
   ks.group = g;
   ks.words = structWords(leaves);
   ks.scanRight = right;
+  ks.pipeSlot = pipeSlot;
   ks.rowsGroup = rowsG;
   return ks;
 }

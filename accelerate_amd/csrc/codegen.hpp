@@ -48,6 +48,9 @@ struct Operand {
   std::string slot;            // when manifest: name of the array slot
 };
 
+// thrown by Codegen::scan for the pipelined variant: the fused producer is not a function of one array's element
+struct ScanNotPipeable {};
+
 // Everything the executor needs to launch a generated kernel.
 struct KernelSource {
   std::string source;                 // full translation unit
@@ -61,6 +64,7 @@ struct KernelSource {
   bool streaming = false;             // has acc_*_stream entry points (non-temporal variant)
   bool xpose = false;                 // backpermute / transform of rank >= 2: has acc_map_xpose (tiles through LDS)
   bool scanRight = false;             // scan only: a right scan
+  std::string pipeSlot;               // pipelined scan only: name of the array slot its loads move
   int rowsGroup = 1;                  // scan only: groups per wave of acc_scan_rows (small-tile variant)
   std::string permuteMode;            // permute only: "atomic", "cas", "lock", "store"
   bool permuteCount = false;          // permute only: has acc_permute_count (sum of a constant per source)

@@ -165,12 +165,13 @@ extern "C" __global__ void __launch_bounds__(ACC_SCAN_BLOCK, ACC_SCAN_MINWAVES)
 acc_scan_pipe(Spec::Env env, Spec::Out out, Spec::Out tot, ScanParams p) {
   typedef Spec S;
   typedef S::Elt Elt;
-  typedef S::Raw Raw;
+  typedef S::Raw Raw;        // what lies in the source array
+  typedef S::RawOut RawOut;  // what goes to the result (the element's one scalar)
   typedef AccScanCfg<S> C;
   constexpr int V = C::V, G = C::G, W = C::W, NW = ACC_SCAN_WAVES;
-  static_assert(sizeof(Raw) * V == 16, "a lane's share of a row is 16 bytes");
+  static_assert(sizeof(Raw) * V == 16 && sizeof(RawOut) == sizeof(Raw), "a lane's share of a row is 16 bytes, in and out");
   static_assert(ACC_SCAN_BLOCK == 1024, "the pipelined scan runs 16 waves");
-  typedef Raw RawRun __attribute__((ext_vector_type(V), aligned(sizeof(Raw))));  // in memory: aligned like an element (scanl shifts by one)
+  typedef RawOut RawRun __attribute__((ext_vector_type(V), aligned(sizeof(RawOut))));  // in memory: aligned like an element (scanl shifts by one)
   typedef Raw RawRow __attribute__((ext_vector_type(V)));                        // in LDS: 16-byte aligned
 
   __shared__ __attribute__((aligned(16))) unsigned char sh_buf[G * 16384];  // load buffer; the rake area lies over it
@@ -274,9 +275,9 @@ acc_scan_pipe(Spec::Env env, Spec::Out out, Spec::Out tot, ScanParams p) {
 #pragma unroll
     for (int g = 0; g < G; ++g) {
       const RawRow r = *(const RawRow*)(myRows + (size_t)(g * ACC_WAVE + lane) * V);
-      x[g][0] = S::from_raw(r[R ? V - 1 : 0]);
+      x[g][0] = S::from_raw(env, r[R ? V - 1 : 0]);
 #pragma unroll
-      for (int k = 1; k < V; ++k) x[g][k] = S::combine(env, x[g][k - 1], S::from_raw(r[R ? V - 1 - k : k]));
+      for (int k = 1; k < V; ++k) x[g][k] = S::combine(env, x[g][k - 1], S::from_raw(env, r[R ? V - 1 - k : k]));
     }
     // ticket of the next tile; nothing looks at the counter's answer before the end of the rake,
     // so the round trip is not waited for

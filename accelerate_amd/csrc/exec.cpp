@@ -650,7 +650,10 @@ ATyP Program::prepare(const Sx& n, TEnv& tenv) {
       Codegen cgp(aenvOf(tenv));
       Plan scratch;
       Operand srcP = operandOf(n.at(4), cgp, tenv, scratch);
-      plan.k3 = ctx_.kernel(cgp.scan(n.at(2), z, srcP, dir == "r", kind, 2));
+      try {
+        plan.k3 = ctx_.kernel(cgp.scan(n.at(2), z, srcP, dir == "r", kind, 2));
+      } catch (const ScanNotPipeable&) {
+      }
     }
     if (prime) {
       ArrayR tr = src.r;
@@ -1635,11 +1638,13 @@ AValP Program::eval(const Sx& n, AEnv& aenv) {
       const KernelSource& pm = plan.k3->meta;
       const int64_t pipeTile = (int64_t)pm.block * pm.group * pm.vec;
       const int64_t eltBytes = 16 / pm.vec;
-      const Sx& so = n.at(4);
-      DArrayP srcArr = so.is("avar") ? aenv[aenv.size() - 1 - (size_t)so.at(1).asInt()] : (temps.empty() ? DArrayP() : temps[0]);
-      // (a right scan's tiles are counted from the end of each row)
+      // the array the kernel moves: the operand itself, or the one array a fused producer reads
+      DArrayP srcArr;
+      for (const ArraySlot& sl : pm.arrays)
+        if (sl.name == pm.pipeSlot) srcArr = sl.temp ? temps.at(sl.index) : aenv.at(aenv.size() - 1 - sl.index);
+      // (a right scan's tiles are counted from the end of each row; a producer must cover its array exactly)
       const bool aligned = srcArr && !srcArr->bufs.empty() && ((uintptr_t)srcArr->bufs[0]->p & 15) == 0 &&
-                           ((rows == 1 && !pm.scanRight) || (len * eltBytes) % 16 == 0);
+                           srcArr->shape == ext && ((rows == 1 && !pm.scanRight) || (len * eltBytes) % 16 == 0);
       const int64_t tprP = (len + pipeTile - 1) / pipeTile;
       // measured on 2^28 elements: Float32 350 us against 395 us for a workgroup per tile, Int64 706
       // against 742; from two tiles per CU on it is level or ahead (Int64 2^23, 512 tiles: 27 against

@@ -87,6 +87,48 @@ def test_right_scan_of_several_rows_with_an_operator_that_is_not_commutative(gpu
         assert np.array_equal(run(x), want), tiles
 
 
+def _scan_of_fused(ty, g, direction="l", seed=None, prime=False, extra=None):
+    """scan (+) over a producer fused into it: \\i -> g (xs ! i), optionally reading a second array too"""
+    sh1 = A.tshape(1)
+    args = [A.tarray(1, ty)] + ([A.tarray(1, ty)] if extra else [])
+
+    def body(a, *more):
+        at_ix = lambda ix: g(A.index(a, A.vexp(ix)), *[A.index(m, A.vexp(ix)) for m in more])
+        at_lin = lambda i: g(A.linearindex(a, i), *[A.linearindex(m, i) for m in more])
+        src = A.delayed(A.tarray(1, ty), A.shape(a), A.lam([sh1], at_ix), A.lam([A.Int], at_lin))
+        z = None if seed is None else A.const(ty, seed)
+        return (A.scan_ if prime else A.scan)(direction, P._binop(A.add, ty), z, src)
+
+    return A.alam(args, body)
+
+
+def test_producers_fused_into_the_scan(gpu_ctx, knobs):
+    # scanl f z (map g xs): a function of one array's element at the scan's own position rides
+    # along in the pipelined kernel (applied to what arrives in LDS); one that reads two arrays
+    # at that position keeps the other kernels.  Both give what numpy gives, in both directions.
+    knobs("scan_tiles", 4)
+    rng = np.random.default_rng(17)
+    twice_plus = lambda v: A.add(A.i64, A.mul(A.i64, v, A.const(A.i64, 2)), A.const(A.i64, 1))
+    for n in (16384 * 3, 16384 * 40 + 8, 16384 * 300):
+        x = rng.integers(-1000, 1000, n).astype(np.int64)
+        y = 2 * x + 1
+        assert np.array_equal(gpu_ctx.compile(_scan_of_fused(A.i64, twice_plus))(x), np.cumsum(y)), n
+        assert np.array_equal(gpu_ctx.compile(_scan_of_fused(A.i64, twice_plus, "r", 5))(x),
+                              np.concatenate([5 + np.cumsum(y[::-1])[::-1], [5]])), n
+        body, total = gpu_ctx.compile(_scan_of_fused(A.i64, twice_plus, "l", 3, True))(x)
+        inc = 3 + np.cumsum(y)
+        assert np.array_equal(body, np.concatenate([[3], inc[:-1]])) and total == inc[-1], n
+        w = rng.integers(-1000, 1000, n).astype(np.int64)
+        both = _scan_of_fused(A.i64, lambda v, u: A.add(A.i64, v, u), extra=True)
+        assert np.array_equal(gpu_ctx.compile(both)(x, w), np.cumsum(x + w)), n
+    # the element's type changes with the function (Int32 -> Float32: same size, so it still rides along)
+    xi = rng.integers(0, 2, 28672 * 20).astype(np.int32)
+    conv = A.alam([A.tarray(1, A.i32)], lambda a: A.scan("l", P._binop(A.add, A.f32), None, A.delayed(
+        A.tarray(1, A.f32), A.shape(a), A.lam([A.tshape(1)], lambda ix: A.fromintegral(A.i32, A.f32, A.index(a, A.vexp(ix)))),
+        A.lam([A.Int], lambda i: A.fromintegral(A.i32, A.f32, A.linearindex(a, i))))))
+    assert np.array_equal(gpu_ctx.compile(conv)(xi), np.cumsum(xi).astype(np.float32))   # (sums below 2^24: exact)
+
+
 @pytest.mark.parametrize("rows,n", [(3, 16384 * 17), (5, 16384 * 16 + 8), (2, 16384 * 20 + 4)])
 def test_several_rows(gpu_ctx, knobs, rows, n):
     # every row starts at a multiple of 16 bytes; rows end in partial tiles, which a second launch takes
