@@ -30,7 +30,7 @@ PIPE_STAMPS = [
      "  for (;;) {\n    u64* lab_stamps = p.stamps; const i64 lab_tile = cur; STAMP(0);\n    const i64 row = cur / tpf;"),
     ("    Elt x[C::G][C::V];\n#pragma unroll\n    for (int g = 0; g < G; ++g) {\n      const RawRow r",
      "    STAMP(1);\n    Elt x[C::G][C::V];\n#pragma unroll\n    for (int g = 0; g < G; ++g) {\n      const RawRow r"),
-    ("    acc_lds_barrier();  // the rake area has been read", "    STAMP(2);\n    acc_lds_barrier();  // the rake area has been read"),
+    ("    if (hasPrev && w != 0) storePrev(S1, S2);\n", "    if (hasPrev && w != 0) storePrev(S1, S2);\n    STAMP(2);\n"),
     ("    // the tile's exclusive prefix: seed or nothing", "    STAMP(3);\n    // the tile's exclusive prefix: seed or nothing"),
     ("      if (lane == 0) {\n        if (successors) {\n          Elt inc;", "      STAMP(4);\n      if (lane == 0) {\n        if (successors) {\n          Elt inc;"),
     ("    const bool hasBase = __builtin_amdgcn_readfirstlane(sh_has_excl) != 0;",
