@@ -592,10 +592,12 @@ ATyP Program::prepare(const Sx& n, TEnv& tenv) {
       bnds = {n.at(4)};
       srcs.push_back(operandOf(n.at(5), cg, tenv, plan));
     } else {
-      pats = {n.at(1), n.at(2)};
+      // (looked up before the lists are built: an operand that is missing throws here, not in the middle of a list)
+      const Sx &p0 = n.at(1), &p1 = n.at(2), &b0 = n.at(5), &b1 = n.at(7);
+      pats = {p0, p1};
       outElt = parseType(n.at(3));
       f = &n.at(4);
-      bnds = {n.at(5), n.at(7)};
+      bnds = {b0, b1};
       srcs.push_back(operandOf(n.at(6), cg, tenv, plan));
       srcs.push_back(operandOf(n.at(8), cg, tenv, plan));
       if (srcs[0].r.rank != srcs[1].r.rank) throw Error("stencil2: operands of different rank");
