@@ -880,7 +880,7 @@ static int vecFor(const std::vector<ST>& leaves, const std::vector<ArraySlot>& a
 }
 
 KernelSource Codegen::finish(const std::string& specBody, const TypeP& elt, const std::vector<ST>& outLeaves,
-                             const std::string& skeleton, int vec) {
+                             const std::string& skeleton, int vec, bool ownStore) {
   KernelSource ks;
   std::string envS = envStruct(ks.arrays);
   ks.outLeaves = outLeaves;
@@ -910,7 +910,7 @@ KernelSource Codegen::finish(const std::string& specBody, const TypeP& elt, cons
   s += specBody;
   // Out <-> Elt when both have the same leaves
   auto el = typeLeaves(elt);
-  if (el == outLeaves) {
+  if (el == outLeaves && !ownStore) {
     s += "  ACC_DEV Elt load(const Out& o, i64 i) {\n    Elt r_;\n";
     for (size_t k = 0; k < el.size(); ++k) s += "    r_.c" + std::to_string(k) + " = o.o" + std::to_string(k) + "[i];\n";
     s += "    return r_;\n  }\n";
@@ -1143,10 +1143,12 @@ bool Codegen::scanPipeable(const Operand& src, bool right) {
   return leaves.size() == 1 && !stIsVec(leaves[0]) && (stSize(leaves[0]) == 4 || stSize(leaves[0]) == 8);
 }
 
-KernelSource Codegen::scan(const Sx& f, const Sx* seed, const Operand& src, bool right, int kind, int variant) {
+KernelSource Codegen::scan(const Sx& f, const Sx* seed, const Operand& src, bool right, int kind, int variant,
+                           const Sx* post, const TypeP& postElt) {
   const TypeP elt = src.r.elt;
   const bool small = variant == 1, pipe = variant == 2;
   if (pipe && !scanPipeable(src, right)) throw Error("scan: this operand cannot take the pipelined kernel");
+  if (post && (pipe || kind == 2)) throw Error("scan: this variant applies no function to its results");
   std::string pipeSlot;  // the array the pipelined kernel moves
   if (kind != 0 && !seed) throw Error("scan: this variant needs a seed");
   std::string body;
@@ -1273,7 +1275,34 @@ KernelSource Codegen::scan(const Sx& f, const Sx* seed, const Operand& src, bool
     if (small && rowsG > 1 && (long)(block / 64) * (64 * (rowsG + 1) + 1) * sz <= 64 * 1024 && !(re && re[0] == '0'))
       body += "#define ACC_ROWS_RAKE 1\n";
   }
-  KernelSource ks = finish(body, elt, leaves, pipe ? "scan.hpp+scan_pipe.hpp" : "scan.hpp+scan_kernel.hpp", vec);
+  std::vector<ST> outLeaves = leaves;
+  if (post) {
+    // the results leave through store / store_run, which here apply the function first.  They are
+    // not handed the environment: a function that reads arrays stays a launch of its own.
+    Emit em;
+    em.ind = 6;
+    ValP r = applyFun(*post, {eltVal(elt, "v")}, {}, em);
+    if (!typeEq(valType(r), postElt)) throw Error("map: function result does not match the declared element type");
+    if (em.code.find("env.") != std::string::npos) throw ScanPostNotFusable();
+    auto lv = leavesOf(r);
+    for (auto& l : lv)
+      if (l->ex.find("env.") != std::string::npos) throw ScanPostNotFusable();
+    outLeaves = typeLeaves(postElt);
+    body += "  template <bool kStream = false>\n  ACC_DEV void store(const Out& o, i64 i, const Elt& v) {\n" + em.code;
+    for (size_t k = 0; k < lv.size(); ++k)
+      body += "      acc_st<kStream>(&o.o" + std::to_string(k) + "[i], (" + stName(outLeaves[k]) + ")(" + lv[k]->ex + "));\n";
+    body += "  }\n";
+    body += "  ACC_DEV void store_run(const Out& o, i64 i, const Elt* vs_) {\n";
+    for (size_t k = 0; k < lv.size(); ++k)
+      body += std::string("    acc_run<") + stName(outLeaves[k]) + ", V> r" + std::to_string(k) + "_;\n";
+    body += "#pragma unroll\n    for (int k_ = 0; k_ < V; ++k_) {\n      const Elt& v = vs_[k_];\n" + em.code;
+    for (size_t k = 0; k < lv.size(); ++k) body += "      r" + std::to_string(k) + "_.e[k_] = " + lv[k]->ex + ";\n";
+    body += "    }\n";
+    for (size_t k = 0; k < lv.size(); ++k)
+      body += std::string("    *(acc_run<") + stName(outLeaves[k]) + ", V>*)&o.o" + std::to_string(k) + "[i] = r" + std::to_string(k) + "_;\n";
+    body += "  }\n";
+  }
+  KernelSource ks = finish(body, elt, outLeaves, pipe ? "scan.hpp+scan_pipe.hpp" : "scan.hpp+scan_kernel.hpp", vec, post != nullptr);
   ks.block = pipe ? 1024 : block;
   ks.group = g;
   ks.words = structWords(leaves);

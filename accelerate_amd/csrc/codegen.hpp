@@ -50,6 +50,8 @@ struct Operand {
 
 // thrown by Codegen::scan for the pipelined variant: the fused producer is not a function of one array's element
 struct ScanNotPipeable {};
+// thrown by Codegen::scan when the function to apply to the results reads arrays
+struct ScanPostNotFusable {};
 
 // Everything the executor needs to launch a generated kernel.
 struct KernelSource {
@@ -92,7 +94,10 @@ class Codegen {
   // small: the variant for short rows (256-thread workgroups)
   // variant 0: large tiles, 1: small tiles (short rows), 2: persistent pipeline for long rows of a plain array
   // (only where scanPipeable holds)
-  KernelSource scan(const Sx& f, const Sx* seed, const Operand& src, bool right, int kind, int variant = 0);
+  // post (with its result type): a function applied to every result on its way to memory -- the
+  // `map g` of `map g (scan f z xs)`, which then costs neither a launch nor an array of its own
+  KernelSource scan(const Sx& f, const Sx* seed, const Operand& src, bool right, int kind, int variant = 0,
+                    const Sx* post = nullptr, const TypeP& postElt = nullptr);
   static bool scanPipeable(const Operand& src, bool right);
   KernelSource foldSeg(const Sx& f, const Sx* seed, const Operand& src, const Operand& seg, ST segType);
   // freshInit: the literal every element of the defaults holds when they are `generate sh (\_ -> c)`
@@ -153,7 +158,7 @@ class Codegen {
   std::string returnElt(const ValP& v, Emit& em);
   bool isCommutative(const Sx& f, std::string* op = nullptr, ST* st = nullptr);
   KernelSource finish(const std::string& specBody, const TypeP& elt, const std::vector<ST>& outLeaves,
-                      const std::string& skeleton, int vec);
+                      const std::string& skeleton, int vec, bool ownStore = false);
 };
 
 // taps a stencil pattern reaches on either side of the focus, per dimension (outermost first)

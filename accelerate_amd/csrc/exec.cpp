@@ -494,6 +494,12 @@ ATyP Program::prepare(const Sx& n, TEnv& tenv) {
   if (h == "use") return atArr(parseArrayR(n.at(1)));
   if (h == "delayed") throw Error("expected manifest array");  // Interpreter.hs:180
 
+  {
+    // a node is planned once, however many variants of its consumer ask for it as an operand
+    // (its own nested operands would otherwise be listed, and evaluated, once per request)
+    auto known = plans_.find(&n);
+    if (known != plans_.end() && known->second.ty) return known->second.ty;
+  }
   Plan& plan = plans_[&n];
   Codegen cg(aenvOf(tenv));
   cg.fastPermuteConst = ctx_.flag(Context::kFastPermuteConst);
@@ -540,6 +546,18 @@ ATyP Program::prepare(const Sx& n, TEnv& tenv) {
     return done(r);
   }
   if (h == "map") {
+    if (n.at(3).is("scan") && ctx_.knobs.scan_post != 0) {
+      // map g (scan f z xs) with the scan written out as an operand (not let-bound: nobody else
+      // reads it): the scan applies g as it stores, where g reads no arrays
+      Plan trial;
+      try {
+        prepareScan(n.at(3), tenv, trial, &n.at(2), parseType(n.at(1)));
+        trial.mode = "scan";
+        plan = std::move(trial);
+        return plan.ty;
+      } catch (const ScanPostNotFusable&) {
+      }
+    }
     Operand src = operandOf(n.at(3), cg, tenv, plan);
     ArrayR r;
     r.rank = src.r.rank;
@@ -631,41 +649,54 @@ ATyP Program::prepare(const Sx& n, TEnv& tenv) {
     plan.k = ctx_.kernel(cg.foldSeg(n.at(2), seedOf(n.at(3)), src, seg, ity));
     return done(src.r);
   }
-  if (h == "scan" || h == "scan'") {
-    bool prime = h == "scan'";
-    const std::string& dir = n.at(1).s;
-    if (dir != "l" && dir != "r") throw Error("scan direction must be l or r");
-    Operand src = operandOf(n.at(4), cg, tenv, plan);
-    if (src.r.rank < 1) throw Error("scan: operand must have rank >= 1");
-    const Sx* z = prime ? &n.at(3) : seedOf(n.at(3));
-    int kind = prime ? 2 : (z ? 1 : 0);
-    plan.k = ctx_.kernel(cg.scan(n.at(2), z, src, dir == "r", kind));
-    {
-      // the same scan with small tiles, chosen at launch for short rows
-      Codegen cgs(aenvOf(tenv));
-      Plan scratch;
-      Operand srcS = operandOf(n.at(4), cgs, tenv, scratch);
-      plan.k2 = ctx_.kernel(cgs.scan(n.at(2), z, srcS, dir == "r", kind, 1));
-    }
-    if (Codegen::scanPipeable(src, dir == "r")) {
-      // and as a pipeline in persistent workgroups, chosen at launch for long rows
-      Codegen cgp(aenvOf(tenv));
-      Plan scratch;
-      Operand srcP = operandOf(n.at(4), cgp, tenv, scratch);
-      try {
-        plan.k3 = ctx_.kernel(cgp.scan(n.at(2), z, srcP, dir == "r", kind, 2));
-      } catch (const ScanNotPipeable&) {
-      }
-    }
-    if (prime) {
-      ArrayR tr = src.r;
-      tr.rank -= 1;
-      plan.ty = atPair(atArr(src.r), atArr(tr));
-      return plan.ty;
-    }
-    return done(src.r);
-  }
+  if (h == "scan" || h == "scan'") return prepareScan(n, tenv, plan, nullptr, nullptr);
   throw Error("unsupported array term '" + h + "'");
+}
+
+// (scan dir f seed operand) and (scan' ...), optionally with the function of a `map` around it
+// applied to the results as they are stored (post; not for scan', whose results are a pair)
+ATyP Program::prepareScan(const Sx& n, TEnv& tenv, Plan& plan, const Sx* post, const TypeP& postElt) {
+  const bool prime = n.is("scan'");
+  auto seedOf = [&](const Sx& s) -> const Sx* {
+    if (s.isAtom("nothing")) return nullptr;
+    if (s.is("just")) return &s.at(1);
+    throw Error("expected (just e) or nothing, got " + s.str());
+  };
+  const std::string& dir = n.at(1).s;
+  if (dir != "l" && dir != "r") throw Error("scan direction must be l or r");
+  Codegen cg(aenvOf(tenv));
+  Operand src = operandOf(n.at(4), cg, tenv, plan);
+  if (src.r.rank < 1) throw Error("scan: operand must have rank >= 1");
+  const Sx* z = prime ? &n.at(3) : seedOf(n.at(3));
+  int kind = prime ? 2 : (z ? 1 : 0);
+  plan.k = ctx_.kernel(cg.scan(n.at(2), z, src, dir == "r", kind, 0, post, postElt));
+  {
+    // the same scan with small tiles, chosen at launch for short rows
+    Codegen cgs(aenvOf(tenv));
+    Plan scratch;
+    Operand srcS = operandOf(n.at(4), cgs, tenv, scratch);
+    plan.k2 = ctx_.kernel(cgs.scan(n.at(2), z, srcS, dir == "r", kind, 1, post, postElt));
+  }
+  if (!post && Codegen::scanPipeable(src, dir == "r")) {
+    // and as a pipeline in persistent workgroups, chosen at launch for long rows
+    Codegen cgp(aenvOf(tenv));
+    Plan scratch;
+    Operand srcP = operandOf(n.at(4), cgp, tenv, scratch);
+    try {
+      plan.k3 = ctx_.kernel(cgp.scan(n.at(2), z, srcP, dir == "r", kind, 2));
+    } catch (const ScanNotPipeable&) {
+    }
+  }
+  if (prime) {
+    ArrayR tr = src.r;
+    tr.rank -= 1;
+    plan.ty = atPair(atArr(src.r), atArr(tr));
+    return plan.ty;
+  }
+  ArrayR r = src.r;
+  if (post) r.elt = postElt;
+  plan.ty = atArr(r);
+  return plan.ty;
 }
 
 // ------------------------------------------------------------------------------------
@@ -1173,7 +1204,7 @@ AValP Program::eval(const Sx& n, AEnv& aenv) {
     launchMap(plan.k, aenv, temps, *out);
     return avArr(out);
   }
-  if (h == "map") {
+  if (h == "map" && plan.mode != "scan") {
     std::vector<DArrayP> temps = evalTemps(plan.temps, aenv);
     size_t cur = 0;
     std::vector<int64_t> ext = operandExtent(n.at(3), aenv, plan, temps, cur);
@@ -1573,12 +1604,13 @@ AValP Program::eval(const Sx& n, AEnv& aenv) {
     }
     return avArr(out);
   }
-  if (h == "scan" || h == "scan'") {
+  if (h == "scan" || h == "scan'" || (h == "map" && plan.mode == "scan")) {
+    const Sx& sn = h == "map" ? n.at(3) : n;  // the scan inside a map whose function it applies itself
     const bool prime = h == "scan'";
-    const int kind = prime ? 2 : (seeded(n.at(3)) ? 1 : 0);
+    const int kind = prime ? 2 : (seeded(sn.at(3)) ? 1 : 0);
     std::vector<DArrayP> temps = evalTemps(plan.temps, aenv);
     size_t cur = 0;
-    std::vector<int64_t> ext = operandExtent(n.at(4), aenv, plan, temps, cur);
+    std::vector<int64_t> ext = operandExtent(sn.at(4), aenv, plan, temps, cur);
     const int64_t len = std::max<int64_t>(ext.back(), 0);
     std::vector<int64_t> outer(ext.begin(), ext.end() - 1);
     std::vector<int64_t> oshape = outer;

@@ -119,6 +119,7 @@ class Program {
   Operand operandOf(const Sx& o, Codegen& cg, TEnv& tenv, Plan& plan);
   void prepareHostExp(const Sx& e, TEnv& tenv, Plan& plan);
   static std::vector<ArrayR> aenvOf(const TEnv& tenv);
+  ATyP prepareScan(const Sx& n, TEnv& tenv, Plan& plan, const Sx* post, const TypeP& postElt);
 
   // execution
   AValP eval(const Sx& n, AEnv& aenv);

@@ -59,7 +59,7 @@ const KnobName kKnobs[] = {
     {"permute_count", &Knobs::permute_count},     {"permute_groups", &Knobs::permute_groups},
     {"permute_partials", &Knobs::permute_partials}, {"permute_fresh", &Knobs::permute_fresh}, {"stencil_chain", &Knobs::stencil_chain},
     {"pool_async", &Knobs::pool_async}, {"fold_one_launch", &Knobs::fold_one_launch},
-    {"foldseg_one_launch", &Knobs::foldseg_one_launch}, {"scan_ticketless", &Knobs::scan_ticketless},
+    {"foldseg_one_launch", &Knobs::foldseg_one_launch}, {"scan_ticketless", &Knobs::scan_ticketless}, {"scan_post", &Knobs::scan_post},
     {"stencil_no2d", &Knobs::stencil_no2d},       {"stencil_no3d", &Knobs::stencil_no3d},
     {"scan_tiles", &Knobs::scan_tiles},           {"scan_spin_limit", &Knobs::scan_spin_limit},
     {"scan_test_skew", &Knobs::scan_test_skew},
