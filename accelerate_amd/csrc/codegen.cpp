@@ -1580,9 +1580,23 @@ KernelSource Codegen::permute(const Sx& f, const ArrayR& dst, const Sx& p, const
     // slow, not an error, as long as the wave's own updates keep landing.
     u += "    u32* lk_ = locks + j;\n    bool done_ = false;\n    u32 rounds_ = 0;\n    while (__ballot(!done_) != 0ull) {\n";
     u += "      if (++rounds_ > ACC_LOCK_SPIN_LIMIT) {\n        if (!done_) __hip_atomic_store(err, 4u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);\n        break;\n      }\n";
-    u += "      const bool won_ = !done_ && __hip_atomic_exchange(lk_, 1u, __ATOMIC_ACQUIRE, __HIP_MEMORY_SCOPE_AGENT) == 0u;\n";
+    // Lock word and element are only ever touched by relaxed device-scope atomics, which go past
+    // the caches that are not coherent across the device; what orders them is that a wave's
+    // accesses have completed before its next ones leave: the exchange's result is waited for by
+    // the branch on it, and the element's stores are waited for (s_waitcnt) before the store that
+    // frees the lock.  Acquire / release orderings on the lock would add a cache invalidation and a
+    // write-back of the whole L2 per update, which nothing here needs: 2^24 pairs into 2^24
+    // elements 17.0 -> 2.3 ms, into 2^20 elements 29.0 -> 2.2 ms.  ACCHIP_LOCK_ORDER=fences
+    // generates the orderings instead.
+    const char* lo = std::getenv("ACCHIP_LOCK_ORDER");
+    const bool relaxedLock = !(lo && std::string(lo) == "fences");
+    if (relaxedLock)
+      u += "      const bool won_ = !done_ && __hip_atomic_exchange(lk_, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == 0u;\n";
+    else
+      u += "      const bool won_ = !done_ && __hip_atomic_exchange(lk_, 1u, __ATOMIC_ACQUIRE, __HIP_MEMORY_SCOPE_AGENT) == 0u;\n";
     u += "      if (__ballot(won_) != 0ull) rounds_ = 0;\n";
     u += "      if (won_) {\n        Elt y_;\n";
+    if (relaxedLock) u += "        asm volatile(\"\" ::: \"memory\");  // (the compiler keeps the element's loads behind the exchange)\n";
     // leaf by leaf (component by component for SIMD vector leaves) through relaxed atomics
     auto each = [&](size_t k, const std::function<void(const std::string& cell, const std::string& field)>& fn) {
       const std::string cell = "out.o" + std::to_string(k) + "[j]", field = ".c" + std::to_string(k);
@@ -1598,7 +1612,10 @@ KernelSource Codegen::permute(const Sx& f, const ArrayR& dst, const Sx& p, const
       each(k, [&](const std::string& cell, const std::string& field) {
         u += "        __hip_atomic_store(&" + cell + ", r_" + field + ", __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);\n";
       });
-    u += "        __hip_atomic_store(lk_, 0u, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_AGENT);\n        done_ = true;\n      }\n    }\n";
+    if (relaxedLock)
+      u += "        asm volatile(\"s_waitcnt vmcnt(0)\" ::: \"memory\");\n        __hip_atomic_store(lk_, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);\n        done_ = true;\n      }\n    }\n";
+    else
+      u += "        __hip_atomic_store(lk_, 0u, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_AGENT);\n        done_ = true;\n      }\n    }\n";
   }
   if (mode == "atomic" || mode == "atomics") {
     // pieces of the LDS-privatised variant (permute.hpp): one private array per component, its
@@ -1635,6 +1652,52 @@ KernelSource Codegen::permute(const Sx& f, const ArrayR& dst, const Sx& p, const
     lds += "  ACC_DEV void lds_init(Priv& p, int i) {\n" + init + "  }\n";
     lds += "  ACC_DEV void lds_update(Priv& p, int i, const Elt& x) {\n" + upd + "  }\n";
     lds += "  ACC_DEV void lds_flush(const Priv& p, int i, const Out& out, i64 j) {\n" + flush + "  }\n";
+  }
+  if (mode == "lock") {
+    // The same privatisation for combinations that need the lock: a private copy of a destination
+    // range in LDS, one state word per element (bit 0: locked, bit 1: holds a value -- no identity
+    // of the function is known, so the first source of an element is stored as it is), updated
+    // under LDS locks; the workgroups leave their copies in memory, and a second launch combines
+    // them element by element.
+    int bytes = 4;
+    for (ST t : leaves) bytes += stSize(t);
+    lds = "#define ACC_PERMUTE_LDS 1\n#define ACC_PERMUTE_LDS_LOCKED 1\n  static constexpr int kPart = 131072 / " + std::to_string(bytes) +
+          ";\n  struct Priv {\n    u32 st[kPart];\n";
+    std::string rd, wr;
+    for (size_t k = 0; k < leaves.size(); ++k) {
+      const std::string T = stName(leaves[k]), K = std::to_string(k);
+      lds += "    " + T + " c" + K + "[kPart];\n";
+      rd += "          y_.c" + K + " = p.c" + K + "[i];\n";
+      wr += "        p.c" + K + "[i] = r_.c" + K + ";\n";
+    }
+    lds += "  };\n";
+    lds += "  ACC_DEV void lds_init(Priv& p, int i) { p.st[i] = 0u; }\n";
+    // (the loop ends for the whole wave at once, like the one of update(), and for the same reason)
+    lds += "  ACC_DEV void lds_update(const Env& env, Priv& p, int i, const Elt& x, u32* err) {\n"
+           "    bool done_ = false;\n    u32 rounds_ = 0;\n    while (__ballot(!done_) != 0ull) {\n"
+           "      if (++rounds_ > ACC_LOCK_SPIN_LIMIT) {\n        if (!done_) __hip_atomic_store(err, 4u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);\n        break;\n      }\n"
+           "      u32 old_ = 1u;\n"
+           "      if (!done_) old_ = __hip_atomic_fetch_or(&p.st[i], 1u, __ATOMIC_ACQUIRE, __HIP_MEMORY_SCOPE_WORKGROUP);\n"
+           "      const bool won_ = (old_ & 1u) == 0u;\n"
+           "      if (__ballot(won_) != 0ull) rounds_ = 0;\n"
+           "      if (won_) {\n        Elt r_ = x;\n        if (old_ & 2u) {\n          Elt y_;\n" + rd +
+           "          r_ = combine(env, x, y_);\n        }\n" + wr +
+           "        __hip_atomic_store(&p.st[i], 2u, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_WORKGROUP);\n        done_ = true;\n      }\n    }\n  }\n";
+    std::string spill, take;
+    for (size_t k = 0; k < leaves.size(); ++k) {
+      const std::string K = std::to_string(k);
+      spill += "      g->c" + K + "[i] = p.c" + K + "[i];\n";
+      take += "      x_.c" + K + " = g[c_].c" + K + "[i];\n";
+    }
+    lds += "  ACC_DEV void lds_spill(const Priv& p, int i, Priv* g) {\n    const u32 s_ = p.st[i];\n    g->st[i] = s_;\n"
+           "    if (s_ & 2u) {\n" + spill + "    }\n  }\n";
+    // (the copies' values are loaded whether they hold one or not, so that the loads of several
+    // copies can be in flight together)
+    lds += "  ACC_DEV void lds_merge(const Env& env, const Out& out, i64 j, const Priv* g, i64 groups, int i) {\n"
+           "    bool have_ = false;\n    Elt acc_{};\n#pragma unroll 4\n    for (i64 c_ = 0; c_ < groups; ++c_) {\n"
+           "      const u32 s_ = g[c_].st[i];\n      Elt x_;\n" + take +
+           "      if (s_ & 2u) {\n        acc_ = have_ ? combine(env, x_, acc_) : x_;\n        have_ = true;\n      }\n    }\n"
+           "    if (have_) store(out, j, combine(env, acc_, load(out, j)));\n  }\n";
   }
   // A sum of one and the same constant per source (a histogram: `permute (+) zeros p ones`, the ones
   // fused into a constant producer): the skeleton only counts, in 16-bit LDS counters, and adds

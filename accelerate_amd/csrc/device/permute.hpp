@@ -72,8 +72,9 @@ struct PermuteLdsParams {
   i64 part;    // elements per range
   i64 dst_n;   // destination elements
   u32* err;    // host-visible word: 2 = a target outside the destination, 4 = a lock never came free
-  // counting variant only: where the workgroups leave their counters for acc_permute_count_reduce,
-  // [nparts][groups][32768 + 16] words (null: every workgroup adds its counters to the destination itself)
+  // counting variant: where the workgroups leave their counters for acc_permute_count_reduce,
+  // [nparts][groups][32768 + 16] words (null: every workgroup adds its counters to the destination itself);
+  // combinations that need the lock: where they leave their private copies, [nparts][groups] of Spec::Priv
   u32* partials;
   i64 groups;  // source chunks
   // != 0: the destination holds nothing yet; its elements all start from one constant, which
@@ -81,6 +82,13 @@ struct PermuteLdsParams {
   // may touch it
   i64 fresh;
 };
+
+// (a combination that needs the lock also needs the environment, for the function, and the error word)
+#ifdef ACC_PERMUTE_LDS_LOCKED
+#define ACC_LDS_UPDATE(idx, x) S::lds_update(env, priv, idx, x, p.err)
+#else
+#define ACC_LDS_UPDATE(idx, x) S::lds_update(priv, idx, x)
+#endif
 
 extern "C" __global__ void __launch_bounds__(ACC_PERMUTE_LDS_BLOCK)
 acc_permute_lds(Spec::Env env, Spec::Out out, PermuteLdsParams p) {
@@ -119,23 +127,47 @@ acc_permute_lds(Spec::Env env, Spec::Out out, PermuteLdsParams p) {
         const i64 i0 = base + ((i64)g * ACC_PERMUTE_LDS_BLOCK + threadIdx.x) * 4;
 #pragma unroll
         for (int k = 0; k < 4; ++k)
-          if (ok[g][k] && j[g][k] >= lo && j[g][k] < hi) S::lds_update(priv, (int)(j[g][k] - lo), S::in_linear(env, i0 + k));
+          if (ok[g][k] && j[g][k] >= lo && j[g][k] < hi) ACC_LDS_UPDATE((int)(j[g][k] - lo), S::in_linear(env, i0 + k));
       }
     } else {
       for (i64 i = base + threadIdx.x; i < end; i += ACC_PERMUTE_LDS_BLOCK) {
         i64 j;
         const int t = S::target(env, i, j);
-        if (t == 1 && j >= lo && j < hi) S::lds_update(priv, (int)(j - lo), S::in_linear(env, i));
+        if (t == 1 && j >= lo && j < hi) ACC_LDS_UPDATE((int)(j - lo), S::in_linear(env, i));
         bad = bad || t == 2;
       }
     }
   }
   __syncthreads();
+#ifdef ACC_PERMUTE_LDS_LOCKED
+  // the private copy goes to memory as it is; acc_permute_lds_merge combines the copies of a range
+  S::Priv* mine = (S::Priv*)p.partials + (range * p.groups + chunkId);
+  for (int i = threadIdx.x; i < (int)(hi - lo); i += ACC_PERMUTE_LDS_BLOCK) S::lds_spill(priv, i, mine);
+#else
   for (int i = threadIdx.x; i < (int)(hi - lo); i += ACC_PERMUTE_LDS_BLOCK) {
     S::lds_flush(priv, i, out, lo + i);  // components that still hold the identity are skipped
   }
+#endif
   if (bad) __hip_atomic_store(p.err, 2u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
 }
+
+#ifdef ACC_PERMUTE_LDS_LOCKED
+// Second launch for combinations that need the lock: a thread per destination element combines
+// what the workgroups' private copies hold for it, then the element itself -- alone, so without
+// the lock.  (Through the global locks instead, every workgroup asking for every element of a
+// small destination at the same time, 2^24 pairs into 384 elements took 7 ms and into 4096 elements
+// 20 ms, against 6.4 s and 0.54 s without private copies.)
+extern "C" __global__ void __launch_bounds__(256)
+acc_permute_lds_merge(Spec::Env env, Spec::Out out, PermuteLdsParams p) {
+  typedef Spec S;
+  const i64 perRange = (p.part + 255) / 256;
+  const i64 range = (i64)blockIdx.x / perRange;
+  const i64 i = ((i64)blockIdx.x - range * perRange) * 256 + threadIdx.x;
+  const i64 j = range * p.part + i;
+  if (i >= p.part || j >= p.dst_n) return;
+  S::lds_merge(env, out, j, (const S::Priv*)p.partials + range * p.groups, p.groups, (int)i);
+}
+#endif
 #endif
 
 #ifdef ACC_PERMUTE_COUNT

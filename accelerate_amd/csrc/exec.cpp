@@ -1398,20 +1398,13 @@ AValP Program::eval(const Sx& n, AEnv& aenv) {
       }
     }
     if (cnt == 0 || out->size() == 0) return avArr(out);
-    DArrayP locks;
-    if (plan.mode == "lock") {
-      ArrayR lr;
-      lr.rank = 1;
-      lr.elt = tScalar(ST::U32);
-      locks = alloc(lr, {out->size()});
-      ctx_.fill0(locks->bufs[0]->p, locks->bufs[0]->bytes);
-    }
     std::vector<uint64_t> args = packArgs(plan.k->meta, aenv, temps, out->shape);
     packOut(args, *out);
     // Many sources into a destination of a few LDS-fuls with a hardware-atomic combination:
     // combine in workgroup-private LDS copies first (see permute.hpp).
     int64_t eltBytes = 0;
     for (ST st : plan.k->meta.outLeaves) eltBytes += stSize(st);
+    if (plan.mode == "lock") eltBytes += 4;  // the private copy's state word
     const int64_t partMax = 131072 / std::max<int64_t>(1, eltBytes);  // Spec::kPart
     // Up to 128 LDS-fuls: every share re-reads the sources (from its XCD's L2), so the cost grows
     // with the destination -- 2^26 keys into 2^20 / 2^22 Int32 bins take 0.5 / 2.0 ms, which is
@@ -1447,7 +1440,9 @@ AValP Program::eval(const Sx& n, AEnv& aenv) {
       if (partials) ctx_.launch(plan.k, "acc_permute_count_reduce", (uint64_t)(nparts * (32768 / 128)), 256, args);
       return avArr(out);
     }
-    if ((plan.mode == "atomic" || plan.mode == "atomics") && many && out->size() <= maxParts * partMax) {
+    // (under the lock, contended elements cost milliseconds each way: 2^24 pairs into 384 elements
+    // took 6.4 s through global locks alone)
+    if ((plan.mode == "atomic" || plan.mode == "atomics" || plan.mode == "lock") && many && out->size() <= maxParts * partMax) {
       const int64_t nparts = (out->size() + partMax - 1) / partMax;
       const int64_t part = (out->size() + nparts - 1) / nparts;
       // one workgroup per CU in total (each holds 128 KiB of LDS): fewer, longer workgroups
@@ -1463,11 +1458,29 @@ AValP Program::eval(const Sx& n, AEnv& aenv) {
       args.push_back((uint64_t)part);
       args.push_back((uint64_t)out->size());
       args.push_back((uint64_t)(uintptr_t)ctx_.errorWord());
-      args.push_back(0);  // (fields of the counting variant)
+      DArrayP copies;
+      if (plan.mode == "lock") {
+        // the workgroups' private copies, one Spec::Priv each (128 KiB and the padding between its arrays at most)
+        ArrayR pr;
+        pr.rank = 1;
+        pr.elt = tScalar(ST::U32);
+        const int64_t privBytes = 131072 + 16 * ((int64_t)plan.k->meta.outLeaves.size() + 2);
+        copies = alloc(pr, {nparts * groups * privBytes / 4});
+      }
+      args.push_back(copies ? (uint64_t)(uintptr_t)copies->bufs[0]->p : 0);  // (otherwise a field of the counting variant)
       args.push_back((uint64_t)groups);
       args.push_back(0);
       ctx_.launch(plan.k, "acc_permute_lds", (uint64_t)(groups * nparts), 1024, args);
+      if (copies) ctx_.launch(plan.k, "acc_permute_lds_merge", (uint64_t)(nparts * ((part + 255) / 256)), 256, args);
       return avArr(out);
+    }
+    DArrayP locks;
+    if (plan.mode == "lock") {
+      ArrayR lr;
+      lr.rank = 1;
+      lr.elt = tScalar(ST::U32);
+      locks = alloc(lr, {out->size()});
+      ctx_.fill0(locks->bufs[0]->p, locks->bufs[0]->bytes);
     }
     args.push_back((uint64_t)cnt);
     args.push_back(locks ? (uint64_t)(uintptr_t)locks->bufs[0]->p : 0);

@@ -235,3 +235,83 @@ def test_counting_permute_writes_constant_defaults_itself(gpu_ctx, knobs):
     for fresh in (1, 0):
         knobs("permute_fresh", fresh)
         assert np.array_equal(gpu_ctx.compile(prog)(keys), want)
+
+
+# -- combinations that need the lock: private copies in LDS under LDS locks, combined by a second launch
+
+def _two_smallest(nbins, a_ty=A.i64, b_ty=A.i64, big=1 << 40):
+    """permute into (inf, inf) pairs: every element ends as the two smallest values sent to it (the
+    merge of Issue137: associative and commutative, but no component is a function of its own
+    component alone, so no hardware atomic fits); a negative target drops the source"""
+    t2 = A.ttup(a_ty, b_ty)
+    sh1 = A.tshape(1)
+    inf_a, inf_b = A.const(a_ty, big), A.const(b_ty, big)
+    conv = (lambda e: e) if a_ty == b_ty else (lambda e: A.fromintegral(a_ty, b_ty, e))
+    back = (lambda e: e) if a_ty == b_ty else (lambda e: A.fromintegral(b_ty, a_ty, e))
+
+    def comb(p, q):
+        a1, a2 = A.untup(p)
+        b1, b2 = A.untup(q)
+        return A.cond(A.lte(a_ty, a1, b1), A.tup(a1, A.min_(b_ty, a2, conv(b1))), A.tup(b1, A.min_(b_ty, b2, conv(a1))))
+
+    def body(xs, to):
+        src = A.delayed(A.tarray(1, t2), A.shape(xs), A.lam([sh1], lambda ix: A.tup(A.index(xs, A.vexp(ix)), inf_b)),
+                        A.lam([A.Int], lambda i: A.tup(A.linearindex(xs, i), inf_b)))
+        tgt = lambda ix: A.cond(A.lt(A.Int, A.index(to, A.vexp(ix)), A.constI(0)), A.nothing(sh1),
+                                A.just(A.sh(A.index(to, A.vexp(ix)))))
+        return A.permute(A.lam([t2, t2], comb),
+                         A.generate(A.tarray(1, t2), A.sh(nbins), A.lam([sh1], lambda ix: A.tup(inf_a, inf_b))),
+                         A.lam([sh1], tgt), src)
+
+    return A.alam([A.tarray(1, a_ty), A.tarray(1, A.Int)], body)
+
+
+def _two_smallest_ref(x, to, nbins, big):
+    keep = to >= 0
+    x, to = x[keep], to[keep]
+    order = np.lexsort((x, to))
+    ts, xs = to[order], x[order]
+    n = len(xs)
+    first = np.searchsorted(ts, np.arange(nbins))
+    cnt = np.diff(np.append(first, n))
+    m1 = np.where(cnt > 0, xs[np.minimum(first, n - 1)], big)
+    m2 = np.where(cnt > 1, xs[np.minimum(first + 1, n - 1)], big)
+    return m1, m2
+
+
+# 6553 elements of (Int64, Int64) and their state word fill 128 KiB of LDS: one range, two ranges,
+# several, and more than the privatised kernel accepts (global locks)
+@pytest.mark.gpu
+@pytest.mark.parametrize("nbins", [1, 7, 384, 6553, 6554, 70000, 300000])
+@pytest.mark.parametrize("order", ["fences", "waits"])
+def test_locked_combination_through_private_copies(gpu_ctx, monkeypatch, nbins, order):
+    if order == "fences":
+        monkeypatch.setenv("ACCHIP_LOCK_ORDER", "fences")   # read when the kernel is generated
+    rng = np.random.default_rng(nbins)
+    n = N
+    x = rng.integers(0, 1 << 30, n, dtype=np.int64)
+    to = rng.integers(-1, nbins, n, dtype=np.int64)         # -1: dropped
+    # a third of the sources want one element (a few thousand of them where the global locks serve: they take turns there)
+    to[rng.random(n) < (0.3 if nbins <= 200000 else 0.002)] = nbins // 2
+    a, b = gpu_ctx.compile(_two_smallest(nbins))(x, to)
+    m1, m2 = _two_smallest_ref(x, to, nbins, 1 << 40)
+    assert np.array_equal(a, m1) and np.array_equal(b, m2)
+
+
+@pytest.mark.gpu
+def test_locked_combination_few_sources_and_mixed_component_types(gpu_ctx):
+    # below the threshold of the privatised kernel: global locks under contention
+    rng = np.random.default_rng(8)
+    x = rng.integers(0, 1 << 30, 3000, dtype=np.int64)
+    to = rng.integers(0, 5, 3000, dtype=np.int64)
+    a, b = gpu_ctx.compile(_two_smallest(5))(x, to)
+    m1, m2 = _two_smallest_ref(x, to, 5, 1 << 40)
+    assert np.array_equal(a, m1) and np.array_equal(b, m2)
+    # (Int32, Int64) pairs: 16 bytes with the state word, 8192 elements per range
+    n = N
+    x = rng.integers(0, 1 << 30, n).astype(np.int32)
+    for nbins in (8192, 8193):
+        to = rng.integers(0, nbins, n, dtype=np.int64)
+        a, b = gpu_ctx.compile(_two_smallest(nbins, A.i32, A.i64, 1 << 30))(x, to)
+        m1, m2 = _two_smallest_ref(x.astype(np.int64), to, nbins, 1 << 30)
+        assert np.array_equal(a, m1.astype(np.int32)) and np.array_equal(b, m2)
