@@ -1653,8 +1653,9 @@ KernelSource Codegen::permute(const Sx& f, const ArrayR& dst, const Sx& p, const
     lds += "  ACC_DEV void lds_update(Priv& p, int i, const Elt& x) {\n" + upd + "  }\n";
     lds += "  ACC_DEV void lds_flush(const Priv& p, int i, const Out& out, i64 j) {\n" + flush + "  }\n";
   }
-  if (mode == "lock") {
-    // The same privatisation for combinations that need the lock: a private copy of a destination
+  if (mode == "lock" || mode == "cas") {
+    // The same privatisation for combinations that need the lock, or the compare-and-swap loop
+    // (2^24 Int64 products into 384 / 4096 elements: 498 / 25 ms of retries): a private copy of a destination
     // range in LDS, one state word per element (bit 0: locked, bit 1: holds a value -- no identity
     // of the function is known, so the first source of an element is stored as it is), updated
     // under LDS locks; the workgroups leave their copies in memory, and a second launch combines

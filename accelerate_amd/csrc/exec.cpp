@@ -1404,13 +1404,15 @@ AValP Program::eval(const Sx& n, AEnv& aenv) {
     // combine in workgroup-private LDS copies first (see permute.hpp).
     int64_t eltBytes = 0;
     for (ST st : plan.k->meta.outLeaves) eltBytes += stSize(st);
-    if (plan.mode == "lock") eltBytes += 4;  // the private copy's state word
+    const bool statefulCopies = plan.mode == "lock" || plan.mode == "cas";
+    if (statefulCopies) eltBytes += 4;  // the private copy's state word
     const int64_t partMax = 131072 / std::max<int64_t>(1, eltBytes);  // Spec::kPart
     // Up to 128 LDS-fuls: every share re-reads the sources (from its XCD's L2), so the cost grows
     // with the destination -- 2^26 keys into 2^20 / 2^22 Int32 bins take 0.5 / 2.0 ms, which is
     // where plain global atomics are for uniform keys (2.5 ms); for Zipf keys those take 110 ms.
     // (the privatised permute: 80 us per range for 2^26 sources, against 2.5 - 3.2 ms of global atomics)
-    const int64_t maxParts = std::min<int64_t>(ctx_.knobs.permute_parts, 32);
+    // (a compare-and-swap loop without contention does 2^24 updates in 0.8 ms, ten ranges' worth)
+    const int64_t maxParts = std::min<int64_t>(ctx_.knobs.permute_parts, plan.mode == "cas" ? 10 : 32);
     // From 2^20 sources on, and from 2^12 on when every destination element receives several of
     // them (few destinations under many sources contend in the memory-side atomic units: 2^16
     // keys into 256 bins take 33 us through global atomics, 2^14 keys into 16 bins 47 us,
@@ -1442,7 +1444,7 @@ AValP Program::eval(const Sx& n, AEnv& aenv) {
     }
     // (under the lock, contended elements cost milliseconds each way: 2^24 pairs into 384 elements
     // took 6.4 s through global locks alone)
-    if ((plan.mode == "atomic" || plan.mode == "atomics" || plan.mode == "lock") && many && out->size() <= maxParts * partMax) {
+    if ((plan.mode == "atomic" || plan.mode == "atomics" || statefulCopies) && many && out->size() <= maxParts * partMax) {
       const int64_t nparts = (out->size() + partMax - 1) / partMax;
       const int64_t part = (out->size() + nparts - 1) / nparts;
       // one workgroup per CU in total (each holds 128 KiB of LDS): fewer, longer workgroups
@@ -1459,7 +1461,7 @@ AValP Program::eval(const Sx& n, AEnv& aenv) {
       args.push_back((uint64_t)out->size());
       args.push_back((uint64_t)(uintptr_t)ctx_.errorWord());
       DArrayP copies;
-      if (plan.mode == "lock") {
+      if (statefulCopies) {
         // the workgroups' private copies, one Spec::Priv each (128 KiB and the padding between its arrays at most)
         ArrayR pr;
         pr.rank = 1;

@@ -315,3 +315,32 @@ def test_locked_combination_few_sources_and_mixed_component_types(gpu_ctx):
         a, b = gpu_ctx.compile(_two_smallest(nbins, A.i32, A.i64, 1 << 30))(x, to)
         m1, m2 = _two_smallest_ref(x.astype(np.int64), to, nbins, 1 << 30)
         assert np.array_equal(a, m1.astype(np.int32)) and np.array_equal(b, m2)
+
+
+# -- scalar combinations without a hardware atomic (compare-and-swap loop): the same private copies
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("nbins", [3, 10922, 10923, 60000, 200000])   # one range, two, six, and the CAS loop in memory
+def test_products_through_private_copies(gpu_ctx, nbins):
+    sh1 = A.tshape(1)
+    prog = A.alam([A.tarray(1, A.i64), A.tarray(1, A.Int), A.tarray(1, A.i64)], lambda xs, to, dfl: A.permute(
+        Q.binop(A.mul, A.i64), dfl, A.lam([sh1], lambda ix: A.just(A.sh(A.index(to, A.vexp(ix))))), xs))
+    rng = np.random.default_rng(nbins)
+    x = rng.integers(0, 1 << 62, N, dtype=np.int64) | 1      # odd factors: the product modulo 2^64 never collapses to 0
+    to = rng.integers(0, nbins, N, dtype=np.int64)
+    to[rng.random(N) < 0.25] = nbins - 1
+    dfl = rng.integers(1, 1000, nbins, dtype=np.int64)
+    want = dfl.astype(np.uint64)
+    np.multiply.at(want, to, x.astype(np.uint64))
+    assert np.array_equal(gpu_ctx.compile(prog)(x, to, dfl).astype(np.uint64), want)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("nbins", [100, 16384, 16385])
+def test_float_maximum_through_private_copies(gpu_ctx, nbins):
+    x = np.random.default_rng(nbins).normal(size=N).astype(np.float32)
+    to = np.random.default_rng(nbins + 1).integers(0, nbins, N, dtype=np.int64)
+    dfl = np.full(nbins, -0.5, dtype=np.float32)
+    want = dfl.copy()
+    np.maximum.at(want, to, x)
+    assert np.array_equal(gpu_ctx.compile(_combine_prog(A.max_, A.f32))(x, to, dfl), want)
