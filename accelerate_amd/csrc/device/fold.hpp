@@ -445,14 +445,24 @@ ACC_DEV void acc_fold_wrows_body(const Spec::Env& env, const Spec::Out& out, con
     S::Elt acc;
     bool have = false;
     if (valid) {
-      i64 e0 = (i64)sub * V;
+      // A commutative operator lets a lane take every L-th run of V elements, so that the wave's
+      // loads cover consecutive memory; any other needs the row in order: a lane takes one stretch
+      // of consecutive elements (a whole number of runs), and the join below, which goes through
+      // the lanes in order, keeps the stretches in theirs.
+      i64 e0 = (i64)sub * V, end = p.n, stp = step;
+      if (!S::kCommutative) {
+        const i64 stretch = ((p.n + L - 1) / L + V - 1) / V * V;
+        e0 = (i64)sub * stretch;
+        end = e0 + stretch < p.n ? e0 + stretch : p.n;
+        stp = V;
+      }
       // four runs at a time, their loads together
-      for (; e0 + 3 * step + V <= p.n; e0 += 4 * step) {
+      for (; e0 + 3 * stp + V <= end; e0 += 4 * stp) {
         S::Elt x[4][S::V];
 #pragma unroll
         for (int u = 0; u < 4; ++u)
 #pragma unroll
-          for (int k = 0; k < V; ++k) x[u][k] = src(off + e0 + u * step + k);
+          for (int k = 0; k < V; ++k) x[u][k] = src(off + e0 + u * stp + k);
 #pragma unroll
         for (int u = 0; u < 4; ++u)
 #pragma unroll
@@ -461,7 +471,7 @@ ACC_DEV void acc_fold_wrows_body(const Spec::Env& env, const Spec::Out& out, con
             have = true;
           }
       }
-      for (; e0 + V <= p.n; e0 += step) {
+      for (; e0 + V <= end; e0 += stp) {
         S::Elt x[S::V];
 #pragma unroll
         for (int k = 0; k < V; ++k) x[k] = src(off + e0 + k);
@@ -471,7 +481,7 @@ ACC_DEV void acc_fold_wrows_body(const Spec::Env& env, const Spec::Out& out, con
           have = true;
         }
       }
-      for (i64 e = e0; e < p.n; ++e) {  // the row's ragged end, in one lane
+      for (i64 e = e0; e < end; ++e) {  // the ragged end of the row (or of the stretch), in one lane
         const S::Elt x = src(off + e);
         acc = have ? S::combine(env, acc, x) : x;
         have = true;
@@ -483,9 +493,9 @@ ACC_DEV void acc_fold_wrows_body(const Spec::Env& env, const Spec::Out& out, con
 
 extern "C" __global__ void __launch_bounds__(ACC_BLOCK)
 acc_fold_wrows(Spec::Env env, Spec::Out out, Spec::Out tmp, FoldWaveRowsParams p) {
-  if constexpr (Spec::kCommutative) acc_fold_wrows_body<false>(env, out, p);
+  acc_fold_wrows_body<false>(env, out, p);
 }
 extern "C" __global__ void __launch_bounds__(ACC_BLOCK)
 acc_fold_wrows_stream(Spec::Env env, Spec::Out out, Spec::Out tmp, FoldWaveRowsParams p) {
-  if constexpr (Spec::kCommutative) acc_fold_wrows_body<true>(env, out, p);
+  acc_fold_wrows_body<true>(env, out, p);
 }

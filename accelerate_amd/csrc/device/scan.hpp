@@ -394,7 +394,8 @@ ACC_DEV void acc_scan_tile(const typename S::Env& env, u64* desc, i64 tiles, i64
             Elt e = load(t);
             x[g][k] = k == 0 ? e : S::combine(env, x[g][k - 1], e);
           } else {
-            x[g][k] = k > 0 ? x[g][k - 1] : filler;
+            if (k > 0) x[g][k] = x[g][k - 1];
+          else x[g][k] = filler;
           }
         }
       }
@@ -601,7 +602,8 @@ ACC_DEV void acc_rows_tile(const typename S::Env& env, int cnt, int n, const Loa
           e.f = t == 0 ? 1u : 0u;
           x[g][k] = k == 0 ? e : SS::combine(env, x[g][k - 1], e);
         } else {
-          x[g][k] = k > 0 ? x[g][k - 1] : filler;
+          if (k > 0) x[g][k] = x[g][k - 1];
+          else x[g][k] = filler;
         }
         if (++t == n) {
           t = 0;
@@ -610,7 +612,11 @@ ACC_DEV void acc_rows_tile(const typename S::Env& env, int cnt, int n, const Loa
       }
     }
   }
-  P waveTot = haveFiller ? filler : x[0][0];
+  // (not `haveFiller ? filler : x[0][0]`: a choice between two objects is a choice between two
+  // addresses, and values of 16 bytes then live in scratch memory -- the rows kernels ran at
+  // 0.84 TB/s for 8-byte elements)
+  P waveTot = x[0][0];
+  if (haveFiller) waveTot = filler;
   bool hasWaveTot = false;
 #ifdef ACC_ROWS_RAKE
   {

@@ -1233,11 +1233,15 @@ AValP Program::eval(const Sx& n, AEnv& aenv) {
     int64_t rows = out->size();
     if (rows == 0) return avArr(out);
     {
-      // many rows of up to a few thousand elements under a commutative operator: a few lanes of
-      // a wave per row (acc_fold_wrows).  fold_rows: 2 forces it, 0 and 1 keep it off.
+      // many rows of up to a few thousand elements: a few lanes of a wave per row (acc_fold_wrows;
+      // under an operator that is not commutative a lane takes a stretch of the row instead of
+      // every so-many-th run).  fold_rows: 2 forces it, 0 and 1 keep it off.
       const KernelSource& m = plan.k->meta;
       const long long fr = ctx_.knobs.fold_rows;
-      const bool wave = m.commutative && len >= 1 && (fr == 2 || (fr < 0 && rows >= 256 && len < 4096));
+      // (in order, a lane's stretch of more than two runs no longer lets the wave's loads cover
+      // consecutive memory: rows of 1024 Int64 1.9 TB/s against 3.9 - 4.5 several rows per workgroup;
+      // rows of 16 / 256: 4.2 / 4.2 against 3.6 / 3.8, Float32 5.2 / 5.3 against 3.9 / 3.9)
+      const bool wave = len >= 1 && (fr == 2 || (fr < 0 && rows >= 256 && (m.commutative ? len < 4096 : len <= 128 * m.vec)));
       if (wave) {
         const int64_t runs = (len + m.vec - 1) / m.vec;
         int64_t lanes = 1;

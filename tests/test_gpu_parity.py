@@ -72,8 +72,8 @@ FOLDS = [(c, g) for cs, g in ((GOLDEN, True), (PARITY, False)) for c in cs
 @pytest.mark.parametrize("rows_kernel", ["0", "1", "2"])
 @pytest.mark.parametrize("case", FOLDS, ids=[c[0][0] for c in FOLDS])
 def test_folds_with_and_without_the_rows_kernel(gpu_ctx, knobs, case, rows_kernel):
-    # short rows are reduced several per workgroup (1), or, under a commutative operator, by a few
-    # lanes of a wave each (2); all paths must give the same answers
+    # short rows are reduced several per workgroup (1), or by a few lanes of a wave each (2); all
+    # paths must give the same answers
     knobs("fold_rows", int(rows_kernel))
     (_, prog, args, last), golden = case
     got = gpu_ctx.compile(prog)(*args)
@@ -114,6 +114,31 @@ def test_rows_reduced_by_a_few_lanes_each(gpu_ctx, knobs):
     assert np.allclose(got, x.astype(np.float64).sum(axis=1), rtol=1e-5)
     x3 = rng.integers(-5, 5, (20, 30, 40)).astype(np.int64)
     assert np.array_equal(gpu_ctx.compile(P.fold_sum(A.i64, 3))(x3), x3.sum(axis=2))
+
+
+@pytest.mark.parametrize("rows_kernel", [2, -1])
+def test_rows_reduced_by_a_few_lanes_each_in_order(gpu_ctx, knobs, rows_kernel):
+    # operators that are not commutative: "the last value that is not zero" and, on pairs, "the first
+    # of the first and the second of the last" -- a lane then takes a stretch of its row, and any
+    # stretch, run or lane joined out of order shows
+    knobs("fold_rows", rows_kernel)
+    rng = np.random.default_rng(32)
+    I = A.i64
+    last = A.lam([I, I], lambda p, q: A.cond(A.neq(I, q, A.constI(0)), q, p))
+    lasts = gpu_ctx.compile(A.alam([A.tarray(2, I)], lambda xs: A.fold(last, A.constI(0), xs)))
+    t2 = A.ttup(I, I)
+    ends = gpu_ctx.compile(A.alam([A.tarray(2, t2)], lambda xs: A.fold(
+        A.lam([t2, t2], lambda p, q: A.tup(A.untup(p)[0], A.untup(q)[1])), None, xs)))
+    for rows, n in [(1, 1), (3, 2), (1000, 3), (64, 5), (999, 17), (4096, 64), (300, 127), (300, 128), (300, 129), (100, 255),
+                    (100, 257), (50, 1000), (33, 4095), (7, 10_001), (300_000, 12), (70_000, 200)]:
+        x = rng.integers(1, 1 << 40, (rows, n)).astype(np.int64)
+        x[rng.random((rows, n)) < 0.7] = 0
+        idx = np.where(x != 0, np.arange(n), -1).max(axis=1)
+        want = np.where(idx >= 0, x[np.arange(rows), np.maximum(idx, 0)], 0)
+        assert np.array_equal(lasts(x), want), (rows, n)
+        y = rng.integers(-1000, 1000, (rows, n)).astype(np.int64)
+        a, b = ends(gpu_ctx.to_device((x, y), A.tarray(2, t2)))
+        assert np.array_equal(a, x[:, 0]) and np.array_equal(b, y[:, -1]), (rows, n)
 
 
 @pytest.mark.parametrize("one_launch", [0, 1])
