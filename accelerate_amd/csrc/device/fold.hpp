@@ -41,7 +41,17 @@ struct FoldParams {
   u32* err;         // host-visible word: 3 = it gave up
 };
 
-template <class S, class Src>
+// tiles the ordered fold turns over in LDS at a time: 128 bytes of elements per lane, none for
+// elements so large that the staging area of a workgroup would pass 40 KiB
+#ifndef ACC_FOLD_STAGE_BYTES
+#define ACC_FOLD_STAGE_BYTES 128
+#endif
+template <class S> struct AccFoldStage {
+  enum { kRun = S::V * (int)sizeof(typename S::Elt),
+         K = S::kCommutative || kRun > 64 ? 1 : ACC_FOLD_STAGE_BYTES / kRun };
+};
+
+template <class S, class Src, bool STAGE = false>
 ACC_DEV bool acc_fold_span(const typename S::Env& env, const Src& src, i64 off, i64 lo, i64 hi,
                            typename S::Elt& result) {
   typedef typename S::Elt Elt;
@@ -88,6 +98,46 @@ ACC_DEV bool acc_fold_span(const typename S::Env& env, const Src& src, i64 off, 
   } else {
     Elt carry;
     i64 base = lo;
+    // Blocks of K tiles, for as long as they last: the wave loads them tile by tile (one load
+    // instruction covers consecutive memory, K of them in flight per lane) and turns them over in
+    // LDS, so that a lane gets K * V consecutive elements to combine in order, and the wave joins
+    // its lanes once per block instead of once per tile -- the join is what a tile costs (a single
+    // row of 2^27 Int64 under "the last value that is not zero": 3.1 TB/s tile by tile).  A lane's
+    // stretch is padded by one element, which keeps its reads off the banks of its neighbours'.
+    // (the staging area costs occupancy, so only the kernels launched for long chunks have it)
+    constexpr int K = STAGE && Src::kBulk ? AccFoldStage<S>::K : 1;
+    if constexpr (K > 1) {
+      constexpr int R = K * V;  // elements a lane combines per block
+      __shared__ Elt sh_stage[ACC_WAVES][ACC_WAVE * (R + 1)];
+      Elt* st = sh_stage[acc_wave()];
+      for (; base + K * T <= hi; base += K * T) {
+        const i64 q = off + base + (i64)lane * V;
+        Elt x[K][S::V];
+#pragma unroll
+        for (int k = 0; k < K; ++k)
+#pragma unroll
+          for (int v = 0; v < V; ++v) x[k][v] = src(q + (i64)k * T + v);
+#pragma unroll
+        for (int k = 0; k < K; ++k)
+#pragma unroll
+          for (int v = 0; v < V; ++v) {
+            const int e = k * (int)T + lane * V + v;
+            st[e + e / R] = x[k][v];
+          }
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+        Elt t = st[lane * (R + 1)];
+#pragma unroll
+        for (int j = 1; j < R; ++j) t = S::combine(env, t, st[lane * (R + 1) + j]);
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+        t = acc_wave_reduce<S>(env, t, lane, ACC_WAVE);
+        carry = have ? S::combine(env, carry, t) : t;
+        have = true;
+      }
+    }
     // full tiles: V unconditional loads per lane (one wide request), all lanes take part
     for (; base + T <= hi; base += T) {
       const i64 q = off + base + (i64)lane * V;
@@ -175,7 +225,7 @@ ACC_DEV bool acc_fold_rows_of_block(const typename S::Env& env, const Src& src, 
 }
 
 // Reduce [lo, hi) of one row with the whole workgroup; the result is valid in thread 0.
-template <class S, class Src>
+template <class S, class Src, bool STAGE = false>
 ACC_DEV bool acc_fold_block(const typename S::Env& env, const Src& src, i64 off, i64 lo, i64 hi,
                             typename S::Elt& result) {
   typedef typename S::Elt Elt;
@@ -191,7 +241,7 @@ ACC_DEV bool acc_fold_block(const typename S::Env& env, const Src& src, i64 off,
   Elt r;
   bool ok;
   if constexpr (S::kCommutative && ACC_FOLD_ROWS) ok = acc_fold_rows_of_block<S>(env, src, off, lo, hi, r);
-  else ok = acc_fold_span<S>(env, src, off, wlo, whi, r);
+  else ok = acc_fold_span<S, Src, STAGE>(env, src, off, wlo, whi, r);
   if (acc_lane() == 0) {
     sh_v[w] = r;
     sh_ok[w] = ok ? 1 : 0;
@@ -211,16 +261,19 @@ ACC_DEV bool acc_fold_block(const typename S::Env& env, const Src& src, i64 off,
 }
 
 template <class S, bool NT = false> struct AccFoldSrcIn {
+  static constexpr bool kBulk = true;  // the operand itself: worth staging blocks of it in LDS
   const typename S::Env& env;
   __device__ __forceinline__ typename S::Elt operator()(i64 i) const { return S::template in_linear<NT>(env, i); }
 };
 template <class S> struct AccFoldSrcTmp {
+  static constexpr bool kBulk = false;
   const typename S::Out& tmp;
   __device__ __forceinline__ typename S::Elt operator()(i64 i) const { return S::load(tmp, i); }
 };
 
 // chunk results published by the workgroups of this launch: waits (bounded) until the words carry the launch's tag
 template <class S> struct AccFoldSrcDesc {
+  static constexpr bool kBulk = false;
   const u64* desc;
   u64 epoch, limit;
   u32* err;
@@ -250,7 +303,7 @@ ACC_DEV void acc_fold_finish(const typename S::Env& env, const typename S::Out& 
   }
 }
 
-template <bool NT>
+template <bool NT, bool STAGE = false>
 ACC_DEV void acc_fold_main_body(const Spec::Env& env, const Spec::Out& out, const Spec::Out& tmp, const FoldParams& p) {
   typedef Spec S;
   i64 bid = p.first + (i64)blockIdx.x;
@@ -260,7 +313,7 @@ ACC_DEV void acc_fold_main_body(const Spec::Env& env, const Spec::Out& out, cons
   i64 hi = lo + p.chunk < p.n ? lo + p.chunk : p.n;
   AccFoldSrcIn<S, NT> src{env};
   S::Elt r;
-  bool have = acc_fold_block<S>(env, src, row * p.n, lo, hi, r);
+  bool have = acc_fold_block<S, AccFoldSrcIn<S, NT>, STAGE>(env, src, row * p.n, lo, hi, r);
   if (p.bpr == 1) {
     acc_fold_finish<S>(env, out, row, have, r);
   } else if (p.desc) {
@@ -289,6 +342,17 @@ acc_fold_main(Spec::Env env, Spec::Out out, Spec::Out tmp, FoldParams p) {
 extern "C" __global__ void __launch_bounds__(ACC_BLOCK)
 acc_fold_main_stream(Spec::Env env, Spec::Out out, Spec::Out tmp, FoldParams p) {
   acc_fold_main_body<true>(env, out, tmp, p);
+}
+
+// the same for operators that are not commutative and chunks of 64 KiB and more: blocks of tiles
+// turned over in LDS (acc_fold_span)
+extern "C" __global__ void __launch_bounds__(ACC_BLOCK)
+acc_fold_main_staged(Spec::Env env, Spec::Out out, Spec::Out tmp, FoldParams p) {
+  acc_fold_main_body<false, (AccFoldStage<Spec>::K > 1)>(env, out, tmp, p);
+}
+extern "C" __global__ void __launch_bounds__(ACC_BLOCK)
+acc_fold_main_staged_stream(Spec::Env env, Spec::Out out, Spec::Out tmp, FoldParams p) {
+  acc_fold_main_body<true, (AccFoldStage<Spec>::K > 1)>(env, out, tmp, p);
 }
 
 extern "C" __global__ void __launch_bounds__(ACC_BLOCK)
@@ -353,11 +417,24 @@ struct AccFoldRowLanes {
     u32 f;
   };
   ACC_DEV Elt combine(const Env& env, const Elt& a, const Elt& b) {
-    if (b.f & 1u) return b;
+    if constexpr (sizeof(Spec::Elt) <= 8) {
+      if (b.f & 1u) return b;
+      Elt r;
+      if ((a.f & 2u) && (b.f & 2u)) r.v = Spec::combine(env, a.v, b.v);
+      else if (b.f & 2u) r.v = b.v;
+      else r.v = a.v;
+      r.f = (a.f & 1u) | ((a.f | b.f) & 2u);
+      return r;
+    }
+    // (larger values: the one kept is chosen word by word, see acc_pick; the function is only
+    // applied to two values that exist: it may read tables with them)
     Elt r;
-    if ((a.f & 2u) && (b.f & 2u)) r.v = Spec::combine(env, a.v, b.v);
-    else r.v = (b.f & 2u) ? b.v : a.v;
-    r.f = (a.f & 1u) | ((a.f | b.f) & 2u);
+    const bool head = (b.f & 1u) != 0u, ha = (a.f & 2u) != 0u, hb = (b.f & 2u) != 0u;
+    u32 wr[AccWords<Spec::Elt>::N];
+    acc_to_words(acc_pick(head || hb, b.v, a.v), wr);
+    if (!head && ha && hb) acc_to_words(Spec::combine(env, a.v, b.v), wr);
+    r.v = acc_from_words<Spec::Elt>(wr);
+    r.f = head ? b.f : ((a.f & 1u) | ((a.f | b.f) & 2u));
     return r;
   }
 };

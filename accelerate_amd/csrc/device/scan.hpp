@@ -527,13 +527,14 @@ template <class S> struct AccSegSpec {
   enum { V = S::V, G = S::G };
   static constexpr bool kSeeded = false;  // z is applied when a segment's value is written
   ACC_DEV Elt combine(const Env& env, const Elt& a, const Elt& b) {
+    // (the value goes through its words, so that `b or the combination` is a choice between
+    // values and not between the addresses of two objects: see acc_pick)
     Elt r;
-    if (b.f) {
-      r = b;
-    } else {
-      r.v = S::combine(env, a.v, b.v);
-      r.f = a.f;
-    }
+    u32 wr[AccWords<typename S::Elt>::N];
+    acc_to_words(b.v, wr);
+    if (!b.f) acc_to_words(S::combine(env, a.v, b.v), wr);
+    r.v = acc_from_words<typename S::Elt>(wr);
+    r.f = b.f ? b.f : a.f;
     return r;
   }
   ACC_DEV Elt seed(const Env&) {

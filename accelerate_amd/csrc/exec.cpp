@@ -1327,10 +1327,19 @@ AValP Program::eval(const Sx& n, AEnv& aenv) {
       for (int k = 0; k < 4; ++k) args.push_back(0);
     }
     const bool st = streams(plan.k->meta, aenv, temps, 0);
+    // An operator that is not commutative over chunks of 64 KiB and more: the kernel that turns
+    // blocks of tiles over in LDS (a wave then joins its lanes once per 8 KiB instead of once per
+    // KiB: a single row of 2^27 Int64 3.1 -> 6.6 TB/s; its staging area would cost shorter rows
+    // their occupancy).  Elements of up to 64 bytes a run (AccFoldStage).
+    int64_t eltBytes = 0;
+    for (ST t : plan.k->meta.outLeaves) eltBytes += stSize(t);
+    const bool staged = !plan.k->meta.commutative && chunk * eltBytes >= 65536 && plan.k->meta.vec * eltBytes <= 64 &&
+                        ctx_.knobs.fold_staged != 0;
+    const char* entry = staged ? (st ? "acc_fold_main_staged_stream" : "acc_fold_main_staged") : (st ? "acc_fold_main_stream" : "acc_fold_main");
     // a launch holds fewer than 2^32 threads: more rows than that many workgroups take several launches
     for (int64_t first = 0; first < rows * bpr; first += most) {
       args[firstAt] = (uint64_t)first;
-      ctx_.launch(plan.k, st ? "acc_fold_main_stream" : "acc_fold_main", (uint64_t)std::min(most, rows * bpr - first), 256, args);
+      ctx_.launch(plan.k, entry, (uint64_t)std::min(most, rows * bpr - first), 256, args);
     }
     args[firstAt] = 0;
     if (bpr > 1 && !oneLaunch) ctx_.launch(plan.k, "acc_fold_final", (uint64_t)rows, 256, args);

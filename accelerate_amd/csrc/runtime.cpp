@@ -55,7 +55,7 @@ struct KnobName {
 const KnobName kKnobs[] = {
     {"stream_bytes", &Knobs::stream_bytes},       {"map_max_blocks", &Knobs::map_max_blocks},
     {"map_tiled", &Knobs::map_tiled},             {"fold_rows", &Knobs::fold_rows},
-    {"fold_target", &Knobs::fold_target},         {"fold_max_blocks", &Knobs::fold_max_blocks},         {"permute_parts", &Knobs::permute_parts},
+    {"fold_target", &Knobs::fold_target},         {"fold_staged", &Knobs::fold_staged},         {"fold_max_blocks", &Knobs::fold_max_blocks},         {"permute_parts", &Knobs::permute_parts},
     {"permute_count", &Knobs::permute_count},     {"permute_groups", &Knobs::permute_groups},
     {"permute_partials", &Knobs::permute_partials}, {"permute_fresh", &Knobs::permute_fresh}, {"stencil_chain", &Knobs::stencil_chain},
     {"pool_async", &Knobs::pool_async}, {"fold_one_launch", &Knobs::fold_one_launch},

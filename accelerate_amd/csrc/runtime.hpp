@@ -52,6 +52,7 @@ struct Knobs {
   long long map_tiled = -1;         // -1: decide per launch, 0 / 1: never / always tile index-permuting producers
   long long fold_rows = -1;         // -1: decide per launch; 0 / 1: never / always the several-rows-per-workgroup fold; 2: always a few lanes per row
   long long fold_target = 2048;     // workgroups a fold aims at
+  long long fold_staged = 1;        // 0: ordered folds never take the kernel that stages blocks of tiles in LDS
   long long scan_post = 1;          // 0: a map around a scan is always a launch of its own
   long long scan_ticketless = 1;    // 0: the tiles of a scan always take their numbers from the ticket counter
   long long foldseg_one_launch = 1; // 0: the ends that reach across tile borders are completed by a launch of their own

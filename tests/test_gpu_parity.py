@@ -141,6 +141,32 @@ def test_rows_reduced_by_a_few_lanes_each_in_order(gpu_ctx, knobs, rows_kernel):
         assert np.array_equal(a, x[:, 0]) and np.array_equal(b, y[:, -1]), (rows, n)
 
 
+@pytest.mark.parametrize("staged", [1, 0])
+def test_long_rows_in_order(gpu_ctx, knobs, staged):
+    # operators that are not commutative over chunks of 64 KiB and more: blocks of eight tiles are
+    # turned over in LDS so that a lane combines a stretch in order; lengths around the block size
+    # (1024 Int64), chunks that end in single tiles and ragged ones, several rows
+    knobs("fold_staged", staged)
+    rng = np.random.default_rng(33)
+    I = A.i64
+    last = A.lam([I, I], lambda p, q: A.cond(A.neq(I, q, A.constI(0)), q, p))
+    t2 = A.ttup(I, I)
+    ends = A.lam([t2, t2], lambda p, q: A.tup(A.untup(p)[0], A.untup(q)[1]))
+    for rank, shape in [(1, (8192,)), (1, (32768,)), (1, (32769,)), (1, (100_003,)), (1, ((1 << 21) + 77,)), (2, (3, 40_000)),
+                        (2, (2, 1 << 19))]:
+        x = rng.integers(1, 1 << 40, shape).astype(np.int64)
+        x[rng.random(shape) < 0.9] = 0
+        n = shape[-1]
+        idx = np.where(x != 0, np.arange(n), -1).max(axis=-1)
+        want = np.where(idx >= 0, np.take_along_axis(x, np.maximum(idx, 0)[..., None], axis=-1)[..., 0], 0)
+        got = gpu_ctx.compile(A.alam([A.tarray(rank, I)], lambda xs: A.fold(last, A.constI(0), xs)))(x)
+        assert np.array_equal(got, want), shape
+        y = rng.integers(-1000, 1000, shape).astype(np.int64)
+        a, b = gpu_ctx.compile(A.alam([A.tarray(rank, t2)], lambda xs: A.fold(ends, None, xs)))(
+            gpu_ctx.to_device((x, y), A.tarray(rank, t2)))
+        assert np.array_equal(a, x[..., 0]) and np.array_equal(b, y[..., -1]), shape
+
+
 @pytest.mark.parametrize("one_launch", [0, 1])
 def test_single_row_with_and_without_the_second_launch(gpu_ctx, knobs, one_launch):
     # a single row cut into chunks: either a second launch combines the chunk results, or the
