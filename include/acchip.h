@@ -130,6 +130,7 @@ int acchip_set_clean_hook(acchip_ctx* ctx, acchip_clean_fn fn, void* user);
  * compiled afterwards), scan_tiles (0 automatic, 1 large, 2 small, 3 rows, 4 pipelined), scan_spin_limit,
  * scan_test_skew, scan_ticketless (0: the tiles of a scan always take their numbers from the counter),
  * scan_post (0: the function of a map around a scan is never applied by the scan itself; read by acchip_compile),
+ * fold_staged (0: folds under operators that are not commutative never stage blocks of tiles in LDS),
  * fold_one_launch and foldseg_one_launch (0: the work that rides behind the main launch
  * takes a launch of its own), pool_async (0: plain hipMalloc / hipFree under the pool).  Fails for a name
  * it does not know.  No counterpart in the reference. */
