@@ -1,0 +1,129 @@
+"""Folds, scans, segmented folds, transpositions and histograms over shapes drawn at random around
+the sizes where the kernels change their ways (powers of two and tile sizes, give or take a few
+elements; one row, a few rows, very many short ones), under launch-time choices drawn at random
+too, against numpy.  Integer data, so every result is exact.  ACCHIP_RANDOM_SHAPES sets the
+number of draws (default 300), ACCHIP_RANDOM_MOST the size of the largest array."""
+from __future__ import annotations
+
+import os
+
+import numpy as np
+import pytest
+
+from accelerate_amd import ir as A
+from accelerate_amd import programs as P
+
+from . import progs as Q
+
+pytestmark = pytest.mark.gpu
+
+I64, I32 = A.i64, A.i32
+DRAWS = int(os.environ.get("ACCHIP_RANDOM_SHAPES", "300"))
+MOST = int(os.environ.get("ACCHIP_RANDOM_MOST", str(1 << 22)))   # elements of the largest array drawn
+
+
+def _length(rng, most):
+    base = int(2 ** (np.log2(most) * rng.uniform(0, 1) ** 0.5))   # more long than short
+    if rng.random() < 0.6:
+        base = 1 << int(round(np.log2(max(base, 1))))          # a power of two ...
+        if rng.random() < 0.3:
+            base = base // 4 * 7 // 2 or 1                     # ... or 7/8 of one (tiles of 112 bytes per lane)
+    return max(1, min(most, base + int(rng.integers(-3, 4))))
+
+
+def _shape(rng, most=MOST):
+    kind = rng.integers(0, 4)
+    if kind == 0:
+        return (_length(rng, most),)
+    n = _length(rng, most if kind == 1 else 1 << 12)
+    rows = _length(rng, max(1, most // n))
+    if kind == 3 and rows * n * 4 <= most:
+        return (int(rng.integers(1, 5)), rows, n)
+    return (rows, n)
+
+
+_last = A.lam([I64, I64], lambda p, q: A.cond(A.neq(I64, q, A.constI(0)), q, p))
+KNOBS = {"scan_tiles": [0, 0, 0, 1, 2, 3, 4], "fold_rows": [-1, -1, -1, 0, 1, 2], "scan_ticketless": [1, 1, 0],
+         "fold_staged": [1, 1, 0], "fold_one_launch": [1, 1, 0], "fold_target": [2048, 2048, 64, 7]}
+
+
+def _last_nonzero(x):
+    n = x.shape[-1]
+    idx = np.where(x != 0, np.arange(n), -1).max(axis=-1)
+    return np.where(idx >= 0, np.take_along_axis(x, np.maximum(idx, 0)[..., None], axis=-1)[..., 0], 0)
+
+
+def _running_last_nonzero(x):
+    n = x.shape[-1]
+    idx = np.maximum.accumulate(np.where(x != 0, np.arange(n), -1), axis=-1)
+    return np.where(idx >= 0, np.take_along_axis(x, np.maximum(idx, 0), axis=-1), 0)
+
+
+def test_shapes_and_launch_choices_drawn_at_random(gpu_ctx, knobs):
+    rng = np.random.default_rng(20240613)
+    progs = {}
+
+    def prog(key, make):
+        if key not in progs:
+            progs[key] = gpu_ctx.compile(make())
+        return progs[key]
+
+    for draw in range(DRAWS):
+        setting = {k: int(rng.choice(v)) for k, v in KNOBS.items()}
+        for k, v in setting.items():
+            knobs(k, v)
+        shape = _shape(rng)
+        rank = len(shape)
+        if setting["scan_tiles"] in (1, 4) and int(np.prod(shape[:-1])) > (1 << 21):
+            knobs("scan_tiles", 0)   # a 1024-thread workgroup per row: more threads than one launch holds (refused)
+        what = ["fold", "fold_last", "scanl1", "scanl", "scanr_prime", "scan_last", "transpose", "histogram", "foldseg"][rng.integers(0, 9)]
+        where = (draw, what, shape, setting)
+        x = rng.integers(-1000, 1000, shape).astype(np.int64)
+        if what == "fold":
+            got = prog(("fold", rank), lambda: P.fold_sum(I64, rank, 5))(x)
+            assert np.array_equal(got, 5 + x.sum(axis=-1)), where
+        elif what == "fold_last":
+            x[rng.random(shape) < 0.8] = 0
+            got = prog(("fold_last", rank), lambda: A.alam([A.tarray(rank, I64)], lambda xs: A.fold(_last, A.constI(0), xs)))(x)
+            assert np.array_equal(got, _last_nonzero(x)), where
+        elif what == "scanl1":
+            got = prog(("scanl1", rank), lambda: P.scanl1_sum(I64, rank))(x)
+            assert np.array_equal(got, np.cumsum(x, axis=-1)), where
+        elif what == "scanl":
+            x32 = x.astype(np.int32)
+            got = prog(("scanl", rank), lambda: P.scan_sum("l", I32, rank, 3))(x32)
+            want = np.concatenate([np.full(shape[:-1] + (1,), 3), 3 + np.cumsum(x, axis=-1)], axis=-1).astype(np.int32)
+            assert np.array_equal(got, want), where
+        elif what == "scanr_prime":
+            body, total = prog(("scanr'", rank), lambda: P.scan_prime_sum("r", I64, rank, 1))(x)
+            inc = 1 + np.cumsum(x[..., ::-1], axis=-1)[..., ::-1]
+            want = np.concatenate([inc[..., 1:], np.full(shape[:-1] + (1,), 1)], axis=-1)
+            assert np.array_equal(body, want) and np.array_equal(total, inc[..., 0]), where
+        elif what == "scan_last":
+            x[rng.random(shape) < 0.9] = 0
+            got = prog(("scan_last", rank), lambda: A.alam([A.tarray(rank, I64)], lambda xs: A.scan("l", _last, None, xs)))(x)
+            assert np.array_equal(got, _running_last_nonzero(x)), where
+        elif what == "transpose":
+            if rank != 2:
+                continue
+            got = prog(("transpose",), lambda: Q.transpose(I64))(x)
+            assert np.array_equal(got, x.T), where
+        elif what == "histogram":
+            # sums into nbins elements (sizes that are set when the program runs); a negative target drops its source
+            nbins = _length(rng, 1 << 18)
+            to = rng.integers(-1, nbins, shape)
+            dfl = rng.integers(-5, 5, nbins).astype(np.int64)
+            got = prog(("accumulate", rank), lambda: Q.accumulate(I64, rank, 1))(x, to.reshape(-1), dfl)
+            want = dfl.copy()
+            np.add.at(want, to[to >= 0], x[to >= 0])
+            assert np.array_equal(got, want), where + (nbins,)
+        else:
+            n = shape[-1]
+            cuts = np.sort(rng.integers(0, n + 1, int(rng.integers(0, max(1, min(n, 5000))))))
+            lens = np.diff(np.concatenate([[0], cuts, [n]])).astype(np.int32)        # empty segments included
+            x32 = x.astype(np.int32)
+            got = prog(("foldseg", rank), lambda: P.foldseg_sum(I32, I32, rank, 2))(x32, lens)
+            ends = np.cumsum(lens)
+            cs = np.concatenate([np.zeros(shape[:-1] + (1,), np.int64), np.cumsum(x, axis=-1)], axis=-1)
+            want = (2 + cs[..., ends] - cs[..., ends - lens]).astype(np.int32)
+            assert np.array_equal(got, want), where
