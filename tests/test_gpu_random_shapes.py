@@ -127,3 +127,50 @@ def test_shapes_and_launch_choices_drawn_at_random(gpu_ctx, knobs):
             cs = np.concatenate([np.zeros(shape[:-1] + (1,), np.int64), np.cumsum(x, axis=-1)], axis=-1)
             want = (2 + cs[..., ends] - cs[..., ends - lens]).astype(np.int32)
             assert np.array_equal(got, want), where
+
+
+def _weighted_reference(x, widths, mode, fill):
+    """numpy restatement of progs.stencil_weighted: tap number k (1-based, the outermost component
+    of the stencil walking the slowest index) weighs k"""
+    rank = x.ndim
+    halo = [w // 2 for w in widths]
+    pad = [(h, h) for h in halo]
+    if mode == "constant":
+        xp = np.pad(x, pad, mode="constant", constant_values=fill)
+    else:
+        xp = np.pad(x, pad, mode={"clamp": "edge", "mirror": "reflect", "wrap": "wrap"}[mode])
+    out = np.zeros_like(x)
+    k = 0
+    for offs in np.ndindex(*widths):
+        k += 1
+        sl = tuple(slice(o, o + n) for o, n in zip(offs, x.shape))
+        out += k * xp[sl]
+    return out
+
+
+def test_stencil_shapes_drawn_at_random(gpu_ctx, knobs):
+    # rank 2 (tiles in LDS) and rank 3 (a ring of planes in LDS) with every boundary condition, on
+    # extents from a single row or plane up to several tiles, mirrored and wrapped halos included
+    # (np.pad needs an extent of at least 2 to mirror)
+    rng = np.random.default_rng(20240614)
+    progs = {}
+    for draw in range(max(20, DRAWS // 5)):
+        rank = int(rng.integers(2, 4))
+        mode = ["clamp", "mirror", "wrap", "constant"][rng.integers(0, 4)]
+        widths = [3] * rank if rng.random() < 0.7 else ([5, 3] if rank == 2 else [3, 5, 3])
+        most = 1 << (21 if rank == 2 else 20)
+        shape = []
+        left = most
+        for d in range(rank):
+            n = max(widths[d] // 2 + 1, _length(rng, max(2, min(left, 3000 if d else 600))))
+            shape.append(n)
+            left = max(2, left // n)
+        shape = tuple(shape)
+        knobs("stencil_chain", int(rng.choice([0, 0, 1, 3])))
+        key = (rank, mode, tuple(widths))
+        if key not in progs:
+            b = A.constant(I64, 7) if mode == "constant" else mode
+            progs[key] = gpu_ctx.compile(Q.stencil_weighted(I64, widths, b))
+        x = rng.integers(-100, 100, shape).astype(np.int64)
+        got = progs[key](x)
+        assert np.array_equal(got, _weighted_reference(x, widths, mode, 7)), (draw, shape, mode, widths)
