@@ -174,3 +174,93 @@ def test_stencil_shapes_drawn_at_random(gpu_ctx, knobs):
         x = rng.integers(-100, 100, shape).astype(np.int64)
         got = progs[key](x)
         assert np.array_equal(got, _weighted_reference(x, widths, mode, 7)), (draw, shape, mode, widths)
+
+
+def _merge_two_smallest():
+    """permute with Issue137's merge into given defaults: an element ends as the two smallest of
+    the values sent to it and its own two (needs the lock: no component stands alone)"""
+    t2 = A.ttup(I64, I64)
+    sh1 = A.tshape(1)
+    big = A.const(I64, 1 << 40)
+
+    def comb(p, q):
+        a1, a2 = A.untup(p)
+        b1, b2 = A.untup(q)
+        return A.cond(A.lte(I64, a1, b1), A.tup(a1, A.min_(I64, a2, b1)), A.tup(b1, A.min_(I64, b2, a1)))
+
+    def body(xs, to, dfl):
+        src = A.delayed(A.tarray(1, t2), A.shape(xs), A.lam([sh1], lambda ix: A.tup(A.index(xs, A.vexp(ix)), big)),
+                        A.lam([A.Int], lambda i: A.tup(A.linearindex(xs, i), big)))
+        tgt = lambda ix: A.cond(A.lt(A.Int, A.index(to, A.vexp(ix)), A.constI(0)), A.nothing(sh1),
+                                A.just(A.sh(A.index(to, A.vexp(ix)))))
+        return A.permute(A.lam([t2, t2], comb), dfl, A.lam([sh1], tgt), src)
+
+    return A.alam([A.tarray(1, I64), A.tarray(1, A.Int), A.tarray(1, t2)], body)
+
+
+def test_permutes_of_every_kind_over_sizes_drawn_at_random(gpu_ctx, knobs):
+    # one hardware atomic (sum), a compare-and-swap loop (product), one atomic per component (sum
+    # and maximum of pairs), the lock (two smallest): sources from a handful to millions, destinations
+    # from one element to more than the private copies take, some sources dropped, some elements popular
+    rng = np.random.default_rng(20240615)
+    sh1 = A.tshape(1)
+    t2 = A.ttup(I64, I64)
+    drop = lambda to: lambda ix: A.cond(A.lt(A.Int, A.index(to, A.vexp(ix)), A.constI(0)), A.nothing(sh1),
+                                       A.just(A.sh(A.index(to, A.vexp(ix)))))
+    scalar = lambda op: A.alam([A.tarray(1, I64), A.tarray(1, A.Int), A.tarray(1, I64)], lambda xs, to, dfl: A.permute(
+        Q.binop(op, I64), dfl, A.lam([sh1], drop(to)), xs))
+    sum_max = A.alam([A.tarray(1, t2), A.tarray(1, A.Int), A.tarray(1, t2)], lambda xs, to, dfl: A.permute(
+        A.lam([t2, t2], lambda p, q: A.tup(A.add(I64, A.untup(p)[0], A.untup(q)[0]), A.max_(I64, A.untup(p)[1], A.untup(q)[1]))),
+        dfl, A.lam([sh1], drop(to)), xs))
+    progs = {"sum": gpu_ctx.compile(scalar(A.add)), "product": gpu_ctx.compile(scalar(A.mul)),
+             "sum_max": gpu_ctx.compile(sum_max), "two_smallest": gpu_ctx.compile(_merge_two_smallest())}
+    for draw in range(max(20, DRAWS // 3)):
+        what = list(progs)[rng.integers(0, 4)]
+        n = _length(rng, 1 << 21)
+        nbins = _length(rng, 1 << 19)
+        parts = int(rng.choice([128, 128, 128, 2, 0]))
+        knobs("permute_parts", parts)
+        to = rng.integers(-1, nbins, n)
+        if rng.random() < 0.5:
+            # a popular element: a fifth of the sources -- a couple of thousand where they take turns at
+            # a lock or a compare-and-swap loop in memory (no private copies: few sources, a large
+            # destination, or the copies switched off)
+            share = 0.2
+            if what in ("two_smallest", "product") and (parts != 128 or nbins > 100_000 or n < (1 << 20)):
+                share = min(share, 2000 / n)
+            to[rng.random(n) < share] = int(rng.integers(0, nbins))
+        keep = to >= 0
+        where = (draw, what, n, nbins)
+        if what == "sum":
+            x = rng.integers(-1000, 1000, n).astype(np.int64)
+            dfl = rng.integers(-5, 5, nbins).astype(np.int64)
+            want = dfl.copy()
+            np.add.at(want, to[keep], x[keep])
+            assert np.array_equal(progs[what](x, to, dfl), want), where
+        elif what == "product":
+            x = rng.integers(0, 1 << 62, n, dtype=np.int64) | 1
+            dfl = rng.integers(1, 1000, nbins).astype(np.int64)
+            want = dfl.astype(np.uint64)
+            np.multiply.at(want, to[keep], x[keep].astype(np.uint64))
+            assert np.array_equal(progs[what](x, to, dfl).astype(np.uint64), want), where
+        elif what == "sum_max":
+            x = rng.integers(-1000, 1000, n).astype(np.int64)
+            y = rng.integers(-1000, 1000, n).astype(np.int64)
+            d0 = rng.integers(-5, 5, nbins).astype(np.int64)
+            d1 = rng.integers(-1000, 1000, nbins).astype(np.int64)
+            w0, w1 = d0.copy(), d1.copy()
+            np.add.at(w0, to[keep], x[keep])
+            np.maximum.at(w1, to[keep], y[keep])
+            a, b = progs[what](gpu_ctx.to_device((x, y), A.tarray(1, t2)), to, gpu_ctx.to_device((d0, d1), A.tarray(1, t2)))
+            assert np.array_equal(a, w0) and np.array_equal(b, w1), where
+        else:
+            x = rng.integers(0, 1 << 30, n, dtype=np.int64)
+            d0 = rng.integers(0, 1 << 31, nbins, dtype=np.int64)
+            d1 = d0 + rng.integers(0, 1 << 31, nbins, dtype=np.int64)        # a pair is (smallest, second smallest)
+            vals = np.concatenate([x[keep], d0, d1])
+            bins = np.concatenate([to[keep], np.arange(nbins), np.arange(nbins)])
+            order = np.lexsort((vals, bins))
+            vs, bs = vals[order], bins[order]
+            first = np.searchsorted(bs, np.arange(nbins))
+            a, b = progs[what](x, to, gpu_ctx.to_device((d0, d1), A.tarray(1, t2)))
+            assert np.array_equal(a, vs[first]) and np.array_equal(b, vs[first + 1]), where
