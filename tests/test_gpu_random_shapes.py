@@ -264,3 +264,66 @@ def test_permutes_of_every_kind_over_sizes_drawn_at_random(gpu_ctx, knobs):
             first = np.searchsorted(bs, np.arange(nbins))
             a, b = progs[what](x, to, gpu_ctx.to_device((d0, d1), A.tarray(1, t2)))
             assert np.array_equal(a, vs[first]) and np.array_equal(b, vs[first + 1]), where
+
+
+def test_scans_with_producers_and_epilogues_over_shapes_drawn_at_random(gpu_ctx, knobs):
+    # a producer fused into the scan (of one array: it may ride in the pipelined kernel; of two: it
+    # may not), a function applied to the results as they are stored, pairs as elements, right scans
+    rng = np.random.default_rng(20240616)
+    t2 = A.ttup(I64, I64)
+    progs = {}
+
+    def fused(rank, two):
+        shr = A.tshape(rank)
+        g = (lambda v, u: A.add(I64, v, u)) if two else (lambda v: A.add(I64, A.mul(I64, v, A.const(I64, 2)), A.const(I64, 1)))
+
+        def body(a, *more):
+            at = lambda ix: g(A.index(a, A.vexp(ix)), *[A.index(m, A.vexp(ix)) for m in more])
+            lin = lambda i: g(A.linearindex(a, i), *[A.linearindex(m, i) for m in more])
+            return A.scan("l", P._binop(A.add, I64), None, A.delayed(A.tarray(rank, I64), A.shape(a), A.lam([shr], at), A.lam([A.Int], lin)))
+        return A.alam([A.tarray(rank, I64)] * (2 if two else 1), body)
+
+    def pairs(rank, direction):
+        f = A.lam([t2, t2], lambda p, q: A.tup(A.add(I64, A.untup(p)[0], A.untup(q)[0]), A.max_(I64, A.untup(p)[1], A.untup(q)[1])))
+        return A.alam([A.tarray(rank, t2)], lambda xs: A.scan(direction, f, None, xs))
+
+    def halved(rank):
+        g = A.lam([I64], lambda v: A.sub(I32, A.fromintegral(I64, I32, v), A.const(I32, 1)))
+        return A.alam([A.tarray(rank, I64)], lambda xs: A.map_(I32, g, A.scan("r", P._binop(A.add, I64), A.const(I64, 2), xs)))
+
+    def prog(key, make):
+        if key not in progs:
+            progs[key] = gpu_ctx.compile(make())
+        return progs[key]
+
+    for draw in range(max(20, DRAWS // 3)):
+        tiles = int(rng.choice([0, 0, 0, 1, 2, 3, 4]))
+        shape = _shape(rng)
+        if len(shape) == 3:
+            shape = shape[1:]
+        rank = len(shape)
+        if tiles in (1, 4) and int(np.prod(shape[:-1])) > (1 << 21):
+            tiles = 0
+        knobs("scan_tiles", tiles)
+        knobs("scan_post", int(rng.choice([1, 1, 0])))
+        what = ["fused1", "fused2", "pairs_l", "pairs_r", "halved"][rng.integers(0, 5)]
+        where = (draw, what, shape, tiles)
+        x = rng.integers(-1000, 1000, shape).astype(np.int64)
+        y = rng.integers(-1000, 1000, shape).astype(np.int64)
+        if what == "fused1":
+            assert np.array_equal(prog((what, rank), lambda: fused(rank, False))(x), np.cumsum(2 * x + 1, axis=-1)), where
+        elif what == "fused2":
+            assert np.array_equal(prog((what, rank), lambda: fused(rank, True))(x, y), np.cumsum(x + y, axis=-1)), where
+        elif what in ("pairs_l", "pairs_r"):
+            d = what[-1]
+            a, b = prog((what, rank), lambda: pairs(rank, d))(gpu_ctx.to_device((x, y), A.tarray(rank, t2)))
+            if d == "l":
+                wa, wb = np.cumsum(x, axis=-1), np.maximum.accumulate(y, axis=-1)
+            else:
+                wa = np.cumsum(x[..., ::-1], axis=-1)[..., ::-1]
+                wb = np.maximum.accumulate(y[..., ::-1], axis=-1)[..., ::-1]
+            assert np.array_equal(a, wa) and np.array_equal(b, wb), where
+        else:
+            inc = 2 + np.cumsum(x[..., ::-1], axis=-1)[..., ::-1]
+            want = np.concatenate([inc, np.full(shape[:-1] + (1,), 2)], axis=-1).astype(np.int32) - np.int32(1)
+            assert np.array_equal(prog((what, rank), lambda: halved(rank))(x), want), where
