@@ -327,3 +327,30 @@ def test_scans_with_producers_and_epilogues_over_shapes_drawn_at_random(gpu_ctx,
             inc = 2 + np.cumsum(x[..., ::-1], axis=-1)[..., ::-1]
             want = np.concatenate([inc, np.full(shape[:-1] + (1,), 2)], axis=-1).astype(np.int32) - np.int32(1)
             assert np.array_equal(prog((what, rank), lambda: halved(rank))(x), want), where
+
+
+def test_axis_permutations_over_extents_drawn_at_random(gpu_ctx, knobs):
+    # transpositions of matrices and the six orders of the dimensions of rank 3, extents from 1 to
+    # a few thousand: tiles of the plane of the two dimensions involved, ragged on every side
+    rng = np.random.default_rng(20240617)
+    perms = [(0, 2, 1), (1, 0, 2), (2, 1, 0), (1, 2, 0), (2, 0, 1)]
+    progs = {}
+    for draw in range(max(20, DRAWS // 3)):
+        knobs("map_tiled", int(rng.choice([-1, -1, -1, 0, 1])))
+        if rng.random() < 0.4:
+            shape = (_length(rng, 5000), _length(rng, 5000))
+            while shape[0] * shape[1] > (1 << 22):
+                shape = (shape[0] // 2 + 1, shape[1])
+            x = rng.integers(-1000, 1000, shape).astype(np.int64)
+            if "t" not in progs:
+                progs["t"] = gpu_ctx.compile(Q.transpose(I64))
+            assert np.array_equal(progs["t"](x), x.T), (draw, shape)
+            continue
+        pm = perms[rng.integers(0, len(perms))]
+        shape = tuple(_length(rng, 300) for _ in range(3))
+        x = rng.integers(-1000, 1000, shape).astype(np.int32)
+        if pm not in progs:
+            inv = [pm.index(k) for k in range(3)]
+            progs[pm] = gpu_ctx.compile(Q.reindex(3, lambda dd, pm=pm: [dd()[pm[0]], dd()[pm[1]], dd()[pm[2]]],
+                                                  lambda ix, dd, inv=inv: [ix[inv[0]], ix[inv[1]], ix[inv[2]]], I32))
+        assert np.array_equal(progs[pm](x), x.transpose(pm)), (draw, shape, pm)
