@@ -648,3 +648,38 @@ def test_wrong_argument_type_is_rejected(gpu_ctx):
     wrong = gpu_ctx.to_device(np.zeros((2, 2), np.float32), A.tarray(2, A.f32))
     with pytest.raises(hip.AccError):
         run.execute(wrong)
+
+
+def test_separable_blur_of_the_stencil_documentation(gpu_ctx):
+    # Language.hs:912-930: a 5x5 Gaussian blur as two passes whose stencils have rows of different
+    # widths -- Stencil5x1 = (Stencil3, Stencil5, Stencil3) reads only its middle row, Stencil1x5 =
+    # five Stencil3 rows only their middle elements -- under clamp, and under mirror and wrap
+    ty = A.f32
+    kern = [0.06136, 0.24477, 0.38774, 0.24477, 0.06136]
+
+    def conv(ts):
+        acc = A.mul(ty, A.const(ty, kern[0]), ts[0])
+        for w, t in zip(kern[1:], ts[1:]):
+            acc = A.add(ty, acc, A.mul(ty, A.const(ty, w), t))
+        return acc
+
+    def blur5x1(b):
+        sr = A.stup(A.sunit(3, ty), A.sunit(5, ty), A.sunit(3, ty))
+        return A.alam([A.tarray(2, ty)], lambda g: A.stencil(
+            sr, ty, A.lam([A.stencil_type(sr)], lambda st: conv(A.untup(A.untup(st)[1]))), b, g))
+
+    def blur1x5(b):
+        sr = A.stup(*[A.sunit(3, ty) for _ in range(5)])
+        return A.alam([A.tarray(2, ty)], lambda g: A.stencil(
+            sr, ty, A.lam([A.stencil_type(sr)], lambda st: conv([A.untup(r)[1] for r in A.untup(st)])), b, g))
+
+    rng = np.random.default_rng(44)
+    for shape in ((7, 9), (300, 517), (3, 40), (40, 3)):
+        x = rng.random(shape, dtype=np.float32)
+        for b in (A.clamp, A.mirror, A.wrap):
+            for prog in (blur5x1(b), blur1x5(b)):
+                assert same(gpu_ctx.compile(prog)(x), O.run_n(prog.text(), x)), (shape, b)
+    # blur = stencil (convolve5x1 gaussian) clamp . stencil (convolve1x5 gaussian) clamp
+    both = A.alam([A.tarray(2, ty)], lambda g: A.apply(blur5x1(A.clamp), A.apply(blur1x5(A.clamp), g)))
+    x = rng.random((64, 70), dtype=np.float32)
+    assert same(gpu_ctx.compile(both)(x), O.run_n(both.text(), x))
