@@ -344,3 +344,20 @@ def test_float_maximum_through_private_copies(gpu_ctx, nbins):
     want = dfl.copy()
     np.maximum.at(want, to, x)
     assert np.array_equal(gpu_ctx.compile(_combine_prog(A.max_, A.f32))(x, to, dfl), want)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("order", ["waits", "fences"])
+def test_locks_in_memory_under_contention(gpu_ctx, knobs, monkeypatch, order):
+    # the private copies switched off: 2^20 sources take turns at the locks of 512 elements (two thousand
+    # each), then of 3 -- every update must see the one before it, whichever way the lock is ordered
+    if order == "fences":
+        monkeypatch.setenv("ACCHIP_LOCK_ORDER", "fences")
+    knobs("permute_parts", 0)
+    rng = np.random.default_rng(99)
+    for n, nbins in ((1 << 20, 512), (1 << 16, 3)):
+        x = rng.integers(0, 1 << 30, n, dtype=np.int64)
+        to = rng.integers(0, nbins, n, dtype=np.int64)
+        a, b = gpu_ctx.compile(_two_smallest(nbins))(x, to)
+        m1, m2 = _two_smallest_ref(x, to, nbins, 1 << 40)
+        assert np.array_equal(a, m1) and np.array_equal(b, m2), (n, nbins)
