@@ -2,7 +2,8 @@
 the sizes where the kernels change their ways (powers of two and tile sizes, give or take a few
 elements; one row, a few rows, very many short ones), under launch-time choices drawn at random
 too, against numpy.  Integer data, so every result is exact.  ACCHIP_RANDOM_SHAPES sets the
-number of draws (default 300), ACCHIP_RANDOM_MOST the size of the largest array."""
+number of draws (default 300), ACCHIP_RANDOM_MOST the size of the largest array, ACCHIP_RANDOM_SEED
+another sequence."""
 from __future__ import annotations
 
 import os
@@ -20,6 +21,7 @@ pytestmark = pytest.mark.gpu
 I64, I32 = A.i64, A.i32
 DRAWS = int(os.environ.get("ACCHIP_RANDOM_SHAPES", "300"))
 MOST = int(os.environ.get("ACCHIP_RANDOM_MOST", str(1 << 22)))   # elements of the largest array drawn
+SEED = int(os.environ.get("ACCHIP_RANDOM_SEED", "0"))             # added to every test's seed
 
 
 def _length(rng, most):
@@ -60,7 +62,7 @@ def _running_last_nonzero(x):
 
 
 def test_shapes_and_launch_choices_drawn_at_random(gpu_ctx, knobs):
-    rng = np.random.default_rng(20240613)
+    rng = np.random.default_rng(20240613 + SEED)
     progs = {}
 
     def prog(key, make):
@@ -152,7 +154,7 @@ def test_stencil_shapes_drawn_at_random(gpu_ctx, knobs):
     # rank 2 (tiles in LDS) and rank 3 (a ring of planes in LDS) with every boundary condition, on
     # extents from a single row or plane up to several tiles, mirrored and wrapped halos included
     # (np.pad needs an extent of at least 2 to mirror)
-    rng = np.random.default_rng(20240614)
+    rng = np.random.default_rng(20240614 + SEED)
     progs = {}
     for draw in range(max(20, DRAWS // 5)):
         rank = int(rng.integers(2, 4))
@@ -202,7 +204,7 @@ def test_permutes_of_every_kind_over_sizes_drawn_at_random(gpu_ctx, knobs):
     # one hardware atomic (sum), a compare-and-swap loop (product), one atomic per component (sum
     # and maximum of pairs), the lock (two smallest): sources from a handful to millions, destinations
     # from one element to more than the private copies take, some sources dropped, some elements popular
-    rng = np.random.default_rng(20240615)
+    rng = np.random.default_rng(20240615 + SEED)
     sh1 = A.tshape(1)
     t2 = A.ttup(I64, I64)
     drop = lambda to: lambda ix: A.cond(A.lt(A.Int, A.index(to, A.vexp(ix)), A.constI(0)), A.nothing(sh1),
@@ -219,6 +221,8 @@ def test_permutes_of_every_kind_over_sizes_drawn_at_random(gpu_ctx, knobs):
         n = _length(rng, 1 << 21)
         nbins = _length(rng, 1 << 19)
         parts = int(rng.choice([128, 128, 128, 2, 0]))
+        if what in ("two_smallest", "product") and n > 3000 * nbins:
+            parts = 128   # (without the private copies these sources would take turns in memory: thousands per element, 20 µs a turn)
         knobs("permute_parts", parts)
         to = rng.integers(-1, nbins, n)
         if rng.random() < 0.5:
@@ -269,7 +273,7 @@ def test_permutes_of_every_kind_over_sizes_drawn_at_random(gpu_ctx, knobs):
 def test_scans_with_producers_and_epilogues_over_shapes_drawn_at_random(gpu_ctx, knobs):
     # a producer fused into the scan (of one array: it may ride in the pipelined kernel; of two: it
     # may not), a function applied to the results as they are stored, pairs as elements, right scans
-    rng = np.random.default_rng(20240616)
+    rng = np.random.default_rng(20240616 + SEED)
     t2 = A.ttup(I64, I64)
     progs = {}
 
@@ -332,7 +336,7 @@ def test_scans_with_producers_and_epilogues_over_shapes_drawn_at_random(gpu_ctx,
 def test_axis_permutations_over_extents_drawn_at_random(gpu_ctx, knobs):
     # transpositions of matrices and the six orders of the dimensions of rank 3, extents from 1 to
     # a few thousand: tiles of the plane of the two dimensions involved, ragged on every side
-    rng = np.random.default_rng(20240617)
+    rng = np.random.default_rng(20240617 + SEED)
     perms = [(0, 2, 1), (1, 0, 2), (2, 1, 0), (1, 2, 0), (2, 0, 1)]
     progs = {}
     for draw in range(max(20, DRAWS // 3)):
