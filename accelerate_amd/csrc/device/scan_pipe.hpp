@@ -161,6 +161,10 @@ ACC_DEV void acc_window_wide(const typename S::Env& env, const u64* rowDesc, i64
   }
 }
 
+#ifndef ACC_PIPE_EXCL
+#define ACC_PIPE_EXCL 1  // 0: scanl / scanl' store their running values one position on (stores off the 16-byte grid)
+#endif
+
 extern "C" __global__ void __launch_bounds__(ACC_SCAN_BLOCK, ACC_SCAN_MINWAVES)
 acc_scan_pipe(Spec::Env env, Spec::Out out, Spec::Out tot, ScanParams p) {
   typedef Spec S;
@@ -191,6 +195,8 @@ acc_scan_pipe(Spec::Env env, Spec::Out out, Spec::Out tot, ScanParams p) {
   // the polling one when the rake area has LDS of its own); the others after the prefixes have
   // been read back.  Sending them before the aggregate is out delays every successor's look-back
   // (Float32, 112 B per lane: 409 us against 353).
+  // left scans with a seed store each lane's results on the 16-byte grid (see where yprev is filled)
+  constexpr bool kExcl = ACC_PIPE_EXCL && !S::kRight && S::kKind != 0;
   constexpr int kRakeBytes = (int)sizeof(Elt) * (G + 1) * ACC_SCAN_BLOCK;
   constexpr int kFirstEarly = kSep ? 1 : (ACC_PIPE_EARLY ? (kRakeBytes + G * 1024 - 1) / (G * 1024) : NW);
 
@@ -332,11 +338,15 @@ acc_scan_pipe(Spec::Env env, Spec::Out out, Spec::Out tot, ScanParams p) {
     if (early && w != 0 && nextLoaded) sendLoads(nxt);
     if (hasPrev && w != 0) storePrev(0, S1);
     acc_lds_barrier();
+    // (left scans with a seed write what lies before each position: the value in front of a lane's
+    // run is this prefix, kept so that the run can be stored on the 16-byte grid, see below)
+    Elt runPre[kExcl ? C::G : 1];
 #pragma unroll
     for (int g = 0; g < G; ++g) {
       const int e = g * ACC_SCAN_BLOCK + tid;
       if (e > 0) {
         const Elt pre = rk[(e / G) * (G + 1) + e % G];
+        if (kExcl) runPre[g] = pre;
 #pragma unroll
         for (int k = 0; k < V; ++k) x[g][k] = S::combine(env, pre, x[g][k]);
       }
@@ -395,7 +405,26 @@ acc_scan_pipe(Spec::Env env, Spec::Out out, Spec::Out tot, ScanParams p) {
     // final values: kept for the next iteration, or written now where a position needs a test
     const i64 shift = S::kKind == 0 ? 0 : 1;
     const bool deferable = S::kKind != 2 || tile + 1 < p.tpr;  // scan' keeps the row's total apart
-    if (deferable) {
+    if (deferable && kExcl) {
+      // scanl / scanl': result u is everything before element u.  A lane's run of results is then
+      // (what lies before its run, its first V - 1 running values) at the positions of its elements,
+      // which are on the 16-byte grid; stored one position on, as the running values themselves,
+      // every store straddled two 16-byte words (2^28 Int64: 749 against 714 us for scanl1).  The
+      // base is there: these scans have a seed.
+#pragma unroll
+      for (int g = 0; g < G; ++g) {
+        yprev[g][0] = g * ACC_SCAN_BLOCK + tid > 0 ? S::combine(env, base, runPre[g]) : base;
+#pragma unroll
+        for (int k = 1; k < V; ++k) yprev[g][k] = S::combine(env, base, x[g][k - 1]);
+      }
+      prevOut = outBase + tile * (i64)C::TILE;
+      hasPrev = true;
+      if (tile + 1 == tpf) {
+        // the value behind the row's last full tile: the row's last result, or the first of its partial tile
+        if (tid == ACC_SCAN_BLOCK - 1) S::store(out, outBase + (tile + 1) * (i64)C::TILE, S::combine(env, base, x[G - 1][V - 1]));
+        tailStores = false;
+      }
+    } else if (deferable) {
 #pragma unroll
       for (int g = 0; g < G; ++g)
 #pragma unroll
@@ -403,6 +432,8 @@ acc_scan_pipe(Spec::Env env, Spec::Out out, Spec::Out tot, ScanParams p) {
       prevOut = R ? outBase + m - shift - V - tile * (i64)C::TILE : outBase + tile * (i64)C::TILE + shift;
       hasPrev = true;
     } else {
+      // (the tile before wrote what lies before its own elements: this tile's first result is still missing)
+      if (kExcl && tid == 0) S::store(out, outBase + tile * (i64)C::TILE, base);
 #pragma unroll
       for (int g = 0; g < G; ++g) {
         const i64 t0 = tile * (i64)C::TILE + ((i64)g * ACC_SCAN_BLOCK + tid) * V;
