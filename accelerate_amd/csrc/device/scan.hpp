@@ -332,7 +332,8 @@ ACC_DEV void acc_rake(const typename S::Env& env, typename S::Elt* mine, const t
 // workgroup (ACC_SCAN_BLOCK threads).  When `plain` holds, a tile that lies completely inside
 // the sequence hands the V consecutive values of a lane to storeRun(t0, y) instead, which
 // can move them with one wide request: a caller whose store tests for a special position
-// (the total of scan') sets it for the tiles that cannot hold that position.  `settle` delays
+// (the total of scan', which is the sequence's last value) sets it for the tiles that cannot hold
+// that position; in the tile that can, only the run that reaches the end goes value by value.  `settle` delays
 // the first look at the predecessors (see acc_lookback).
 template <class S, class Load, class Store, class StoreRun>
 ACC_DEV void acc_scan_tile(const typename S::Env& env, u64* desc, i64 tiles, i64 tile, i64 n, u64 epoch, u64 limit,
@@ -499,7 +500,7 @@ ACC_DEV void acc_scan_tile(const typename S::Env& env, u64* desc, i64 tiles, i64
       Elt y[C::V];
 #pragma unroll
       for (int k = 0; k < V; ++k) y[k] = hasBase ? S::combine(env, base, x[g][k]) : x[g][k];
-      if (plain) {
+      if (plain || t0 + V < n) {  // (the special position is the sequence's last)
         storeRun(t0, y);
       } else {
 #pragma unroll
