@@ -404,7 +404,9 @@ acc_scan_pipe(Spec::Env env, Spec::Out out, Spec::Out tot, ScanParams p) {
     const Elt base = sh_excl;
     // final values: kept for the next iteration, or written now where a position needs a test
     const i64 shift = S::kKind == 0 ? 0 : 1;
-    const bool deferable = S::kKind != 2 || tile + 1 < p.tpr;  // scan' keeps the row's total apart
+    // scan' keeps the row's total apart: the tile that holds it stores value by value -- unless the
+    // results go out as `what lies before`, which never touches the position of the total
+    const bool deferable = kExcl || S::kKind != 2 || tile + 1 < p.tpr;
     if (deferable && kExcl) {
       // scanl / scanl': result u is everything before element u.  A lane's run of results is then
       // (what lies before its run, its first V - 1 running values) at the positions of its elements,
@@ -421,7 +423,12 @@ acc_scan_pipe(Spec::Env env, Spec::Out out, Spec::Out tot, ScanParams p) {
       hasPrev = true;
       if (tile + 1 == tpf) {
         // the value behind the row's last full tile: the row's last result, or the first of its partial tile
-        if (tid == ACC_SCAN_BLOCK - 1) S::store(out, outBase + (tile + 1) * (i64)C::TILE, S::combine(env, base, x[G - 1][V - 1]));
+        if (tid == ACC_SCAN_BLOCK - 1) {
+          const Elt behind = S::combine(env, base, x[G - 1][V - 1]);
+          const i64 u = (tile + 1) * (i64)C::TILE;
+          if (S::kKind == 2 && u == n) S::store(tot, row, behind);  // scanl': the row's total
+          else S::store(out, outBase + u, behind);
+        }
         tailStores = false;
       }
     } else if (deferable) {
@@ -432,8 +439,6 @@ acc_scan_pipe(Spec::Env env, Spec::Out out, Spec::Out tot, ScanParams p) {
       prevOut = R ? outBase + m - shift - V - tile * (i64)C::TILE : outBase + tile * (i64)C::TILE + shift;
       hasPrev = true;
     } else {
-      // (the tile before wrote what lies before its own elements: this tile's first result is still missing)
-      if (kExcl && tid == 0) S::store(out, outBase + tile * (i64)C::TILE, base);
 #pragma unroll
       for (int g = 0; g < G; ++g) {
         const i64 t0 = tile * (i64)C::TILE + ((i64)g * ACC_SCAN_BLOCK + tid) * V;
