@@ -162,7 +162,7 @@ ACC_DEV void acc_window_wide(const typename S::Env& env, const u64* rowDesc, i64
 }
 
 #ifndef ACC_PIPE_EXCL
-#define ACC_PIPE_EXCL 1  // 0: scanl / scanl' store their running values one position on (stores off the 16-byte grid)
+#define ACC_PIPE_EXCL 1  // 0: scanl / scanl' / scanr' store their running values one position on (stores off the 16-byte grid)
 #endif
 
 extern "C" __global__ void __launch_bounds__(ACC_SCAN_BLOCK, ACC_SCAN_MINWAVES)
@@ -195,8 +195,9 @@ acc_scan_pipe(Spec::Env env, Spec::Out out, Spec::Out tot, ScanParams p) {
   // the polling one when the rake area has LDS of its own); the others after the prefixes have
   // been read back.  Sending them before the aggregate is out delays every successor's look-back
   // (Float32, 112 B per lane: 409 us against 353).
-  // left scans with a seed store each lane's results on the 16-byte grid (see where yprev is filled)
-  constexpr bool kExcl = ACC_PIPE_EXCL && !S::kRight && S::kKind != 0;
+  // scans whose result u is the running value u - 1 store each lane's results on the 16-byte grid (see where yprev is filled)
+  // (scanr writes its running values at its elements' own positions already; scanr' does not)
+  constexpr bool kExcl = ACC_PIPE_EXCL && S::kKind != 0 && !(S::kRight && S::kKind == 1);
   constexpr int kRakeBytes = (int)sizeof(Elt) * (G + 1) * ACC_SCAN_BLOCK;
   constexpr int kFirstEarly = kSep ? 1 : (ACC_PIPE_EARLY ? (kRakeBytes + G * 1024 - 1) / (G * 1024) : NW);
 
@@ -338,7 +339,7 @@ acc_scan_pipe(Spec::Env env, Spec::Out out, Spec::Out tot, ScanParams p) {
     if (early && w != 0 && nextLoaded) sendLoads(nxt);
     if (hasPrev && w != 0) storePrev(0, S1);
     acc_lds_barrier();
-    // (left scans with a seed write what lies before each position: the value in front of a lane's
+    // (scanl, scanl' and scanr' write what lies before each position: the value in front of a lane's
     // run is this prefix, kept so that the run can be stored on the 16-byte grid, see below)
     Elt runPre[kExcl ? C::G : 1];
 #pragma unroll
@@ -408,7 +409,7 @@ acc_scan_pipe(Spec::Env env, Spec::Out out, Spec::Out tot, ScanParams p) {
     // results go out as `what lies before`, which never touches the position of the total
     const bool deferable = kExcl || S::kKind != 2 || tile + 1 < p.tpr;
     if (deferable && kExcl) {
-      // scanl / scanl': result u is everything before element u.  A lane's run of results is then
+      // scanl / scanl' / scanr': result u is everything before element u (in the scan's direction).  A lane's run of results is then
       // (what lies before its run, its first V - 1 running values) at the positions of its elements,
       // which are on the 16-byte grid; stored one position on, as the running values themselves,
       // every store straddled two 16-byte words (2^28 Int64: 749 against 714 us for scanl1).  The
@@ -419,15 +420,15 @@ acc_scan_pipe(Spec::Env env, Spec::Out out, Spec::Out tot, ScanParams p) {
 #pragma unroll
         for (int k = 1; k < V; ++k) yprev[g][k] = S::combine(env, base, x[g][k - 1]);
       }
-      prevOut = outBase + tile * (i64)C::TILE;
+      prevOut = R ? outBase + m - V - tile * (i64)C::TILE : outBase + tile * (i64)C::TILE;
       hasPrev = true;
       if (tile + 1 == tpf) {
         // the value behind the row's last full tile: the row's last result, or the first of its partial tile
         if (tid == ACC_SCAN_BLOCK - 1) {
           const Elt behind = S::combine(env, base, x[G - 1][V - 1]);
           const i64 u = (tile + 1) * (i64)C::TILE;
-          if (S::kKind == 2 && u == n) S::store(tot, row, behind);  // scanl': the row's total
-          else S::store(out, outBase + u, behind);
+          if (S::kKind == 2 && u == n) S::store(tot, row, behind);  // scanl' / scanr': the row's total
+          else S::store(out, outBase + (R ? m - 1 - u : u), behind);
         }
         tailStores = false;
       }
